@@ -1,0 +1,226 @@
+/*
+ * sparse_hip.h -- C ABI of the MI355X (gfx950) MoE-layer execution path.
+ *
+ * The reference (louislichen/SPARSE) has no FFI: its MoE layer is a Python class
+ * (`DistributedSparseMoeBlock`, utils/eval_core.py:4407-17215) that issues ATen calls.
+ * Each entry point below replaces one run of those ATen calls; the comment on each
+ * names the reference lines it stands in for.  The Python host in `sparse_amd/`
+ * binds them with ctypes; any other host can bind them the same way.
+ *
+ * Conventions
+ *   - Every function returns 0 on success, a negative SPARSE_HIP_E* code otherwise;
+ *     `sparse_hip_last_error()` returns a thread-local message for the last failure.
+ *   - All pointers named *_dev are device (HBM) pointers; *_host are host pointers.
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream).
+ *   - Nothing here allocates device memory or synchronises the host unless its
+ *     comment says so: callers pass workspaces and outputs.  Launches are
+ *     asynchronous with respect to the host and may be captured into a HIP graph.
+ *   - Row-major everywhere.  Weight matrices are [out_features, in_features] as in
+ *     torch.nn.Linear.
+ *   - dtype codes: SPARSE_HIP_F32 = 0, SPARSE_HIP_BF16 = 1.
+ */
+#ifndef SPARSE_HIP_H
+#define SPARSE_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SPARSE_HIP_ABI_VERSION 1
+
+#define SPARSE_HIP_F32 0
+#define SPARSE_HIP_BF16 1
+
+#define SPARSE_HIP_OK 0
+#define SPARSE_HIP_EINVAL (-1)   /* bad argument (shape, dtype, alignment, NULL) */
+#define SPARSE_HIP_ELAUNCH (-2)  /* HIP runtime reported an error */
+#define SPARSE_HIP_ENOTREADY 1   /* event_query: work still in flight (not an error) */
+
+/* Largest expert count / top-k / decode batch the kernels are built for. */
+#define SPARSE_HIP_MAX_EXPERTS 256
+#define SPARSE_HIP_MAX_TOPK 16
+#define SPARSE_HIP_DECODE_MAX_TOKENS 32
+
+/* ---- library identity ------------------------------------------------------ */
+
+/* ABI version of the loaded library (SPARSE_HIP_ABI_VERSION at build time). */
+int sparse_hip_version(void);
+/* Code-object architecture the kernels were built for ("gfx950"). */
+const char* sparse_hip_arch(void);
+/* Message of the last failure on the calling thread ("" if none). */
+const char* sparse_hip_last_error(void);
+
+/* ---- expert weight slab ---------------------------------------------------- */
+
+/*
+ * Where the routed experts of one layer live in HBM.  One slot holds one expert:
+ * gate [I,H], up [I,H], down [H,I], contiguous in that order, `slot_stride` bytes
+ * apart.  `expert_slot_dev[e]` is the slot that currently holds expert e (any value
+ * for experts that are not touched by the call).  An all-resident layer uses the
+ * identity table.  Replaces the per-expert tensors the reference keeps in
+ * `local_gate_cpu/local_up_cpu/local_down_cpu2` and in cache payload tuples
+ * (utils/eval_core.py:5097-5123, :11427-11435).
+ */
+typedef struct sparse_hip_experts {
+  const void* slab_dev;            /* base of slot 0 */
+  uint64_t slot_stride;            /* bytes between slots (>= 3*I*H*elem) */
+  const int32_t* expert_slot_dev;  /* [E] expert id -> slot */
+  int32_t num_experts;             /* E */
+  int32_t hidden;                  /* H */
+  int32_t inter;                   /* I */
+  int32_t dtype;                   /* SPARSE_HIP_F32 | SPARSE_HIP_BF16 */
+} sparse_hip_experts;
+
+/*
+ * Which expert segments one launch executes, in launch order.  If `eids_dev` is
+ * non-NULL the list is read on the device: `eids_dev[0 .. *count_dev)` with at most
+ * `n` entries (the grid is sized for n).  Otherwise the first `n` entries of `eids`
+ * are used.  A segment is the run of permuted rows of one expert
+ * (utils/eval_core.py:13240-13262).
+ */
+typedef struct sparse_hip_seglist {
+  const int32_t* eids_dev;
+  const int32_t* count_dev;
+  int32_t n;
+  int16_t eids[SPARSE_HIP_MAX_EXPERTS];
+} sparse_hip_seglist;
+
+/* ---- A1: router ------------------------------------------------------------ */
+
+/*
+ * logits[t,e] = sum_h x[t,h] * wg[e,h], accumulated in fp32 and rounded once to
+ * `logits_dtype` -- `router_logits = self.gate(x)` (utils/eval_core.py:9519) when
+ * logits_dtype == dtype; the DeepSeek gate's fp32 logits when logits_dtype is F32.
+ * If `wsg_dev` is non-NULL also writes shared_gate_dev[t] = sum_h x[t,h]*wsg[h] in
+ * `dtype` -- `self.shared_expert_gate(x)` (utils/eval_core.py:9461).
+ * x [T,H], wg [E,H], wsg [H] in `dtype`.  H % 8 == 0.
+ */
+int sparse_hip_router_logits(const void* x_dev, const void* wg_dev, const void* wsg_dev,
+                             int dtype, int logits_dtype, int T, int H, int E,
+                             void* logits_dev, void* shared_gate_dev, void* stream);
+
+/*
+ * probs = softmax(logits, fp32); (topv, topi) = top-K of probs, descending, ties to
+ * the lower expert id; optional renormalisation topv /= max(sum topv, 1e-12); topv is
+ * rounded to `out_dtype`, topi is int64 -- utils/eval_core.py:9520, :9590-9595.
+ * logits [T,E] in `logits_dtype`; topv [T,K]; topi [T,K].  E <= 256, K <= 16, K <= E.
+ */
+int sparse_hip_gate_topk(const void* logits_dev, int logits_dtype, int T, int E, int K,
+                         int renorm, int out_dtype, void* topv_dev, int64_t* topi_dev,
+                         void* stream);
+
+/* ---- A5: token x K expansion + permutation --------------------------------- */
+
+/*
+ * Stable bucketing of the flat routed items f = t*K + k by expert id:
+ *   perm[p] = f of the p-th item in (expert id, f) order,  inv_perm[f] = p,
+ *   seg_offsets[e] .. seg_offsets[e+1] = rows of expert e (exclusive prefix sum of
+ *   the per-expert counts), active_eids[0 .. *n_active) = ids with >= 1 item,
+ *   ascending.
+ * Stands in for `argsort(flat_i)` + segment scan + `out[order] = out_sorted`
+ * (utils/eval_core.py:14728-14730, :13240-13262, :13359-13360) without host syncs.
+ * topi [T,K] int64 with 0 <= id < E.  Outputs int32: perm [T*K], inv_perm [T*K],
+ * seg_offsets [E+1], active_eids [E], n_active [1].  `ws_dev` is a workspace of
+ * sparse_hip_permute_ws_bytes(T, K, E) bytes.
+ */
+size_t sparse_hip_permute_ws_bytes(int T, int K, int E);
+int sparse_hip_permute_build(const int64_t* topi_dev, int T, int K, int E, int32_t* perm_dev,
+                             int32_t* inv_perm_dev, int32_t* seg_offsets_dev,
+                             int32_t* active_eids_dev, int32_t* n_active_dev, void* ws_dev,
+                             void* stream);
+
+/* ---- A4/A6: grouped SwiGLU expert FFN -------------------------------------- */
+
+/*
+ * For every segment in `segs` (expert e, rows p in [seg_offsets[e], seg_offsets[e+1])):
+ *   cur   = x[perm[p] / K]
+ *   inter = act(gate_e(cur)) * up_e(cur)         (each Linear rounded to dtype, the
+ *                                                 activation and the product too)
+ *   parts[p] = down_e(inter) * topv_flat[perm[p]]  (rounded to dtype twice)
+ * i.e. `_plain_ep_compute_segment` / `_module_expert_forward`
+ * (utils/eval_core.py:11700-11793) over segments, writing rows in permuted order.
+ * Rows of segments that are not in `segs` are left untouched.
+ *
+ * `_decode` is the HBM-bandwidth path: T <= SPARSE_HIP_DECODE_MAX_TOKENS, weights are
+ * streamed once.  `_prefill` is the MFMA grouped-GEMM path for any T (bf16), and the
+ * tiled FMA path for fp32.  Both produce the same rows up to fp32 summation order.
+ * x [T,H]; topv [T,K] in dtype; inter_ws [T*K, I] and parts [T*K, H] in dtype.
+ * H % 64 == 0 and I % 64 == 0.
+ */
+int sparse_hip_grouped_swiglu_decode(const sparse_hip_experts* experts, const void* x_dev,
+                                     const void* topv_dev, const int32_t* perm_dev,
+                                     const int32_t* seg_offsets_dev,
+                                     const sparse_hip_seglist* segs, int T, int K,
+                                     void* inter_ws_dev, void* parts_dev, void* stream);
+int sparse_hip_grouped_swiglu_prefill(const sparse_hip_experts* experts, const void* x_dev,
+                                      const void* topv_dev, const int32_t* perm_dev,
+                                      const int32_t* seg_offsets_dev,
+                                      const sparse_hip_seglist* segs, int T, int K,
+                                      void* inter_ws_dev, void* parts_dev, void* stream);
+
+/* ---- A8: shared expert ----------------------------------------------------- */
+
+/*
+ * shared[t] = down_s(act(gate_s(x[t])) * up_s(x[t])), times
+ * sigmoid(shared_gate[t]) when `shared_gate_dev` is non-NULL (each step rounded to
+ * dtype) -- `_shared_expert_forward` (utils/eval_core.py:9455-9463).
+ * gate_s, up_s [Is,H], down_s [H,Is]; inter_ws [T,Is]; shared [T,H].
+ * Uses the decode kernels when T <= SPARSE_HIP_DECODE_MAX_TOKENS, the prefill
+ * kernels otherwise.
+ */
+int sparse_hip_shared_expert(const void* x_dev, const void* gate_w_dev, const void* up_w_dev,
+                             const void* down_w_dev, const void* shared_gate_dev, int dtype,
+                             int T, int H, int Is, void* inter_ws_dev, void* shared_dev,
+                             void* stream);
+
+/* ---- A7: combine ----------------------------------------------------------- */
+
+/*
+ * out[t] = (((0 + parts[p_0]) + parts[p_1]) + ...) (+ shared[t]) with p_j the rows of
+ * token t in ascending expert id and every add rounded to dtype: the accumulation
+ * order of `final.index_add_` in `_experts_world1_exact` (utils/eval_core.py:14720)
+ * and of `combine_expert_outputs` (utils/eval_core.py:523-538), followed by
+ * `expert_out + shared_out` (utils/eval_core.py:16526).  `shared_dev` may be NULL.
+ * parts [T*K,H], inv_perm [T*K], out [T,H].  H % 8 == 0.
+ */
+int sparse_hip_combine(const void* parts_dev, const int32_t* inv_perm_dev,
+                       const void* shared_dev, int dtype, int T, int K, int H, void* out_dev,
+                       void* stream);
+
+/* ---- A11/A12/A13: expert residency ----------------------------------------- */
+
+/*
+ * Enqueue a pinned-host -> HBM copy of one expert (`bytes` from `src_host` to
+ * `dst_dev`) on `stream`, then record `event` (a hipEvent_t as void*, may be NULL) on
+ * it.  Stands in for the three `pinned_cpu.to(device, non_blocking=True)` copies and
+ * `_record_prefetch_event` (utils/eval_core.py:11427-11429, :9970-9984, :11234-11242,
+ * :11621-11634).  Safe to call from a second host thread.
+ */
+int sparse_hip_expert_upload_async(void* dst_dev, const void* src_host, size_t bytes,
+                                   void* stream, void* event);
+
+/* Events and streams used to gate readiness (utils/eval_core.py:11176-11210,
+ * :5028-5055).  Events are created without timing unless `timing` is non-zero. */
+int sparse_hip_event_create(int timing, void** event_out);
+int sparse_hip_event_destroy(void* event);
+int sparse_hip_event_record(void* event, void* stream);
+/* 0 = complete, SPARSE_HIP_ENOTREADY = still in flight. */
+int sparse_hip_event_query(void* event);
+/* Make `stream` wait for `event` without blocking the host. */
+int sparse_hip_stream_wait_event(void* stream, void* event);
+int sparse_hip_event_elapsed_ms(void* start, void* stop, float* ms_out);
+/* Streams are created at the default priority. */
+int sparse_hip_stream_create(void** stream_out);
+int sparse_hip_stream_destroy(void* stream);
+int sparse_hip_stream_synchronize(void* stream);
+/* Pinned host arena for offloaded experts (hipHostMalloc / hipHostFree). */
+int sparse_hip_host_alloc(size_t bytes, void** ptr_out);
+int sparse_hip_host_free(void* ptr);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SPARSE_HIP_H */

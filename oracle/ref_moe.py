@@ -1,0 +1,184 @@
+"""CPU oracle for the arithmetic of the MoE layer path.  TEST INFRASTRUCTURE ONLY.
+
+This file restates, with PyTorch CPU ops, what louislichen/SPARSE's
+``DistributedSparseMoeBlock`` computes on the all-resident path.  Only ``tests/``,
+``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of ``bench.py`` may import it,
+and only as the checker or the timed CPU baseline -- never the product path.
+
+Every function cites the reference lines it follows (paths relative to the reference
+checkout, ``utils/eval_core.py`` unless stated).
+
+How each function is pinned (see tests/test_oracle_moe.py):
+  routing_router            closed form (fp64 softmax + brute-force top-k on small E),
+                            invariants (distinct ids, descending, sum <= 1), the chosen
+                            tie rule on hand-made ties.  torch.topk leaves tie order
+                            unspecified; the rule here is "higher probability first, then
+                            lower expert id".
+  deepseek_router           parity unpinned: the reference delegates to the model's own
+                            ``MoEGate`` (third-party, loaded with trust_remote_code, no
+                            version pin, source not in the reference tree).  Restated from
+                            the published DeepSeek-V2 gate: fp32 logits, fp32 softmax,
+                            top-k, times routed_scaling_factor.  Tests compare per-token
+                            index sets.
+  experts_world1_exact      fp64 per-token closed form sum_k w_k*down(silu(gate x)*up x)
+                            (the expected value of the reference's own
+                            tests/test_lightweight_policy.py:122-127), permutation
+                            invariance, equality with execute_sorted_segments+combine.
+  combine_expert_outputs    brute force on tiny inputs, order sensitivity in bf16.
+  shared_expert_forward     closed form.
+"""
+from __future__ import annotations
+
+from typing import List, Optional, Sequence, Tuple
+
+import torch
+import torch.nn.functional as F
+
+ExpertWeights = Tuple[torch.Tensor, torch.Tensor, torch.Tensor]  # gate [I,H], up [I,H], down [H,I]
+
+
+def topk_lower_id_first(probs: torch.Tensor, k: int) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Top-k along the last dim, descending, ties resolved to the lower index."""
+    order = torch.sort(probs, dim=-1, descending=True, stable=True)
+    return order.values[..., :k].contiguous(), order.indices[..., :k].contiguous()
+
+
+def routing_router(x: torch.Tensor, gate_w: torch.Tensor, top_k: int, norm_topk_prob: bool = False,
+                   router_logits: Optional[torch.Tensor] = None):
+    """Qwen-family router, :9519-9520 and :9590-9595.
+
+    ``router_logits = gate(x)`` in x.dtype, fp32 softmax, top-k, optional renorm, cast.
+    ``router_logits`` may be supplied to route on given logits (the parity contract is
+    "bit-exact indices given identical router logits").
+    Returns (topv [T,K] x.dtype, topi [T,K] int64, router_logits [T,E]).
+    """
+    if router_logits is None:
+        router_logits = F.linear(x, gate_w)
+    probs = torch.softmax(router_logits, dim=-1, dtype=torch.float32)
+    topv, topi = topk_lower_id_first(probs, top_k)
+    if norm_topk_prob:
+        topv = topv / topv.sum(dim=-1, keepdim=True).clamp_min(1e-12)
+    return topv.to(dtype=x.dtype), topi.to(torch.long), router_logits
+
+
+def deepseek_router(x: torch.Tensor, gate_w: torch.Tensor, top_k: int, routed_scaling_factor: float = 1.0,
+                    router_logits: Optional[torch.Tensor] = None):
+    """DeepSeek-family router as seen at the reference's call site :9503-9517.
+
+    The gate itself is third-party (parity unpinned, see the module docstring): fp32
+    logits from fp32-cast x and W, fp32 softmax, greedy top-k, weights scaled and cast to
+    x.dtype.  Returns (topv, topi, pseudo_logits) with pseudo_logits built as :9490-9499.
+    """
+    if router_logits is None:
+        router_logits = F.linear(x.to(torch.float32), gate_w.to(torch.float32))
+    probs = torch.softmax(router_logits, dim=-1, dtype=torch.float32)
+    topv, topi = topk_lower_id_first(probs, top_k)
+    topv = (topv * routed_scaling_factor).to(dtype=x.dtype)
+    pseudo = torch.full((x.shape[0], gate_w.shape[0]), float("-inf"), dtype=torch.float32)
+    pseudo.scatter_(1, topi, topv.to(torch.float32).clamp_min(1e-12).log())
+    return topv, topi.to(torch.long), pseudo
+
+
+def expert_forward(cur: torch.Tensor, weights: ExpertWeights) -> torch.Tensor:
+    """``down(act(gate(cur)) * up(cur))`` with SiLU, :11793-11796 (module layout)."""
+    gw, uw, dw = weights
+    return F.linear(F.silu(F.linear(cur, gw)) * F.linear(cur, uw), dw)
+
+
+def experts_world1_exact(x: torch.Tensor, idx: torch.Tensor, w: torch.Tensor,
+                         experts: Sequence[ExpertWeights]) -> torch.Tensor:
+    """All-resident expert loop, :14690-14721: ascending expert id, rows of an expert in
+    (slot, token) order, ``index_add_`` in x.dtype."""
+    T, H = x.shape
+    E = len(experts)
+    final = torch.zeros((T, H), dtype=x.dtype)
+    mask = F.one_hot(idx.to(torch.long), num_classes=E).permute(2, 1, 0)
+    for e in range(E):
+        slot, tok = torch.where(mask[e])
+        if tok.numel() == 0:
+            continue
+        cur = x[None, tok].reshape(-1, H)
+        y = expert_forward(cur, experts[e])
+        y = y * w[tok, slot, None]
+        final.index_add_(0, tok, y.to(x.dtype))
+    return final
+
+
+def combine_expert_outputs(parts: torch.Tensor, expert_ids: torch.Tensor) -> torch.Tensor:
+    """Per-token sum of the K slot outputs in ascending expert id, accumulated in the
+    activation dtype, :523-538."""
+    T, K, H = parts.shape
+    if tuple(expert_ids.shape) != (T, K):
+        raise ValueError("expert output/ID shape mismatch")
+    by_id = torch.argsort(expert_ids, dim=1, stable=True)
+    total = parts.new_zeros((T, H))
+    tok = torch.arange(T)
+    for j in range(K):
+        total.add_(parts[tok, by_id[:, j]])
+    return total
+
+
+def execute_sorted_segments(x: torch.Tensor, idx: torch.Tensor, w: torch.Tensor,
+                            experts: Sequence[ExpertWeights],
+                            order: Optional[Sequence[int]] = None) -> torch.Tensor:
+    """World-size-1 form of the EP executor: token x K expansion (:14728-14730), sort by
+    expert id and contiguous segments (:13240-13262), per-segment SwiGLU times route
+    weight (:13340-13357, :11700-11765), un-permute (:13359-13360), then
+    ``combine_expert_outputs`` (:14861-14863).  ``order`` optionally gives the expert
+    execution order (EPIPE changes the order, never the values).  The sort is the stable
+    one; the reference's ``argsort`` leaves ties unspecified and only row order inside a
+    segment depends on it."""
+    T, H = x.shape
+    K = idx.shape[1]
+    expanded = x.unsqueeze(1).expand(-1, K, -1).reshape(-1, H)
+    flat_i = idx.reshape(-1).to(torch.long)
+    flat_w = w.reshape(-1).to(expanded.dtype)
+    perm = torch.argsort(flat_i, stable=True)
+    sorted_i = flat_i[perm]
+    hidden_sorted = expanded[perm]
+    w_sorted = flat_w[perm]
+    out_sorted = torch.zeros_like(hidden_sorted)
+    bounds = {}
+    n = int(sorted_i.numel())
+    start = 0
+    while start < n:
+        e = int(sorted_i[start])
+        end = start
+        while end < n and int(sorted_i[end]) == e:
+            end += 1
+        bounds[e] = (start, end)
+        start = end
+    for e in (sorted(bounds) if order is None else order):
+        s, t = bounds[e]
+        y = expert_forward(hidden_sorted[s:t], experts[e])
+        out_sorted[s:t] = y * w_sorted[s:t].unsqueeze(1)
+    out = torch.zeros_like(expanded)
+    out[perm] = out_sorted
+    return combine_expert_outputs(out.view(T, K, H), idx)
+
+
+def shared_expert_forward(x: torch.Tensor, shared: Optional[ExpertWeights],
+                          shared_gate_w: Optional[torch.Tensor]) -> torch.Tensor:
+    """:9455-9463.  Qwen: ``sigmoid(shared_expert_gate(x)) * shared_expert(x)``; DeepSeek:
+    ``shared_experts(x)`` (pass ``shared_gate_w=None``); no shared expert: zeros."""
+    if shared is None:
+        return torch.zeros_like(x)
+    out = expert_forward(x, shared)
+    if shared_gate_w is not None:
+        out = torch.sigmoid(F.linear(x, shared_gate_w.reshape(1, -1))) * out
+    return out
+
+
+def moe_forward(x: torch.Tensor, gate_w: torch.Tensor, experts: Sequence[ExpertWeights], top_k: int,
+                shared: Optional[ExpertWeights] = None, shared_gate_w: Optional[torch.Tensor] = None,
+                norm_topk_prob: bool = False, family: str = "qwen_shared",
+                router_logits: Optional[torch.Tensor] = None):
+    """``forward`` at world size 1, :16488 and :16520-16526: route, expert loop, shared
+    expert, sum.  Returns (out [T,H], topv, topi, router_logits)."""
+    if family == "deepseek_shared":
+        topv, topi, logits = deepseek_router(x, gate_w, top_k, router_logits=router_logits)
+    else:
+        topv, topi, logits = routing_router(x, gate_w, top_k, norm_topk_prob, router_logits=router_logits)
+    expert_out = experts_world1_exact(x, topi, topv, experts)
+    shared_out = shared_expert_forward(x, shared, shared_gate_w)
+    return expert_out + shared_out, topv, topi, logits

@@ -1,0 +1,123 @@
+// C ABI entry points of the grouped SwiGLU FFN and the shared expert: argument
+// checks, then dispatch to the decode (HBM-bound, bf16 MFMA 16x16x32), prefill
+// (bf16 MFMA grouped GEMM) or fp32 tiled kernels.
+#include "common.h"
+
+namespace sparse {
+
+int decode_routed_bf16(const sparse_hip_experts*, const void*, const void*, const int32_t*, const int32_t*,
+                       const sparse_hip_seglist*, int, int, void*, void*, hipStream_t);
+int decode_shared_bf16(const void*, const void*, const void*, const void*, const void*, int, int, int, void*,
+                       void*, hipStream_t);
+int prefill_routed_bf16(const sparse_hip_experts*, const void*, const void*, const int32_t*, const int32_t*,
+                        const sparse_hip_seglist*, int, int, void*, void*, hipStream_t);
+int prefill_shared_bf16(const void*, const void*, const void*, const void*, const void*, int, int, int, void*,
+                        void*, hipStream_t);
+template <typename T>
+int tiled_routed(const sparse_hip_experts*, const void*, const void*, const int32_t*, const int32_t*,
+                 const sparse_hip_seglist*, int, int, void*, void*, hipStream_t);
+template <typename T>
+int tiled_shared(const void*, const void*, const void*, const void*, const void*, int, int, int, void*, void*,
+                 hipStream_t);
+
+static int check_routed(const char* fn, const sparse_hip_experts* ex, const void* x, const void* topv,
+                        const int32_t* perm, const int32_t* seg_offsets, const sparse_hip_seglist* segs, int T,
+                        int K, void* inter_ws, void* parts) {
+  SP_REQUIRE(ex != nullptr && segs != nullptr, "%s: NULL descriptor", fn);
+  SP_REQUIRE(valid_dtype(ex->dtype), "%s: unknown dtype %d", fn, ex->dtype);
+  SP_REQUIRE(ex->num_experts >= 1 && ex->num_experts <= SPARSE_HIP_MAX_EXPERTS, "%s: E=%d outside [1,%d]", fn,
+             ex->num_experts, SPARSE_HIP_MAX_EXPERTS);
+  SP_REQUIRE(ex->hidden > 0 && ex->hidden % 64 == 0, "%s: H=%d must be a positive multiple of 64", fn,
+             ex->hidden);
+  SP_REQUIRE(ex->inter > 0 && ex->inter % 64 == 0, "%s: I=%d must be a positive multiple of 64", fn, ex->inter);
+  SP_REQUIRE(ex->slot_stride >= 3ull * ex->hidden * ex->inter * elem_size(ex->dtype) &&
+                 ex->slot_stride % 16 == 0,
+             "%s: slot_stride=%llu too small or not 16-byte aligned", fn,
+             static_cast<unsigned long long>(ex->slot_stride));
+  SP_REQUIRE(ex->slab_dev && ex->expert_slot_dev, "%s: NULL weight slab or slot table", fn);
+  SP_REQUIRE((reinterpret_cast<uintptr_t>(ex->slab_dev) & 15) == 0, "%s: slab not 16-byte aligned", fn);
+  SP_REQUIRE(T >= 1, "%s: T=%d must be >= 1", fn, T);
+  SP_REQUIRE(K >= 1 && K <= SPARSE_HIP_MAX_TOPK, "%s: K=%d outside [1,%d]", fn, K, SPARSE_HIP_MAX_TOPK);
+  SP_REQUIRE(x && topv && perm && seg_offsets && inter_ws && parts, "%s: NULL pointer", fn);
+  SP_REQUIRE((reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(inter_ws) & 15) == 0 &&
+                 (reinterpret_cast<uintptr_t>(parts) & 15) == 0,
+             "%s: activations must be 16-byte aligned", fn);
+  SP_REQUIRE(segs->n >= 0 && segs->n <= SPARSE_HIP_MAX_EXPERTS, "%s: segment count %d outside [0,%d]", fn,
+             segs->n, SPARSE_HIP_MAX_EXPERTS);
+  SP_REQUIRE(segs->eids_dev == nullptr || segs->count_dev != nullptr, "%s: device segment list without count",
+             fn);
+  if (segs->eids_dev == nullptr) {
+    for (int i = 0; i < segs->n; ++i)
+      SP_REQUIRE(segs->eids[i] >= 0 && segs->eids[i] < ex->num_experts, "%s: segment %d names expert %d", fn, i,
+                 static_cast<int>(segs->eids[i]));
+  }
+  return SPARSE_HIP_OK;
+}
+
+}  // namespace sparse
+
+using namespace sparse;
+
+extern "C" {
+
+int sparse_hip_grouped_swiglu_decode(const sparse_hip_experts* experts, const void* x_dev, const void* topv_dev,
+                                     const int32_t* perm_dev, const int32_t* seg_offsets_dev,
+                                     const sparse_hip_seglist* segs, int T, int K, void* inter_ws_dev,
+                                     void* parts_dev, void* stream) {
+  int rc = check_routed("grouped_swiglu_decode", experts, x_dev, topv_dev, perm_dev, seg_offsets_dev, segs, T, K,
+                        inter_ws_dev, parts_dev);
+  if (rc != SPARSE_HIP_OK) return rc;
+  SP_REQUIRE(T <= SPARSE_HIP_DECODE_MAX_TOKENS, "grouped_swiglu_decode: T=%d exceeds %d; use the prefill entry",
+             T, SPARSE_HIP_DECODE_MAX_TOKENS);
+  if (segs->n == 0) return SPARSE_HIP_OK;
+  hipStream_t st = as_stream(stream);
+  if (experts->dtype == SPARSE_HIP_BF16)
+    return decode_routed_bf16(experts, x_dev, topv_dev, perm_dev, seg_offsets_dev, segs, T, K, inter_ws_dev,
+                              parts_dev, st);
+  return tiled_routed<float>(experts, x_dev, topv_dev, perm_dev, seg_offsets_dev, segs, T, K, inter_ws_dev,
+                             parts_dev, st);
+}
+
+int sparse_hip_grouped_swiglu_prefill(const sparse_hip_experts* experts, const void* x_dev, const void* topv_dev,
+                                      const int32_t* perm_dev, const int32_t* seg_offsets_dev,
+                                      const sparse_hip_seglist* segs, int T, int K, void* inter_ws_dev,
+                                      void* parts_dev, void* stream) {
+  int rc = check_routed("grouped_swiglu_prefill", experts, x_dev, topv_dev, perm_dev, seg_offsets_dev, segs, T,
+                        K, inter_ws_dev, parts_dev);
+  if (rc != SPARSE_HIP_OK) return rc;
+  if (segs->n == 0) return SPARSE_HIP_OK;
+  hipStream_t st = as_stream(stream);
+  if (experts->dtype == SPARSE_HIP_BF16)
+    return prefill_routed_bf16(experts, x_dev, topv_dev, perm_dev, seg_offsets_dev, segs, T, K, inter_ws_dev,
+                               parts_dev, st);
+  return tiled_routed<float>(experts, x_dev, topv_dev, perm_dev, seg_offsets_dev, segs, T, K, inter_ws_dev,
+                             parts_dev, st);
+}
+
+int sparse_hip_shared_expert(const void* x_dev, const void* gate_w_dev, const void* up_w_dev,
+                             const void* down_w_dev, const void* shared_gate_dev, int dtype, int T, int H,
+                             int Is, void* inter_ws_dev, void* shared_dev, void* stream) {
+  SP_REQUIRE(valid_dtype(dtype), "shared_expert: unknown dtype %d", dtype);
+  SP_REQUIRE(T >= 1, "shared_expert: T=%d must be >= 1", T);
+  SP_REQUIRE(H > 0 && H % 64 == 0 && Is > 0 && Is % 64 == 0,
+             "shared_expert: H=%d and Is=%d must be positive multiples of 64", H, Is);
+  SP_REQUIRE(x_dev && gate_w_dev && up_w_dev && down_w_dev && inter_ws_dev && shared_dev,
+             "shared_expert: NULL pointer");
+  SP_REQUIRE(((reinterpret_cast<uintptr_t>(x_dev) | reinterpret_cast<uintptr_t>(gate_w_dev) |
+               reinterpret_cast<uintptr_t>(up_w_dev) | reinterpret_cast<uintptr_t>(down_w_dev) |
+               reinterpret_cast<uintptr_t>(inter_ws_dev) | reinterpret_cast<uintptr_t>(shared_dev)) &
+              15) == 0,
+             "shared_expert: pointers must be 16-byte aligned");
+  hipStream_t st = as_stream(stream);
+  if (dtype == SPARSE_HIP_BF16) {
+    if (T <= SPARSE_HIP_DECODE_MAX_TOKENS)
+      return decode_shared_bf16(x_dev, gate_w_dev, up_w_dev, down_w_dev, shared_gate_dev, T, H, Is, inter_ws_dev,
+                                shared_dev, st);
+    return prefill_shared_bf16(x_dev, gate_w_dev, up_w_dev, down_w_dev, shared_gate_dev, T, H, Is, inter_ws_dev,
+                               shared_dev, st);
+  }
+  return tiled_shared<float>(x_dev, gate_w_dev, up_w_dev, down_w_dev, shared_gate_dev, T, H, Is, inter_ws_dev,
+                             shared_dev, st);
+}
+
+}  // extern "C"

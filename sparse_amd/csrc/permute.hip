@@ -1,0 +1,167 @@
+// Token x K expansion and stable bucketing by expert id, staged in LDS.
+//
+// A block owns 256 consecutive tokens.  Inside a block the rank of item (t, k) among
+// the items of its expert is the number of earlier tokens of the block that picked
+// the same expert (a token picks an expert at most once), read off a per-expert
+// token bitmap in LDS with popcounts.  Across blocks the ranks are offset by the
+// per-block histograms of a first pass.  The result is the (expert id, t*K+k)
+// order of a stable sort, with no atomics on positions, so it is deterministic.
+#include "common.h"
+
+namespace sparse {
+
+constexpr int kPermThreads = 256;
+constexpr int kMaskWords = kPermThreads / 32;
+
+__global__ __launch_bounds__(kPermThreads) void permute_count_kernel(const int64_t* __restrict__ topi, int T,
+                                                                     int K, int E,
+                                                                     int32_t* __restrict__ block_counts) {
+  __shared__ int32_t hist[SPARSE_HIP_MAX_EXPERTS];
+  for (int e = threadIdx.x; e < E; e += kPermThreads) hist[e] = 0;
+  __syncthreads();
+  const int t = blockIdx.x * kPermThreads + threadIdx.x;
+  if (t < T) {
+    for (int k = 0; k < K; ++k) {
+      const int64_t e = topi[static_cast<size_t>(t) * K + k];
+      if (e >= 0 && e < E) atomicAdd(&hist[e], 1);
+    }
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < E; e += kPermThreads)
+    block_counts[static_cast<size_t>(blockIdx.x) * E + e] = hist[e];
+}
+
+template <bool kSingleBlock>
+__global__ __launch_bounds__(kPermThreads) void permute_scatter_kernel(
+    const int64_t* __restrict__ topi, int T, int K, int E, const int32_t* __restrict__ block_counts,
+    int32_t* __restrict__ perm, int32_t* __restrict__ inv_perm, int32_t* __restrict__ seg_offsets,
+    int32_t* __restrict__ active_eids, int32_t* __restrict__ n_active) {
+  __shared__ uint32_t mask[SPARSE_HIP_MAX_EXPERTS][kMaskWords];
+  __shared__ int32_t scan_tot[SPARSE_HIP_MAX_EXPERTS];   // inclusive scan of per-expert totals
+  __shared__ int32_t scan_act[SPARSE_HIP_MAX_EXPERTS];   // inclusive scan of (total > 0)
+  __shared__ int32_t base[SPARSE_HIP_MAX_EXPERTS];       // first row of this block's items of e
+
+  const int tid = threadIdx.x;
+  for (int i = tid; i < E * kMaskWords; i += kPermThreads) (&mask[0][0])[i] = 0u;
+  __syncthreads();
+
+  const int t = blockIdx.x * kPermThreads + tid;
+  int64_t my_e[SPARSE_HIP_MAX_TOPK];
+  if (t < T) {
+#pragma unroll
+    for (int k = 0; k < SPARSE_HIP_MAX_TOPK; ++k) {
+      if (k < K) {
+        const int64_t e = topi[static_cast<size_t>(t) * K + k];
+        my_e[k] = e;
+        if (e >= 0 && e < E) atomicOr(&mask[e][tid >> 5], 1u << (tid & 31));
+      }
+    }
+  }
+  __syncthreads();
+
+  // per-expert totals and the number of items in earlier blocks
+  int32_t total = 0, before = 0;
+  if (tid < E) {
+    if (kSingleBlock) {
+#pragma unroll
+      for (int w = 0; w < kMaskWords; ++w) total += __popc(mask[tid][w]);
+    } else {
+      const int nb = gridDim.x;
+      for (int b = 0; b < nb; ++b) {
+        const int32_t c = block_counts[static_cast<size_t>(b) * E + tid];
+        total += c;
+        if (b < static_cast<int>(blockIdx.x)) before += c;
+      }
+    }
+  }
+  scan_tot[tid] = (tid < E) ? total : 0;
+  scan_act[tid] = (tid < E && total > 0) ? 1 : 0;
+  __syncthreads();
+  // Hillis-Steele inclusive scans over the 256 entries
+  for (int off = 1; off < kPermThreads; off <<= 1) {
+    int32_t a = 0, b = 0;
+    if (tid >= off) {
+      a = scan_tot[tid - off];
+      b = scan_act[tid - off];
+    }
+    __syncthreads();
+    scan_tot[tid] += a;
+    scan_act[tid] += b;
+    __syncthreads();
+  }
+  if (tid < E) {
+    const int32_t excl = scan_tot[tid] - total;
+    base[tid] = excl + before;
+    if (blockIdx.x == 0) {
+      seg_offsets[tid] = excl;
+      if (tid == E - 1) seg_offsets[E] = scan_tot[tid];
+      if (total > 0) active_eids[scan_act[tid] - 1] = tid;
+      if (tid == E - 1) n_active[0] = scan_act[tid];
+    }
+  }
+  __syncthreads();
+
+  if (t < T) {
+    const int word = tid >> 5;
+    const uint32_t below = (1u << (tid & 31)) - 1u;
+#pragma unroll
+    for (int k = 0; k < SPARSE_HIP_MAX_TOPK; ++k) {
+      if (k < K) {
+        const int64_t e = my_e[k];
+        if (e >= 0 && e < E) {
+          int32_t rank = __popc(mask[e][word] & below);
+          for (int w = 0; w < word; ++w) rank += __popc(mask[e][w]);
+          const int32_t f = t * K + k;
+          const int32_t pos = base[e] + rank;
+          perm[pos] = f;
+          inv_perm[f] = pos;
+        }
+      }
+    }
+  }
+}
+
+}  // namespace sparse
+
+using namespace sparse;
+
+extern "C" {
+
+size_t sparse_hip_permute_ws_bytes(int T, int K, int E) {
+  (void)K;
+  if (T <= 0 || E <= 0) return 0;
+  const size_t nb = (static_cast<size_t>(T) + kPermThreads - 1) / kPermThreads;
+  return nb * static_cast<size_t>(E) * sizeof(int32_t);
+}
+
+int sparse_hip_permute_build(const int64_t* topi_dev, int T, int K, int E, int32_t* perm_dev,
+                             int32_t* inv_perm_dev, int32_t* seg_offsets_dev, int32_t* active_eids_dev,
+                             int32_t* n_active_dev, void* ws_dev, void* stream) {
+  SP_REQUIRE(T >= 1, "permute_build: T=%d must be >= 1", T);
+  SP_REQUIRE(E >= 1 && E <= SPARSE_HIP_MAX_EXPERTS, "permute_build: E=%d outside [1,%d]", E,
+             SPARSE_HIP_MAX_EXPERTS);
+  SP_REQUIRE(K >= 1 && K <= SPARSE_HIP_MAX_TOPK && K <= E, "permute_build: K=%d outside [1,min(%d,E)]", K,
+             SPARSE_HIP_MAX_TOPK);
+  SP_REQUIRE(static_cast<int64_t>(T) * K < (1ll << 31), "permute_build: T*K overflows int32");
+  SP_REQUIRE(topi_dev && perm_dev && inv_perm_dev && seg_offsets_dev && active_eids_dev && n_active_dev,
+             "permute_build: NULL pointer");
+  hipStream_t st = as_stream(stream);
+  const int nb = (T + kPermThreads - 1) / kPermThreads;
+  if (nb == 1) {
+    hipLaunchKernelGGL((permute_scatter_kernel<true>), dim3(1), dim3(kPermThreads), 0, st, topi_dev, T, K, E,
+                       static_cast<const int32_t*>(nullptr), perm_dev, inv_perm_dev, seg_offsets_dev,
+                       active_eids_dev, n_active_dev);
+    SP_LAUNCH_CHECK("permute_scatter_kernel<single>");
+    return SPARSE_HIP_OK;
+  }
+  SP_REQUIRE(ws_dev != nullptr, "permute_build: workspace is NULL for T=%d", T);
+  int32_t* counts = static_cast<int32_t*>(ws_dev);
+  hipLaunchKernelGGL(permute_count_kernel, dim3(nb), dim3(kPermThreads), 0, st, topi_dev, T, K, E, counts);
+  SP_LAUNCH_CHECK("permute_count_kernel");
+  hipLaunchKernelGGL((permute_scatter_kernel<false>), dim3(nb), dim3(kPermThreads), 0, st, topi_dev, T, K, E,
+                     counts, perm_dev, inv_perm_dev, seg_offsets_dev, active_eids_dev, n_active_dev);
+  SP_LAUNCH_CHECK("permute_scatter_kernel");
+  return SPARSE_HIP_OK;
+}
+
+}  // extern "C"

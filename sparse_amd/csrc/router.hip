@@ -1,0 +1,227 @@
+// Router: gate projection (logits) and fused softmax + top-k with wavefront shuffles.
+#include "common.h"
+
+namespace sparse {
+
+// ---------------------------------------------------------------------------
+// logits[t, e] = <x[t, :], wg[e, :]>, one workgroup per (expert row, 32-token tile).
+// Row `E` of the grid (when present) is the shared-expert gate vector.
+// Every thread owns 8 consecutive h per 2048-wide sweep so that one sweep of the
+// workgroup reads a weight row with 16-byte (bf16) / 32-byte (fp32) loads per lane.
+// ---------------------------------------------------------------------------
+constexpr int kRouterThreads = 256;
+constexpr int kRouterTokTile = 32;
+
+template <typename T>
+__device__ __forceinline__ void load8(const T* p, float (&v)[8]);
+template <>
+__device__ __forceinline__ void load8<float>(const float* p, float (&v)[8]) {
+  const float4 a = *reinterpret_cast<const float4*>(p);
+  const float4 b = *reinterpret_cast<const float4*>(p + 4);
+  v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+  v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+}
+template <>
+__device__ __forceinline__ void load8<uint16_t>(const uint16_t* p, float (&v)[8]) {
+  const u32x4 a = *reinterpret_cast<const u32x4*>(p);
+  v[0] = __uint_as_float(a.x << 16); v[1] = __uint_as_float(a.x & 0xffff0000u);
+  v[2] = __uint_as_float(a.y << 16); v[3] = __uint_as_float(a.y & 0xffff0000u);
+  v[4] = __uint_as_float(a.z << 16); v[5] = __uint_as_float(a.z & 0xffff0000u);
+  v[6] = __uint_as_float(a.w << 16); v[7] = __uint_as_float(a.w & 0xffff0000u);
+}
+
+template <typename T, typename TL>
+__global__ __launch_bounds__(kRouterThreads) void router_logits_kernel(
+    const T* __restrict__ x, const T* __restrict__ wg, const T* __restrict__ wsg, int Ttok, int H,
+    int E, TL* __restrict__ logits, T* __restrict__ shared_gate) {
+  const int row = blockIdx.x;  // expert id, or E for the shared gate
+  const int t0 = blockIdx.y * kRouterTokTile;
+  const int nt = min(kRouterTokTile, Ttok - t0);
+  const T* w = (row < E) ? wg + static_cast<size_t>(row) * H : wsg;
+
+  float acc[kRouterTokTile];
+#pragma unroll
+  for (int i = 0; i < kRouterTokTile; ++i) acc[i] = 0.f;
+
+  for (int h = threadIdx.x * 8; h < H; h += kRouterThreads * 8) {
+    float wv[8];
+    load8<T>(w + h, wv);
+#pragma unroll
+    for (int i = 0; i < kRouterTokTile; ++i) {
+      if (i < nt) {
+        float xv[8];
+        load8<T>(x + static_cast<size_t>(t0 + i) * H + h, xv);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[i] = fmaf(xv[j], wv[j], acc[i]);
+      }
+    }
+  }
+
+  __shared__ float red[kRouterThreads / 64][kRouterTokTile];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+#pragma unroll
+  for (int i = 0; i < kRouterTokTile; ++i) {
+    const float s = wave_sum(acc[i]);
+    if (lane == 0) red[wave][i] = s;
+  }
+  __syncthreads();
+  if (threadIdx.x < nt) {
+    float s = 0.f;
+#pragma unroll
+    for (int wv = 0; wv < kRouterThreads / 64; ++wv) s += red[wv][threadIdx.x];
+    const int t = t0 + threadIdx.x;
+    if (row < E) {
+      Elem<TL>::store(logits + static_cast<size_t>(t) * E + row, s);
+    } else {
+      Elem<T>::store(shared_gate + t, s);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Fused softmax(fp32) + top-k.  One wavefront per token; lane l holds experts
+// l, l+64, l+128, l+192.  Selection runs K rounds of a wave-wide arg-max whose
+// order is (probability descending, expert id ascending).
+// ---------------------------------------------------------------------------
+constexpr int kTopkWaves = 4;
+constexpr int kTopkNV = SPARSE_HIP_MAX_EXPERTS / 64;
+
+template <typename TL, typename TO>
+__global__ __launch_bounds__(kTopkWaves * 64) void gate_topk_kernel(
+    const TL* __restrict__ logits, int Ttok, int E, int K, int renorm, TO* __restrict__ topv,
+    int64_t* __restrict__ topi) {
+  const int lane = threadIdx.x & 63;
+  const int t = blockIdx.x * kTopkWaves + (threadIdx.x >> 6);
+  if (t >= Ttok) return;
+  const TL* row = logits + static_cast<size_t>(t) * E;
+
+  float p[kTopkNV];
+  float m = -INFINITY;
+#pragma unroll
+  for (int j = 0; j < kTopkNV; ++j) {
+    const int e = lane + 64 * j;
+    p[j] = (e < E) ? Elem<TL>::load(row + e) : -INFINITY;
+    m = fmaxf(m, p[j]);
+  }
+  m = wave_max(m);
+  float s = 0.f;
+#pragma unroll
+  for (int j = 0; j < kTopkNV; ++j) {
+    const int e = lane + 64 * j;
+    p[j] = (e < E) ? expf(p[j] - m) : 0.f;
+    s += p[j];
+  }
+  s = wave_sum(s);
+#pragma unroll
+  for (int j = 0; j < kTopkNV; ++j) {
+    const int e = lane + 64 * j;
+    p[j] = (e < E) ? p[j] / s : -1.f;  // -1 marks "not a candidate"
+  }
+
+  float sel_v = 0.f;  // lane r keeps the r-th selection
+  int sel_i = 0;
+  float sum_sel = 0.f;
+  for (int r = 0; r < K; ++r) {
+    float bv = -1.f;
+    int bi = 0x7fffffff;
+#pragma unroll
+    for (int j = 0; j < kTopkNV; ++j) {
+      const int e = lane + 64 * j;
+      if (p[j] > bv) {  // ascending j == ascending id, so strict > keeps the lower id
+        bv = p[j];
+        bi = e;
+      }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+      const float ov = __shfl_xor(bv, off, 64);
+      const int oi = __shfl_xor(bi, off, 64);
+      if (ov > bv || (ov == bv && oi < bi)) {
+        bv = ov;
+        bi = oi;
+      }
+    }
+    // every lane now holds the winner; its owner retires it
+    if ((bi & 63) == lane) {
+#pragma unroll
+      for (int j = 0; j < kTopkNV; ++j)
+        if ((bi >> 6) == j) p[j] = -1.f;
+    }
+    if (lane == r) {
+      sel_v = bv;
+      sel_i = bi;
+    }
+    sum_sel += bv;
+  }
+  if (lane < K) {
+    float v = sel_v;
+    if (renorm) v = v / fmaxf(sum_sel, 1e-12f);
+    Elem<TO>::store(topv + static_cast<size_t>(t) * K + lane, v);
+    topi[static_cast<size_t>(t) * K + lane] = static_cast<int64_t>(sel_i);
+  }
+}
+
+template <typename T, typename TL>
+static int launch_router_logits(const void* x, const void* wg, const void* wsg, int Ttok, int H, int E,
+                                void* logits, void* shared_gate, hipStream_t st) {
+  dim3 grid(E + (wsg != nullptr ? 1 : 0), (Ttok + kRouterTokTile - 1) / kRouterTokTile);
+  hipLaunchKernelGGL((router_logits_kernel<T, TL>), grid, dim3(kRouterThreads), 0, st,
+                     static_cast<const T*>(x), static_cast<const T*>(wg), static_cast<const T*>(wsg), Ttok,
+                     H, E, static_cast<TL*>(logits), static_cast<T*>(shared_gate));
+  SP_LAUNCH_CHECK("router_logits_kernel");
+  return SPARSE_HIP_OK;
+}
+
+template <typename TL, typename TO>
+static int launch_gate_topk(const void* logits, int Ttok, int E, int K, int renorm, void* topv,
+                            int64_t* topi, hipStream_t st) {
+  dim3 grid((Ttok + kTopkWaves - 1) / kTopkWaves);
+  hipLaunchKernelGGL((gate_topk_kernel<TL, TO>), grid, dim3(kTopkWaves * 64), 0, st,
+                     static_cast<const TL*>(logits), Ttok, E, K, renorm, static_cast<TO*>(topv), topi);
+  SP_LAUNCH_CHECK("gate_topk_kernel");
+  return SPARSE_HIP_OK;
+}
+
+}  // namespace sparse
+
+using namespace sparse;
+
+extern "C" {
+
+int sparse_hip_router_logits(const void* x_dev, const void* wg_dev, const void* wsg_dev, int dtype,
+                             int logits_dtype, int T, int H, int E, void* logits_dev,
+                             void* shared_gate_dev, void* stream) {
+  SP_REQUIRE(valid_dtype(dtype) && valid_dtype(logits_dtype), "router_logits: unknown dtype");
+  SP_REQUIRE(logits_dtype == dtype || logits_dtype == SPARSE_HIP_F32,
+             "router_logits: logits_dtype must equal dtype or be fp32");
+  SP_REQUIRE(T >= 0 && H > 0 && E > 0, "router_logits: bad shape T=%d H=%d E=%d", T, H, E);
+  SP_REQUIRE(H % 8 == 0, "router_logits: H=%d must be a multiple of 8", H);
+  SP_REQUIRE(x_dev && wg_dev && logits_dev, "router_logits: NULL pointer");
+  SP_REQUIRE(wsg_dev == nullptr || shared_gate_dev != nullptr, "router_logits: shared gate output is NULL");
+  if (T == 0) return SPARSE_HIP_OK;
+  hipStream_t st = as_stream(stream);
+  if (dtype == SPARSE_HIP_F32)
+    return launch_router_logits<float, float>(x_dev, wg_dev, wsg_dev, T, H, E, logits_dev, shared_gate_dev, st);
+  if (logits_dtype == SPARSE_HIP_F32)
+    return launch_router_logits<uint16_t, float>(x_dev, wg_dev, wsg_dev, T, H, E, logits_dev, shared_gate_dev, st);
+  return launch_router_logits<uint16_t, uint16_t>(x_dev, wg_dev, wsg_dev, T, H, E, logits_dev, shared_gate_dev, st);
+}
+
+int sparse_hip_gate_topk(const void* logits_dev, int logits_dtype, int T, int E, int K, int renorm,
+                         int out_dtype, void* topv_dev, int64_t* topi_dev, void* stream) {
+  SP_REQUIRE(valid_dtype(logits_dtype) && valid_dtype(out_dtype), "gate_topk: unknown dtype");
+  SP_REQUIRE(T >= 0, "gate_topk: T=%d", T);
+  SP_REQUIRE(E >= 1 && E <= SPARSE_HIP_MAX_EXPERTS, "gate_topk: E=%d outside [1,%d]", E, SPARSE_HIP_MAX_EXPERTS);
+  SP_REQUIRE(K >= 1 && K <= SPARSE_HIP_MAX_TOPK && K <= E, "gate_topk: K=%d outside [1,min(%d,E)]", K,
+             SPARSE_HIP_MAX_TOPK);
+  SP_REQUIRE(logits_dev && topv_dev && topi_dev, "gate_topk: NULL pointer");
+  if (T == 0) return SPARSE_HIP_OK;
+  hipStream_t st = as_stream(stream);
+  const bool lb = logits_dtype == SPARSE_HIP_BF16, ob = out_dtype == SPARSE_HIP_BF16;
+  if (lb && ob) return launch_gate_topk<uint16_t, uint16_t>(logits_dev, T, E, K, renorm, topv_dev, topi_dev, st);
+  if (lb) return launch_gate_topk<uint16_t, float>(logits_dev, T, E, K, renorm, topv_dev, topi_dev, st);
+  if (ob) return launch_gate_topk<float, uint16_t>(logits_dev, T, E, K, renorm, topv_dev, topi_dev, st);
+  return launch_gate_topk<float, float>(logits_dev, T, E, K, renorm, topv_dev, topi_dev, st);
+}
+
+}  // extern "C"

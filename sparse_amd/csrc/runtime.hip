@@ -1,0 +1,118 @@
+// Library identity, error reporting, and the residency primitives of the C ABI:
+// pinned-host -> HBM expert uploads on a caller-chosen stream, and the event/stream
+// wrappers that gate readiness without host synchronisation.
+#include "common.h"
+
+#include <string.h>
+
+namespace sparse {
+
+static thread_local char g_err[512] = {0};
+
+void set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+}
+
+int hip_fail(hipError_t err, const char* what) {
+  set_error("%s: %s (%d)", what, hipGetErrorString(err), static_cast<int>(err));
+  return SPARSE_HIP_ELAUNCH;
+}
+
+}  // namespace sparse
+
+using namespace sparse;
+
+extern "C" {
+
+int sparse_hip_version(void) { return SPARSE_HIP_ABI_VERSION; }
+
+const char* sparse_hip_arch(void) { return "gfx950"; }
+
+const char* sparse_hip_last_error(void) { return g_err; }
+
+int sparse_hip_expert_upload_async(void* dst_dev, const void* src_host, size_t bytes, void* stream,
+                                   void* event) {
+  SP_REQUIRE(dst_dev != nullptr && src_host != nullptr, "expert_upload_async: NULL pointer");
+  SP_REQUIRE(bytes > 0, "expert_upload_async: bytes must be > 0");
+  SP_HIP(hipMemcpyAsync(dst_dev, src_host, bytes, hipMemcpyHostToDevice, as_stream(stream)));
+  if (event != nullptr) SP_HIP(hipEventRecord(reinterpret_cast<hipEvent_t>(event), as_stream(stream)));
+  return SPARSE_HIP_OK;
+}
+
+int sparse_hip_event_create(int timing, void** event_out) {
+  SP_REQUIRE(event_out != nullptr, "event_create: NULL out pointer");
+  hipEvent_t ev;
+  SP_HIP(hipEventCreateWithFlags(&ev, timing ? hipEventDefault : hipEventDisableTiming));
+  *event_out = ev;
+  return SPARSE_HIP_OK;
+}
+
+int sparse_hip_event_destroy(void* event) {
+  SP_REQUIRE(event != nullptr, "event_destroy: NULL event");
+  SP_HIP(hipEventDestroy(reinterpret_cast<hipEvent_t>(event)));
+  return SPARSE_HIP_OK;
+}
+
+int sparse_hip_event_record(void* event, void* stream) {
+  SP_REQUIRE(event != nullptr, "event_record: NULL event");
+  SP_HIP(hipEventRecord(reinterpret_cast<hipEvent_t>(event), as_stream(stream)));
+  return SPARSE_HIP_OK;
+}
+
+int sparse_hip_event_query(void* event) {
+  SP_REQUIRE(event != nullptr, "event_query: NULL event");
+  hipError_t e = hipEventQuery(reinterpret_cast<hipEvent_t>(event));
+  if (e == hipSuccess) return SPARSE_HIP_OK;
+  if (e == hipErrorNotReady) return SPARSE_HIP_ENOTREADY;
+  return hip_fail(e, "hipEventQuery");
+}
+
+int sparse_hip_stream_wait_event(void* stream, void* event) {
+  SP_REQUIRE(event != nullptr, "stream_wait_event: NULL event");
+  SP_HIP(hipStreamWaitEvent(as_stream(stream), reinterpret_cast<hipEvent_t>(event), 0));
+  return SPARSE_HIP_OK;
+}
+
+int sparse_hip_event_elapsed_ms(void* start, void* stop, float* ms_out) {
+  SP_REQUIRE(start != nullptr && stop != nullptr && ms_out != nullptr, "event_elapsed_ms: NULL argument");
+  SP_HIP(hipEventElapsedTime(ms_out, reinterpret_cast<hipEvent_t>(start), reinterpret_cast<hipEvent_t>(stop)));
+  return SPARSE_HIP_OK;
+}
+
+int sparse_hip_stream_create(void** stream_out) {
+  SP_REQUIRE(stream_out != nullptr, "stream_create: NULL out pointer");
+  hipStream_t s;
+  SP_HIP(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+  *stream_out = s;
+  return SPARSE_HIP_OK;
+}
+
+int sparse_hip_stream_destroy(void* stream) {
+  SP_REQUIRE(stream != nullptr, "stream_destroy: NULL stream");
+  SP_HIP(hipStreamDestroy(as_stream(stream)));
+  return SPARSE_HIP_OK;
+}
+
+int sparse_hip_stream_synchronize(void* stream) {
+  SP_HIP(hipStreamSynchronize(as_stream(stream)));
+  return SPARSE_HIP_OK;
+}
+
+int sparse_hip_host_alloc(size_t bytes, void** ptr_out) {
+  SP_REQUIRE(ptr_out != nullptr && bytes > 0, "host_alloc: bad argument");
+  void* p = nullptr;
+  SP_HIP(hipHostMalloc(&p, bytes, hipHostMallocDefault));
+  *ptr_out = p;
+  return SPARSE_HIP_OK;
+}
+
+int sparse_hip_host_free(void* ptr) {
+  SP_REQUIRE(ptr != nullptr, "host_free: NULL pointer");
+  SP_HIP(hipHostFree(ptr));
+  return SPARSE_HIP_OK;
+}
+
+}  // extern "C"

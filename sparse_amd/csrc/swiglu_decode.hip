@@ -1,0 +1,302 @@
+// Decode-time grouped SwiGLU expert FFN (bf16): the HBM-bandwidth path.
+//
+// With at most 32 tokens per call every expert sees a handful of rows, so the FFN is a
+// stream of weight rows past a tiny activation block.  A workgroup owns 32 output
+// rows of one expert (two 16-row MFMA tiles) and all of the expert's tokens (one or
+// two 16-token MFMA column tiles).  Weights go HBM -> registers in the MFMA A-operand
+// layout with no LDS hop: lane (r, q) of a wave loads 32 contiguous bytes of row r at
+// k = d*64 + q*16, so four lanes cover one 128-byte line of a row, the four waves of
+// the workgroup cover four adjacent lines, and every line is consumed by two
+// back-to-back loads.  The reduction dimension is split across the four waves
+// (64-wide slices dealt round-robin); partial 16x16 tiles meet in LDS once, in a
+// fixed order, and the epilogue (rounding, SiLU*up or *route-weight) runs there.
+//
+// MFMA 16x16x32 bf16 operand layout (lane l, r = l & 15, q = l >> 4):
+//   A: row r, k = q*8 .. q*8+7      B: column r, k = q*8 .. q*8+7
+//   D: column r, rows q*4 .. q*4+3
+// A and B use the same k mapping, so any permutation of k inside a 64-wide slice
+// applied to both leaves the product unchanged; the 32-byte-per-lane load relies on it.
+#include "common.h"
+
+namespace sparse {
+
+constexpr int kDecThreads = 256;
+constexpr int kDecWaves = 4;
+constexpr int kDecTiles = 2;                    // 16-row tiles per workgroup
+constexpr int kDecRows = kDecTiles * 16;        // output rows per workgroup
+
+struct DecodeArgs {
+  // routed experts
+  const uint16_t* slab;         // slot 0
+  uint64_t slot_stride;         // elements between slots
+  uint64_t mat_offset;          // element offset of the (first) matrix inside a slot
+  uint64_t mat2_offset;         // element offset of the second matrix (gate-up only)
+  const int32_t* expert_slot;   // [E]
+  const int32_t* perm;          // [T*K]
+  const int32_t* seg_offsets;   // [E+1]
+  const uint16_t* topv;         // [T*K] route weights (down only)
+  const uint16_t* act_r;        // gate-up: x [T,Kdim]; down: inter [T*K,Kdim]
+  uint16_t* out_r;              // gate-up: inter [T*K,Ndim]; down: parts [T*K,Ndim]
+  int32_t topk;
+  int32_t Kdim;                 // reduction length of the routed matrices
+  int32_t Ndim;                 // output rows of the routed matrices
+  int32_t tiles_r;              // Ndim / kDecRows
+  // shared expert (tiles_s == 0 when absent)
+  const uint16_t* w_s;          // first matrix [Ndim_s, Kdim_s]
+  const uint16_t* w2_s;         // second matrix (gate-up only)
+  const uint16_t* act_s;        // [T, Kdim_s]
+  const uint16_t* gate_s;       // [T] shared gate logits or NULL (down only)
+  uint16_t* out_s;              // [T, Ndim_s]
+  int32_t Kdim_s;
+  int32_t Ndim_s;
+  int32_t tiles_s;
+  int32_t T;
+  sparse_hip_seglist segs;
+};
+
+__device__ __forceinline__ bf16x8 ld_bf16x8(const uint16_t* p) {
+  return *reinterpret_cast<const bf16x8*>(p);
+}
+
+template <bool kGateUp, int NT>
+__global__ __launch_bounds__(kDecThreads) void decode_ffn_kernel(const DecodeArgs a) {
+  constexpr int NM = kGateUp ? 2 : 1;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int r = lane & 15, q = lane >> 4;
+
+  // ---- which tile of which matrix ------------------------------------------
+  const bool is_shared = static_cast<int>(blockIdx.x) < a.tiles_s;
+  const uint16_t *w0, *w1 = nullptr;
+  int Kdim, Ndim, row0, M, r0 = 0;
+  if (is_shared) {
+    Kdim = a.Kdim_s;
+    Ndim = a.Ndim_s;
+    row0 = blockIdx.x * kDecRows;
+    M = a.T;
+    w0 = a.w_s;
+    w1 = a.w2_s;
+  } else {
+    const int b = blockIdx.x - a.tiles_s;
+    const int si = b / a.tiles_r;
+    int eid;
+    if (a.segs.eids_dev != nullptr) {
+      const int cnt = min(a.segs.count_dev[0], a.segs.n);
+      if (si >= cnt) return;
+      eid = a.segs.eids_dev[si];
+    } else {
+      if (si >= a.segs.n) return;
+      eid = a.segs.eids[si];
+    }
+    Kdim = a.Kdim;
+    Ndim = a.Ndim;
+    row0 = (b - si * a.tiles_r) * kDecRows;
+    r0 = a.seg_offsets[eid];
+    M = a.seg_offsets[eid + 1] - r0;
+    if (M <= 0) return;
+    const uint16_t* slot = a.slab + static_cast<uint64_t>(a.expert_slot[eid]) * a.slot_stride;
+    w0 = slot + a.mat_offset;
+    w1 = slot + a.mat2_offset;
+  }
+
+  // ---- B operand rows (activations) ----------------------------------------
+  const uint16_t* brow[NT];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    const int n = r + 16 * nt;
+    brow[nt] = nullptr;
+    if (n < M) {
+      if (is_shared) {
+        brow[nt] = a.act_s + static_cast<size_t>(n) * Kdim;
+      } else if (kGateUp) {
+        brow[nt] = a.act_r + static_cast<size_t>(a.perm[r0 + n] / a.topk) * Kdim;
+      } else {
+        brow[nt] = a.act_r + static_cast<size_t>(r0 + n) * Kdim;
+      }
+    }
+  }
+
+  f32x4 acc[NM][kDecTiles][NT];
+#pragma unroll
+  for (int m = 0; m < NM; ++m)
+#pragma unroll
+    for (int tl = 0; tl < kDecTiles; ++tl)
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) acc[m][tl][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  const uint16_t* wrow0 = w0 + static_cast<size_t>(row0 + r) * Kdim + (q << 4);
+  const uint16_t* wrow1 = kGateUp ? w1 + static_cast<size_t>(row0 + r) * Kdim + (q << 4) : nullptr;
+  const size_t tile_step = static_cast<size_t>(16) * Kdim;
+  const int ND = Kdim >> 6;
+
+#pragma unroll 2
+  for (int d = wave; d < ND; d += kDecWaves) {
+    const int koff = d << 6;
+    bf16x8 b0[NT], b1[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      if (brow[nt] != nullptr) {
+        b0[nt] = ld_bf16x8(brow[nt] + koff + (q << 4));
+        b1[nt] = ld_bf16x8(brow[nt] + koff + (q << 4) + 8);
+      } else {
+        b0[nt] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+        b1[nt] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+      }
+    }
+#pragma unroll
+    for (int tl = 0; tl < kDecTiles; ++tl) {
+      const bf16x8 g0 = ld_bf16x8(wrow0 + tl * tile_step + koff);
+      const bf16x8 g1 = ld_bf16x8(wrow0 + tl * tile_step + koff + 8);
+      bf16x8 u0, u1;
+      if (kGateUp) {
+        u0 = ld_bf16x8(wrow1 + tl * tile_step + koff);
+        u1 = ld_bf16x8(wrow1 + tl * tile_step + koff + 8);
+      }
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
+        acc[0][tl][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(g0, b0[nt], acc[0][tl][nt], 0, 0, 0);
+        acc[0][tl][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(g1, b1[nt], acc[0][tl][nt], 0, 0, 0);
+        if (kGateUp) {
+          acc[1][tl][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(u0, b0[nt], acc[1][tl][nt], 0, 0, 0);
+          acc[1][tl][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(u1, b1[nt], acc[1][tl][nt], 0, 0, 0);
+        }
+      }
+    }
+  }
+
+  // ---- split-K partials meet in LDS ----------------------------------------
+  constexpr int NFRAG = kDecTiles * NT;
+  __shared__ f32x4 red[kDecWaves][NFRAG * NM][64];
+#pragma unroll
+  for (int tl = 0; tl < kDecTiles; ++tl)
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+      for (int m = 0; m < NM; ++m) red[wave][(tl * NT + nt) * NM + m][lane] = acc[m][tl][nt];
+  __syncthreads();
+
+  for (int f = wave; f < NFRAG; f += kDecWaves) {
+    const int tl = f / NT, nt = f - tl * NT;
+    const int n = r + 16 * nt;
+    if (n >= M) continue;
+    f32x4 s0 = red[0][f * NM][lane];
+    f32x4 s1 = kGateUp ? red[0][f * NM + 1][lane] : f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int w = 1; w < kDecWaves; ++w) {
+      s0 += red[w][f * NM][lane];
+      if (kGateUp) s1 += red[w][f * NM + 1][lane];
+    }
+    const int orow = row0 + tl * 16 + q * 4;
+    float scale = 1.f;
+    bool has_scale = false;
+    if (!kGateUp) {
+      if (is_shared) {
+        if (a.gate_s != nullptr) {
+          scale = round_bf16(sigmoid_f32(bf16_bits_to_f32(a.gate_s[n])));
+          has_scale = true;
+        }
+      } else {
+        scale = bf16_bits_to_f32(a.topv[a.perm[r0 + n]]);
+        has_scale = true;
+      }
+    }
+    uint16_t o[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      float v;
+      if (kGateUp) {
+        const float g = round_bf16(s0[j]);
+        const float u = round_bf16(s1[j]);
+        v = round_bf16(silu_f32(g)) * u;
+      } else {
+        v = round_bf16(s0[j]);
+        if (has_scale) v = v * scale;
+      }
+      o[j] = f32_to_bf16_bits(v);
+    }
+    uint16_t* dst = is_shared ? a.out_s + static_cast<size_t>(n) * Ndim + orow
+                              : a.out_r + static_cast<size_t>(r0 + n) * Ndim + orow;
+    uint2 pk;
+    pk.x = static_cast<uint32_t>(o[0]) | (static_cast<uint32_t>(o[1]) << 16);
+    pk.y = static_cast<uint32_t>(o[2]) | (static_cast<uint32_t>(o[3]) << 16);
+    *reinterpret_cast<uint2*>(dst) = pk;
+  }
+}
+
+template <bool kGateUp>
+static int launch_decode(const DecodeArgs& a, int n_seg, hipStream_t st) {
+  const int grid = a.tiles_s + n_seg * a.tiles_r;
+  if (grid == 0) return SPARSE_HIP_OK;
+  if (a.T <= 16) {
+    hipLaunchKernelGGL((decode_ffn_kernel<kGateUp, 1>), dim3(grid), dim3(kDecThreads), 0, st, a);
+  } else {
+    hipLaunchKernelGGL((decode_ffn_kernel<kGateUp, 2>), dim3(grid), dim3(kDecThreads), 0, st, a);
+  }
+  SP_LAUNCH_CHECK("decode_ffn_kernel");
+  return SPARSE_HIP_OK;
+}
+
+// Routed experts, bf16.  Two launches: gate-up into inter_ws, down into parts.
+int decode_routed_bf16(const sparse_hip_experts* ex, const void* x, const void* topv, const int32_t* perm,
+                       const int32_t* seg_offsets, const sparse_hip_seglist* segs, int T, int K,
+                       void* inter_ws, void* parts, hipStream_t st) {
+  const uint64_t H = ex->hidden, I = ex->inter;
+  DecodeArgs a = {};
+  a.slab = static_cast<const uint16_t*>(ex->slab_dev);
+  a.slot_stride = ex->slot_stride / 2;
+  a.expert_slot = ex->expert_slot_dev;
+  a.perm = perm;
+  a.seg_offsets = seg_offsets;
+  a.topk = K;
+  a.T = T;
+  a.segs = *segs;
+  // gate-up
+  a.mat_offset = 0;
+  a.mat2_offset = I * H;
+  a.act_r = static_cast<const uint16_t*>(x);
+  a.out_r = static_cast<uint16_t*>(inter_ws);
+  a.Kdim = static_cast<int32_t>(H);
+  a.Ndim = static_cast<int32_t>(I);
+  a.tiles_r = a.Ndim / kDecRows;
+  int rc = launch_decode<true>(a, segs->n, st);
+  if (rc != SPARSE_HIP_OK) return rc;
+  // down
+  a.mat_offset = 2 * I * H;
+  a.mat2_offset = 0;
+  a.topv = static_cast<const uint16_t*>(topv);
+  a.act_r = static_cast<const uint16_t*>(inter_ws);
+  a.out_r = static_cast<uint16_t*>(parts);
+  a.Kdim = static_cast<int32_t>(I);
+  a.Ndim = static_cast<int32_t>(H);
+  a.tiles_r = a.Ndim / kDecRows;
+  return launch_decode<false>(a, segs->n, st);
+}
+
+// Shared expert, bf16, T <= 32.
+int decode_shared_bf16(const void* x, const void* gate_w, const void* up_w, const void* down_w,
+                       const void* shared_gate, int T, int H, int Is, void* inter_ws, void* shared_out,
+                       hipStream_t st) {
+  DecodeArgs a = {};
+  a.T = T;
+  a.topk = 1;
+  a.tiles_r = 1;
+  a.w_s = static_cast<const uint16_t*>(gate_w);
+  a.w2_s = static_cast<const uint16_t*>(up_w);
+  a.act_s = static_cast<const uint16_t*>(x);
+  a.out_s = static_cast<uint16_t*>(inter_ws);
+  a.Kdim_s = H;
+  a.Ndim_s = Is;
+  a.tiles_s = Is / kDecRows;
+  int rc = launch_decode<true>(a, 0, st);
+  if (rc != SPARSE_HIP_OK) return rc;
+  a.w_s = static_cast<const uint16_t*>(down_w);
+  a.w2_s = nullptr;
+  a.act_s = static_cast<const uint16_t*>(inter_ws);
+  a.gate_s = static_cast<const uint16_t*>(shared_gate);
+  a.out_s = static_cast<uint16_t*>(shared_out);
+  a.Kdim_s = Is;
+  a.Ndim_s = H;
+  a.tiles_s = H / kDecRows;
+  return launch_decode<false>(a, 0, st);
+}
+
+}  // namespace sparse

@@ -1,0 +1,281 @@
+"""Operator-level Python wrappers over the C ABI.
+
+PyTorch supplies device memory (``Tensor.data_ptr()``) and the current HIP stream; all
+arithmetic happens in ``libsparse_hip.so``.  Every wrapper takes its outputs and
+workspaces from the caller (or allocates them with torch when ``None`` is passed) and
+launches asynchronously on ``torch.cuda.current_stream()``.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Optional, Sequence, Tuple
+
+import torch
+
+from . import _lib
+from ._lib import BF16, F32, DECODE_MAX_TOKENS, Experts, SegList
+
+
+def dtype_code(dtype: torch.dtype) -> int:
+    if dtype == torch.bfloat16:
+        return BF16
+    if dtype == torch.float32:
+        return F32
+    raise ValueError(f"unsupported dtype {dtype}: the MoE kernels take bfloat16 or float32")
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _need(t: torch.Tensor, name: str, dtype=None, shape=None) -> None:
+    if not t.is_cuda:
+        raise ValueError(f"{name} must be a device tensor")
+    if not t.is_contiguous():
+        raise ValueError(f"{name} must be contiguous")
+    if dtype is not None and t.dtype != dtype:
+        raise ValueError(f"{name} must be {dtype}, got {t.dtype}")
+    if shape is not None and tuple(t.shape) != tuple(shape):
+        raise ValueError(f"{name} must have shape {tuple(shape)}, got {tuple(t.shape)}")
+
+
+# --------------------------------------------------------------------------- router
+def router_logits(x: torch.Tensor, wg: torch.Tensor, wsg: Optional[torch.Tensor] = None,
+                  logits_dtype: Optional[torch.dtype] = None,
+                  out: Optional[torch.Tensor] = None,
+                  shared_gate_out: Optional[torch.Tensor] = None):
+    """``gate(x)`` (and ``shared_expert_gate(x)`` when ``wsg`` is given)."""
+    lib = _lib.load()
+    T, H = x.shape
+    E = wg.shape[0]
+    _need(x, "x")
+    _need(wg, "wg", x.dtype, (E, H))
+    ldt = logits_dtype or x.dtype
+    if out is None:
+        out = torch.empty((T, E), device=x.device, dtype=ldt)
+    _need(out, "logits", ldt, (T, E))
+    if wsg is not None:
+        _need(wsg, "wsg", x.dtype)
+        if wsg.numel() != H:
+            raise ValueError("wsg must hold H elements")
+        if shared_gate_out is None:
+            shared_gate_out = torch.empty((T,), device=x.device, dtype=x.dtype)
+    rc = lib.sparse_hip_router_logits(_ptr(x), _ptr(wg), _ptr(wsg), dtype_code(x.dtype), dtype_code(ldt),
+                                      T, H, E, _ptr(out), _ptr(shared_gate_out), _stream())
+    _lib.check(rc, "sparse_hip_router_logits")
+    return out, shared_gate_out
+
+
+def gate_topk(logits: torch.Tensor, k: int, renorm: bool = False, out_dtype: Optional[torch.dtype] = None,
+              topv: Optional[torch.Tensor] = None, topi: Optional[torch.Tensor] = None):
+    """Fused softmax(fp32) + top-k: returns ``(topv [T,k] out_dtype, topi [T,k] int64)``."""
+    lib = _lib.load()
+    _need(logits, "logits")
+    T, E = logits.shape
+    odt = out_dtype or logits.dtype
+    if topv is None:
+        topv = torch.empty((T, k), device=logits.device, dtype=odt)
+    if topi is None:
+        topi = torch.empty((T, k), device=logits.device, dtype=torch.int64)
+    _need(topv, "topv", odt, (T, k))
+    _need(topi, "topi", torch.int64, (T, k))
+    rc = lib.sparse_hip_gate_topk(_ptr(logits), dtype_code(logits.dtype), T, E, int(k), int(bool(renorm)),
+                                  dtype_code(odt), _ptr(topv), _ptr(topi), _stream())
+    _lib.check(rc, "sparse_hip_gate_topk")
+    return topv, topi
+
+
+# --------------------------------------------------------------------------- permute
+class Permutation:
+    """Outputs of ``permute_build`` (all int32 device tensors)."""
+
+    __slots__ = ("perm", "inv_perm", "seg_offsets", "active_eids", "n_active", "ws")
+
+    def __init__(self, T: int, K: int, E: int, device) -> None:
+        self.perm = torch.empty((T * K,), device=device, dtype=torch.int32)
+        self.inv_perm = torch.empty((T * K,), device=device, dtype=torch.int32)
+        self.seg_offsets = torch.empty((E + 1,), device=device, dtype=torch.int32)
+        self.active_eids = torch.empty((E,), device=device, dtype=torch.int32)
+        self.n_active = torch.empty((1,), device=device, dtype=torch.int32)
+        nbytes = _lib.load().sparse_hip_permute_ws_bytes(T, K, E)
+        self.ws = torch.empty((max(1, nbytes // 4),), device=device, dtype=torch.int32)
+
+
+def permute_build(topi: torch.Tensor, num_experts: int, out: Optional[Permutation] = None) -> Permutation:
+    lib = _lib.load()
+    _need(topi, "topi", torch.int64)
+    T, K = topi.shape
+    if out is None:
+        out = Permutation(T, K, num_experts, topi.device)
+    rc = lib.sparse_hip_permute_build(_ptr(topi), T, K, int(num_experts), _ptr(out.perm), _ptr(out.inv_perm),
+                                      _ptr(out.seg_offsets), _ptr(out.active_eids), _ptr(out.n_active),
+                                      _ptr(out.ws), _stream())
+    _lib.check(rc, "sparse_hip_permute_build")
+    return out
+
+
+# --------------------------------------------------------------------------- experts
+def make_experts(slab: torch.Tensor, expert_slot: torch.Tensor, num_experts: int, hidden: int, inter: int,
+                 slot_stride_bytes: Optional[int] = None) -> Experts:
+    """Describe a weight slab ``[slots, 3*I*H]`` (gate | up | down per slot)."""
+    _need(slab, "slab")
+    _need(expert_slot, "expert_slot", torch.int32, (num_experts,))
+    es = slab.element_size()
+    stride = slot_stride_bytes if slot_stride_bytes is not None else 3 * hidden * inter * es
+    return Experts(slab.data_ptr(), stride, expert_slot.data_ptr(), num_experts, hidden, inter,
+                   dtype_code(slab.dtype))
+
+
+def seglist_device(perm: Permutation, max_segments: int) -> SegList:
+    """Segment list read on the device: the active experts in ascending id."""
+    s = SegList()
+    s.eids_dev = perm.active_eids.data_ptr()
+    s.count_dev = perm.n_active.data_ptr()
+    s.n = int(max_segments)
+    return s
+
+
+def seglist_host(eids: Sequence[int]) -> SegList:
+    """Segment list passed by value, in the given execution order."""
+    s = SegList()
+    s.eids_dev = None
+    s.count_dev = None
+    s.n = len(eids)
+    if s.n > _lib.MAX_EXPERTS:
+        raise ValueError("too many segments")
+    for i, e in enumerate(eids):
+        s.eids[i] = int(e)
+    return s
+
+
+def grouped_swiglu(experts: Experts, x: torch.Tensor, topv: torch.Tensor, perm: Permutation, segs: SegList,
+                   inter_ws: torch.Tensor, parts: torch.Tensor, *, decode: Optional[bool] = None) -> None:
+    """Routed-expert FFN over the segments in ``segs``; rows land in ``parts`` (permuted order)."""
+    lib = _lib.load()
+    T, H = x.shape
+    K = topv.shape[1]
+    _need(x, "x")
+    _need(topv, "topv", x.dtype, (T, K))
+    _need(inter_ws, "inter_ws", x.dtype, (T * K, experts.inter))
+    _need(parts, "parts", x.dtype, (T * K, H))
+    if H != experts.hidden:
+        raise ValueError(f"x has hidden {H}, the expert slab has {experts.hidden}")
+    use_decode = (T <= DECODE_MAX_TOKENS) if decode is None else bool(decode)
+    fn = lib.sparse_hip_grouped_swiglu_decode if use_decode else lib.sparse_hip_grouped_swiglu_prefill
+    rc = fn(C.byref(experts), _ptr(x), _ptr(topv), _ptr(perm.perm), _ptr(perm.seg_offsets), C.byref(segs), T, K,
+            _ptr(inter_ws), _ptr(parts), _stream())
+    _lib.check(rc, "sparse_hip_grouped_swiglu_" + ("decode" if use_decode else "prefill"))
+
+
+def shared_expert(x: torch.Tensor, gate_w: torch.Tensor, up_w: torch.Tensor, down_w: torch.Tensor,
+                  shared_gate: Optional[torch.Tensor], inter_ws: torch.Tensor, out: torch.Tensor) -> None:
+    lib = _lib.load()
+    T, H = x.shape
+    Is = gate_w.shape[0]
+    _need(x, "x")
+    _need(gate_w, "shared gate_proj", x.dtype, (Is, H))
+    _need(up_w, "shared up_proj", x.dtype, (Is, H))
+    _need(down_w, "shared down_proj", x.dtype, (H, Is))
+    _need(inter_ws, "shared inter_ws", x.dtype, (T, Is))
+    _need(out, "shared out", x.dtype, (T, H))
+    if shared_gate is not None:
+        _need(shared_gate, "shared gate logits", x.dtype)
+        if shared_gate.numel() != T:
+            raise ValueError("shared gate logits must hold T elements")
+    rc = lib.sparse_hip_shared_expert(_ptr(x), _ptr(gate_w), _ptr(up_w), _ptr(down_w), _ptr(shared_gate),
+                                      dtype_code(x.dtype), T, H, Is, _ptr(inter_ws), _ptr(out), _stream())
+    _lib.check(rc, "sparse_hip_shared_expert")
+
+
+def combine(parts: torch.Tensor, perm: Permutation, shared: Optional[torch.Tensor], T: int, K: int,
+            out: torch.Tensor) -> None:
+    lib = _lib.load()
+    H = parts.shape[1]
+    _need(parts, "parts", None, (T * K, H))
+    _need(out, "out", parts.dtype, (T, H))
+    if shared is not None:
+        _need(shared, "shared", parts.dtype, (T, H))
+    rc = lib.sparse_hip_combine(_ptr(parts), _ptr(perm.inv_perm), _ptr(shared), dtype_code(parts.dtype), T, K, H,
+                                _ptr(out), _stream())
+    _lib.check(rc, "sparse_hip_combine")
+
+
+# --------------------------------------------------------------------------- residency
+class Event:
+    """A HIP event owned through the C ABI (no timing unless asked)."""
+
+    def __init__(self, timing: bool = False) -> None:
+        h = C.c_void_p()
+        _lib.check(_lib.load().sparse_hip_event_create(int(timing), C.byref(h)), "sparse_hip_event_create")
+        self.handle = h.value
+
+    def record(self, stream: Optional[int] = None) -> None:
+        _lib.check(_lib.load().sparse_hip_event_record(self.handle, _stream() if stream is None else stream),
+                   "sparse_hip_event_record")
+
+    def query(self) -> bool:
+        rc = _lib.load().sparse_hip_event_query(self.handle)
+        if rc == _lib.ENOTREADY:
+            return False
+        _lib.check(rc, "sparse_hip_event_query")
+        return True
+
+    def wait(self, stream: Optional[int] = None) -> None:
+        """Make ``stream`` (default: torch's current stream) wait; the host does not block."""
+        _lib.check(_lib.load().sparse_hip_stream_wait_event(_stream() if stream is None else stream, self.handle),
+                   "sparse_hip_stream_wait_event")
+
+    def elapsed_ms(self, end: "Event") -> float:
+        ms = C.c_float()
+        _lib.check(_lib.load().sparse_hip_event_elapsed_ms(self.handle, end.handle, C.byref(ms)),
+                   "sparse_hip_event_elapsed_ms")
+        return float(ms.value)
+
+    def __del__(self) -> None:
+        try:
+            if self.handle:
+                _lib.load().sparse_hip_event_destroy(self.handle)
+                self.handle = None
+        except Exception:
+            pass
+
+
+class SideStream:
+    """A non-blocking HIP stream at the default priority, for expert uploads."""
+
+    def __init__(self) -> None:
+        h = C.c_void_p()
+        _lib.check(_lib.load().sparse_hip_stream_create(C.byref(h)), "sparse_hip_stream_create")
+        self.handle = h.value
+
+    def synchronize(self) -> None:
+        _lib.check(_lib.load().sparse_hip_stream_synchronize(self.handle), "sparse_hip_stream_synchronize")
+
+    def __del__(self) -> None:
+        try:
+            if self.handle:
+                _lib.load().sparse_hip_stream_destroy(self.handle)
+                self.handle = None
+        except Exception:
+            pass
+
+
+def expert_upload_async(dst_dev_ptr: int, src_host_ptr: int, nbytes: int, stream: int,
+                        event: Optional[Event]) -> None:
+    rc = _lib.load().sparse_hip_expert_upload_async(dst_dev_ptr, src_host_ptr, nbytes, stream,
+                                                    None if event is None else event.handle)
+    _lib.check(rc, "sparse_hip_expert_upload_async")
+
+
+def host_alloc(nbytes: int) -> int:
+    p = C.c_void_p()
+    _lib.check(_lib.load().sparse_hip_host_alloc(nbytes, C.byref(p)), "sparse_hip_host_alloc")
+    return p.value
+
+
+def host_free(ptr: int) -> None:
+    _lib.check(_lib.load().sparse_hip_host_free(ptr), "sparse_hip_host_free")

@@ -1,0 +1,82 @@
+"""Expert weight storage: HBM slot slab and pinned-host arena.
+
+One slot holds one routed expert as three row-major matrices back to back,
+``gate [I,H] | up [I,H] | down [H,I]`` (the module layout of the reference,
+utils/eval_core.py:5115-5123, made contiguous so that one expert is one H2D copy).
+All-resident layers use ``E`` slots with the identity slot table; cached layers use
+``capacity (+ staging)`` slots and rewrite ``expert_slot`` as experts move.
+"""
+from __future__ import annotations
+
+from typing import Optional, Sequence, Tuple
+
+import torch
+
+ExpertWeights = Tuple[torch.Tensor, torch.Tensor, torch.Tensor]
+
+
+def expert_numel(hidden: int, inter: int) -> int:
+    return 3 * hidden * inter
+
+
+def pack_expert_into(dst_row: torch.Tensor, weights: ExpertWeights, hidden: int, inter: int) -> None:
+    """Copy (gate, up, down) into one flat slot row."""
+    gw, uw, dw = weights
+    if tuple(gw.shape) != (inter, hidden) or tuple(uw.shape) != (inter, hidden) or tuple(dw.shape) != (hidden, inter):
+        raise ValueError(
+            f"expert weights must be gate/up [{inter},{hidden}] and down [{hidden},{inter}], got "
+            f"{tuple(gw.shape)}, {tuple(uw.shape)}, {tuple(dw.shape)}")
+    n = hidden * inter
+    dst_row[0:n].copy_(gw.reshape(-1))
+    dst_row[n:2 * n].copy_(uw.reshape(-1))
+    dst_row[2 * n:3 * n].copy_(dw.reshape(-1))
+
+
+class HostExpertArena:
+    """All routed experts of a layer in pinned host memory, one row per expert id."""
+
+    def __init__(self, experts: Sequence[ExpertWeights], hidden: int, inter: int, dtype: torch.dtype,
+                 pin: bool = True) -> None:
+        self.hidden, self.inter, self.dtype = hidden, inter, dtype
+        self.num_experts = len(experts)
+        self.rows = torch.empty((self.num_experts, expert_numel(hidden, inter)), dtype=dtype, pin_memory=pin)
+        for e, w in enumerate(experts):
+            pack_expert_into(self.rows[e], tuple(t.to(dtype) for t in w), hidden, inter)
+        self.expert_bytes = self.rows[0].numel() * self.rows.element_size()
+
+    def host_ptr(self, eid: int) -> int:
+        return self.rows[eid].data_ptr()
+
+
+class ExpertSlab:
+    """``num_slots`` expert slots in HBM plus the device-side expert -> slot table."""
+
+    def __init__(self, num_slots: int, num_experts: int, hidden: int, inter: int, dtype: torch.dtype,
+                 device: torch.device) -> None:
+        self.hidden, self.inter, self.dtype = hidden, inter, dtype
+        self.num_slots, self.num_experts = num_slots, num_experts
+        self.data = torch.empty((num_slots, expert_numel(hidden, inter)), dtype=dtype, device=device)
+        self.expert_bytes = self.data[0].numel() * self.data.element_size()
+        # host mirror of the table; pushed to the device whenever it changes
+        self.slot_of = [-1] * num_experts
+        self.expert_slot = torch.zeros((num_experts,), dtype=torch.int32, device=device)
+
+    @classmethod
+    def resident(cls, experts: Sequence[ExpertWeights], hidden: int, inter: int, dtype: torch.dtype,
+                 device: torch.device) -> "ExpertSlab":
+        """All experts resident, slot == expert id."""
+        slab = cls(len(experts), len(experts), hidden, inter, dtype, device)
+        staging = torch.empty((expert_numel(hidden, inter),), dtype=dtype)
+        for e, w in enumerate(experts):
+            pack_expert_into(staging, tuple(t.detach().to("cpu", dtype) for t in w), hidden, inter)
+            slab.data[e].copy_(staging)
+            slab.slot_of[e] = e
+        slab.push_table()
+        return slab
+
+    def slot_ptr(self, slot: int) -> int:
+        return self.data.data_ptr() + slot * self.expert_bytes
+
+    def push_table(self) -> None:
+        table = torch.tensor([max(0, s) for s in self.slot_of], dtype=torch.int32)
+        self.expert_slot.copy_(table)

@@ -1,0 +1,26 @@
+"""Seeded synthetic MoE layers shared by the tests (weights ~N(0, 0.02), hidden ~N(0, 1))."""
+from __future__ import annotations
+
+import torch
+
+Q_SHAPE = dict(H=2048, E=60, I=1408, K=4, Is=5632, shared_gate=True)
+D_SHAPE = dict(H=2048, E=64, I=1408, K=6, Is=2816, shared_gate=False)
+
+
+def make_layer(H, E, I, K, Is=0, shared_gate=False, dtype=torch.float32, seed=0, std=0.02):
+    g = torch.Generator().manual_seed(seed)
+
+    def w(*shape):
+        return (torch.randn(*shape, generator=g) * std).to(dtype)
+
+    layer = dict(H=H, E=E, I=I, K=K, Is=Is, dtype=dtype)
+    layer["gate_w"] = w(E, H)
+    layer["experts"] = [(w(I, H), w(I, H), w(H, I)) for _ in range(E)]
+    layer["shared"] = (w(Is, H), w(Is, H), w(H, Is)) if Is else None
+    layer["shared_gate_w"] = w(H) if (Is and shared_gate) else None
+    return layer
+
+
+def make_hidden(T, H, dtype=torch.float32, seed=1000):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn(T, H, generator=g).to(dtype)

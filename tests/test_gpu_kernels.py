@@ -1,0 +1,276 @@
+"""GPU parity tests of the individual C-ABI operators against the CPU oracle.
+
+Bit-exact for indices and permutations; bf16 outputs within rtol 2e-2 / atol 1e-2 and fp32
+outputs within rtol/atol 1e-5 of the oracle (the tolerances the north star states).
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import ref_moe, ref_permute
+from tests.helpers import make_hidden, make_layer
+
+pytestmark = pytest.mark.gpu
+
+BF16_TOL = dict(rtol=2e-2, atol=1e-2)
+F32_TOL = dict(rtol=1e-5, atol=1e-5)
+
+
+def tol(dtype):
+    return BF16_TOL if dtype == torch.bfloat16 else F32_TOL
+
+
+def _ops():
+    from sparse_amd import ops
+    return ops
+
+
+def _boundary_safe(probs: torch.Tensor, k: int, eps: float = 1e-6) -> torch.Tensor:
+    """Tokens whose selected set cannot flip under ulp-level differences in exp/sum:
+    every adjacent pair among the k+1 largest probabilities is separated (relative)."""
+    s = torch.sort(probs, dim=-1, descending=True).values[:, : k + 1]
+    gap = (s[:, :-1] - s[:, 1:]) / s[:, :-1].clamp_min(1e-30)
+    return (gap > eps).all(dim=1)
+
+
+# ------------------------------------------------------------------ gate_topk
+@pytest.mark.parametrize("E,K", [(60, 4), (64, 6), (16, 2), (200, 8)])
+@pytest.mark.parametrize("ldt", [torch.float32, torch.bfloat16])
+def test_gate_topk_matches_oracle(device, E, K, ldt):
+    ops = _ops()
+    g = torch.Generator().manual_seed(E * 100 + K)
+    logits = (torch.randn(257, E, generator=g) * 2.0).to(ldt)
+    probs = torch.softmax(logits, dim=-1, dtype=torch.float32)
+    ref_v, ref_i = ref_moe.topk_lower_id_first(probs, K)
+    topv, topi = ops.gate_topk(logits.to(device), K, out_dtype=ldt)
+    topv, topi = topv.cpu(), topi.cpu()
+    safe = _boundary_safe(probs, K)
+    assert safe.float().mean() > 0.9
+    assert torch.equal(topi[safe], ref_i[safe])
+    # tokens with a near-tie still pick a valid top-k set
+    both = torch.sort(topi, dim=1).values
+    assert (both[:, 1:] != both[:, :-1]).all()
+    torch.testing.assert_close(topv.float()[safe], ref_v.to(ldt).float()[safe], rtol=1e-2, atol=1e-6)
+
+
+def test_gate_topk_ties_go_to_lower_id(device):
+    ops = _ops()
+    logits = torch.zeros(5, 60)
+    logits[1, [7, 3, 50]] = 2.0          # three-way tie at the top, K=4 takes all + id 0
+    logits[2, [59, 58, 57, 56, 55]] = 1.0  # five-way tie, K=4 takes the four lowest ids
+    logits[3, 10] = 5.0
+    logits[4] = torch.arange(60, dtype=torch.float32).flip(0) * 0.0  # all equal
+    for ldt in (torch.float32, torch.bfloat16):
+        probs = torch.softmax(logits.to(ldt), dim=-1, dtype=torch.float32)
+        ref_v, ref_i = ref_moe.topk_lower_id_first(probs, 4)
+        topv, topi = ops.gate_topk(logits.to(ldt).to(device), 4)
+        assert torch.equal(topi.cpu(), ref_i)
+        assert topi.cpu()[0].tolist() == [0, 1, 2, 3]
+        assert topi.cpu()[1].tolist() == [3, 7, 50, 0]
+        assert topi.cpu()[2].tolist() == [55, 56, 57, 58]
+        assert topi.cpu()[3].tolist() == [10, 0, 1, 2]
+
+
+def test_gate_topk_renorm(device):
+    ops = _ops()
+    g = torch.Generator().manual_seed(5)
+    logits = torch.randn(33, 60, generator=g)
+    topv, topi = ops.gate_topk(logits.to(device), 4, renorm=True)
+    torch.testing.assert_close(topv.cpu().sum(dim=1), torch.ones(33), rtol=1e-5, atol=1e-5)
+    x = torch.zeros(33, 8)
+    ref_v, ref_i, _ = ref_moe.routing_router(x, torch.zeros(60, 8), 4, True, router_logits=logits)
+    safe = _boundary_safe(torch.softmax(logits, -1), 4)
+    assert torch.equal(topi.cpu()[safe], ref_i[safe])
+    torch.testing.assert_close(topv.cpu()[safe], ref_v[safe], rtol=1e-5, atol=1e-6)
+
+
+def test_gate_topk_rejects_bad_arguments(device):
+    ops = _ops()
+    logits = torch.zeros(4, 300, device=device)
+    with pytest.raises(ValueError):
+        ops.gate_topk(logits, 4)
+    with pytest.raises(ValueError):
+        ops.gate_topk(torch.zeros(4, 8, device=device), 9)
+
+
+# ------------------------------------------------------------------ router logits
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("T", [1, 8, 33, 128])
+def test_router_logits(device, dtype, T):
+    ops = _ops()
+    layer = make_layer(2048, 60, 64, 4, Is=64, shared_gate=True, dtype=dtype, seed=3)
+    x = make_hidden(T, 2048, dtype, seed=4)
+    ref = torch.nn.functional.linear(x.float(), layer["gate_w"].float())
+    ref_sg = torch.nn.functional.linear(x.float(), layer["shared_gate_w"].float().reshape(1, -1)).reshape(-1)
+    logits, sg = ops.router_logits(x.to(device), layer["gate_w"].to(device), layer["shared_gate_w"].to(device))
+    assert logits.dtype == dtype and sg.dtype == dtype
+    t = dict(rtol=1e-2, atol=1e-2) if dtype == torch.bfloat16 else dict(rtol=1e-4, atol=1e-5)
+    torch.testing.assert_close(logits.float().cpu(), ref, **t)
+    torch.testing.assert_close(sg.float().cpu(), ref_sg, **t)
+    if dtype == torch.bfloat16:
+        l32, _ = ops.router_logits(x.to(device), layer["gate_w"].to(device), logits_dtype=torch.float32)
+        assert l32.dtype == torch.float32
+        torch.testing.assert_close(l32.cpu(), ref, rtol=1e-4, atol=1e-4)
+
+
+# ------------------------------------------------------------------ permute
+@pytest.mark.parametrize("T,E,K", [(1, 60, 4), (8, 60, 4), (32, 60, 4), (255, 64, 6), (256, 64, 6),
+                                    (257, 64, 6), (2048, 64, 6), (4096, 64, 6), (1000, 256, 16), (3, 4, 4)])
+def test_permute_build_bit_exact(device, T, E, K):
+    ops = _ops()
+    g = torch.Generator().manual_seed(T * 7 + E)
+    scores = torch.rand(T, E, generator=g)
+    if T >= 255:
+        scores[:, : E // 4] += 0.5  # skewed popularity, some experts possibly empty
+        scores[:, E - 1] = -1.0     # one expert never chosen
+    topi = torch.topk(scores, K, dim=1).indices.to(torch.int64)
+    p = ops.permute_build(topi.to(device), E)
+    perm, inv, off, active = ref_permute.permute_build(topi.numpy(), E)
+    torch.cuda.synchronize()
+    assert np.array_equal(p.perm.cpu().numpy(), perm)
+    assert np.array_equal(p.inv_perm.cpu().numpy(), inv)
+    assert np.array_equal(p.seg_offsets.cpu().numpy(), off)
+    n = int(p.n_active.cpu().item())
+    assert n == active.size
+    assert np.array_equal(p.active_eids.cpu().numpy()[:n], active)
+
+
+# ------------------------------------------------------------------ FFN helpers
+def _run_routed(ops, layer, x, topv, topi, device, decode, order=None):
+    from sparse_amd.weights import ExpertSlab
+    H, E, I, K = layer["H"], layer["E"], layer["I"], layer["K"]
+    dtype = layer["dtype"]
+    T = x.shape[0]
+    slab = ExpertSlab.resident(layer["experts"], H, I, dtype, device)
+    ex = ops.make_experts(slab.data, slab.expert_slot, E, H, I)
+    xd, tvd, tid = x.to(device), topv.to(device), topi.to(device)
+    p = ops.permute_build(tid, E)
+    inter = torch.zeros((T * K, I), device=device, dtype=dtype)
+    parts = torch.zeros((T * K, H), device=device, dtype=dtype)
+    if order is None:
+        segs = ops.seglist_device(p, min(E, T * K))
+    else:
+        segs = ops.seglist_host(order)
+    ops.grouped_swiglu(ex, xd, tvd, p, segs, inter, parts, decode=decode)
+    out = torch.empty((T, H), device=device, dtype=dtype)
+    ops.combine(parts, p, None, T, K, out)
+    torch.cuda.synchronize()
+    return out.cpu(), parts.cpu(), p
+
+
+def _routing(layer, x):
+    topv, topi, _ = ref_moe.routing_router(x, layer["gate_w"], layer["K"])
+    return topv, topi
+
+
+@pytest.mark.parametrize("T", [1, 2, 8, 16, 17, 32])
+def test_decode_ffn_bf16_matches_oracle(device, T):
+    ops = _ops()
+    layer = make_layer(512, 12, 256, 4, dtype=torch.bfloat16, seed=11, std=0.05)
+    x = make_hidden(T, 512, torch.bfloat16, seed=12)
+    topv, topi = _routing(layer, x)
+    out, _, _ = _run_routed(ops, layer, x, topv, topi, device, decode=True)
+    ref = ref_moe.experts_world1_exact(x, topi, topv, layer["experts"])
+    torch.testing.assert_close(out.float(), ref.float(), **BF16_TOL)
+    # a wrong row/column mapping would give O(1) relative error; check it is tight
+    err = (out.float() - ref.float()).abs().max() / ref.float().abs().max()
+    assert err < 2e-2
+
+
+def test_decode_ffn_bf16_qwen_shape(device):
+    ops = _ops()
+    layer = make_layer(2048, 60, 1408, 4, dtype=torch.bfloat16, seed=0)
+    x = make_hidden(8, 2048, torch.bfloat16, seed=1000)
+    topv, topi = _routing(layer, x)
+    out, _, _ = _run_routed(ops, layer, x, topv, topi, device, decode=True)
+    ref = ref_moe.experts_world1_exact(x, topi, topv, layer["experts"])
+    torch.testing.assert_close(out.float(), ref.float(), **BF16_TOL)
+    assert (out.float() - ref.float()).abs().max() / ref.float().abs().max() < 2e-2
+
+
+@pytest.mark.parametrize("T", [40, 128, 300])
+def test_prefill_ffn_bf16_matches_oracle(device, T):
+    ops = _ops()
+    layer = make_layer(512, 12, 256, 4, dtype=torch.bfloat16, seed=21, std=0.05)
+    x = make_hidden(T, 512, torch.bfloat16, seed=22)
+    topv, topi = _routing(layer, x)
+    out, _, _ = _run_routed(ops, layer, x, topv, topi, device, decode=False)
+    ref = ref_moe.experts_world1_exact(x, topi, topv, layer["experts"])
+    torch.testing.assert_close(out.float(), ref.float(), **BF16_TOL)
+    assert (out.float() - ref.float()).abs().max() / ref.float().abs().max() < 2e-2
+
+
+def test_prefill_and_decode_kernels_agree(device):
+    ops = _ops()
+    layer = make_layer(512, 12, 256, 4, dtype=torch.bfloat16, seed=31, std=0.05)
+    x = make_hidden(24, 512, torch.bfloat16, seed=32)
+    topv, topi = _routing(layer, x)
+    a, _, _ = _run_routed(ops, layer, x, topv, topi, device, decode=True)
+    b, _, _ = _run_routed(ops, layer, x, topv, topi, device, decode=False)
+    torch.testing.assert_close(a.float(), b.float(), **BF16_TOL)
+
+
+@pytest.mark.parametrize("T,decode", [(8, True), (128, False)])
+def test_ffn_fp32_matches_oracle(device, T, decode):
+    ops = _ops()
+    layer = make_layer(256, 10, 128, 3, dtype=torch.float32, seed=41, std=0.05)
+    x = make_hidden(T, 256, torch.float32, seed=42)
+    topv, topi = _routing(layer, x)
+    out, _, _ = _run_routed(ops, layer, x, topv, topi, device, decode=decode)
+    ref = ref_moe.experts_world1_exact(x, topi, topv, layer["experts"])
+    torch.testing.assert_close(out, ref, **F32_TOL)
+
+
+def test_segment_order_changes_nothing(device):
+    """EPIPE reorders expert execution; values must not move (host-ordered segment list)."""
+    ops = _ops()
+    layer = make_layer(512, 12, 256, 4, dtype=torch.bfloat16, seed=51, std=0.05)
+    x = make_hidden(16, 512, torch.bfloat16, seed=52)
+    topv, topi = _routing(layer, x)
+    base, _, _ = _run_routed(ops, layer, x, topv, topi, device, decode=True)
+    active = sorted(set(topi.reshape(-1).tolist()))
+    shuffled = list(reversed(active))
+    other, _, _ = _run_routed(ops, layer, x, topv, topi, device, decode=True, order=shuffled)
+    assert torch.equal(base, other)
+    pre, _, _ = _run_routed(ops, layer, x, topv, topi, device, decode=False, order=shuffled)
+    pre2, _, _ = _run_routed(ops, layer, x, topv, topi, device, decode=False)
+    assert torch.equal(pre, pre2)
+
+
+# ------------------------------------------------------------------ shared expert + combine
+@pytest.mark.parametrize("dtype,T", [(torch.bfloat16, 8), (torch.bfloat16, 32), (torch.bfloat16, 200),
+                                     (torch.float32, 8), (torch.float32, 100)])
+@pytest.mark.parametrize("gated", [True, False])
+def test_shared_expert(device, dtype, T, gated):
+    ops = _ops()
+    layer = make_layer(512, 4, 64, 2, Is=384, shared_gate=gated, dtype=dtype, seed=61, std=0.05)
+    x = make_hidden(T, 512, dtype, seed=62)
+    ref = ref_moe.shared_expert_forward(x, layer["shared"], layer["shared_gate_w"])
+    xd = x.to(device)
+    sg = None
+    if gated:
+        _, sg = ops.router_logits(xd, layer["gate_w"].to(device), layer["shared_gate_w"].to(device))
+    gw, uw, dw = (t.to(device) for t in layer["shared"])
+    inter = torch.empty((T, 384), device=device, dtype=dtype)
+    out = torch.empty((T, 512), device=device, dtype=dtype)
+    ops.shared_expert(xd, gw, uw, dw, sg, inter, out)
+    torch.testing.assert_close(out.cpu().float(), ref.float(), **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_combine_is_ordered_sum(device, dtype):
+    ops = _ops()
+    T, K, H, E = 37, 4, 256, 20
+    g = torch.Generator().manual_seed(71)
+    scores = torch.rand(T, E, generator=g)
+    topi = torch.topk(scores, K, dim=1).indices.to(torch.int64)
+    parts_tkh = (torch.randn(T, K, H, generator=g) * 3).to(dtype)
+    shared = torch.randn(T, H, generator=g).to(dtype)
+    ref = ref_moe.combine_expert_outputs(parts_tkh, topi) + shared
+    p = ops.permute_build(topi.to(device), E)
+    perm = p.perm.cpu().long()
+    parts_sorted = parts_tkh.reshape(T * K, H)[perm].contiguous().to(device)
+    out = torch.empty((T, H), device=device, dtype=dtype)
+    ops.combine(parts_sorted, p, shared.to(device), T, K, out)
+    # same adds in the same order: bit-exact
+    assert torch.equal(out.cpu(), ref)
