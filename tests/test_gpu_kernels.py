@@ -25,12 +25,17 @@ def _ops():
     return ops
 
 
-def _boundary_safe(probs: torch.Tensor, k: int, eps: float = 1e-6) -> torch.Tensor:
-    """Tokens whose selected set cannot flip under ulp-level differences in exp/sum:
-    every adjacent pair among the k+1 largest probabilities is separated (relative)."""
-    s = torch.sort(probs, dim=-1, descending=True).values[:, : k + 1]
-    gap = (s[:, :-1] - s[:, 1:]) / s[:, :-1].clamp_min(1e-30)
-    return (gap > eps).all(dim=1)
+def _boundary_safe(logits: torch.Tensor, k: int, eps: float = 1e-6) -> torch.Tensor:
+    """Tokens whose top-k cannot flip under ulp-level differences in exp/sum: every
+    adjacent pair among the k+1 largest is either an exact logit tie (equal inputs give
+    equal probabilities everywhere, the id rule decides) or clearly separated."""
+    srt = torch.sort(logits.float(), dim=-1, descending=True, stable=True)
+    top_l = srt.values[:, : k + 1]
+    probs = torch.softmax(logits, dim=-1, dtype=torch.float32)
+    top_p = torch.gather(probs, 1, srt.indices[:, : k + 1])
+    gap = (top_p[:, :-1] - top_p[:, 1:]) / top_p[:, :-1].clamp_min(1e-30)
+    ok = (top_l[:, :-1] == top_l[:, 1:]) | (gap > eps)
+    return ok.all(dim=1)
 
 
 # ------------------------------------------------------------------ gate_topk
@@ -44,7 +49,7 @@ def test_gate_topk_matches_oracle(device, E, K, ldt):
     ref_v, ref_i = ref_moe.topk_lower_id_first(probs, K)
     topv, topi = ops.gate_topk(logits.to(device), K, out_dtype=ldt)
     topv, topi = topv.cpu(), topi.cpu()
-    safe = _boundary_safe(probs, K)
+    safe = _boundary_safe(logits, K)
     assert safe.float().mean() > 0.9
     assert torch.equal(topi[safe], ref_i[safe])
     # tokens with a near-tie still pick a valid top-k set
@@ -79,7 +84,7 @@ def test_gate_topk_renorm(device):
     torch.testing.assert_close(topv.cpu().sum(dim=1), torch.ones(33), rtol=1e-5, atol=1e-5)
     x = torch.zeros(33, 8)
     ref_v, ref_i, _ = ref_moe.routing_router(x, torch.zeros(60, 8), 4, True, router_logits=logits)
-    safe = _boundary_safe(torch.softmax(logits, -1), 4)
+    safe = _boundary_safe(logits, 4)
     assert torch.equal(topi.cpu()[safe], ref_i[safe])
     torch.testing.assert_close(topv.cpu()[safe], ref_v[safe], rtol=1e-5, atol=1e-6)
 
