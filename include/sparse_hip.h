@@ -67,7 +67,7 @@ const char* sparse_hip_last_error(void);
 typedef struct sparse_hip_experts {
   const void* slab_dev;            /* base of slot 0 */
   uint64_t slot_stride;            /* bytes between slots (>= 3*I*H*elem) */
-  const int32_t* expert_slot_dev;  /* [E] expert id -> slot */
+  const int32_t* expert_slot_dev;  /* [E] expert id -> slot (device segment lists only) */
   int32_t num_experts;             /* E */
   int32_t hidden;                  /* H */
   int32_t inter;                   /* I */
@@ -77,15 +77,18 @@ typedef struct sparse_hip_experts {
 /*
  * Which expert segments one launch executes, in launch order.  If `eids_dev` is
  * non-NULL the list is read on the device: `eids_dev[0 .. *count_dev)` with at most
- * `n` entries (the grid is sized for n).  Otherwise the first `n` entries of `eids`
- * are used.  A segment is the run of permuted rows of one expert
- * (utils/eval_core.py:13240-13262).
+ * `n` entries (the grid is sized for n), and the weights of expert e are in slot
+ * `expert_slot_dev[e]`.  Otherwise the first `n` entries of `eids` are used and the
+ * weights of `eids[i]` are in slot `slots[i]`: the host decides order and residency
+ * per launch and nothing on the device has to be rewritten between launches.  A
+ * segment is the run of permuted rows of one expert (utils/eval_core.py:13240-13262).
  */
 typedef struct sparse_hip_seglist {
   const int32_t* eids_dev;
   const int32_t* count_dev;
   int32_t n;
   int16_t eids[SPARSE_HIP_MAX_EXPERTS];
+  int16_t slots[SPARSE_HIP_MAX_EXPERTS];
 } sparse_hip_seglist;
 
 /* ---- A1: router ------------------------------------------------------------ */

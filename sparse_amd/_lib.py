@@ -49,6 +49,7 @@ class SegList(C.Structure):
         ("count_dev", C.c_void_p),
         ("n", C.c_int32),
         ("eids", C.c_int16 * MAX_EXPERTS),
+        ("slots", C.c_int16 * MAX_EXPERTS),
     ]
 
 

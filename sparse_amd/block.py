@@ -1,0 +1,486 @@
+"""``DistributedSparseMoeBlock``: the MoE layer of louislichen/SPARSE on one MI355X.
+
+Keeps the reference block's constructor keywords, ``forward(hidden[B,S,H])`` signature,
+return convention and lifecycle hooks (utils/eval_core.py:4408-4440, :16418-16563,
+:6097-6147, :16565-16659) and runs the layer through the HIP kernels behind the C ABI:
+
+    router_logits -> gate_topk -> permute_build -> shared_expert
+                  -> grouped_swiglu (resident: one device-ordered launch pair;
+                     offloaded: batches ordered by the residency policy)
+                  -> combine
+
+``expert_offload="gpu"`` keeps every expert in an HBM slab and never touches the host
+during ``forward`` (capturable in a HIP graph).  ``expert_offload="cpu"`` keeps experts in
+pinned host memory and a per-layer HBM cache of ``expert_cache`` slots; ``forward`` then
+synchronises once per call to learn which experts were routed, exactly where the
+reference's ``torch.where`` / ``.tolist()`` calls synchronise.
+"""
+from __future__ import annotations
+
+import os
+from typing import Any, Dict, List, Optional, Sequence, Tuple
+
+import torch
+import torch.nn.functional as F
+from torch import nn
+
+from . import ops
+from .context import DistEnv, Metrics, SparseContext
+from .residency import Backend, LayerResidency, ResidencyConfig
+from .weights import ExpertSlab, HostExpertArena
+
+
+def _is_silu(fn: Any) -> bool:
+    return fn is None or fn is F.silu or isinstance(fn, nn.SiLU) or getattr(fn, "__name__", "") == "silu"
+
+
+def _mlp_weights(mod: Any) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    return mod.gate_proj.weight.detach(), mod.up_proj.weight.detach(), mod.down_proj.weight.detach()
+
+
+def extract_experts(experts: Any) -> Tuple[str, List[Tuple[torch.Tensor, torch.Tensor, torch.Tensor]]]:
+    """Accept the two expert containers the reference accepts (:4350-4362): a fused object
+    (``gate_up_proj [E,2I,H]``, ``down_proj [E,H,I]``) or a list of modules."""
+    if hasattr(experts, "gate_up_proj") and hasattr(experts, "down_proj"):
+        gu, dn = experts.gate_up_proj.detach(), experts.down_proj.detach()
+        inter = gu.shape[1] // 2
+        if not _is_silu(getattr(experts, "act_fn", None)):
+            raise NotImplementedError("only SiLU experts are built")
+        return "fused", [(gu[e, :inter], gu[e, inter:], dn[e]) for e in range(gu.shape[0])]
+    try:
+        mods = list(experts)
+    except TypeError:
+        mods = []
+    if mods and all(hasattr(m, "gate_proj") and hasattr(m, "up_proj") and hasattr(m, "down_proj") for m in mods):
+        for m in mods:
+            if not _is_silu(getattr(m, "act_fn", None)):
+                raise NotImplementedError("only SiLU experts are built")
+        return "modulelist", [_mlp_weights(m) for m in mods]
+    raise RuntimeError("Unsupported experts container. Need fused or modulelist experts.")
+
+
+class _Workspace:
+    """Activation buffers for one (T, layer shape); shared by all layers of that shape."""
+
+    _cache: Dict[Tuple, "_Workspace"] = {}
+
+    def __init__(self, T: int, K: int, E: int, H: int, I: int, Is: int, dtype, logits_dtype, device) -> None:
+        self.logits_dtype = logits_dtype
+        self.shared_gate = torch.empty((T,), device=device, dtype=dtype)
+        self.topv = torch.empty((T, K), device=device, dtype=dtype)
+        self.topi = torch.empty((T, K), device=device, dtype=torch.int64)
+        self.perm = ops.Permutation(T, K, E, device)
+        self.inter = torch.empty((T * K, I), device=device, dtype=dtype)
+        self.parts = torch.empty((T * K, H), device=device, dtype=dtype)
+        self.shared_inter = torch.empty((T, Is), device=device, dtype=dtype) if Is else None
+        self.shared_out = torch.empty((T, H), device=device, dtype=dtype) if Is else None
+        self.segs_dev = ops.seglist_device(self.perm, min(E, T * K))
+        # host mirrors for the offloaded path (pinned, written by async D2H copies)
+        self.host_offsets = torch.empty((E + 1,), dtype=torch.int32, pin_memory=True)
+        self.host_rs_topi = torch.empty((T * E,), dtype=torch.int64, pin_memory=True)
+        self.host_rs_topv = torch.empty((T * E,), dtype=torch.float32, pin_memory=True)
+
+    @classmethod
+    def get(cls, *key) -> "_Workspace":
+        ws = cls._cache.get(key)
+        if ws is None:
+            ws = cls(*key)
+            cls._cache[key] = ws
+        return ws
+
+
+class _EventRing:
+    """Reusable events of one lane.  An event is only ever re-recorded on the same
+    in-order lane, so waiting on a recycled event still implies the older work is done."""
+
+    def __init__(self, n: int = 512) -> None:
+        self._events = [ops.Event() for _ in range(n)]
+        self._next = 0
+
+    def take(self) -> ops.Event:
+        ev = self._events[self._next]
+        self._next = (self._next + 1) % len(self._events)
+        return ev
+
+
+class _SideStreams:
+    """Upload streams shared by all layers (default priority)."""
+
+    _inst: Optional["_SideStreams"] = None
+
+    def __init__(self) -> None:
+        self.prefetch = ops.SideStream()
+        self.epipe = ops.SideStream()
+        self.rings = {"compute": _EventRing(2048), "prefetch": _EventRing(2048), "epipe": _EventRing(512)}
+
+    @classmethod
+    def get(cls) -> "_SideStreams":
+        if cls._inst is None:
+            cls._inst = cls()
+        return cls._inst
+
+
+class _HipBackend(Backend):
+    """Uploads, events and FFN launches for one layer's residency policy."""
+
+    def __init__(self, block: "DistributedSparseMoeBlock") -> None:
+        self.block = block
+        self.streams = _SideStreams.get()
+        self.rings = self.streams.rings
+        self.x: Optional[torch.Tensor] = None
+        self.ws: Optional[_Workspace] = None
+        self.launches = 0
+
+    def _stream(self, lane: str) -> int:
+        if lane == "compute":
+            return torch.cuda.current_stream().cuda_stream
+        return self.streams.prefetch.handle if lane == "prefetch" else self.streams.epipe.handle
+
+    def bind(self, x: torch.Tensor, ws: _Workspace) -> None:
+        self.x, self.ws = x, ws
+
+    def upload(self, eid: int, slot: int, lane: str):
+        blk = self.block
+        ev = self.rings[lane].take()
+        ops.expert_upload_async(blk.slab.slot_ptr(slot), blk.arena.host_ptr(eid), blk.arena.expert_bytes,
+                                self._stream(lane), ev)
+        return ev
+
+    def event_done(self, event) -> bool:
+        return event.query()
+
+    def wait_event(self, event, lane: str) -> None:
+        event.wait(self._stream(lane))
+
+    def run_segments(self, segments: Sequence[Tuple[int, int]]) -> None:
+        blk, ws = self.block, self.ws
+        segs = ops.seglist_host([e for e, _ in segments], [s for _, s in segments])
+        ops.grouped_swiglu(blk._experts_desc, self.x, ws.topv, ws.perm, segs, ws.inter, ws.parts)
+        self.launches += 1
+
+    def fence(self):
+        ev = self.rings["compute"].take()
+        ev.record(self._stream("compute"))
+        return ev
+
+
+class DistributedSparseMoeBlock(nn.Module):
+    """Drop-in for the reference block on a single GPU (world size 1)."""
+
+    def __init__(
+        self,
+        layer_idx: int,
+        mlp_block: Any,
+        scp_map: Any = None,
+        env: Optional[DistEnv] = None,
+        num_layers: int = 1,
+        num_experts: Optional[int] = None,
+        top_k: int = 1,
+        dtype: torch.dtype = torch.bfloat16,
+        expert_offload: str = "gpu",
+        expert_cache: int = 10,
+        routing_mode: str = "router",
+        rs_dir: Optional[str] = None,
+        rs_require_complete: bool = False,
+        rs_prob_to_logit_eps: float = 1e-12,
+        log_routing_stats: bool = False,
+        rs_group: int = 3,
+        rs_debug: bool = False,
+        metrics: Optional[Metrics] = None,
+        debug_a2a_checks: bool = False,
+        collect_per_layer: bool = False,
+        log_per_layer: bool = False,
+        planner_mode: str = "none",
+        prefetch_top_m: int = 1,
+        oracle_mode: str = "none",
+        oracle_ignore_cache_capacity: bool = True,
+        placement_mode: str = "scp",
+        expert_source: str = "router",
+        cache_policy: str = "lru",
+        runtime_mode: str = "baseline",
+        topology: Any = None,
+        residency_config: Optional[ResidencyConfig] = None,
+    ) -> None:
+        super().__init__()
+        self.layer_idx = int(layer_idx)
+        self.env = env if env is not None else DistEnv()
+        self.device = torch.device(self.env.device)
+        self.rank, self.world = int(self.env.rank), int(self.env.world)
+        if self.world != 1:
+            raise NotImplementedError("this build runs the MoE layer on one GPU (world size 1)")
+        self.num_layers = int(num_layers)
+        self.top_k = int(top_k)
+        self.dtype = dtype
+        self.norm_topk_prob = bool(getattr(mlp_block, "norm_topk_prob", False))
+        # enum validation, same messages as the reference (:4475-4498, :4799-4804)
+        self.exec_routing_mode = str(routing_mode)
+        if self.exec_routing_mode not in ("router", "rs"):
+            raise ValueError(f"routing_mode must be router|rs, got {self.exec_routing_mode}")
+        self.placement_mode = str(placement_mode)
+        if self.placement_mode not in ("scp", "scp_ep", "round_robin", "weighted_random_balanced"):
+            raise ValueError(
+                f"placement_mode must be scp|scp_ep|round_robin|weighted_random_balanced, got {self.placement_mode}")
+        self.planner_mode = str(planner_mode)
+        if self.planner_mode not in ("none", "rs_prefetch"):
+            raise ValueError(f"planner_mode must be none|rs_prefetch, got {self.planner_mode}")
+        self.expert_source = str(expert_source)
+        if self.expert_source not in ("router", "rs"):
+            raise ValueError(f"expert_source must be router|rs, got {self.expert_source}")
+        if str(runtime_mode) != "baseline":
+            raise ValueError(f"Unsupported runtime_mode: {runtime_mode}")
+        self.runtime_mode = "baseline"
+        if self.expert_source == "rs" and not (self.exec_routing_mode == "rs" or self.planner_mode == "rs_prefetch"):
+            raise ValueError(
+                "expert_source=rs requires RS cache available, so routing_mode must be 'rs' "
+                "or planner_mode must be 'rs_prefetch'.")
+        self.expert_offload = str(expert_offload)
+        if self.expert_offload not in ("cpu", "gpu"):
+            raise ValueError(f"expert_offload must be cpu|gpu, got {self.expert_offload}")
+        self.cache_policy = str(cache_policy).lower()
+        if self.cache_policy not in ("lru", "lfu", "tiered"):
+            raise ValueError(f"cache_policy must be lru|lfu|tiered, got {self.cache_policy}")
+        if self.cache_policy != "lru":
+            raise NotImplementedError(f"cache_policy={self.cache_policy} is not built; formal runs use lru")
+        if self.dtype not in (torch.bfloat16, torch.float32):
+            raise ValueError(f"dtype must be bfloat16 or float32, got {self.dtype}")
+        self.rs_group = int(rs_group)
+        self.prefetch_top_m = int(prefetch_top_m)
+        self.metrics = metrics if metrics is not None else Metrics()
+
+        # ---- weights --------------------------------------------------------
+        if not hasattr(mlp_block, "gate") or not hasattr(mlp_block, "experts"):
+            raise RuntimeError("mlp_block needs .gate and .experts")
+        self.moe_family = "qwen_shared" if hasattr(mlp_block, "shared_expert") else "deepseek_shared"
+        self.routed_scaling_factor = float(getattr(mlp_block.gate, "routed_scaling_factor",
+                                                   getattr(mlp_block, "routed_scaling_factor", 1.0)) or 1.0)
+        self.gate_weight = mlp_block.gate.weight.detach().to(self.device, self.dtype).contiguous()
+        self.experts_kind, expert_weights = extract_experts(mlp_block.experts)
+        self.num_experts = int(num_experts) if num_experts is not None else len(expert_weights)
+        if self.num_experts != len(expert_weights) or self.gate_weight.shape[0] != self.num_experts:
+            raise ValueError("num_experts does not match the gate / experts container")
+        self.hidden_size = int(self.gate_weight.shape[1])
+        self.inter_size = int(expert_weights[0][0].shape[0])
+        shared_mod = getattr(mlp_block, "shared_expert", None) or getattr(mlp_block, "shared_experts", None)
+        self.shared_weights = None
+        self.shared_inter_size = 0
+        if shared_mod is not None:
+            if not _is_silu(getattr(shared_mod, "act_fn", None)):
+                raise NotImplementedError("only SiLU shared experts are built")
+            self.shared_weights = tuple(t.to(self.device, self.dtype).contiguous() for t in _mlp_weights(shared_mod))
+            self.shared_inter_size = int(self.shared_weights[0].shape[0])
+        sg = getattr(mlp_block, "shared_expert_gate", None)
+        self.shared_gate_weight = (
+            sg.weight.detach().to(self.device, self.dtype).reshape(-1).contiguous() if sg is not None else None)
+        self.logits_dtype = torch.float32 if self.moe_family == "deepseek_shared" else self.dtype
+
+        E, H, I = self.num_experts, self.hidden_size, self.inter_size
+        self.local_expert_ids = list(range(E))
+        self._local_eid_set = set(self.local_expert_ids)
+        self.residency: Optional[LayerResidency] = None
+        self.arena: Optional[HostExpertArena] = None
+        if self.expert_offload == "gpu":
+            self.slab = ExpertSlab.resident(expert_weights, H, I, self.dtype, self.device)
+        else:
+            cfg = residency_config if residency_config is not None else ResidencyConfig.from_env(
+                capacity=int(expert_cache), planner_mode=self.planner_mode, prefetch_top_m=int(prefetch_top_m))
+            cfg.capacity = int(expert_cache) if residency_config is None else cfg.capacity
+            self.arena = HostExpertArena(expert_weights, H, I, self.dtype, pin=True)
+            self._backend = _HipBackend(self)
+            self.residency = LayerResidency(self.layer_idx, E, self.top_k, cfg, self._backend, self.metrics,
+                                            expert_bytes=self.arena.expert_bytes)
+            self.slab = ExpertSlab(self.residency.num_slots, E, H, I, self.dtype, self.device)
+        self._experts_desc = ops.make_experts(self.slab.data, self.slab.expert_slot, E, H, I)
+        self._cache = self.residency.cache if self.residency is not None else None
+        self._current_forward_batch_size = 0
+        self._current_forward_seq_len = 0
+        SparseContext.register_layer_block(self.layer_idx, self)
+
+    # ------------------------------------------------------------------ helpers
+    def _return_tensor_only_mlp(self) -> bool:
+        return self.moe_family == "deepseek_shared"
+
+    def _current_stage(self, seq_len: Optional[int] = None) -> str:
+        """Reference :6149-6158."""
+        phase = str(SparseContext.current_phase or "none").strip().lower()
+        if phase in ("prefill", "decode"):
+            return phase
+        seq = int(seq_len) if seq_len is not None else int(self._current_forward_seq_len or 0)
+        if seq > 0:
+            return "decode" if seq == 1 else "prefill"
+        return "decode"
+
+    def _workspace(self, T: int) -> _Workspace:
+        return _Workspace.get(T, self.top_k, self.num_experts, self.hidden_size, self.inter_size,
+                              self.shared_inter_size, self.dtype, self.logits_dtype, self.device)
+
+    # ------------------------------------------------------------------ routing
+    def _route(self, x: torch.Tensor, ws: _Workspace) -> torch.Tensor:
+        """Router logits (+ shared gate), fused softmax/top-k, permutation (:9519-9595).
+        Returns the logits, a fresh tensor the caller owns."""
+        logits = torch.empty((x.shape[0], self.num_experts), device=x.device, dtype=self.logits_dtype)
+        ops.router_logits(x, self.gate_weight, self.shared_gate_weight, self.logits_dtype, out=logits,
+                          shared_gate_out=ws.shared_gate if self.shared_gate_weight is not None else None)
+        ops.gate_topk(logits, self.top_k, self.norm_topk_prob, out_dtype=self.dtype, topv=ws.topv, topi=ws.topi)
+        if self.routed_scaling_factor != 1.0:
+            ws.topv.mul_(self.routed_scaling_factor)
+        ops.permute_build(ws.topi, self.num_experts, out=ws.perm)
+        return logits
+
+    def _routing_router(self, x: torch.Tensor):
+        """``(topv, topi, router_logits)`` like the reference's method (:9502-9595)."""
+        ws = self._workspace(int(x.shape[0]))
+        logits = self._route(x.contiguous(), ws)
+        if self.moe_family == "deepseek_shared":
+            logits = torch.full_like(logits, float("-inf"), dtype=torch.float32)
+            logits.scatter_(1, ws.topi, ws.topv.float().clamp_min(1e-12).log())
+        return ws.topv, ws.topi, logits
+
+    # ------------------------------------------------------------------ RS prefetch
+    def _rs_begin(self, x: torch.Tensor, seq_len: int, ws: _Workspace):
+        """Device half of ``_compute_and_schedule_next_layer_rs`` (:10916-11010): budget on
+        the host, predictor + top-k on the device, async copy of the top-k to the host."""
+        if self.planner_mode != "rs_prefetch" or SparseContext.rs_bank is None:
+            return None
+        if SparseContext.rs_bank_layout != "next_layer":
+            return None
+        target = self.layer_idx + 1
+        if target >= self.num_layers:
+            return None
+        src = SparseContext.rs_bank_source_layers
+        if target >= len(src) or int(src[target]) != self.layer_idx:
+            return None
+        tblk = SparseContext.layer_blocks.get(target)
+        if tblk is None or tblk.residency is None or target >= len(SparseContext.rs_bank):
+            return None
+        tres = tblk.residency
+        if int(seq_len) != 1 and not tres.cfg.rs_prefetch_prefill:
+            return None
+        tres.phase, tres.call_id = str(SparseContext.current_phase), int(SparseContext.runtime_call_id)
+        key = ("next_layer_rs", str(SparseContext.current_phase), int(SparseContext.runtime_call_id),
+               self.layer_idx, target)
+        budget = tres.prefetch_budget(key)
+        if budget <= 0:
+            return None
+        pred = SparseContext.rs_bank[target](x.float()).to(torch.float32)
+        self.metrics.rs_next_layer_pred_calls += 1
+        self.metrics.rs_mlp_calls += 1
+        pred_k = min(int(pred.shape[-1]), int(tres.predict_topk()))
+        topv, topi = torch.topk(pred, k=pred_k, dim=-1)
+        if self.norm_topk_prob:
+            topv = topv / topv.sum(dim=-1, keepdim=True).clamp_min(1e-12)
+        T = int(x.shape[0])
+        ws.host_rs_topi[:T * pred_k].view(T, pred_k).copy_(topi, non_blocking=True)
+        ws.host_rs_topv[:T * pred_k].view(T, pred_k).copy_(topv.to(x.dtype).float(), non_blocking=True)
+        return (tres, budget, T, pred_k)
+
+    def _rs_finish(self, job, ws: _Workspace) -> None:
+        """Host half: score, plan, admit; uploads go to the prefetch stream."""
+        tres, budget, T, pred_k = job
+        ids = ws.host_rs_topi[:T * pred_k].tolist()
+        probs = ws.host_rs_topv[:T * pred_k].tolist()
+        if self.metrics.events is not None:
+            self.metrics.bump("rs_plans")
+        plan = tres.schedule_prefetch(ids, probs, budget)
+        hook = getattr(self, "_rs_plan_hook", None)
+        if hook is not None:
+            hook(self.layer_idx, ids, probs, budget, plan)
+
+    # ------------------------------------------------------------------ forward
+    @torch.no_grad()
+    def forward(self, hidden_states: torch.Tensor):
+        if hidden_states.dim() != 3:
+            raise ValueError("hidden_states must be [B, S, H]")
+        B, S, H = hidden_states.shape
+        if H != self.hidden_size:
+            raise ValueError(f"hidden size {H} does not match the layer's {self.hidden_size}")
+        if hidden_states.dtype != self.dtype:
+            raise ValueError(f"hidden_states must be {self.dtype}, got {hidden_states.dtype}")
+        x = hidden_states.view(-1, H)
+        T = int(x.shape[0])
+        self._current_forward_batch_size, self._current_forward_seq_len = int(B), int(S)
+        SparseContext.current_moe_layer_idx = self.layer_idx
+        if T == 0:
+            logits = torch.empty((0, self.num_experts), device=x.device, dtype=self.logits_dtype)
+            return hidden_states if self._return_tensor_only_mlp() else (hidden_states, logits)
+        ws = self._workspace(T)
+        rs_job = self._rs_begin(x, S, ws)
+
+        logits = self._route(x, ws)
+        if self.shared_weights is not None:
+            gw, uw, dw = self.shared_weights
+            ops.shared_expert(x, gw, uw, dw, ws.shared_gate if self.shared_gate_weight is not None else None,
+                              ws.shared_inter, ws.shared_out)
+
+        if self.residency is None:
+            ops.grouped_swiglu(self._experts_desc, x, ws.topv, ws.perm, ws.segs_dev, ws.inter, ws.parts)
+        else:
+            ws.host_offsets.copy_(ws.perm.seg_offsets, non_blocking=True)
+            torch.cuda.current_stream().synchronize()
+            if rs_job is not None:
+                self._rs_finish(rs_job, ws)
+            off = ws.host_offsets.tolist()
+            segments = [(e, off[e + 1] - off[e]) for e in range(self.num_experts) if off[e + 1] > off[e]]
+            res = self.residency
+            res.phase, res.call_id = str(SparseContext.current_phase), int(SparseContext.runtime_call_id)
+            res.stage = self._current_stage(S)
+            self._backend.bind(x, ws)
+            self.last_executor = res.execute(segments)
+        if self.residency is None and rs_job is not None:
+            torch.cuda.current_stream().synchronize()
+            self._rs_finish(rs_job, ws)
+
+        out = torch.empty((T, H), device=x.device, dtype=self.dtype)
+        ops.combine(ws.parts, ws.perm, ws.shared_out, T, self.top_k, out)
+        out = out.view(B, S, H)
+        if self._return_tensor_only_mlp():
+            return out
+        return out, logits
+
+    # ------------------------------------------------------------------ lifecycle hooks
+    def _finalize_prev_group_prefetch(self) -> None:
+        if self.residency is not None:
+            self.residency.finalize_prev_group_prefetch()
+
+    def reset_runtime_state_for_new_request(self, *, clear_expert_cache: bool = False,
+                                            clear_cache_metadata: bool = True, demote_hot: bool = False) -> None:
+        """Reference :6097-6147."""
+        if self.residency is not None:
+            self.residency.reset_for_new_request(clear_expert_cache=clear_expert_cache,
+                                                 clear_cache_metadata=clear_cache_metadata)
+
+    @classmethod
+    def clear_all_expert_caches(cls) -> None:
+        for blk in SparseContext.layer_blocks.values():
+            if blk.residency is not None:
+                blk.residency.clear()
+
+    @classmethod
+    def demote_prefill_scp_transients_for_decode(cls, metrics: Optional[Any] = None) -> None:
+        """Once per request, at the prefill -> decode boundary (:16565-16601).  At world
+        size 1 no entry is ever transient, so this only flips the request flag."""
+        if SparseContext.prefill_scp_transient_demoted_for_decode:
+            return
+        resident = demoted = 0
+        for blk in SparseContext.layer_blocks.values():
+            cache = getattr(blk, "_cache", None)
+            if cache is None:
+                continue
+            resident += len(cache.prefill_scp_transient_ids())
+            demoted += int(cache.demote_prefill_scp_transients())
+        if metrics is not None:
+            metrics.bump("prefill_scp_transient_resident_at_decode_start", resident)
+            metrics.bump("prefill_scp_transient_demote_count", demoted)
+        SparseContext.prefill_scp_transient_demoted_for_decode = True
+
+    @classmethod
+    def handle_epipe_prefill_extra_cache_decode_boundary(cls, metrics: Optional[Any] = None) -> None:
+        """Drop prefill-staged payloads before decode (:16603-16640)."""
+        for blk in SparseContext.layer_blocks.values():
+            res = blk.residency
+            if res is None or res.extra_cache.capacity <= 0:
+                continue
+            for eid in res.extra_cache.resident_ids():
+                res._release_slot(res.extra_cache.peek(eid))
+            n = res.extra_cache.clear()
+            if metrics is not None:
+                metrics.bump("epipe_prefill_extra_cache_cleared", n)

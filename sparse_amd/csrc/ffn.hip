@@ -34,7 +34,7 @@ static int check_routed(const char* fn, const sparse_hip_experts* ex, const void
                  ex->slot_stride % 16 == 0,
              "%s: slot_stride=%llu too small or not 16-byte aligned", fn,
              static_cast<unsigned long long>(ex->slot_stride));
-  SP_REQUIRE(ex->slab_dev && ex->expert_slot_dev, "%s: NULL weight slab or slot table", fn);
+  SP_REQUIRE(ex->slab_dev != nullptr, "%s: NULL weight slab", fn);
   SP_REQUIRE((reinterpret_cast<uintptr_t>(ex->slab_dev) & 15) == 0, "%s: slab not 16-byte aligned", fn);
   SP_REQUIRE(T >= 1, "%s: T=%d must be >= 1", fn, T);
   SP_REQUIRE(K >= 1 && K <= SPARSE_HIP_MAX_TOPK, "%s: K=%d outside [1,%d]", fn, K, SPARSE_HIP_MAX_TOPK);
@@ -47,9 +47,13 @@ static int check_routed(const char* fn, const sparse_hip_experts* ex, const void
   SP_REQUIRE(segs->eids_dev == nullptr || segs->count_dev != nullptr, "%s: device segment list without count",
              fn);
   if (segs->eids_dev == nullptr) {
-    for (int i = 0; i < segs->n; ++i)
+    for (int i = 0; i < segs->n; ++i) {
       SP_REQUIRE(segs->eids[i] >= 0 && segs->eids[i] < ex->num_experts, "%s: segment %d names expert %d", fn, i,
                  static_cast<int>(segs->eids[i]));
+      SP_REQUIRE(segs->slots[i] >= 0, "%s: segment %d has slot %d", fn, i, static_cast<int>(segs->slots[i]));
+    }
+  } else {
+    SP_REQUIRE(ex->expert_slot_dev != nullptr, "%s: device segment list needs expert_slot_dev", fn);
   }
   return SPARSE_HIP_OK;
 }

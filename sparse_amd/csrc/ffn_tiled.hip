@@ -41,7 +41,7 @@ __global__ __launch_bounds__(kTlThreads) void ffn_tiled_kernel(const TiledArgs a
   constexpr int NM = kGateUp ? 2 : 1;
   __shared__ float As[kTlBK][kTlBM + 4];
   __shared__ float Bs[NM][kTlBK][kTlBN + 4];
-  __shared__ int32_t s_seg[3];  // eid, first row, rows
+  __shared__ int32_t s_seg[4];  // eid, first row, rows, slot
 
   const int tid = threadIdx.x;
   const int bn = blockIdx.x % a.ntiles_n;
@@ -49,7 +49,7 @@ __global__ __launch_bounds__(kTlThreads) void ffn_tiled_kernel(const TiledArgs a
 
   // ---- find (segment, m-tile) ------------------------------------------------
   if (tid == 0) {
-    int eid = -1, r0 = 0, M = 0;
+    int eid = -1, r0 = 0, M = 0, slot_id = 0;
     if (a.shared) {
       if (bm_global * kTlBM < a.T) {
         eid = 0;
@@ -66,6 +66,7 @@ __global__ __launch_bounds__(kTlThreads) void ffn_tiled_kernel(const TiledArgs a
         const int nt = (m + kTlBM - 1) / kTlBM;
         if (left < nt) {
           eid = e;
+          slot_id = (a.segs.eids_dev != nullptr) ? a.expert_slot[e] : a.segs.slots[s];
           r0 = b + left * kTlBM;
           M = min(kTlBM, m - left * kTlBM);
           break;
@@ -76,6 +77,7 @@ __global__ __launch_bounds__(kTlThreads) void ffn_tiled_kernel(const TiledArgs a
     s_seg[0] = eid;
     s_seg[1] = r0;
     s_seg[2] = M;
+    s_seg[3] = slot_id;
   }
   __syncthreads();
   const int eid = s_seg[0], r0 = s_seg[1], M = s_seg[2];
@@ -87,7 +89,7 @@ __global__ __launch_bounds__(kTlThreads) void ffn_tiled_kernel(const TiledArgs a
     w0 = static_cast<const T*>(a.w_s);
     w1 = static_cast<const T*>(a.w2_s);
   } else {
-    const T* slot = static_cast<const T*>(a.slab) + static_cast<uint64_t>(a.expert_slot[eid]) * a.slot_stride;
+    const T* slot = static_cast<const T*>(a.slab) + static_cast<uint64_t>(s_seg[3]) * a.slot_stride;
     w0 = slot + a.mat_offset;
     w1 = slot + a.mat2_offset;
   }

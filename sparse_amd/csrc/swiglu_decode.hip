@@ -78,14 +78,16 @@ __global__ __launch_bounds__(kDecThreads) void decode_ffn_kernel(const DecodeArg
   } else {
     const int b = blockIdx.x - a.tiles_s;
     const int si = b / a.tiles_r;
-    int eid;
+    int eid, slot_id;
     if (a.segs.eids_dev != nullptr) {
       const int cnt = min(a.segs.count_dev[0], a.segs.n);
       if (si >= cnt) return;
       eid = a.segs.eids_dev[si];
+      slot_id = a.expert_slot[eid];
     } else {
       if (si >= a.segs.n) return;
       eid = a.segs.eids[si];
+      slot_id = a.segs.slots[si];
     }
     Kdim = a.Kdim;
     Ndim = a.Ndim;
@@ -93,7 +95,7 @@ __global__ __launch_bounds__(kDecThreads) void decode_ffn_kernel(const DecodeArg
     r0 = a.seg_offsets[eid];
     M = a.seg_offsets[eid + 1] - r0;
     if (M <= 0) return;
-    const uint16_t* slot = a.slab + static_cast<uint64_t>(a.expert_slot[eid]) * a.slot_stride;
+    const uint16_t* slot = a.slab + static_cast<uint64_t>(slot_id) * a.slot_stride;
     w0 = slot + a.mat_offset;
     w1 = slot + a.mat2_offset;
   }

@@ -58,7 +58,7 @@ template <bool kGateUp>
 __global__ __launch_bounds__(kPfThreads, 2) void prefill_ffn_kernel(const PrefillArgs a) {
   __shared__ __attribute__((aligned(16))) uint8_t lds[kPfLdsA + kPfLdsB];
   __shared__ float s_scale[kPfBM];
-  __shared__ int32_t s_seg[4];  // eid, first row, rows, n-tile
+  __shared__ int32_t s_seg[5];  // eid, first row, rows, n-tile, slot
 
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63;
@@ -69,7 +69,7 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_ffn_kernel(const Prefil
     const int nblk = gridDim.x;
     const int per_xcd = (nblk + kPfXcds - 1) / kPfXcds;
     const int logical = (blockIdx.x % kPfXcds) * per_xcd + blockIdx.x / kPfXcds;
-    int eid = -1, r0 = 0, M = 0, bn = 0;
+    int eid = -1, r0 = 0, M = 0, bn = 0, slot_id = 0;
     if (a.shared) {
       // n-tile major, m fastest
       const int mt = (a.T + kPfBM - 1) / kPfBM;
@@ -93,6 +93,7 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_ffn_kernel(const Prefil
           bn = left / mt;
           const int bm = left - bn * mt;
           eid = e;
+          slot_id = (a.segs.eids_dev != nullptr) ? a.expert_slot[e] : a.segs.slots[s];
           r0 = b + bm * kPfBM;
           M = min(kPfBM, m - bm * kPfBM);
           break;
@@ -104,6 +105,7 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_ffn_kernel(const Prefil
     s_seg[1] = r0;
     s_seg[2] = M;
     s_seg[3] = bn;
+    s_seg[4] = slot_id;
   }
   __syncthreads();
   const int eid = s_seg[0], r0 = s_seg[1], M = s_seg[2], bn = s_seg[3];
@@ -115,7 +117,7 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_ffn_kernel(const Prefil
     w0 = a.w_s;
     w1 = a.w2_s;
   } else {
-    const uint16_t* slot = a.slab + static_cast<uint64_t>(a.expert_slot[eid]) * a.slot_stride;
+    const uint16_t* slot = a.slab + static_cast<uint64_t>(s_seg[4]) * a.slot_stride;
     w0 = slot + a.mat_offset;
     w1 = slot + a.mat2_offset;
   }

@@ -139,8 +139,9 @@ def seglist_device(perm: Permutation, max_segments: int) -> SegList:
     return s
 
 
-def seglist_host(eids: Sequence[int]) -> SegList:
-    """Segment list passed by value, in the given execution order."""
+def seglist_host(eids: Sequence[int], slots: Optional[Sequence[int]] = None) -> SegList:
+    """Segment list passed by value, in the given execution order; ``slots[i]`` is the slab
+    slot holding ``eids[i]`` (default: slot == expert id)."""
     s = SegList()
     s.eids_dev = None
     s.count_dev = None
@@ -149,6 +150,7 @@ def seglist_host(eids: Sequence[int]) -> SegList:
         raise ValueError("too many segments")
     for i, e in enumerate(eids):
         s.eids[i] = int(e)
+        s.slots[i] = int(e) if slots is None else int(slots[i])
     return s
 
 

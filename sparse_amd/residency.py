@@ -1,0 +1,871 @@
+"""Per-layer expert residency: HBM slot pool, demand loads, RS prefetch planning and
+EPIPE readiness-ordered execution.
+
+Pure Python over a small device ``Backend`` (uploads, events, kernel launches), so the
+whole state machine also runs on the CPU with a fake backend.  Behaviour follows the
+reference's block methods (utils/eval_core.py): demand path :11388-11435, prefetch cycle
+:9619-9665, budget :9754-9810, scoring and planning :10031-10262, admission :10433-10527,
+EPIPE upfront scan :11867-12167 and residual scan :12169-12512.  Cache hit / miss events
+and the resulting residency are the same as the reference's for the same accesses; what
+differs is physical: an expert lives in a numbered HBM slot, experts of one call are run
+in batched launches, and a slot is reused only after the launches that read it.
+
+Slots.  ``capacity`` cache slots plus ``staging_slots`` spares.  A spare holds an expert
+that the policy has already evicted but an un-launched batch still reads, or an EPIPE
+transient.  When no slot is free the pending batch is launched, which releases them.
+"""
+from __future__ import annotations
+
+import os
+from dataclasses import dataclass, field
+from typing import Any, Callable, Dict, List, Optional, Sequence, Set, Tuple
+
+from .cache import EpipePrefillExtraCache, ExpertWeightCache
+from .context import Metrics
+
+Segment = Tuple[int, int]  # (expert id, routed rows)
+
+
+def _env_flag(name: str, default: str) -> bool:
+    return str(os.environ.get(name, default)).strip().lower() in ("1", "true", "yes", "on")
+
+
+def _env_int(name: str, default: int) -> int:
+    try:
+        return int(os.environ.get(name, str(default)) or default)
+    except ValueError:
+        return int(default)
+
+
+def _env_float(name: str, default: float) -> float:
+    try:
+        return float(os.environ.get(name, str(default)) or default)
+    except ValueError:
+        return float(default)
+
+
+@dataclass
+class ResidencyConfig:
+    """Knobs of the cache / prefetch / EPIPE machinery with the reference's defaults
+    (utils/eval_core.py:4939-5075); ``from_env`` reads the same ``SPARSE_*`` variables."""
+
+    capacity: int = 10
+    staging_slots: int = 4
+    planner_mode: str = "none"            # none | rs_prefetch
+    prefetch_top_m: int = 4
+    pred_topk: Optional[int] = None        # SPARSE_RS_PREFETCH_PRED_TOPK
+    rs_policy: str = "default"             # default | cache_safe
+    min_candidate_score: float = 0.02
+    replace_advantage: float = 0.02
+    replace_margin: float = 1.05
+    cache_safe_min_score: float = 0.03
+    cache_safe_replace_advantage: float = 0.05
+    cache_safe_replace_margin: float = 1.10
+    allow_active_replace: bool = True
+    recent_protect_steps: int = 0
+    protect_mode: str = "default"
+    wait_before_evict: bool = True
+    rs_prefetch_prefill: bool = False
+    cache_ttl_steps: int = 0
+    # EPIPE
+    epipe_enable: bool = False
+    epipe_prefill_enable: bool = False
+    epipe_mode: str = "upfront_scan"
+    epipe_decode_rs_mode: str = "late_only"
+    epipe_no_evict: bool = True
+    epipe_transient_staging: bool = True
+    epipe_max_staged_experts: int = 1
+    epipe_min_ready_experts: int = 1
+    epipe_min_ready_items: int = 1
+    epipe_min_missing_experts: int = 1
+    epipe_sort_ready_by_work: bool = False
+    epipe_prefill_commit: bool = True
+    epipe_rs_handle_late_prefetch: bool = True
+    epipe_rs_handle_demand_miss: bool = False
+    epipe_rs_force_demand_stage: bool = False
+    epipe_rs_demand_commit: bool = True
+    epipe_deferred_lru_commit: bool = True
+    epipe_rs_min_buffer_groups: int = 1
+    epipe_rs_min_buffer_items: int = 1
+    epipe_rs_rolling_gate: bool = True
+    epipe_rs_gate_window: int = 16
+    epipe_rs_gate_min_triggers: int = 1
+    epipe_rs_gate_skip_steps: int = 8
+    epipe_prefill_extra_cache_slots: int = 0
+    # execution order for plain EP: unique_mask | full_mask | sorted_segment (same events)
+    plain_ep_exec_mode: str = "unique_mask"
+
+    @classmethod
+    def from_env(cls, **overrides) -> "ResidencyConfig":
+        c = cls()
+        c.staging_slots = max(1, _env_int("SPARSE_HIP_STAGING_SLOTS", c.staging_slots))
+        raw = os.environ.get("SPARSE_RS_PREFETCH_PRED_TOPK", "").strip()
+        c.pred_topk = int(raw) if raw else None
+        c.rs_policy = str(os.environ.get("SPARSE_RS_PREFETCH_POLICY", "default") or "default").strip().lower()
+        c.min_candidate_score = _env_float("SPARSE_PREFETCH_MIN_CAND_SCORE", 0.02)
+        c.replace_advantage = _env_float("SPARSE_PREFETCH_REPLACE_ADVANTAGE", 0.02)
+        c.replace_margin = _env_float("SPARSE_PREFETCH_REPLACE_MARGIN", 1.05)
+        c.cache_safe_min_score = _env_float("SPARSE_RS_CACHE_SAFE_MIN_SCORE", 0.03)
+        c.cache_safe_replace_advantage = _env_float("SPARSE_RS_CACHE_SAFE_REPLACE_ADVANTAGE", 0.05)
+        c.cache_safe_replace_margin = _env_float("SPARSE_RS_CACHE_SAFE_REPLACE_MARGIN", 1.10)
+        c.allow_active_replace = _env_flag("SPARSE_PREFETCH_ALLOW_ACTIVE_REPLACE", "1")
+        c.recent_protect_steps = _env_int("SPARSE_RS_PREFETCH_RECENT_PROTECT_STEPS", 0)
+        c.protect_mode = str(os.environ.get("SPARSE_PREFETCH_PROTECT_MODE", "default") or "default").strip().lower()
+        c.wait_before_evict = _env_flag("SPARSE_PREFETCH_WAIT_BEFORE_EVICT", "1")
+        c.rs_prefetch_prefill = _env_flag("SPARSE_RS_PREFETCH_PREFILL", "0")
+        c.cache_ttl_steps = _env_int("SPARSE_CACHE_TTL_STEPS", 0)
+        c.epipe_enable = _env_flag("SPARSE_EPIPE_ENABLE", "0")
+        c.epipe_prefill_enable = _env_flag("SPARSE_EPIPE_PREFILL_ENABLE", "0")
+        c.epipe_mode = str(os.environ.get("SPARSE_EPIPE_MODE", "upfront_scan") or "upfront_scan").strip().lower()
+        c.epipe_decode_rs_mode = str(
+            os.environ.get("SPARSE_EPIPE_DECODE_RS_MODE", "late_only") or "late_only").strip().lower()
+        c.epipe_no_evict = _env_flag("SPARSE_EPIPE_NO_EVICT", "1")
+        c.epipe_transient_staging = _env_flag("SPARSE_EPIPE_TRANSIENT_STAGING", "1")
+        c.epipe_max_staged_experts = _env_int("SPARSE_EPIPE_MAX_STAGED_EXPERTS", 1)
+        c.epipe_sort_ready_by_work = _env_flag("SPARSE_EPIPE_SORT_READY_BY_WORK", "0")
+        c.epipe_prefill_commit = _env_flag("SPARSE_EPIPE_PREFILL_COMMIT", "1")
+        c.epipe_rs_handle_late_prefetch = _env_flag("SPARSE_EPIPE_RS_HANDLE_LATE_PREFETCH", "1")
+        c.epipe_rs_handle_demand_miss = _env_flag("SPARSE_EPIPE_RS_HANDLE_DEMAND_MISS", "0")
+        c.epipe_rs_force_demand_stage = _env_flag("SPARSE_EPIPE_RS_FORCE_DEMAND_STAGE", "0")
+        c.epipe_rs_min_buffer_groups = _env_int("SPARSE_EPIPE_RS_MIN_BUFFER_GROUPS", 1)
+        c.epipe_rs_min_buffer_items = _env_int("SPARSE_EPIPE_RS_MIN_BUFFER_ITEMS", 1)
+        c.epipe_rs_rolling_gate = _env_flag("SPARSE_EPIPE_RS_ROLLING_GATE", "1")
+        c.epipe_rs_gate_window = _env_int("SPARSE_EPIPE_RS_GATE_WINDOW", 16)
+        c.epipe_rs_gate_min_triggers = _env_int("SPARSE_EPIPE_RS_GATE_MIN_TRIGGERS", 1)
+        c.epipe_rs_gate_skip_steps = _env_int("SPARSE_EPIPE_RS_GATE_SKIP_STEPS", 8)
+        c.epipe_prefill_extra_cache_slots = _env_int("SPARSE_EPIPE_PREFILL_EXTRA_CACHE_SLOTS", 0)
+        c.plain_ep_exec_mode = str(
+            os.environ.get("SPARSE_PLAIN_EP_EXEC_MODE", "unique_mask") or "unique_mask").strip().lower()
+        for k, v in overrides.items():
+            if not hasattr(c, k):
+                raise ValueError(f"unknown residency option {k}")
+            setattr(c, k, v)
+        return c
+
+
+class Backend:
+    """Device services the policy needs.  Lanes: ``compute`` (the stream the layer's
+    kernels run on), ``prefetch`` and ``epipe`` (side streams for uploads)."""
+
+    def upload(self, eid: int, slot: int, lane: str) -> Any:
+        """Enqueue the H2D copy of expert ``eid`` into ``slot`` on ``lane``; return an event
+        recorded behind the copy."""
+        raise NotImplementedError
+
+    def event_done(self, event: Any) -> bool:
+        raise NotImplementedError
+
+    def wait_event(self, event: Any, lane: str) -> None:
+        """Make ``lane`` wait for ``event`` (never blocks the host)."""
+        raise NotImplementedError
+
+    def run_segments(self, segments: Sequence[Tuple[int, int]]) -> None:
+        """Launch the expert FFN for ``(expert id, slot)`` pairs, in this order."""
+        raise NotImplementedError
+
+    def fence(self) -> Any:
+        """Event recorded on the compute lane now."""
+        raise NotImplementedError
+
+    def free_device_bytes(self) -> Optional[int]:
+        return None
+
+
+class LayerResidency:
+    """Residency state of one layer's routed experts."""
+
+    def __init__(self, layer_idx: int, num_experts: int, top_k: int, config: ResidencyConfig,
+                 backend: Backend, metrics: Optional[Metrics] = None, expert_bytes: int = 0) -> None:
+        self.layer_idx = int(layer_idx)
+        self.num_experts = int(num_experts)
+        self.top_k = int(top_k)
+        self.cfg = config
+        self.backend = backend
+        self.metrics = metrics if metrics is not None else Metrics()
+        self.expert_bytes = int(expert_bytes)
+        self.cache = ExpertWeightCache(int(config.capacity))
+        self.extra_cache = EpipePrefillExtraCache(int(config.epipe_prefill_extra_cache_slots))
+        self.num_slots = max(0, int(config.capacity)) + max(1, int(config.staging_slots)) + \
+            max(0, int(config.epipe_prefill_extra_cache_slots))
+        self._free_slots: List[int] = list(range(self.num_slots - 1, -1, -1))
+        self._retired: List[int] = []           # evicted, still read by the pending batch
+        self._pending: List[Tuple[int, int]] = []  # (eid, slot) not launched yet
+        self._pending_slots: Set[int] = set()
+        self._slot_fence: Dict[int, Any] = {}    # compute-lane event after the last read
+        self._slot_upload: Dict[int, Tuple[Any, str]] = {}  # last upload (event, lane)
+        self._slot_of: Dict[int, int] = {}       # resident expert -> slot (mirrors the cache)
+        # prefetch cycle state (reference :5056-5083)
+        self.prefetched_ids: Set[int] = set()
+        self.prefetch_used_ids: Set[int] = set()
+        self.prefetch_events: Dict[int, Any] = {}
+        self.cycle_key: Optional[Tuple[Any, ...]] = None
+        self.access_freq: Dict[int, int] = {}
+        self.last_used_decode_step: Dict[int, int] = {}
+        # rolling gate of the residual scan (reference :4989-4998)
+        self._gate_calls = 0
+        self._gate_triggers = 0
+        self._gate_skip_remaining = 0
+        # harness state, set by the block before each call
+        self.phase = "none"
+        self.call_id = -1
+        self.stage = "decode"
+
+    # ------------------------------------------------------------------ events / counters
+    def _event(self, kind: str, eid: int) -> None:
+        m = self.metrics
+        if kind == "hit":
+            m.cache_hit_count += 1
+        elif kind == "prefetch_hit":
+            m.prefetch_hit_count += 1
+        else:
+            m.cache_miss_count += 1
+        if m.events is not None:
+            m.events.append((kind, self.layer_idx, int(eid)))
+
+    # ------------------------------------------------------------------ slot pool
+    def _release_slot(self, slot: int) -> None:
+        if slot in self._pending_slots:
+            self._retired.append(slot)
+        else:
+            self._free_slots.append(slot)
+
+    def _acquire_slot(self) -> int:
+        if not self._free_slots:
+            self.flush()
+        if not self._free_slots:
+            raise RuntimeError(
+                f"Insufficient HBM slots before expert H2D: layer={self.layer_idx} "
+                f"slots={self.num_slots} capacity={self.cache.capacity}")
+        return self._free_slots.pop()
+
+    def _upload(self, eid: int, slot: int, lane: str) -> Any:
+        fence = self._slot_fence.pop(slot, None)
+        if fence is not None and lane != "compute":
+            self.backend.wait_event(fence, lane)
+        prev = self._slot_upload.get(slot)
+        if prev is not None and prev[1] != lane:
+            self.backend.wait_event(prev[0], lane)
+        ev = self.backend.upload(int(eid), int(slot), lane)
+        self._slot_upload[slot] = (ev, lane)
+        return ev
+
+    def _enqueue(self, eid: int, slot: int) -> None:
+        self._pending.append((int(eid), int(slot)))
+        self._pending_slots.add(int(slot))
+
+    def flush(self) -> None:
+        """Launch the pending batch; slots it alone kept alive become free."""
+        if self._pending:
+            self.backend.run_segments(self._pending)
+            fence = self.backend.fence()
+            for _eid, slot in self._pending:
+                self._slot_fence[slot] = fence
+            self._pending = []
+            self._pending_slots = set()
+        if self._retired:
+            self._free_slots.extend(self._retired)
+            self._retired = []
+
+    # ------------------------------------------------------------------ demand path
+    def _cache_protect_ids(self) -> Set[int]:
+        """TTL protection (reference :5929-5938); off by default."""
+        protect: Set[int] = set()
+        ttl = int(self.cfg.cache_ttl_steps)
+        if ttl > 0 and self.phase == "decode" and self.call_id >= 0:
+            for eid, last in self.last_used_decode_step.items():
+                if self.call_id - int(last) <= ttl:
+                    protect.add(int(eid))
+        return protect
+
+    def _protect_with_fallback(self, new_eid: int) -> Set[int]:
+        protect = self._cache_protect_ids()
+        protect.discard(int(new_eid))
+        resident = set(self.cache.resident_ids())
+        if resident and resident.issubset(protect):
+            self.metrics.bump("cache_eviction_fallback_all_protected")
+            return set()
+        return protect
+
+    def _on_demand_access(self, eid: int) -> None:
+        """Reference :11213-11221."""
+        self.access_freq[eid] = int(self.access_freq.get(eid, 0)) + 1
+        if self.phase == "decode":
+            self.last_used_decode_step[int(eid)] = int(self.call_id)
+        if self.access_freq[eid] >= 2:
+            self.cache.promote_hot(eid)
+
+    def _sync_slots(self) -> None:
+        """Release the slot of every expert the cache no longer holds."""
+        if len(self._slot_of) == len(self.cache):
+            return
+        for eid in [e for e in self._slot_of if not self.cache.has(e)]:
+            self.prefetch_events.pop(eid, None)
+            self._release_slot(self._slot_of.pop(eid))
+
+    def _cache_put(self, eid: int, slot: int) -> None:
+        """``_cache_put_guarded`` (reference :5985-6022) plus slot bookkeeping."""
+        if self.cache.capacity <= 0:
+            # nothing is ever stored: the slot only lives until the batch is launched
+            self._pending_slots.add(slot)
+            self._retired.append(slot)
+            return
+        protect = self._protect_with_fallback(eid)
+        self.cache.put(int(eid), slot, pinned=False, protect_ids=protect)
+        self._slot_of[int(eid)] = slot
+        self._sync_slots()
+
+    def _record_cached_use(self, eid: int, wait_prefetch: bool) -> None:
+        """Hit accounting shared by the demand path and EPIPE (reference :11395-11412,
+        :11652-11670)."""
+        if eid in self.prefetched_ids:
+            self._event("prefetch_hit", eid)
+            self.prefetch_used_ids.add(eid)
+            self.cache.unpin(eid)
+            self.cache.promote_hot(eid)
+        else:
+            self._event("hit", eid)
+        if wait_prefetch:
+            self._maybe_wait_prefetch(eid)
+
+    def _maybe_wait_prefetch(self, eid: int) -> None:
+        """Reference :11176-11210: the compute lane waits the copy event, the host never."""
+        ev = self.prefetch_events.pop(eid, None)
+        if ev is None:
+            return
+        if self.backend.event_done(ev):
+            self.metrics.prefetch_complete_before_use_count += 1
+        self.backend.wait_event(ev, "compute")
+        self.metrics.prefetch_completed_count += 1
+
+    def _demand(self, eid: int) -> int:
+        """``_get_local_module_weights`` (reference :11388-11435): returns the slot."""
+        slot = self.cache.get(eid)
+        if slot is not None:
+            self._record_cached_use(eid, wait_prefetch=True)
+            return slot
+        extra = self.extra_cache.get(eid)
+        if extra is not None:
+            return extra
+        self._event("miss", eid)
+        slot = self._acquire_slot()
+        self._upload(eid, slot, "compute")
+        self.metrics.demand_h2d_bytes += self.expert_bytes
+        self._on_demand_access(eid)
+        self._cache_put(eid, slot)
+        return slot
+
+    def _compute(self, eid: int, slot: Optional[int] = None) -> None:
+        """Queue expert ``eid`` for execution, loading it on demand when no slot is given."""
+        if slot is None:
+            slot = self._demand(eid)
+        self._enqueue(eid, slot)
+
+    # ------------------------------------------------------------------ executors
+    def execute(self, segments: Sequence[Segment]) -> str:
+        """Run the routed experts of one call; ``segments`` is ``(eid, rows)`` ascending by
+        expert id.  Picks the executor like ``_execute_local_recv_groups`` (reference
+        :13264-13357) and returns its name."""
+        if not segments:
+            return "empty"
+        name = None
+        if self._epipe_stage_enabled() and self.cfg.epipe_mode != "off":
+            rs_active = self.cfg.planner_mode == "rs_prefetch"
+            mode = self.cfg.epipe_decode_rs_mode
+            if self.stage == "decode" and rs_active and mode == "off":
+                name = None
+            elif self.stage == "decode" and rs_active and mode == "residual_scan":
+                name = self._epipe_rs_residual_scan(segments)
+            elif self.stage == "decode" and rs_active:
+                raise NotImplementedError(
+                    f"SPARSE_EPIPE_DECODE_RS_MODE={mode} is not built; use off or residual_scan")
+            elif self.stage == "decode" and self.cfg.epipe_mode != "miss_triggered":
+                name = self._epipe_upfront_scan(segments)
+            elif self.cfg.epipe_mode == "upfront_scan":
+                name = self._epipe_upfront_scan(segments)
+            else:
+                raise NotImplementedError("SPARSE_EPIPE_MODE=miss_triggered is not built")
+        if name is None:
+            for eid, _rows in segments:
+                self._compute(eid)
+            name = "plain"
+        self.flush()
+        return name
+
+    def _epipe_stage_enabled(self) -> bool:
+        """Reference :5585-5598 (shadow modes are not built)."""
+        if self.stage == "prefill":
+            return bool(self.cfg.epipe_prefill_enable)
+        if self.stage == "decode":
+            if self.cfg.planner_mode == "rs_prefetch":
+                return bool(self.cfg.epipe_enable and self.cfg.epipe_decode_rs_mode not in ("off", "disabled"))
+            return bool(self.cfg.epipe_enable)
+        return False
+
+    def _contains_no_touch(self, eid: int) -> bool:
+        """Reference :5815-5851."""
+        return self.extra_cache.has(eid) or self.cache.has(eid)
+
+    def _headroom_ok(self) -> bool:
+        """A transient needs a slot that no cache entry owns."""
+        return bool(self._free_slots) or bool(self._retired) or bool(self._pending)
+
+    def _fallback(self, reason: str) -> None:
+        self.metrics.bump("epipe_fallback_count")
+        if reason:
+            self.metrics.bump(reason)
+
+    # ---- EPIPE without RS, and prefill: upfront scan (reference :11867-12167) ----------
+    def _epipe_upfront_scan(self, segments: Sequence[Segment]) -> Optional[str]:
+        cfg, m = self.cfg, self.metrics
+        stage = self.stage
+        enabled = bool(cfg.epipe_enable if stage == "decode" else cfg.epipe_prefill_enable)
+        if not enabled:
+            return None
+        ready = [s for s in segments if self._contains_no_touch(s[0])]
+        missing = [s for s in segments if not self._contains_no_touch(s[0])]
+        ready_items = sum(r for _, r in ready)
+        free_cache_slots = max(0, self.cache.capacity - len(self.cache))
+        if not cfg.epipe_no_evict:
+            raise NotImplementedError("SPARSE_EPIPE_NO_EVICT=0 is not implemented in EPIPE-Lite.")
+        if cfg.epipe_max_staged_experts != 1:
+            raise NotImplementedError("EPIPE-Lite currently supports only one staged missing expert.")
+        if len(ready) < cfg.epipe_min_ready_experts or ready_items < cfg.epipe_min_ready_items:
+            self._fallback("epipe_fallback_no_ready")
+            return None
+        if len(missing) < cfg.epipe_min_missing_experts:
+            self._fallback("epipe_fallback_no_missing")
+            return None
+        staged_eid = missing[0][0]
+        can_insert = free_cache_slots > 0 and not (stage == "prefill" and not cfg.epipe_prefill_commit)
+        use_transient = not can_insert
+        if use_transient:
+            if not cfg.epipe_transient_staging:
+                self._fallback("epipe_fallback_cache_full_no_temp")
+                return None
+            if not self._headroom_ok():
+                self._fallback("epipe_fallback_no_memory_headroom")
+                return None
+        # stage the first missing expert on the EPIPE lane
+        slot = self._acquire_slot()
+        stage_event = self._upload(staged_eid, slot, "epipe")
+        ready_order = list(ready)
+        if cfg.epipe_sort_ready_by_work:
+            ready_order.sort(key=lambda s: s[1], reverse=True)
+        for eid, _rows in ready_order:
+            self._compute(eid)
+        # the ready batch must be on the device before the compute lane waits the copy
+        self.flush()
+        self.backend.wait_event(stage_event, "compute")
+        self._event("miss", staged_eid)
+        if stage != "prefill":
+            self._on_demand_access(staged_eid)
+        m.demand_h2d_bytes += self.expert_bytes
+        m.bump("epipe_staged_missing_count")
+        m.bump("epipe_enabled_count")
+        kept = False  # does some cache keep the staged slot alive after this call?
+        if can_insert:
+            if len(self.cache) < self.cache.capacity:
+                if stage == "prefill":
+                    self._on_demand_access(staged_eid)
+                self._enqueue(staged_eid, slot)
+                self._cache_put(staged_eid, slot)
+                m.bump("epipe_cache_insert_count")
+                kept = True
+            else:
+                use_transient = True
+        if not kept:
+            self._enqueue(staged_eid, slot)
+            if use_transient and stage == "prefill" and self.extra_cache.capacity > 0:
+                old_extra = {e: self.extra_cache.peek(e) for e in self.extra_cache.resident_ids()}
+                kept, _upd, _ev = self.extra_cache.put(staged_eid, slot, nbytes=self.expert_bytes)
+                for e, s_old in old_extra.items():
+                    if not self.extra_cache.has(e) or (e == staged_eid and s_old != slot):
+                        self._release_slot(s_old)
+            if not kept:
+                m.bump("epipe_transient_payload_count")
+                self._retired.append(slot)  # back to the pool once this batch is launched
+        for eid, _rows in missing[1:]:
+            self._compute(eid)
+        return "epipe_upfront"
+
+    # ---- EPIPE on top of RS prefetch: residual scan (reference :12169-12512) -----------
+    def _pending_prefetch_event(self, eid: int):
+        """Reference :11636-11650: an event that is still in flight, else None."""
+        ev = self.prefetch_events.get(eid)
+        if ev is None:
+            return None
+        if self.backend.event_done(ev):
+            self.prefetch_events.pop(eid, None)
+            self.metrics.prefetch_complete_before_use_count += 1
+            self.metrics.prefetch_completed_count += 1
+            return None
+        return ev
+
+    def _demand_gate_can_open(self) -> bool:
+        """Reference :5880-5893; the exposed-stall threshold variant is not built."""
+        return bool(self.cfg.epipe_rs_handle_demand_miss and self.cfg.epipe_rs_force_demand_stage)
+
+    def _residual_present(self, segments: Sequence[Segment]) -> bool:
+        for eid, _rows in segments:
+            ev = self.prefetch_events.get(eid)
+            if ev is not None and self.cfg.epipe_rs_handle_late_prefetch and not self.backend.event_done(ev):
+                return True
+            if self._demand_gate_can_open() and not self._contains_no_touch(eid):
+                return True
+        return False
+
+    def _maybe_skip_gate(self, segments: Sequence[Segment]) -> bool:
+        cfg = self.cfg
+        if not cfg.epipe_rs_rolling_gate:
+            return False
+        if self._gate_skip_remaining > 0:
+            if self._residual_present(segments):
+                self._gate_skip_remaining = 0
+                self.metrics.bump("epipe_rs_gate_reenable_count")
+                return False
+            self._gate_skip_remaining -= 1
+            self.metrics.bump("epipe_rs_gate_skip_count")
+            return True
+        self._gate_calls += 1
+        if self._gate_calls >= cfg.epipe_rs_gate_window and self._gate_triggers < cfg.epipe_rs_gate_min_triggers:
+            self._gate_calls = 0
+            self._gate_triggers = 0
+            self._gate_skip_remaining = int(cfg.epipe_rs_gate_skip_steps)
+            if self._gate_skip_remaining > 0:
+                self.metrics.bump("epipe_rs_gate_skip_count")
+                self._gate_skip_remaining -= 1
+                return True
+        if self._gate_calls >= cfg.epipe_rs_gate_window:
+            self._gate_calls = 0
+            self._gate_triggers = 0
+        return False
+
+    def _epipe_rs_residual_scan(self, segments: Sequence[Segment]) -> Optional[str]:
+        cfg, m = self.cfg, self.metrics
+        if self.stage != "decode" or cfg.planner_mode != "rs_prefetch" or not cfg.epipe_enable:
+            return None
+        m.bump("epipe_rs_residual_scan_calls")
+        if self._maybe_skip_gate(segments):
+            return None
+        ready_idx: List[int] = []
+        late_idx: List[int] = []
+        demand_idx: List[int] = []
+        for i, (eid, _rows) in enumerate(segments):
+            pending_ev = self._pending_prefetch_event(eid)
+            cached = self._contains_no_touch(eid)
+            if cached and pending_ev is None:
+                ready_idx.append(i)
+            elif cached and pending_ev is not None and cfg.epipe_rs_handle_late_prefetch:
+                late_idx.append(i)
+            elif (not cached) and cfg.epipe_rs_handle_demand_miss and self._demand_gate_can_open():
+                demand_idx.append(i)
+        ready_items = sum(segments[i][1] for i in ready_idx)
+        if len(ready_idx) < cfg.epipe_rs_min_buffer_groups or ready_items < cfg.epipe_rs_min_buffer_items:
+            m.bump("epipe_rs_residual_scan_no_ready_count")
+            return None
+        residual: Optional[int] = None
+        kind = ""
+        if late_idx:
+            residual, kind = late_idx[0], "late"
+        elif demand_idx and self._demand_gate_open(ready_items):
+            residual, kind = demand_idx[0], "demand"
+        if residual is None:
+            m.bump("epipe_fallback_no_miss_trigger")
+            return None
+        residual_eid = segments[residual][0]
+        cover = [i for i in ready_idx if i != residual]
+        if len(cover) < cfg.epipe_rs_min_buffer_groups:
+            m.bump("epipe_rs_residual_scan_no_ready_count")
+            return None
+        m.bump("epipe_rs_trigger_count")
+        m.bump("epipe_rs_residual_scan_late_count" if kind == "late" else "epipe_rs_residual_scan_demand_count")
+        if cfg.epipe_rs_rolling_gate:
+            self._gate_triggers += 1
+
+        def compute_ready(indices: Sequence[int]) -> None:
+            for i in indices:
+                eid = segments[i][0]
+                slot = self.cache.get(eid)
+                if slot is None:
+                    self._compute(eid)
+                else:
+                    self._record_cached_use(eid, wait_prefetch=False)
+                    self._compute(eid, slot)
+
+        done: Set[int] = set()
+        if kind == "late":
+            slot = self.cache.get(residual_eid)
+            if slot is None:
+                return None
+            compute_ready(cover)
+            done.update(cover)
+            self.flush()  # resident experts run while the late copy lands
+            self._maybe_wait_prefetch(residual_eid)
+            self._record_cached_use(residual_eid, wait_prefetch=False)
+            m.bump("epipe_enabled_count")
+            m.bump("epipe_rs_late_prefetch_overlap_count")
+            self._compute(residual_eid, slot)
+            done.add(residual)
+        else:
+            if not self._headroom_ok():
+                self._fallback("epipe_fallback_memory")
+                return None
+            slot = self._acquire_slot()
+            stage_event = self._upload(residual_eid, slot, "epipe")
+            compute_ready(cover)
+            done.update(cover)
+            self.flush()
+            self.backend.wait_event(stage_event, "compute")
+            self._event("miss", residual_eid)
+            self._on_demand_access(residual_eid)
+            m.demand_h2d_bytes += self.expert_bytes
+            free_cache_slots = max(0, self.cache.capacity - len(self.cache))
+            commit = bool(cfg.epipe_rs_demand_commit and cfg.epipe_deferred_lru_commit
+                          and (free_cache_slots > 0 or not cfg.epipe_no_evict))
+            self._enqueue(residual_eid, slot)
+            if commit and self.cache.capacity > 0:
+                self._cache_put(residual_eid, slot)
+                m.bump("epipe_cache_insert_count")
+            else:
+                self._retired.append(slot)
+                m.bump("epipe_transient_payload_count")
+            m.bump("epipe_enabled_count")
+            m.bump("epipe_staged_missing_count")
+            done.add(residual)
+        for i, (eid, _rows) in enumerate(segments):
+            if i not in done:
+                self._compute(eid)
+        if cfg.epipe_rs_rolling_gate and self._gate_skip_remaining > 0:
+            self._gate_skip_remaining = 0
+            m.bump("epipe_rs_gate_reenable_count")
+        return "epipe_rs_residual_scan"
+
+    def _demand_gate_open(self, ready_items: int) -> bool:
+        """Reference :5895-5907."""
+        if not self.cfg.epipe_rs_handle_demand_miss:
+            return False
+        if ready_items < self.cfg.epipe_rs_min_buffer_items:
+            return False
+        return self._demand_gate_can_open()
+
+    # ------------------------------------------------------------------ RS prefetch
+    def effective_top_m(self) -> int:
+        return max(0, int(self.cfg.prefetch_top_m))
+
+    def predict_topk(self) -> int:
+        """Reference :10888-10901."""
+        if self.cfg.pred_topk is not None:
+            return max(1, min(int(self.cfg.pred_topk), self.num_experts))
+        return max(self.top_k, min(self.num_experts, self.effective_top_m()))
+
+    def finalize_prev_group_prefetch(self) -> None:
+        """Reference :9619-9635."""
+        for eid, ev in list(self.prefetch_events.items()):
+            if self.backend.event_done(ev):
+                self.metrics.prefetch_completed_count += 1
+                self.prefetch_events.pop(eid, None)
+        self.metrics.prefetch_wasted_count += len(self.prefetched_ids - self.prefetch_used_ids)
+        self.cache.unpin_all()
+        self.prefetched_ids.clear()
+        self.prefetch_used_ids.clear()
+        self.cycle_key = None
+
+    def _begin_cycle(self, key: Tuple[Any, ...]) -> None:
+        if self.cycle_key == key:
+            return
+        self.finalize_prev_group_prefetch()
+        self.cycle_key = key
+
+    def prefetch_protect_ids(self) -> Set[int]:
+        """Reference :9651-9665."""
+        if self.cfg.protect_mode in ("minimal", "current_next", "current-next"):
+            protect = set(self.prefetch_used_ids)
+        else:
+            protect = set(self.prefetched_ids) | set(self.prefetch_used_ids)
+        protect.update(self._cache_protect_ids())
+        recent = int(self.cfg.recent_protect_steps)
+        if recent > 0 and self.phase == "decode" and self.call_id >= 0:
+            for eid, last in self.last_used_decode_step.items():
+                if self.call_id - int(last) <= recent:
+                    protect.add(int(eid))
+        return protect
+
+    def prefetch_budget(self, cycle_key: Tuple[Any, ...]) -> int:
+        """``_prefetch_target_budget`` (reference :9785-9810)."""
+        top_m = self.effective_top_m()
+        if self.cfg.planner_mode != "rs_prefetch" or top_m <= 0 or self.num_experts == 0:
+            return 0
+        self._begin_cycle(cycle_key)
+        protect = self.prefetch_protect_ids()
+        room = self.cache.prefetch_free_slots()
+        if self.cfg.allow_active_replace:
+            room += len(self.cache.evictable_prefetch_ids(protect))
+        budget = max(0, min(max(0, top_m - len(self.prefetched_ids)), room))
+        if budget <= 0:
+            self.metrics.prefetch_budget_zero_count += 1
+        else:
+            self.metrics.prefetch_budget_positive_count += 1
+        return budget
+
+    @staticmethod
+    def score_map(flat_ids: Sequence[int], flat_probs: Sequence[float]) -> Dict[int, float]:
+        """Aggregate predicted probabilities per expert (reference :10040-10107):
+        ``sum * (1 + 0.15*(count-1)) + 0.05*max``, keyed in first-seen order."""
+        total: Dict[int, float] = {}
+        count: Dict[int, int] = {}
+        peak: Dict[int, float] = {}
+        for eid, p in zip(flat_ids, flat_probs):
+            eid, p = int(eid), float(p)
+            total[eid] = total.get(eid, 0.0) + p
+            count[eid] = count.get(eid, 0) + 1
+            peak[eid] = max(peak.get(eid, 0.0), p)
+        return {eid: total[eid] * (1.0 + 0.15 * float(max(count[eid] - 1, 0))) + 0.05 * peak[eid]
+                for eid in total}
+
+    def _keep_bias(self, eid: int) -> float:
+        """Reference :10031-10038 (no hot tier in the plain LRU)."""
+        bias = 0.02 * float(min(self.access_freq.get(int(eid), 0), 16))
+        if int(eid) in self.prefetched_ids:
+            bias += 0.10
+        return bias
+
+    def build_plan(self, scores: Dict[int, float], protect: Set[int],
+                   budget: int) -> List[Tuple[int, Optional[int]]]:
+        """``_build_prefetch_plan_from_score_map`` (reference :10144-10262)."""
+        cfg, m = self.cfg, self.metrics
+        if budget <= 0 or not scores:
+            return []
+        min_score, adv, margin = cfg.min_candidate_score, cfg.replace_advantage, cfg.replace_margin
+        if cfg.rs_policy in ("cache_safe", "cache-safe", "benefit_gate", "benefit-gate"):
+            min_score = max(min_score, cfg.cache_safe_min_score)
+            adv = max(adv, cfg.cache_safe_replace_advantage)
+            margin = max(margin, cfg.cache_safe_replace_margin)
+        candidates: List[Tuple[float, int]] = []
+        for eid, score in scores.items():
+            if self.cache.has(eid):
+                m.bump("rs_candidate_filter_out_cached_count")
+                continue
+            if float(score) < min_score:
+                m.bump("prefetch_rejected_low_score")
+                continue
+            candidates.append((float(score), int(eid)))
+        if not candidates:
+            return []
+        candidates.sort(key=lambda c: c[0], reverse=True)
+        free = self.cache.prefetch_free_slots()
+        ranked = []
+        for order, eid in enumerate(self.cache.evictable_prefetch_ids(protect)):
+            ranked.append((float(scores.get(eid, 0.0)) + self._keep_bias(eid), order, eid))
+        ranked.sort(key=lambda v: (v[0], v[1]))
+        victims = [eid for _, _, eid in ranked]
+        plan: List[Tuple[int, Optional[int]]] = []
+        pos = 0
+        for _ in range(min(free, budget, len(candidates))):
+            plan.append((candidates[pos][1], None))
+            pos += 1
+        remaining = budget - len(plan)
+        if remaining <= 0:
+            return plan
+        if not cfg.allow_active_replace:
+            m.bump("prefetch_rejected_active_replace", min(remaining, max(0, len(candidates) - pos)))
+            return plan
+        vpos = 0
+        while pos < len(candidates) and vpos < len(victims) and remaining > 0:
+            cand_score, cand = candidates[pos]
+            victim = victims[vpos]
+            victim_score = float(scores.get(victim, 0.0)) + self._keep_bias(victim)
+            if cand_score >= victim_score * margin or (cand_score - victim_score) >= adv:
+                plan.append((cand, victim))
+                remaining -= 1
+                pos += 1
+                vpos += 1
+            else:
+                m.bump("prefetch_rejected_margin", max(1, len(candidates) - pos))
+                break
+        if remaining > 0 and pos < len(candidates) and vpos >= len(victims):
+            m.bump("prefetch_rejected_cache_full", min(remaining, len(candidates) - pos))
+        return plan
+
+    def admit_plan(self, plan: Sequence[Tuple[int, Optional[int]]]) -> None:
+        """``_admit_prefetch_plan`` (reference :10433-10527): uploads ride the prefetch lane."""
+        if not plan:
+            return
+        m = self.metrics
+        m.prefetch_issued_count += len(plan)
+        protect = self.prefetch_protect_ids()
+        for eid, victim in plan:
+            eid = int(eid)
+            if self.cache.has(eid):
+                slot = self.cache.get(eid)
+                if not self.cache.admit_prefetch(eid, slot, protect_ids=protect, preferred_victim=victim):
+                    continue
+                self.prefetched_ids.add(eid)
+                protect.add(eid)
+                m.prefetch_admitted_count += 1
+                continue
+            if victim is not None:
+                self._discard_before_prefetch(int(victim))
+            if not self._free_slots and not self._retired and not self._pending:
+                # every slot is owned by a resident that may not go: skip, demand loads it later
+                m.bump("prefetch_oom_skip_count")
+                continue
+            slot = self._acquire_slot()
+            ev = self._upload(eid, slot, "prefetch")
+            m.prefetch_h2d_bytes += self.expert_bytes
+            ok = self.cache.admit_prefetch(eid, slot, protect_ids=protect, preferred_victim=victim)
+            if not ok:
+                self._free_slots.append(slot)
+                continue
+            self._slot_of[eid] = slot
+            self._sync_slots()
+            self.prefetch_events[eid] = ev
+            self.prefetched_ids.add(eid)
+            protect.add(eid)
+            if self.cfg.protect_mode in ("minimal", "current_next", "current-next"):
+                self.cache.unpin(eid)
+            m.prefetch_admitted_count += 1
+
+    def _discard_before_prefetch(self, eid: int) -> None:
+        """Reference :10011-10026."""
+        ev = self.prefetch_events.pop(eid, None)
+        if ev is not None and self.cfg.wait_before_evict:
+            self.backend.wait_event(ev, "prefetch")
+        if self.cache.discard(eid):
+            self._release_slot(self._slot_of.pop(eid))
+        self.prefetched_ids.discard(eid)
+        self.prefetch_used_ids.discard(eid)
+
+    def schedule_prefetch(self, flat_ids: Sequence[int], flat_probs: Sequence[float], budget: int) -> \
+            List[Tuple[int, Optional[int]]]:
+        """Plan and admit from the predictor's flattened ``[T, pred_k]`` top-k
+        (reference :10996-11010, :10413-10431)."""
+        protect = self.prefetch_protect_ids()
+        plan = self.build_plan(self.score_map(flat_ids, flat_probs), protect, int(budget))
+        self.admit_plan(plan)
+        return plan
+
+    # ------------------------------------------------------------------ lifecycle
+    def reset_for_new_request(self, *, clear_expert_cache: bool = False, clear_cache_metadata: bool = True) -> None:
+        """Reference :6097-6147."""
+        self.metrics.prefetch_completed_count += len(self.prefetch_events)
+        for ev in self.prefetch_events.values():
+            self.backend.wait_event(ev, "compute")  # nothing may read a slot before its copy lands
+        self.prefetch_events.clear()
+        self.prefetched_ids.clear()
+        self.prefetch_used_ids.clear()
+        self.access_freq.clear()
+        self.last_used_decode_step.clear()
+        self.cycle_key = None
+        if clear_expert_cache:
+            self.clear()
+        elif clear_cache_metadata:
+            self.cache.reset_request_metadata(unpin=True)
+
+    def clear(self) -> None:
+        """Drop every resident expert; all slots return to the pool."""
+        self.flush()
+        self.cache.clear()
+        self.extra_cache.clear()
+        self._slot_of.clear()
+        self._free_slots = list(range(self.num_slots - 1, -1, -1))
+        self._retired = []

@@ -66,10 +66,8 @@ class ExpertSlab:
                  device: torch.device) -> "ExpertSlab":
         """All experts resident, slot == expert id."""
         slab = cls(len(experts), len(experts), hidden, inter, dtype, device)
-        staging = torch.empty((expert_numel(hidden, inter),), dtype=dtype)
         for e, w in enumerate(experts):
-            pack_expert_into(staging, tuple(t.detach().to("cpu", dtype) for t in w), hidden, inter)
-            slab.data[e].copy_(staging)
+            pack_expert_into(slab.data[e], tuple(t.detach() for t in w), hidden, inter)
             slab.slot_of[e] = e
         slab.push_table()
         return slab

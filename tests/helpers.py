@@ -24,3 +24,29 @@ def make_layer(H, E, I, K, Is=0, shared_gate=False, dtype=torch.float32, seed=0,
 def make_hidden(T, H, dtype=torch.float32, seed=1000):
     g = torch.Generator().manual_seed(seed)
     return torch.randn(T, H, generator=g).to(dtype)
+
+
+def oracle_layer(mlp_block):
+    """CPU tensors of a duck-typed ``mlp_block`` in the oracle's argument format."""
+    def cpu(t):
+        return t.detach().cpu()
+
+    def triple(m):
+        return (cpu(m.gate_proj.weight), cpu(m.up_proj.weight), cpu(m.down_proj.weight))
+
+    experts = mlp_block.experts
+    if hasattr(experts, "gate_up_proj"):
+        gu, dn = cpu(experts.gate_up_proj), cpu(experts.down_proj)
+        inter = gu.shape[1] // 2
+        ex = [(gu[e, :inter].contiguous(), gu[e, inter:].contiguous(), dn[e].contiguous()) for e in range(gu.shape[0])]
+    else:
+        ex = [triple(m) for m in experts]
+    shared_mod = getattr(mlp_block, "shared_expert", None) or getattr(mlp_block, "shared_experts", None)
+    sg = getattr(mlp_block, "shared_expert_gate", None)
+    return dict(
+        gate_w=cpu(mlp_block.gate.weight),
+        experts=ex,
+        shared=triple(shared_mod) if shared_mod is not None else None,
+        shared_gate_w=cpu(sg.weight).reshape(-1) if sg is not None else None,
+        family="qwen_shared" if hasattr(mlp_block, "shared_expert") else "deepseek_shared",
+    )

@@ -54,4 +54,4 @@ def test_identity_and_error_channel():
 def test_struct_layouts_match_the_header():
     # sparse_hip_experts: ptr, u64, ptr, 4 x i32 ; sparse_hip_seglist: 2 ptr, i32, 256 x i16
     assert ctypes.sizeof(_lib.Experts) == 8 + 8 + 8 + 16
-    assert ctypes.sizeof(_lib.SegList) == 8 + 8 + 4 + 2 * 256 + 4  # tail padding to 8
+    assert ctypes.sizeof(_lib.SegList) == 8 + 8 + 4 + 2 * 256 + 2 * 256 + 4  # tail padding to 8
