@@ -179,6 +179,21 @@ int sparse_hip_shared_expert(const void* x_dev, const void* gate_w_dev, const vo
                              int T, int H, int Is, void* inter_ws_dev, void* shared_dev,
                              void* stream);
 
+/*
+ * Decode fast path: sparse_hip_grouped_swiglu_decode and sparse_hip_shared_expert of one
+ * call in a single launch pair (gate/up of every routed segment and of the shared
+ * expert, then all down projections), so the chip sees one fat stream of weights
+ * instead of four thinner launches.  Results are identical to the two separate calls.
+ * bf16 only, T <= SPARSE_HIP_DECODE_MAX_TOKENS.  Arguments as in those two functions;
+ * `sh_*` are the shared expert's (utils/eval_core.py:16520-16526).
+ */
+int sparse_hip_moe_ffn_decode(const sparse_hip_experts* experts, const void* x_dev, const void* topv_dev,
+                              const int32_t* perm_dev, const int32_t* seg_offsets_dev,
+                              const sparse_hip_seglist* segs, int T, int K, void* inter_ws_dev,
+                              void* parts_dev, const void* sh_gate_w_dev, const void* sh_up_w_dev,
+                              const void* sh_down_w_dev, const void* shared_gate_dev, int Is,
+                              void* sh_inter_ws_dev, void* shared_dev, void* stream);
+
 /* ---- A7: combine ----------------------------------------------------------- */
 
 /*
@@ -222,6 +237,34 @@ int sparse_hip_stream_synchronize(void* stream);
 /* Pinned host arena for offloaded experts (hipHostMalloc / hipHostFree). */
 int sparse_hip_host_alloc(size_t bytes, void** ptr_out);
 int sparse_hip_host_free(void* ptr);
+
+/* ---- measurement ---------------------------------------------------------- */
+
+/*
+ * Per-kernel timing with HIP events on the stream each kernel is launched on (no
+ * counterpart in the reference, which times whole segments with cuda.Event pairs,
+ * utils/eval_core.py:14655-14688).  While enabled, every kernel launch made through
+ * this library is bracketed by an event pair; `profile_read` waits for the recorded
+ * pairs of one kernel and returns their summed duration and count.  Leave it off in
+ * timed runs and under graph capture: the event records add launch gaps.
+ */
+#define SPARSE_HIP_K_ROUTER_LOGITS 0
+#define SPARSE_HIP_K_GATE_TOPK 1
+#define SPARSE_HIP_K_PERMUTE 2
+#define SPARSE_HIP_K_DECODE_GATEUP 3
+#define SPARSE_HIP_K_DECODE_DOWN 4
+#define SPARSE_HIP_K_PREFILL_GATEUP 5
+#define SPARSE_HIP_K_PREFILL_DOWN 6
+#define SPARSE_HIP_K_TILED_GATEUP 7
+#define SPARSE_HIP_K_TILED_DOWN 8
+#define SPARSE_HIP_K_COMBINE 9
+#define SPARSE_HIP_K_COUNT 10
+int sparse_hip_profile_enable(int on);
+int sparse_hip_profile_reset(void);
+int sparse_hip_profile_read(int kernel, double* total_ms_out, int64_t* launches_out);
+/* Name of the __global__ function behind a kernel id (as rocprofv3 prints it, without
+ * template arguments). */
+const char* sparse_hip_kernel_name(int kernel);
 
 #ifdef __cplusplus
 }

@@ -68,6 +68,9 @@ SIGNATURES = {
         _i, [C.POINTER(Experts), _vp, _vp, _vp, _vp, C.POINTER(SegList), _i, _i, _vp, _vp, _vp]),
     "sparse_hip_grouped_swiglu_prefill": (
         _i, [C.POINTER(Experts), _vp, _vp, _vp, _vp, C.POINTER(SegList), _i, _i, _vp, _vp, _vp]),
+    "sparse_hip_moe_ffn_decode": (
+        _i, [C.POINTER(Experts), _vp, _vp, _vp, _vp, C.POINTER(SegList), _i, _i, _vp, _vp,
+             _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp]),
     "sparse_hip_shared_expert": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp, _vp]),
     "sparse_hip_combine": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp]),
     "sparse_hip_expert_upload_async": (_i, [_vp, _vp, _sz, _vp, _vp]),
@@ -82,7 +85,14 @@ SIGNATURES = {
     "sparse_hip_stream_synchronize": (_i, [_vp]),
     "sparse_hip_host_alloc": (_i, [_sz, C.POINTER(_vp)]),
     "sparse_hip_host_free": (_i, [_vp]),
+    "sparse_hip_profile_enable": (_i, [_i]),
+    "sparse_hip_profile_reset": (_i, []),
+    "sparse_hip_profile_read": (_i, [_i, C.POINTER(C.c_double), C.POINTER(C.c_int64)]),
+    "sparse_hip_kernel_name": (C.c_char_p, [_i]),
 }
+
+KERNELS = ("router_logits", "gate_topk", "permute", "decode_gateup", "decode_down", "prefill_gateup",
+           "prefill_down", "tiled_gateup", "tiled_down", "combine")
 
 _lib = None
 

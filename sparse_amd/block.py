@@ -406,12 +406,17 @@ class DistributedSparseMoeBlock(nn.Module):
         rs_job = self._rs_begin(x, S, ws)
 
         logits = self._route(x, ws)
-        if self.shared_weights is not None:
+        shared_gate = ws.shared_gate if self.shared_gate_weight is not None else None
+        fused = (self.residency is None and self.shared_weights is not None and self.dtype == torch.bfloat16
+                 and T <= ops.DECODE_MAX_TOKENS)
+        if self.shared_weights is not None and not fused:
             gw, uw, dw = self.shared_weights
-            ops.shared_expert(x, gw, uw, dw, ws.shared_gate if self.shared_gate_weight is not None else None,
-                              ws.shared_inter, ws.shared_out)
+            ops.shared_expert(x, gw, uw, dw, shared_gate, ws.shared_inter, ws.shared_out)
 
-        if self.residency is None:
+        if fused:
+            ops.moe_ffn_decode(self._experts_desc, x, ws.topv, ws.perm, ws.segs_dev, ws.inter, ws.parts,
+                               self.shared_weights, shared_gate, ws.shared_inter, ws.shared_out)
+        elif self.residency is None:
             ops.grouped_swiglu(self._experts_desc, x, ws.topv, ws.perm, ws.segs_dev, ws.inter, ws.parts)
         else:
             ws.host_offsets.copy_(ws.perm.seg_offsets, non_blocking=True)

@@ -67,6 +67,7 @@ extern "C" int sparse_hip_combine(const void* parts_dev, const int32_t* inv_perm
   const int64_t nblk = static_cast<int64_t>((H / 8 + kCombThreads - 1) / kCombThreads) * T;
   SP_REQUIRE(nblk < (1ll << 31), "combine: grid too large");
   dim3 grid(static_cast<unsigned>(nblk));
+  ProfScope prof(SPARSE_HIP_K_COMBINE, as_stream(stream));
   if (dtype == SPARSE_HIP_BF16) {
     hipLaunchKernelGGL((combine_kernel<uint16_t>), grid, dim3(kCombThreads), 0, as_stream(stream),
                        static_cast<const uint16_t*>(parts_dev), inv_perm_dev,

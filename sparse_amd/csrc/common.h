@@ -34,6 +34,15 @@ int hip_fail(hipError_t err, const char* what);
     if (_e != hipSuccess) return sparse::hip_fail(_e, name);      \
   } while (0)
 
+// Brackets one kernel launch with an event pair while profiling is enabled.
+struct ProfScope {
+  ProfScope(int kernel, hipStream_t stream);
+  ~ProfScope();
+  int kernel_;
+  hipStream_t stream_;
+  hipEvent_t start_;
+};
+
 inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
 inline size_t elem_size(int dtype) { return dtype == SPARSE_HIP_BF16 ? 2 : 4; }
 inline bool valid_dtype(int dtype) { return dtype == SPARSE_HIP_F32 || dtype == SPARSE_HIP_BF16; }

@@ -9,6 +9,9 @@ int decode_routed_bf16(const sparse_hip_experts*, const void*, const void*, cons
                        const sparse_hip_seglist*, int, int, void*, void*, hipStream_t);
 int decode_shared_bf16(const void*, const void*, const void*, const void*, const void*, int, int, int, void*,
                        void*, hipStream_t);
+int decode_fused_bf16(const sparse_hip_experts*, const void*, const void*, const int32_t*, const int32_t*,
+                      const sparse_hip_seglist*, int, int, void*, void*, const void*, const void*, const void*,
+                      const void*, int, void*, void*, hipStream_t);
 int prefill_routed_bf16(const sparse_hip_experts*, const void*, const void*, const int32_t*, const int32_t*,
                         const sparse_hip_seglist*, int, int, void*, void*, hipStream_t);
 int prefill_shared_bf16(const void*, const void*, const void*, const void*, const void*, int, int, int, void*,
@@ -96,6 +99,31 @@ int sparse_hip_grouped_swiglu_prefill(const sparse_hip_experts* experts, const v
                                parts_dev, st);
   return tiled_routed<float>(experts, x_dev, topv_dev, perm_dev, seg_offsets_dev, segs, T, K, inter_ws_dev,
                              parts_dev, st);
+}
+
+int sparse_hip_moe_ffn_decode(const sparse_hip_experts* experts, const void* x_dev, const void* topv_dev,
+                              const int32_t* perm_dev, const int32_t* seg_offsets_dev,
+                              const sparse_hip_seglist* segs, int T, int K, void* inter_ws_dev, void* parts_dev,
+                              const void* sh_gate_w_dev, const void* sh_up_w_dev, const void* sh_down_w_dev,
+                              const void* shared_gate_dev, int Is, void* sh_inter_ws_dev, void* shared_dev,
+                              void* stream) {
+  int rc = check_routed("moe_ffn_decode", experts, x_dev, topv_dev, perm_dev, seg_offsets_dev, segs, T, K,
+                        inter_ws_dev, parts_dev);
+  if (rc != SPARSE_HIP_OK) return rc;
+  SP_REQUIRE(experts->dtype == SPARSE_HIP_BF16, "moe_ffn_decode: bf16 only; use the separate entry points");
+  SP_REQUIRE(T <= SPARSE_HIP_DECODE_MAX_TOKENS, "moe_ffn_decode: T=%d exceeds %d", T,
+             SPARSE_HIP_DECODE_MAX_TOKENS);
+  SP_REQUIRE(Is > 0 && Is % 64 == 0, "moe_ffn_decode: Is=%d must be a positive multiple of 64", Is);
+  SP_REQUIRE(sh_gate_w_dev && sh_up_w_dev && sh_down_w_dev && sh_inter_ws_dev && shared_dev,
+             "moe_ffn_decode: NULL shared-expert pointer");
+  SP_REQUIRE(((reinterpret_cast<uintptr_t>(sh_gate_w_dev) | reinterpret_cast<uintptr_t>(sh_up_w_dev) |
+               reinterpret_cast<uintptr_t>(sh_down_w_dev) | reinterpret_cast<uintptr_t>(sh_inter_ws_dev) |
+               reinterpret_cast<uintptr_t>(shared_dev)) &
+              15) == 0,
+             "moe_ffn_decode: shared-expert pointers must be 16-byte aligned");
+  return decode_fused_bf16(experts, x_dev, topv_dev, perm_dev, seg_offsets_dev, segs, T, K, inter_ws_dev,
+                           parts_dev, sh_gate_w_dev, sh_up_w_dev, sh_down_w_dev, shared_gate_dev, Is,
+                           sh_inter_ws_dev, shared_dev, as_stream(stream));
 }
 
 int sparse_hip_shared_expert(const void* x_dev, const void* gate_w_dev, const void* up_w_dev,

@@ -193,6 +193,7 @@ static int launch_tiled(TiledArgs& a, int max_mtiles, hipStream_t st) {
   const int64_t grid = static_cast<int64_t>(a.ntiles_n) * max_mtiles;
   if (grid == 0) return SPARSE_HIP_OK;
   SP_REQUIRE(grid < (1ll << 31), "ffn_tiled: grid too large");
+  ProfScope prof(kGateUp ? SPARSE_HIP_K_TILED_GATEUP : SPARSE_HIP_K_TILED_DOWN, st);
   hipLaunchKernelGGL((ffn_tiled_kernel<T, kGateUp>), dim3(static_cast<unsigned>(grid)), dim3(kTlThreads), 0,
                      st, a);
   SP_LAUNCH_CHECK("ffn_tiled_kernel");

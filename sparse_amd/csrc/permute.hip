@@ -147,6 +147,7 @@ int sparse_hip_permute_build(const int64_t* topi_dev, int T, int K, int E, int32
              "permute_build: NULL pointer");
   hipStream_t st = as_stream(stream);
   const int nb = (T + kPermThreads - 1) / kPermThreads;
+  ProfScope prof(SPARSE_HIP_K_PERMUTE, st);
   if (nb == 1) {
     hipLaunchKernelGGL((permute_scatter_kernel<true>), dim3(1), dim3(kPermThreads), 0, st, topi_dev, T, K, E,
                        static_cast<const int32_t*>(nullptr), perm_dev, inv_perm_dev, seg_offsets_dev,

@@ -165,6 +165,7 @@ template <typename T, typename TL>
 static int launch_router_logits(const void* x, const void* wg, const void* wsg, int Ttok, int H, int E,
                                 void* logits, void* shared_gate, hipStream_t st) {
   dim3 grid(E + (wsg != nullptr ? 1 : 0), (Ttok + kRouterTokTile - 1) / kRouterTokTile);
+  ProfScope prof(SPARSE_HIP_K_ROUTER_LOGITS, st);
   hipLaunchKernelGGL((router_logits_kernel<T, TL>), grid, dim3(kRouterThreads), 0, st,
                      static_cast<const T*>(x), static_cast<const T*>(wg), static_cast<const T*>(wsg), Ttok,
                      H, E, static_cast<TL*>(logits), static_cast<T*>(shared_gate));
@@ -176,6 +177,7 @@ template <typename TL, typename TO>
 static int launch_gate_topk(const void* logits, int Ttok, int E, int K, int renorm, void* topv,
                             int64_t* topi, hipStream_t st) {
   dim3 grid((Ttok + kTopkWaves - 1) / kTopkWaves);
+  ProfScope prof(SPARSE_HIP_K_GATE_TOPK, st);
   hipLaunchKernelGGL((gate_topk_kernel<TL, TO>), grid, dim3(kTopkWaves * 64), 0, st,
                      static_cast<const TL*>(logits), Ttok, E, K, renorm, static_cast<TO*>(topv), topi);
   SP_LAUNCH_CHECK("gate_topk_kernel");

@@ -5,6 +5,9 @@
 
 #include <string.h>
 
+#include <mutex>
+#include <vector>
+
 namespace sparse {
 
 static thread_local char g_err[512] = {0};
@@ -19,6 +22,45 @@ void set_error(const char* fmt, ...) {
 int hip_fail(hipError_t err, const char* what) {
   set_error("%s: %s (%d)", what, hipGetErrorString(err), static_cast<int>(err));
   return SPARSE_HIP_ELAUNCH;
+}
+
+// ---- per-kernel event timing ---------------------------------------------------
+struct ProfRec {
+  hipEvent_t start, stop;
+};
+static std::mutex g_prof_mu;
+static bool g_prof_on = false;
+static std::vector<ProfRec> g_prof_recs[SPARSE_HIP_K_COUNT];
+static std::vector<hipEvent_t> g_prof_free;
+
+static hipEvent_t prof_take_event() {
+  if (!g_prof_free.empty()) {
+    hipEvent_t e = g_prof_free.back();
+    g_prof_free.pop_back();
+    return e;
+  }
+  hipEvent_t e = nullptr;
+  if (hipEventCreate(&e) != hipSuccess) return nullptr;
+  return e;
+}
+
+ProfScope::ProfScope(int kernel, hipStream_t stream) : kernel_(kernel), stream_(stream), start_(nullptr) {
+  if (!g_prof_on) return;
+  std::lock_guard<std::mutex> lk(g_prof_mu);
+  start_ = prof_take_event();
+  if (start_ != nullptr) (void)hipEventRecord(start_, stream_);
+}
+
+ProfScope::~ProfScope() {
+  if (start_ == nullptr) return;
+  std::lock_guard<std::mutex> lk(g_prof_mu);
+  hipEvent_t stop = prof_take_event();
+  if (stop == nullptr) {
+    g_prof_free.push_back(start_);
+    return;
+  }
+  (void)hipEventRecord(stop, stream_);
+  g_prof_recs[kernel_].push_back(ProfRec{start_, stop});
 }
 
 }  // namespace sparse
@@ -113,6 +155,50 @@ int sparse_hip_host_free(void* ptr) {
   SP_REQUIRE(ptr != nullptr, "host_free: NULL pointer");
   SP_HIP(hipHostFree(ptr));
   return SPARSE_HIP_OK;
+}
+
+int sparse_hip_profile_enable(int on) {
+  std::lock_guard<std::mutex> lk(g_prof_mu);
+  g_prof_on = on != 0;
+  return SPARSE_HIP_OK;
+}
+
+int sparse_hip_profile_reset(void) {
+  std::lock_guard<std::mutex> lk(g_prof_mu);
+  for (auto& recs : g_prof_recs) {
+    for (auto& r : recs) {
+      g_prof_free.push_back(r.start);
+      g_prof_free.push_back(r.stop);
+    }
+    recs.clear();
+  }
+  return SPARSE_HIP_OK;
+}
+
+int sparse_hip_profile_read(int kernel, double* total_ms_out, int64_t* launches_out) {
+  SP_REQUIRE(kernel >= 0 && kernel < SPARSE_HIP_K_COUNT, "profile_read: kernel id %d outside [0,%d)", kernel,
+             SPARSE_HIP_K_COUNT);
+  SP_REQUIRE(total_ms_out != nullptr && launches_out != nullptr, "profile_read: NULL output");
+  std::lock_guard<std::mutex> lk(g_prof_mu);
+  double total = 0.0;
+  for (auto& r : g_prof_recs[kernel]) {
+    SP_HIP(hipEventSynchronize(r.stop));
+    float ms = 0.f;
+    SP_HIP(hipEventElapsedTime(&ms, r.start, r.stop));
+    total += ms;
+  }
+  *total_ms_out = total;
+  *launches_out = static_cast<int64_t>(g_prof_recs[kernel].size());
+  return SPARSE_HIP_OK;
+}
+
+const char* sparse_hip_kernel_name(int kernel) {
+  static const char* names[SPARSE_HIP_K_COUNT] = {
+      "router_logits_kernel", "gate_topk_kernel",   "permute_scatter_kernel", "decode_ffn_kernel<true>",
+      "decode_ffn_kernel<false>", "prefill_ffn_kernel<true>", "prefill_ffn_kernel<false>",
+      "ffn_tiled_kernel<gate_up>", "ffn_tiled_kernel<down>", "combine_kernel"};
+  if (kernel < 0 || kernel >= SPARSE_HIP_K_COUNT) return "";
+  return names[kernel];
 }
 
 }  // extern "C"

@@ -228,6 +228,7 @@ template <bool kGateUp>
 static int launch_decode(const DecodeArgs& a, int n_seg, hipStream_t st) {
   const int grid = a.tiles_s + n_seg * a.tiles_r;
   if (grid == 0) return SPARSE_HIP_OK;
+  ProfScope prof(kGateUp ? SPARSE_HIP_K_DECODE_GATEUP : SPARSE_HIP_K_DECODE_DOWN, st);
   if (a.T <= 16) {
     hipLaunchKernelGGL((decode_ffn_kernel<kGateUp, 1>), dim3(grid), dim3(kDecThreads), 0, st, a);
   } else {
@@ -270,6 +271,59 @@ int decode_routed_bf16(const sparse_hip_experts* ex, const void* x, const void* 
   a.Kdim = static_cast<int32_t>(I);
   a.Ndim = static_cast<int32_t>(H);
   a.tiles_r = a.Ndim / kDecRows;
+  return launch_decode<false>(a, segs->n, st);
+}
+
+// Routed experts and the shared expert in one launch pair, bf16, T <= 32.  The shared
+// expert's tiles lead the grid (largest, known amount of work), routed segments follow.
+int decode_fused_bf16(const sparse_hip_experts* ex, const void* x, const void* topv, const int32_t* perm,
+                      const int32_t* seg_offsets, const sparse_hip_seglist* segs, int T, int K, void* inter_ws,
+                      void* parts, const void* sh_gate_w, const void* sh_up_w, const void* sh_down_w,
+                      const void* shared_gate, int Is, void* sh_inter_ws, void* shared_out, hipStream_t st) {
+  const uint64_t H = ex->hidden, I = ex->inter;
+  DecodeArgs a = {};
+  a.slab = static_cast<const uint16_t*>(ex->slab_dev);
+  a.slot_stride = ex->slot_stride / 2;
+  a.expert_slot = ex->expert_slot_dev;
+  a.perm = perm;
+  a.seg_offsets = seg_offsets;
+  a.topk = K;
+  a.T = T;
+  a.segs = *segs;
+  // gate-up
+  a.mat_offset = 0;
+  a.mat2_offset = I * H;
+  a.act_r = static_cast<const uint16_t*>(x);
+  a.out_r = static_cast<uint16_t*>(inter_ws);
+  a.Kdim = static_cast<int32_t>(H);
+  a.Ndim = static_cast<int32_t>(I);
+  a.tiles_r = a.Ndim / kDecRows;
+  a.w_s = static_cast<const uint16_t*>(sh_gate_w);
+  a.w2_s = static_cast<const uint16_t*>(sh_up_w);
+  a.act_s = static_cast<const uint16_t*>(x);
+  a.out_s = static_cast<uint16_t*>(sh_inter_ws);
+  a.Kdim_s = static_cast<int32_t>(H);
+  a.Ndim_s = Is;
+  a.tiles_s = Is / kDecRows;
+  int rc = launch_decode<true>(a, segs->n, st);
+  if (rc != SPARSE_HIP_OK) return rc;
+  // down
+  a.mat_offset = 2 * I * H;
+  a.mat2_offset = 0;
+  a.topv = static_cast<const uint16_t*>(topv);
+  a.act_r = static_cast<const uint16_t*>(inter_ws);
+  a.out_r = static_cast<uint16_t*>(parts);
+  a.Kdim = static_cast<int32_t>(I);
+  a.Ndim = static_cast<int32_t>(H);
+  a.tiles_r = a.Ndim / kDecRows;
+  a.w_s = static_cast<const uint16_t*>(sh_down_w);
+  a.w2_s = nullptr;
+  a.act_s = static_cast<const uint16_t*>(sh_inter_ws);
+  a.gate_s = static_cast<const uint16_t*>(shared_gate);
+  a.out_s = static_cast<uint16_t*>(shared_out);
+  a.Kdim_s = Is;
+  a.Ndim_s = static_cast<int32_t>(H);
+  a.tiles_s = a.Ndim_s / kDecRows;
   return launch_decode<false>(a, segs->n, st);
 }
 

@@ -265,6 +265,7 @@ static int launch_prefill(PrefillArgs& a, hipStream_t st) {
   grid = (grid + kPfXcds - 1) / kPfXcds * kPfXcds;
   if (grid == 0) return SPARSE_HIP_OK;
   SP_REQUIRE(grid < (1ll << 31), "prefill_ffn: grid too large");
+  ProfScope prof(kGateUp ? SPARSE_HIP_K_PREFILL_GATEUP : SPARSE_HIP_K_PREFILL_DOWN, st);
   hipLaunchKernelGGL((prefill_ffn_kernel<kGateUp>), dim3(static_cast<unsigned>(grid)), dim3(kPfThreads), 0, st,
                      a);
   SP_LAUNCH_CHECK("prefill_ffn_kernel");

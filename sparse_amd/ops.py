@@ -281,3 +281,48 @@ def host_alloc(nbytes: int) -> int:
 
 def host_free(ptr: int) -> None:
     _lib.check(_lib.load().sparse_hip_host_free(ptr), "sparse_hip_host_free")
+
+
+# --------------------------------------------------------------------------- measurement
+def profile_enable(on: bool) -> None:
+    _lib.check(_lib.load().sparse_hip_profile_enable(int(bool(on))), "sparse_hip_profile_enable")
+
+
+def profile_reset() -> None:
+    _lib.check(_lib.load().sparse_hip_profile_reset(), "sparse_hip_profile_reset")
+
+
+def profile_read() -> dict:
+    """``{kernel: (total_ms, launches, device function name)}`` for every kernel id."""
+    lib = _lib.load()
+    out = {}
+    for kid, name in enumerate(_lib.KERNELS):
+        ms, n = C.c_double(), C.c_int64()
+        _lib.check(lib.sparse_hip_profile_read(kid, C.byref(ms), C.byref(n)), "sparse_hip_profile_read")
+        out[name] = (float(ms.value), int(n.value), lib.sparse_hip_kernel_name(kid).decode())
+    return out
+
+
+def moe_ffn_decode(experts: Experts, x: torch.Tensor, topv: torch.Tensor, perm: Permutation, segs: SegList,
+                   inter_ws: torch.Tensor, parts: torch.Tensor, shared_w, shared_gate: Optional[torch.Tensor],
+                   shared_inter_ws: torch.Tensor, shared_out: torch.Tensor) -> None:
+    """Routed experts + shared expert of a decode call in one launch pair (bf16, T <= 32)."""
+    lib = _lib.load()
+    T, H = x.shape
+    K = topv.shape[1]
+    gw, uw, dw = shared_w
+    Is = gw.shape[0]
+    _need(x, "x", torch.bfloat16)
+    _need(topv, "topv", x.dtype, (T, K))
+    _need(inter_ws, "inter_ws", x.dtype, (T * K, experts.inter))
+    _need(parts, "parts", x.dtype, (T * K, H))
+    _need(gw, "shared gate_proj", x.dtype, (Is, H))
+    _need(uw, "shared up_proj", x.dtype, (Is, H))
+    _need(dw, "shared down_proj", x.dtype, (H, Is))
+    _need(shared_inter_ws, "shared inter_ws", x.dtype, (T, Is))
+    _need(shared_out, "shared out", x.dtype, (T, H))
+    rc = lib.sparse_hip_moe_ffn_decode(C.byref(experts), _ptr(x), _ptr(topv), _ptr(perm.perm),
+                                       _ptr(perm.seg_offsets), C.byref(segs), T, K, _ptr(inter_ws), _ptr(parts),
+                                       _ptr(gw), _ptr(uw), _ptr(dw), _ptr(shared_gate), Is, _ptr(shared_inter_ws),
+                                       _ptr(shared_out), _stream())
+    _lib.check(rc, "sparse_hip_moe_ffn_decode")
