@@ -15,8 +15,16 @@
  *   - Nothing here allocates device memory or synchronises the host unless its
  *     comment says so: callers pass workspaces and outputs.  Launches are
  *     asynchronous with respect to the host and may be captured into a HIP graph.
- *   - Row-major everywhere.  Weight matrices are [out_features, in_features] as in
- *     torch.nn.Linear.
+ *   - Activations, logits and outputs are row-major.  Weight matrices are
+ *     [out_features, in_features] = [R, K] as in torch.nn.Linear, but stored TILED
+ *     (R % 16 == 0, K % 64 == 0): element (row, k) lives at element offset
+ *         (row/16)*16*K + (k/64)*1024 + ((k/8)%2)*512 + ((k/16)%4)*128 + (row%16)*8 + k%8
+ *     i.e. the K extent of a 16-row group is one contiguous run, cut into 2 KB (bf16)
+ *     blocks of 64 k whose two halves are the A operands of two 16x16x32 MFMAs in lane
+ *     order.  Streaming a weight matrix is then a sequence of contiguous 1 KB wave
+ *     loads; row-major rows 4 KB apart would pile onto the same HBM channels.
+ *     `sparse_hip_tile_weight` converts.  The router gate matrix `wg` and the shared
+ *     gate vector stay row-major.
  *   - dtype codes: SPARSE_HIP_F32 = 0, SPARSE_HIP_BF16 = 1.
  */
 #ifndef SPARSE_HIP_H
@@ -170,7 +178,7 @@ int sparse_hip_grouped_swiglu_prefill(const sparse_hip_experts* experts, const v
  * shared[t] = down_s(act(gate_s(x[t])) * up_s(x[t])), times
  * sigmoid(shared_gate[t]) when `shared_gate_dev` is non-NULL (each step rounded to
  * dtype) -- `_shared_expert_forward` (utils/eval_core.py:9455-9463).
- * gate_s, up_s [Is,H], down_s [H,Is]; inter_ws [T,Is]; shared [T,H].
+ * gate_s, up_s [Is,H], down_s [H,Is] (tiled); inter_ws [T,Is]; shared [T,H].
  * Uses the decode kernels when T <= SPARSE_HIP_DECODE_MAX_TOKENS, the prefill
  * kernels otherwise.
  */
@@ -237,6 +245,21 @@ int sparse_hip_stream_synchronize(void* stream);
 /* Pinned host arena for offloaded experts (hipHostMalloc / hipHostFree). */
 int sparse_hip_host_alloc(size_t bytes, void** ptr_out);
 int sparse_hip_host_free(void* ptr);
+
+/* ---- weight layout ---------------------------------------------------------- */
+
+/*
+ * Convert one [rows, cols] matrix between row-major and the tiled layout described at the
+ * top of this file (to_tiled != 0: row-major -> tiled).  src and dst must not alias.
+ * The reference keeps weights row-major (utils/eval_core.py:5115-5123); packing is a
+ * load-time step of this library's host.
+ */
+int sparse_hip_tile_weight(const void* src_dev, void* dst_dev, int rows, int cols, int dtype, int to_tiled,
+                           void* stream);
+
+/* Plain device copy of `bytes` (multiple of 16) by a grid-stride kernel: the known-size
+ * reference point for scaling HBM traffic counters.  No counterpart in the reference. */
+int sparse_hip_calib_copy(const void* src_dev, void* dst_dev, size_t bytes, void* stream);
 
 /* ---- measurement ---------------------------------------------------------- */
 

@@ -27,7 +27,7 @@ from torch import nn
 from . import ops
 from .context import DistEnv, Metrics, SparseContext
 from .residency import Backend, LayerResidency, ResidencyConfig
-from .weights import ExpertSlab, HostExpertArena
+from .weights import ExpertSlab, HostExpertArena, tile_weight
 
 
 def _is_silu(fn: Any) -> bool:
@@ -266,7 +266,10 @@ class DistributedSparseMoeBlock(nn.Module):
         if shared_mod is not None:
             if not _is_silu(getattr(shared_mod, "act_fn", None)):
                 raise NotImplementedError("only SiLU shared experts are built")
-            self.shared_weights = tuple(t.to(self.device, self.dtype).contiguous() for t in _mlp_weights(shared_mod))
+            # tiled content, logical [rows, cols] shape kept for argument checks
+            self.shared_weights = tuple(
+                tile_weight(t.to(self.device, self.dtype)).reshape(t.shape).contiguous()
+                for t in _mlp_weights(shared_mod))
             self.shared_inter_size = int(self.shared_weights[0].shape[0])
         sg = getattr(mlp_block, "shared_expert_gate", None)
         self.shared_gate_weight = (

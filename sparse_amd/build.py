@@ -28,6 +28,7 @@ SOURCES = [
     "ffn_tiled.hip",
     "ffn.hip",
     "combine.hip",
+    "layout.hip",
 ]
 
 # Packed-fp32 VALU ops are switched off for the device pass; the host pass does not know

@@ -110,8 +110,9 @@ __global__ __launch_bounds__(kTlThreads) void ffn_tiled_kernel(const TiledArgs a
     }
   }
   const bool brow_ok = (n0 + lrow) < Ndim;
-  const T* brow0 = w0 + static_cast<size_t>(brow_ok ? n0 + lrow : 0) * Kdim;
-  const T* brow1 = kGateUp ? w1 + static_cast<size_t>(brow_ok ? n0 + lrow : 0) * Kdim : nullptr;
+  // weights are tiled: 16-row groups, blocks of 64 k, (half, k-quarter, row, 8 k) inside
+  const int wrow = brow_ok ? n0 + lrow : 0;
+  const size_t wbase = static_cast<size_t>(wrow >> 4) * 16 * Kdim + (wrow & 15) * 8;
 
   const int ty = tid >> 4, tx = tid & 15;
   float acc[NM][4][4];
@@ -126,8 +127,11 @@ __global__ __launch_bounds__(kTlThreads) void ffn_tiled_kernel(const TiledArgs a
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       As[lk + j][lrow] = (arow != nullptr) ? Elem<T>::load(arow + k0 + lk + j) : 0.f;
-      Bs[0][lk + j][lrow] = brow_ok ? Elem<T>::load(brow0 + k0 + lk + j) : 0.f;
-      if (kGateUp) Bs[1][lk + j][lrow] = brow_ok ? Elem<T>::load(brow1 + k0 + lk + j) : 0.f;
+      const int kk = k0 + lk + j;
+      const size_t wo = wbase + static_cast<size_t>(kk >> 6) * 1024 + ((kk >> 3) & 1) * 512 +
+                        ((kk >> 4) & 3) * 128 + (kk & 7);
+      Bs[0][lk + j][lrow] = brow_ok ? Elem<T>::load(w0 + wo) : 0.f;
+      if (kGateUp) Bs[1][lk + j][lrow] = brow_ok ? Elem<T>::load(w1 + wo) : 0.f;
     }
     __syncthreads();
 #pragma unroll

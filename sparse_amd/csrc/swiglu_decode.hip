@@ -125,45 +125,70 @@ __global__ __launch_bounds__(kDecThreads) void decode_ffn_kernel(const DecodeArg
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt) acc[m][tl][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  const uint16_t* wrow0 = w0 + static_cast<size_t>(row0 + r) * Kdim + (q << 4);
-  const uint16_t* wrow1 = kGateUp ? w1 + static_cast<size_t>(row0 + r) * Kdim + (q << 4) : nullptr;
-  const size_t tile_step = static_cast<size_t>(16) * Kdim;
+  // Weights are tiled: the K extent of a 16-row group is contiguous, cut into 2 KB blocks
+  // of 64 k; the first KB of a block is the first MFMA's A operand in lane order, the
+  // second KB the second MFMA's, so every load instruction of a wave reads 1 KB straight.
+  const size_t group_stride = static_cast<size_t>(16) * Kdim;
+  const uint16_t* wt0 = w0 + static_cast<size_t>(row0 >> 4) * group_stride + lane * 8;
+  const uint16_t* wt1 = kGateUp ? w1 + static_cast<size_t>(row0 >> 4) * group_stride + lane * 8 : nullptr;
   const int ND = Kdim >> 6;
 
-#pragma unroll 2
-  for (int d = wave; d < ND; d += kDecWaves) {
-    const int koff = d << 6;
-    bf16x8 b0[NT], b1[NT];
+  bf16x8 cb[NT][2], cw[NM][kDecTiles][2];  // fragments being multiplied
+  bf16x8 nb[NT][2], nw[NM][kDecTiles][2];  // fragments in flight for the next slice
+
+#define SP_DEC_LOAD(B, W, d)                                                             \
+  do {                                                                                   \
+    const int koff_ = (d) << 6;                                                          \
+    _Pragma("unroll") for (int nt = 0; nt < NT; ++nt) {                                  \
+      if (brow[nt] != nullptr) {                                                         \
+        B[nt][0] = ld_bf16x8(brow[nt] + koff_ + (q << 4));                               \
+        B[nt][1] = ld_bf16x8(brow[nt] + koff_ + (q << 4) + 8);                           \
+      } else {                                                                           \
+        B[nt][0] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};                                       \
+        B[nt][1] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};                                       \
+      }                                                                                  \
+    }                                                                                    \
+    _Pragma("unroll") for (int tl = 0; tl < kDecTiles; ++tl) {                           \
+      const size_t o_ = tl * group_stride + (static_cast<size_t>(d) << 10);              \
+      W[0][tl][0] = ld_bf16x8(wt0 + o_);                                                 \
+      W[0][tl][1] = ld_bf16x8(wt0 + o_ + 512);                                           \
+      if (kGateUp) {                                                                     \
+        W[NM - 1][tl][0] = ld_bf16x8(wt1 + o_);                                          \
+        W[NM - 1][tl][1] = ld_bf16x8(wt1 + o_ + 512);                                    \
+      }                                                                                  \
+    }                                                                                    \
+  } while (0)
+
+  int d = wave;
+  if (d < ND) SP_DEC_LOAD(cb, cw, d);
+  for (; d < ND; d += kDecWaves) {
+    const bool more = d + kDecWaves < ND;
+    if (more) SP_DEC_LOAD(nb, nw, d + kDecWaves);
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-      if (brow[nt] != nullptr) {
-        b0[nt] = ld_bf16x8(brow[nt] + koff + (q << 4));
-        b1[nt] = ld_bf16x8(brow[nt] + koff + (q << 4) + 8);
-      } else {
-        b0[nt] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
-        b1[nt] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
-      }
-    }
+    for (int tl = 0; tl < kDecTiles; ++tl)
 #pragma unroll
-    for (int tl = 0; tl < kDecTiles; ++tl) {
-      const bf16x8 g0 = ld_bf16x8(wrow0 + tl * tile_step + koff);
-      const bf16x8 g1 = ld_bf16x8(wrow0 + tl * tile_step + koff + 8);
-      bf16x8 u0, u1;
-      if (kGateUp) {
-        u0 = ld_bf16x8(wrow1 + tl * tile_step + koff);
-        u1 = ld_bf16x8(wrow1 + tl * tile_step + koff + 8);
-      }
+      for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int m = 0; m < NM; ++m) {
+          acc[m][tl][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cw[m][tl][0], cb[nt][0], acc[m][tl][nt], 0, 0, 0);
+          acc[m][tl][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cw[m][tl][1], cb[nt][1], acc[m][tl][nt], 0, 0, 0);
+        }
+    if (more) {
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt) {
-        acc[0][tl][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(g0, b0[nt], acc[0][tl][nt], 0, 0, 0);
-        acc[0][tl][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(g1, b1[nt], acc[0][tl][nt], 0, 0, 0);
-        if (kGateUp) {
-          acc[1][tl][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(u0, b0[nt], acc[1][tl][nt], 0, 0, 0);
-          acc[1][tl][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(u1, b1[nt], acc[1][tl][nt], 0, 0, 0);
-        }
+        cb[nt][0] = nb[nt][0];
+        cb[nt][1] = nb[nt][1];
       }
+#pragma unroll
+      for (int m = 0; m < NM; ++m)
+#pragma unroll
+        for (int tl = 0; tl < kDecTiles; ++tl) {
+          cw[m][tl][0] = nw[m][tl][0];
+          cw[m][tl][1] = nw[m][tl][1];
+        }
     }
   }
+#undef SP_DEC_LOAD
 
   // ---- split-K partials meet in LDS ----------------------------------------
   constexpr int NFRAG = kDecTiles * NT;

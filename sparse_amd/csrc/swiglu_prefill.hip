@@ -153,22 +153,28 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_ffn_kernel(const Prefil
     }
     aptr[i] = a.act + row * Kdim + lchunk * 8;
   }
+  // Weight rows are tiled (16-row groups, 2 KB blocks of 64 k in MFMA lane order): a pass
+  // of the workgroup copies two whole blocks, 128 sixteen-byte units each, so global reads
+  // are 2 KB runs; unit u = h*64 + q*16 + r is row r, k = q*16 + h*8 .. +7 of its block.
+  const int bu = tid & 127, bgrp = tid >> 7;
+  const int br = bu & 15, bq = (bu >> 4) & 3, bh = bu >> 6;
   const uint16_t* bptr[8];
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
-    const int rr = lrow + 32 * i;  // row inside the 256-row weight tile
+    const int g = 2 * i + bgrp;  // 16-row group inside the 256-row weight tile
     const uint16_t* base;
     int n;
     if (kGateUp) {
-      base = (rr < kPfBR / 2) ? w0 : w1;
-      n = n0 + (rr & (kPfBR / 2 - 1));
+      base = (g < 8) ? w0 : w1;
+      n = n0 + (g & 7) * 16;
     } else {
       base = w0;
-      n = n0 + rr;
+      n = n0 + g * 16;
     }
-    n = min(n, Ndim - 1);
-    bptr[i] = base + static_cast<size_t>(n) * Kdim + lchunk * 8;
+    n = min(n, Ndim - 16);
+    bptr[i] = base + static_cast<size_t>(n >> 4) * 16 * Kdim + bu * 8;
   }
+  const int lds_wr_b = (bgrp * 16 + br) * kPfRowBytes + (bq * 2 + bh) * 16;
   const int lds_wr = lrow * kPfRowBytes + lchunk * 16;
 
   f32x16 acc[4][2];
@@ -202,14 +208,14 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_ffn_kernel(const Prefil
       *reinterpret_cast<u32x4*>(lds + lds_wr + i * 32 * kPfRowBytes) = ra[i];
 #pragma unroll
     for (int i = 0; i < 8; ++i)
-      *reinterpret_cast<u32x4*>(lds + kPfLdsA + lds_wr + i * 32 * kPfRowBytes) = rb[i];
+      *reinterpret_cast<u32x4*>(lds + kPfLdsA + lds_wr_b + i * 32 * kPfRowBytes) = rb[i];
     __syncthreads();
     if (kt + 1 < nk) {
       const int ko = (kt + 1) * kPfBK;
 #pragma unroll
       for (int i = 0; i < 4; ++i) ra[i] = *reinterpret_cast<const u32x4*>(aptr[i] + ko);
 #pragma unroll
-      for (int i = 0; i < 8; ++i) rb[i] = *reinterpret_cast<const u32x4*>(bptr[i] + ko);
+      for (int i = 0; i < 8; ++i) rb[i] = *reinterpret_cast<const u32x4*>(bptr[i] + (kt + 1) * 1024);
     }
 #pragma unroll
     for (int ks = 0; ks < kPfBK / 16; ++ks) {

@@ -1,8 +1,10 @@
 """Expert weight storage: HBM slot slab and pinned-host arena.
 
-One slot holds one routed expert as three row-major matrices back to back,
+One slot holds one routed expert as three matrices back to back,
 ``gate [I,H] | up [I,H] | down [H,I]`` (the module layout of the reference,
-utils/eval_core.py:5115-5123, made contiguous so that one expert is one H2D copy).
+utils/eval_core.py:5115-5123, made contiguous so that one expert is one H2D copy), each
+stored in the kernels' tiled order (``tile_weight``) so that weight streaming is a run of
+contiguous wave loads.
 All-resident layers use ``E`` slots with the identity slot table; cached layers use
 ``capacity (+ staging)`` slots and rewrite ``expert_slot`` as experts move.
 """
@@ -19,17 +21,36 @@ def expert_numel(hidden: int, inter: int) -> int:
     return 3 * hidden * inter
 
 
+def tile_weight(w: torch.Tensor) -> torch.Tensor:
+    """Row-major ``[R, K]`` -> the library's tiled layout, flattened (R % 16 == 0, K % 64 == 0).
+
+    Element (row, k) goes to ``(row//16)*16*K + (k//64)*1024 + ((k//8)%2)*512 +
+    ((k//16)%4)*128 + (row%16)*8 + k%8``: per 16-row group and 64-wide k block, the
+    order is (8-k half, k quarter, row, k within 8)."""
+    R, K = w.shape
+    if R % 16 or K % 64:
+        raise ValueError(f"tiled weights need rows % 16 == 0 and cols % 64 == 0, got {tuple(w.shape)}")
+    v = w.reshape(R // 16, 16, K // 64, 4, 2, 8)       # [group, row, block, quarter, half, k8]
+    return v.permute(0, 2, 4, 3, 1, 5).reshape(-1)      # [group, block, half, quarter, row, k8]
+
+
+def untile_weight(flat: torch.Tensor, rows: int, cols: int) -> torch.Tensor:
+    """Inverse of ``tile_weight``."""
+    v = flat.reshape(rows // 16, cols // 64, 2, 4, 16, 8)
+    return v.permute(0, 4, 1, 3, 2, 5).reshape(rows, cols)
+
+
 def pack_expert_into(dst_row: torch.Tensor, weights: ExpertWeights, hidden: int, inter: int) -> None:
-    """Copy (gate, up, down) into one flat slot row."""
+    """Copy (gate, up, down), each tiled, into one flat slot row."""
     gw, uw, dw = weights
     if tuple(gw.shape) != (inter, hidden) or tuple(uw.shape) != (inter, hidden) or tuple(dw.shape) != (hidden, inter):
         raise ValueError(
             f"expert weights must be gate/up [{inter},{hidden}] and down [{hidden},{inter}], got "
             f"{tuple(gw.shape)}, {tuple(uw.shape)}, {tuple(dw.shape)}")
     n = hidden * inter
-    dst_row[0:n].copy_(gw.reshape(-1))
-    dst_row[n:2 * n].copy_(uw.reshape(-1))
-    dst_row[2 * n:3 * n].copy_(dw.reshape(-1))
+    dst_row[0:n].copy_(tile_weight(gw))
+    dst_row[n:2 * n].copy_(tile_weight(uw))
+    dst_row[2 * n:3 * n].copy_(tile_weight(dw))
 
 
 class HostExpertArena:

@@ -242,6 +242,30 @@ def test_segment_order_changes_nothing(device):
     assert torch.equal(pre, pre2)
 
 
+# ------------------------------------------------------------------ weight layout
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_tile_weight_kernel_matches_host_packing(device, dtype):
+    from sparse_amd import _lib, ops
+    from sparse_amd.weights import tile_weight, untile_weight
+    w = torch.randn(48, 192).to(dtype)
+    ref = tile_weight(w)
+    assert torch.equal(untile_weight(ref, 48, 192), w)
+    src = w.to(device)
+    dst = torch.empty(48 * 192, device=device, dtype=dtype)
+    lib = _lib.load()
+    stream = torch.cuda.current_stream().cuda_stream
+    _lib.check(lib.sparse_hip_tile_weight(src.data_ptr(), dst.data_ptr(), 48, 192, ops.dtype_code(dtype), 1, stream),
+               "tile")
+    assert torch.equal(dst.cpu(), ref)
+    back = torch.empty_like(src)
+    _lib.check(lib.sparse_hip_tile_weight(dst.data_ptr(), back.data_ptr(), 48, 192, ops.dtype_code(dtype), 0, stream),
+               "untile")
+    assert torch.equal(back.cpu(), w)
+    with pytest.raises(ValueError):
+        _lib.check(lib.sparse_hip_tile_weight(src.data_ptr(), dst.data_ptr(), 40, 192, ops.dtype_code(dtype), 1,
+                                              stream), "tile")
+
+
 # ------------------------------------------------------------------ shared expert + combine
 @pytest.mark.parametrize("dtype,T", [(torch.bfloat16, 8), (torch.bfloat16, 32), (torch.bfloat16, 200),
                                      (torch.float32, 8), (torch.float32, 100)])
@@ -255,7 +279,8 @@ def test_shared_expert(device, dtype, T, gated):
     sg = None
     if gated:
         _, sg = ops.router_logits(xd, layer["gate_w"].to(device), layer["shared_gate_w"].to(device))
-    gw, uw, dw = (t.to(device) for t in layer["shared"])
+    from sparse_amd.weights import tile_weight
+    gw, uw, dw = (tile_weight(t).reshape(t.shape).contiguous().to(device) for t in layer["shared"])
     inter = torch.empty((T, 384), device=device, dtype=dtype)
     out = torch.empty((T, 512), device=device, dtype=dtype)
     ops.shared_expert(xd, gw, uw, dw, sg, inter, out)
