@@ -143,6 +143,21 @@ int sparse_hip_permute_build(const int64_t* topi_dev, int T, int K, int E, int32
                              int32_t* active_eids_dev, int32_t* n_active_dev, void* ws_dev,
                              void* stream);
 
+/*
+ * Decode fast path: sparse_hip_router_logits + sparse_hip_gate_topk +
+ * sparse_hip_permute_build in ONE launch for T <= SPARSE_HIP_DECODE_MAX_TOKENS (topv is
+ * written in `dtype`).  Each workgroup computes one column of the logits; the workgroup
+ * that finishes last (counted in `counter_dev` behind a device-scope fence) does the
+ * top-k and the permutation.  `counter_dev` is one int32 that must be zero before the
+ * first call; every call leaves it zero.  Same outputs, bit for bit, as the three
+ * separate calls (utils/eval_core.py:9519-9595, :14728-14730, :13240-13262).
+ */
+int sparse_hip_route_decode(const void* x_dev, const void* wg_dev, const void* wsg_dev, int dtype,
+                            int logits_dtype, int T, int H, int E, int K, int renorm, void* logits_dev,
+                            void* shared_gate_dev, void* topv_dev, int64_t* topi_dev, int32_t* perm_dev,
+                            int32_t* inv_perm_dev, int32_t* seg_offsets_dev, int32_t* active_eids_dev,
+                            int32_t* n_active_dev, int32_t* counter_dev, void* stream);
+
 /* ---- A4/A6: grouped SwiGLU expert FFN -------------------------------------- */
 
 /*
@@ -281,7 +296,8 @@ int sparse_hip_calib_copy(const void* src_dev, void* dst_dev, size_t bytes, void
 #define SPARSE_HIP_K_TILED_GATEUP 7
 #define SPARSE_HIP_K_TILED_DOWN 8
 #define SPARSE_HIP_K_COMBINE 9
-#define SPARSE_HIP_K_COUNT 10
+#define SPARSE_HIP_K_ROUTE_DECODE 10
+#define SPARSE_HIP_K_COUNT 11
 int sparse_hip_profile_enable(int on);
 int sparse_hip_profile_reset(void);
 int sparse_hip_profile_read(int kernel, double* total_ms_out, int64_t* launches_out);

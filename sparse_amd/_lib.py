@@ -62,6 +62,8 @@ SIGNATURES = {
     "sparse_hip_last_error": (C.c_char_p, []),
     "sparse_hip_router_logits": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _vp, _vp]),
     "sparse_hip_gate_topk": (_i, [_vp, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp]),
+    "sparse_hip_route_decode": (
+        _i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "sparse_hip_permute_ws_bytes": (_sz, [_i, _i, _i]),
     "sparse_hip_permute_build": (_i, [_vp, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "sparse_hip_grouped_swiglu_decode": (
@@ -94,7 +96,7 @@ SIGNATURES = {
 }
 
 KERNELS = ("router_logits", "gate_topk", "permute", "decode_gateup", "decode_down", "prefill_gateup",
-           "prefill_down", "tiled_gateup", "tiled_down", "combine")
+           "prefill_down", "tiled_gateup", "tiled_down", "combine", "route_decode")
 
 _lib = None
 

@@ -75,6 +75,7 @@ class _Workspace:
         self.shared_inter = torch.empty((T, Is), device=device, dtype=dtype) if Is else None
         self.shared_out = torch.empty((T, H), device=device, dtype=dtype) if Is else None
         self.segs_dev = ops.seglist_device(self.perm, min(E, T * K))
+        self.route_counter = torch.zeros((1,), device=device, dtype=torch.int32)
         # host mirrors for the offloaded path (pinned, written by async D2H copies)
         self.host_offsets = torch.empty((E + 1,), dtype=torch.int32, pin_memory=True)
         self.host_rs_topi = torch.empty((T * E,), dtype=torch.int64, pin_memory=True)
@@ -321,8 +322,13 @@ class DistributedSparseMoeBlock(nn.Module):
         """Router logits (+ shared gate), fused softmax/top-k, permutation (:9519-9595).
         Returns the logits, a fresh tensor the caller owns."""
         logits = torch.empty((x.shape[0], self.num_experts), device=x.device, dtype=self.logits_dtype)
+        shared_gate = ws.shared_gate if self.shared_gate_weight is not None else None
+        if x.shape[0] <= ops.DECODE_MAX_TOKENS and self.routed_scaling_factor == 1.0:
+            ops.route_decode(x, self.gate_weight, self.shared_gate_weight, self.top_k, self.norm_topk_prob, logits,
+                             shared_gate, ws.topv, ws.topi, ws.perm, ws.route_counter)
+            return logits
         ops.router_logits(x, self.gate_weight, self.shared_gate_weight, self.logits_dtype, out=logits,
-                          shared_gate_out=ws.shared_gate if self.shared_gate_weight is not None else None)
+                          shared_gate_out=shared_gate)
         ops.gate_topk(logits, self.top_k, self.norm_topk_prob, out_dtype=self.dtype, topv=ws.topv, topi=ws.topi)
         if self.routed_scaling_factor != 1.0:
             ws.topv.mul_(self.routed_scaling_factor)

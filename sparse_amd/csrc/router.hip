@@ -1,5 +1,6 @@
-// Router: gate projection (logits) and fused softmax + top-k with wavefront shuffles.
-#include "common.h"
+// Router: gate projection (logits), fused softmax + top-k with wavefront shuffles, and
+// the single-launch decode router (logits -> top-k -> permutation).
+#include "permute_device.h"
 
 namespace sparse {
 
@@ -30,19 +31,14 @@ __device__ __forceinline__ void load8<uint16_t>(const uint16_t* p, float (&v)[8]
   v[6] = __uint_as_float(a.w << 16); v[7] = __uint_as_float(a.w & 0xffff0000u);
 }
 
-template <typename T, typename TL>
-__global__ __launch_bounds__(kRouterThreads) void router_logits_kernel(
-    const T* __restrict__ x, const T* __restrict__ wg, const T* __restrict__ wsg, int Ttok, int H,
-    int E, TL* __restrict__ logits, T* __restrict__ shared_gate) {
-  const int row = blockIdx.x;  // expert id, or E for the shared gate
-  const int t0 = blockIdx.y * kRouterTokTile;
-  const int nt = min(kRouterTokTile, Ttok - t0);
-  const T* w = (row < E) ? wg + static_cast<size_t>(row) * H : wsg;
-
+// Dot products of one weight row with up to 32 token rows; the workgroup's result for
+// token i lands in thread i (i < nt) and is stored by `store(token, value)`.
+template <typename T, typename Store>
+__device__ __forceinline__ void router_row_dots(const T* __restrict__ x, const T* __restrict__ w, int t0, int nt,
+                                                int H, Store store) {
   float acc[kRouterTokTile];
 #pragma unroll
   for (int i = 0; i < kRouterTokTile; ++i) acc[i] = 0.f;
-
   for (int h = threadIdx.x * 8; h < H; h += kRouterThreads * 8) {
     float wv[8];
     load8<T>(w + h, wv);
@@ -56,30 +52,43 @@ __global__ __launch_bounds__(kRouterThreads) void router_logits_kernel(
       }
     }
   }
-
   __shared__ float red[kRouterThreads / 64][kRouterTokTile];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
 #pragma unroll
   for (int i = 0; i < kRouterTokTile; ++i) {
-    const float s = wave_sum(acc[i]);
-    if (lane == 0) red[wave][i] = s;
+    if (i < nt) {
+      const float s = wave_sum(acc[i]);
+      if (lane == 0) red[wave][i] = s;
+    }
   }
   __syncthreads();
-  if (threadIdx.x < nt) {
+  if (static_cast<int>(threadIdx.x) < nt) {
     float s = 0.f;
 #pragma unroll
     for (int wv = 0; wv < kRouterThreads / 64; ++wv) s += red[wv][threadIdx.x];
-    const int t = t0 + threadIdx.x;
+    store(t0 + static_cast<int>(threadIdx.x), s);
+  }
+}
+
+template <typename T, typename TL>
+__global__ __launch_bounds__(kRouterThreads) void router_logits_kernel(
+    const T* __restrict__ x, const T* __restrict__ wg, const T* __restrict__ wsg, int Ttok, int H,
+    int E, TL* __restrict__ logits, T* __restrict__ shared_gate) {
+  const int row = blockIdx.x;  // expert id, or E for the shared gate
+  const int t0 = blockIdx.y * kRouterTokTile;
+  const int nt = min(kRouterTokTile, Ttok - t0);
+  const T* w = (row < E) ? wg + static_cast<size_t>(row) * H : wsg;
+  router_row_dots<T>(x, w, t0, nt, H, [&](int t, float s) {
     if (row < E) {
       Elem<TL>::store(logits + static_cast<size_t>(t) * E + row, s);
     } else {
       Elem<T>::store(shared_gate + t, s);
     }
-  }
+  });
 }
 
 // ---------------------------------------------------------------------------
-// Fused softmax(fp32) + top-k.  One wavefront per token; lane l holds experts
+// Fused softmax(fp32) + top-k of one token by one wavefront; lane l holds experts
 // l, l+64, l+128, l+192.  Selection runs K rounds of a wave-wide arg-max whose
 // order is (probability descending, expert id ascending).
 // ---------------------------------------------------------------------------
@@ -87,14 +96,8 @@ constexpr int kTopkWaves = 4;
 constexpr int kTopkNV = SPARSE_HIP_MAX_EXPERTS / 64;
 
 template <typename TL, typename TO>
-__global__ __launch_bounds__(kTopkWaves * 64) void gate_topk_kernel(
-    const TL* __restrict__ logits, int Ttok, int E, int K, int renorm, TO* __restrict__ topv,
-    int64_t* __restrict__ topi) {
-  const int lane = threadIdx.x & 63;
-  const int t = blockIdx.x * kTopkWaves + (threadIdx.x >> 6);
-  if (t >= Ttok) return;
-  const TL* row = logits + static_cast<size_t>(t) * E;
-
+__device__ __forceinline__ void topk_token(const TL* __restrict__ row, int E, int K, int renorm,
+                                           TO* __restrict__ topv_row, int64_t* __restrict__ topi_row, int lane) {
   float p[kTopkNV];
   float m = -INFINITY;
 #pragma unroll
@@ -156,9 +159,82 @@ __global__ __launch_bounds__(kTopkWaves * 64) void gate_topk_kernel(
   if (lane < K) {
     float v = sel_v;
     if (renorm) v = v / fmaxf(sum_sel, 1e-12f);
-    Elem<TO>::store(topv + static_cast<size_t>(t) * K + lane, v);
-    topi[static_cast<size_t>(t) * K + lane] = static_cast<int64_t>(sel_i);
+    Elem<TO>::store(topv_row + lane, v);
+    topi_row[lane] = static_cast<int64_t>(sel_i);
   }
+}
+
+template <typename TL, typename TO>
+__global__ __launch_bounds__(kTopkWaves * 64) void gate_topk_kernel(
+    const TL* __restrict__ logits, int Ttok, int E, int K, int renorm, TO* __restrict__ topv,
+    int64_t* __restrict__ topi) {
+  const int t = blockIdx.x * kTopkWaves + (threadIdx.x >> 6);
+  if (t >= Ttok) return;
+  topk_token<TL, TO>(logits + static_cast<size_t>(t) * E, E, K, renorm, topv + static_cast<size_t>(t) * K,
+                     topi + static_cast<size_t>(t) * K, threadIdx.x & 63);
+}
+
+// ---------------------------------------------------------------------------
+// Decode router in one launch (T <= 32).  Workgroup e computes logits[:, e] (workgroup E
+// the shared gate); the workgroup that finishes last -- counted with a device atomic
+// behind a fence -- runs softmax/top-k for every token and the single-block
+// permutation, then puts the counter back to zero for the next launch.
+// ---------------------------------------------------------------------------
+struct RouteArgs {
+  const void* x;
+  const void* wg;
+  const void* wsg;
+  void* logits;
+  void* shared_gate;
+  void* topv;
+  int64_t* topi;
+  int32_t* perm;
+  int32_t* inv_perm;
+  int32_t* seg_offsets;
+  int32_t* active_eids;
+  int32_t* n_active;
+  int32_t* counter;
+  int32_t T, H, E, K, renorm;
+};
+
+template <typename T, typename TL>
+__global__ __launch_bounds__(kRouterThreads) void route_decode_kernel(const RouteArgs a) {
+  const int row = blockIdx.x;
+  const T* x = static_cast<const T*>(a.x);
+  const T* w = (row < a.E) ? static_cast<const T*>(a.wg) + static_cast<size_t>(row) * a.H
+                           : static_cast<const T*>(a.wsg);
+  TL* logits = static_cast<TL*>(a.logits);
+  T* shared_gate = static_cast<T*>(a.shared_gate);
+  const int E = a.E;
+  router_row_dots<T>(x, w, 0, a.T, a.H, [&](int t, float s) {
+    if (row < E) {
+      Elem<TL>::store(logits + static_cast<size_t>(t) * E + row, s);
+    } else {
+      Elem<T>::store(shared_gate + t, s);
+    }
+  });
+
+  __shared__ int s_last;
+  __threadfence();  // this block's logits are visible device-wide before it is counted
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const int prev = atomicAdd(a.counter, 1);
+    s_last = (prev == static_cast<int>(gridDim.x) - 1);
+  }
+  __syncthreads();
+  if (!s_last) return;
+  __threadfence();
+  if (threadIdx.x == 0) a.counter[0] = 0;
+
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  for (int t = wave; t < a.T; t += kRouterThreads / 64)
+    topk_token<TL, T>(logits + static_cast<size_t>(t) * E, E, a.K, a.renorm,
+                      static_cast<T*>(a.topv) + static_cast<size_t>(t) * a.K, a.topi + static_cast<size_t>(t) * a.K,
+                      lane);
+  __threadfence_block();
+  __syncthreads();
+  permute_scatter_block<true>(a.topi, a.T, a.K, E, nullptr, 0, 1, a.perm, a.inv_perm, a.seg_offsets,
+                              a.active_eids, a.n_active);
 }
 
 template <typename T, typename TL>
@@ -181,6 +257,15 @@ static int launch_gate_topk(const void* logits, int Ttok, int E, int K, int reno
   hipLaunchKernelGGL((gate_topk_kernel<TL, TO>), grid, dim3(kTopkWaves * 64), 0, st,
                      static_cast<const TL*>(logits), Ttok, E, K, renorm, static_cast<TO*>(topv), topi);
   SP_LAUNCH_CHECK("gate_topk_kernel");
+  return SPARSE_HIP_OK;
+}
+
+template <typename T, typename TL>
+static int launch_route_decode(const RouteArgs& a, hipStream_t st) {
+  const int grid = a.E + (a.wsg != nullptr ? 1 : 0);
+  ProfScope prof(SPARSE_HIP_K_ROUTE_DECODE, st);
+  hipLaunchKernelGGL((route_decode_kernel<T, TL>), dim3(grid), dim3(kRouterThreads), 0, st, a);
+  SP_LAUNCH_CHECK("route_decode_kernel");
   return SPARSE_HIP_OK;
 }
 
@@ -224,6 +309,33 @@ int sparse_hip_gate_topk(const void* logits_dev, int logits_dtype, int T, int E,
   if (lb) return launch_gate_topk<uint16_t, float>(logits_dev, T, E, K, renorm, topv_dev, topi_dev, st);
   if (ob) return launch_gate_topk<float, uint16_t>(logits_dev, T, E, K, renorm, topv_dev, topi_dev, st);
   return launch_gate_topk<float, float>(logits_dev, T, E, K, renorm, topv_dev, topi_dev, st);
+}
+
+int sparse_hip_route_decode(const void* x_dev, const void* wg_dev, const void* wsg_dev, int dtype,
+                            int logits_dtype, int T, int H, int E, int K, int renorm, void* logits_dev,
+                            void* shared_gate_dev, void* topv_dev, int64_t* topi_dev, int32_t* perm_dev,
+                            int32_t* inv_perm_dev, int32_t* seg_offsets_dev, int32_t* active_eids_dev,
+                            int32_t* n_active_dev, int32_t* counter_dev, void* stream) {
+  SP_REQUIRE(valid_dtype(dtype) && valid_dtype(logits_dtype), "route_decode: unknown dtype");
+  SP_REQUIRE(logits_dtype == dtype || logits_dtype == SPARSE_HIP_F32,
+             "route_decode: logits_dtype must equal dtype or be fp32");
+  SP_REQUIRE(T >= 1 && T <= SPARSE_HIP_DECODE_MAX_TOKENS, "route_decode: T=%d outside [1,%d]", T,
+             SPARSE_HIP_DECODE_MAX_TOKENS);
+  SP_REQUIRE(H > 0 && H % 8 == 0, "route_decode: H=%d must be a positive multiple of 8", H);
+  SP_REQUIRE(E >= 1 && E <= SPARSE_HIP_MAX_EXPERTS, "route_decode: E=%d outside [1,%d]", E, SPARSE_HIP_MAX_EXPERTS);
+  SP_REQUIRE(K >= 1 && K <= SPARSE_HIP_MAX_TOPK && K <= E, "route_decode: K=%d outside [1,min(%d,E)]", K,
+             SPARSE_HIP_MAX_TOPK);
+  SP_REQUIRE(x_dev && wg_dev && logits_dev && topv_dev && topi_dev && perm_dev && inv_perm_dev && seg_offsets_dev &&
+                 active_eids_dev && n_active_dev && counter_dev,
+             "route_decode: NULL pointer");
+  SP_REQUIRE(wsg_dev == nullptr || shared_gate_dev != nullptr, "route_decode: shared gate output is NULL");
+  RouteArgs a = {x_dev,     wg_dev,       wsg_dev,         logits_dev,      shared_gate_dev, topv_dev,   topi_dev,
+                 perm_dev,  inv_perm_dev, seg_offsets_dev, active_eids_dev, n_active_dev,    counter_dev,
+                 T,         H,            E,               K,               renorm};
+  hipStream_t st = as_stream(stream);
+  if (dtype == SPARSE_HIP_F32) return launch_route_decode<float, float>(a, st);
+  if (logits_dtype == SPARSE_HIP_F32) return launch_route_decode<uint16_t, float>(a, st);
+  return launch_route_decode<uint16_t, uint16_t>(a, st);
 }
 
 }  // extern "C"

@@ -196,7 +196,7 @@ const char* sparse_hip_kernel_name(int kernel) {
   static const char* names[SPARSE_HIP_K_COUNT] = {
       "router_logits_kernel", "gate_topk_kernel",   "permute_scatter_kernel", "decode_ffn_kernel<true>",
       "decode_ffn_kernel<false>", "prefill_ffn_kernel<true>", "prefill_ffn_kernel<false>",
-      "ffn_tiled_kernel<gate_up>", "ffn_tiled_kernel<down>", "combine_kernel"};
+      "ffn_tiled_kernel<gate_up>", "ffn_tiled_kernel<down>", "combine_kernel", "route_decode_kernel"};
   if (kernel < 0 || kernel >= SPARSE_HIP_K_COUNT) return "";
   return names[kernel];
 }

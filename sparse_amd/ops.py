@@ -118,6 +118,31 @@ def permute_build(topi: torch.Tensor, num_experts: int, out: Optional[Permutatio
     return out
 
 
+def route_decode(x: torch.Tensor, wg: torch.Tensor, wsg: Optional[torch.Tensor], k: int, renorm: bool,
+                 logits: torch.Tensor, shared_gate: Optional[torch.Tensor], topv: torch.Tensor,
+                 topi: torch.Tensor, perm: Permutation, counter: torch.Tensor) -> None:
+    """Router logits + top-k + permutation in one launch (T <= 32).  ``counter`` is a zeroed
+    int32[1] the kernel uses to find its last workgroup and leaves at zero."""
+    lib = _lib.load()
+    T, H = x.shape
+    E = wg.shape[0]
+    _need(x, "x")
+    _need(wg, "wg", x.dtype, (E, H))
+    _need(logits, "logits", None, (T, E))
+    _need(topv, "topv", x.dtype, (T, k))
+    _need(topi, "topi", torch.int64, (T, k))
+    _need(counter, "counter", torch.int32, (1,))
+    if wsg is not None:
+        _need(wsg, "wsg", x.dtype)
+        _need(shared_gate, "shared gate logits", x.dtype, (T,))
+    rc = lib.sparse_hip_route_decode(_ptr(x), _ptr(wg), _ptr(wsg), dtype_code(x.dtype), dtype_code(logits.dtype),
+                                     T, H, E, int(k), int(bool(renorm)), _ptr(logits), _ptr(shared_gate),
+                                     _ptr(topv), _ptr(topi), _ptr(perm.perm), _ptr(perm.inv_perm),
+                                     _ptr(perm.seg_offsets), _ptr(perm.active_eids), _ptr(perm.n_active),
+                                     _ptr(counter), _stream())
+    _lib.check(rc, "sparse_hip_route_decode")
+
+
 # --------------------------------------------------------------------------- experts
 def make_experts(slab: torch.Tensor, expert_slot: torch.Tensor, num_experts: int, hidden: int, inter: int,
                  slot_stride_bytes: Optional[int] = None) -> Experts:

@@ -118,6 +118,38 @@ def test_router_logits(device, dtype, T):
         torch.testing.assert_close(l32.cpu(), ref, rtol=1e-4, atol=1e-4)
 
 
+@pytest.mark.parametrize("dtype,ldt", [(torch.bfloat16, torch.bfloat16), (torch.bfloat16, torch.float32),
+                                       (torch.float32, torch.float32)])
+@pytest.mark.parametrize("T", [1, 8, 32])
+def test_route_decode_equals_the_three_separate_calls(device, dtype, ldt, T):
+    """The single-launch decode router must reproduce router_logits + gate_topk +
+    permute_build bit for bit, call after call (its counter goes back to zero)."""
+    ops = _ops()
+    E, K, H = 60, 4, 2048
+    layer = make_layer(H, E, 64, K, Is=64, shared_gate=True, dtype=dtype, seed=7)
+    wg, wsg = layer["gate_w"].to(device), layer["shared_gate_w"].to(device)
+    counter = torch.zeros(1, dtype=torch.int32, device=device)
+    for rep in range(3):
+        x = make_hidden(T, H, dtype, seed=100 + rep).to(device)
+        logits_a, sg_a = ops.router_logits(x, wg, wsg, logits_dtype=ldt)
+        topv_a, topi_a = ops.gate_topk(logits_a, K, out_dtype=dtype)
+        perm_a = ops.permute_build(topi_a, E)
+        logits_b = torch.empty_like(logits_a)
+        sg_b = torch.empty_like(sg_a)
+        topv_b, topi_b = torch.empty_like(topv_a), torch.empty_like(topi_a)
+        perm_b = ops.Permutation(T, K, E, device)
+        ops.route_decode(x, wg, wsg, K, False, logits_b, sg_b, topv_b, topi_b, perm_b, counter)
+        torch.cuda.synchronize()
+        assert int(counter.item()) == 0
+        assert torch.equal(logits_a, logits_b) and torch.equal(sg_a, sg_b)
+        assert torch.equal(topv_a, topv_b) and torch.equal(topi_a, topi_b)
+        n = int(perm_a.n_active.item())
+        assert n == int(perm_b.n_active.item())
+        for name in ("perm", "inv_perm", "seg_offsets"):
+            assert torch.equal(getattr(perm_a, name), getattr(perm_b, name)), name
+        assert torch.equal(perm_a.active_eids[:n], perm_b.active_eids[:n])
+
+
 # ------------------------------------------------------------------ permute
 @pytest.mark.parametrize("T,E,K", [(1, 60, 4), (8, 60, 4), (32, 60, 4), (255, 64, 6), (256, 64, 6),
                                     (257, 64, 6), (2048, 64, 6), (4096, 64, 6), (1000, 256, 16), (3, 4, 4)])
