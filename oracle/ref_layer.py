@@ -1,0 +1,579 @@
+"""CPU oracle of one layer's cache / prefetch / EPIPE state machine.  TEST INFRASTRUCTURE
+ONLY: only ``tests/``, ``__graft_entry__.smoke()`` and ``bench.py``'s ``cpu_baseline`` leg
+may import this.
+
+``RefLayer`` restates, method by method, the parts of the reference's
+``DistributedSparseMoeBlock`` that decide residency and execution order on one GPU
+(world size 1, ``cache_policy=lru``, ``expert_offload=cpu``), without any device work.
+Every method names the reference lines it follows (utils/eval_core.py).  Device effects
+are recorded in ``trace`` as tuples:
+
+    ("hit" | "prefetch_hit" | "miss", eid)       cache events (:5400-5418)
+    ("h2d", lane, eid)                           a copy enqueued on compute/prefetch/epipe
+    ("wait", eid)                                the compute stream waits a copy event
+    ("compute", eid)                             the expert's segment is executed
+    ("plan", ((eid, victim), ...))               an admitted prefetch plan
+
+Copy completion is not modelled by time: ``copy_done(eid)`` (a callable given by the
+test, default "always complete") answers ``event.query()``.
+
+Pinned by (tests/test_oracle_residency.py and tests/golden/):
+  score map          the reference's known-answer tests of the same formula through
+                     ``select_candidates`` (tests/test_rs_staging.py:147-150, :308-312)
+                     and golden vectors from the reference's own
+                     ``_build_target_layer_prob_score_map``.
+  plan / victims     golden vectors from the reference's own
+                     ``_build_prefetch_plan_from_score_map`` and
+                     ``_pick_victims_by_low_value`` on random states; invariants (plan
+                     never exceeds the budget, never names a cached expert, victims are
+                     evictable and unprotected).
+  demand path        reference test tests/test_rs_staging.py:74-92 (in-flight prefetch hit:
+                     exactly one wait, ``is_prefetch_hit``, no second load) restated;
+                     textbook LRU replay.
+  EPIPE executors    parity unpinned against executed reference code: all four executors
+                     return None unless ``device.type == "cuda"`` (:11881, :12184), so they
+                     cannot run in a GPU-less container.  Pinned only by restatement plus
+                     invariants: every segment computed exactly once, the staged expert
+                     counts exactly one miss, resident experts run before the wait,
+                     outputs equal the plain path.
+"""
+from __future__ import annotations
+
+from typing import Any, Callable, Dict, List, Optional, Sequence, Set, Tuple
+
+from .ref_cache import RefEpipePrefillExtraCache, RefExpertWeightCache
+
+Segment = Tuple[int, int]  # (expert id, rows)
+
+
+class RefConfig:
+    """Reference defaults (:4939-5075, :5066-5075, :10162-10183)."""
+
+    def __init__(self, **kw: Any) -> None:
+        self.capacity = 10
+        self.planner_mode = "none"
+        self.prefetch_top_m = 4
+        self.pred_topk: Optional[int] = None
+        self.rs_policy = "default"
+        self.min_candidate_score = 0.02
+        self.replace_advantage = 0.02
+        self.replace_margin = 1.05
+        self.cache_safe_min_score = 0.03
+        self.cache_safe_replace_advantage = 0.05
+        self.cache_safe_replace_margin = 1.10
+        self.allow_active_replace = True
+        self.recent_protect_steps = 0
+        self.protect_mode = "default"
+        self.wait_before_evict = True
+        self.cache_ttl_steps = 0
+        self.epipe_enable = False
+        self.epipe_prefill_enable = False
+        self.epipe_mode = "upfront_scan"
+        self.epipe_decode_rs_mode = "late_only"
+        self.epipe_no_evict = True
+        self.epipe_transient_staging = True
+        self.epipe_min_ready_experts = 1
+        self.epipe_min_ready_items = 1
+        self.epipe_min_missing_experts = 1
+        self.epipe_sort_ready_by_work = False
+        self.epipe_prefill_commit = True
+        self.epipe_rs_handle_late_prefetch = True
+        self.epipe_rs_handle_demand_miss = False
+        self.epipe_rs_force_demand_stage = False
+        self.epipe_rs_demand_commit = True
+        self.epipe_deferred_lru_commit = True
+        self.epipe_rs_min_buffer_groups = 1
+        self.epipe_rs_min_buffer_items = 1
+        self.epipe_rs_rolling_gate = True
+        self.epipe_rs_gate_window = 16
+        self.epipe_rs_gate_min_triggers = 1
+        self.epipe_rs_gate_skip_steps = 8
+        self.epipe_prefill_extra_cache_slots = 0
+        for k, v in kw.items():
+            if not hasattr(self, k):
+                raise ValueError(f"unknown option {k}")
+            setattr(self, k, v)
+
+
+class RefLayer:
+    def __init__(self, layer_idx: int, num_experts: int, top_k: int, cfg: RefConfig,
+                 copy_done: Optional[Callable[[int], bool]] = None) -> None:
+        self.layer_idx, self.num_experts, self.top_k, self.cfg = layer_idx, num_experts, top_k, cfg
+        self.cache = RefExpertWeightCache(cfg.capacity)
+        self.extra = RefEpipePrefillExtraCache(cfg.epipe_prefill_extra_cache_slots)
+        self.copy_done = copy_done or (lambda eid: True)
+        self.prefetched: Set[int] = set()        # _prefetched_ids_this_group
+        self.used: Set[int] = set()              # _prefetch_used_ids_this_group
+        self.events: Dict[int, int] = {}         # _prefetch_events: eid -> token
+        self.cycle_key = None
+        self.freq: Dict[int, int] = {}           # _expert_access_freq
+        self.last_used: Dict[int, int] = {}      # _last_used_decode_step
+        self.gate_calls = self.gate_triggers = self.gate_skip = 0
+        self.phase, self.call_id, self.stage = "none", -1, "decode"
+        self.trace: List[Tuple] = []
+        self.counters: Dict[str, int] = {}
+
+    def _count(self, name: str, n: int = 1) -> None:
+        self.counters[name] = self.counters.get(name, 0) + n
+
+    # ------------------------------------------------------------ demand path
+    def _protect_ttl(self) -> Set[int]:
+        """:5929-5938."""
+        out: Set[int] = set()
+        if self.cfg.cache_ttl_steps > 0 and self.phase == "decode" and self.call_id >= 0:
+            for eid, last in self.last_used.items():
+                if self.call_id - last <= self.cfg.cache_ttl_steps:
+                    out.add(eid)
+        return out
+
+    def on_demand_access(self, eid: int) -> None:
+        """:11213-11221."""
+        self.freq[eid] = self.freq.get(eid, 0) + 1
+        if self.phase == "decode":
+            self.last_used[eid] = self.call_id
+        if self.freq[eid] >= 2:
+            self.cache.promote_hot(eid)
+
+    def cache_put_guarded(self, eid: int) -> None:
+        """:5985-6022 with :5940-5951."""
+        protect = self._protect_ttl()
+        protect.discard(eid)
+        resident = set(self.cache.resident_ids())
+        if resident and resident.issubset(protect):
+            protect = set()
+        self.cache.put(eid, ("w", eid), pinned=False, protect_ids=protect)
+
+    def maybe_wait_prefetch(self, eid: int) -> None:
+        """:11176-11210."""
+        if eid in self.events:
+            del self.events[eid]
+            if self.copy_done(eid):
+                self._count("prefetch_complete_before_use")
+            self.trace.append(("wait", eid))
+            self._count("prefetch_completed")
+
+    def record_cached_use(self, eid: int, wait: bool) -> None:
+        """:11395-11412 and :11652-11670."""
+        if eid in self.prefetched:
+            self.trace.append(("prefetch_hit", eid))
+            self.used.add(eid)
+            self.cache.unpin(eid)
+            self.cache.promote_hot(eid)
+        else:
+            self.trace.append(("hit", eid))
+        if wait:
+            self.maybe_wait_prefetch(eid)
+
+    def demand(self, eid: int) -> None:
+        """``_get_local_module_weights`` :11388-11435."""
+        if self.cache.get(eid) is not None:
+            self.record_cached_use(eid, wait=True)
+            return
+        if self.extra.get(eid) is not None:
+            return
+        self.trace.append(("miss", eid))
+        self.trace.append(("h2d", "compute", eid))
+        self.on_demand_access(eid)
+        self.cache_put_guarded(eid)
+
+    def compute(self, eid: int, have_payload: bool = False) -> None:
+        if not have_payload:
+            self.demand(eid)
+        self.trace.append(("compute", eid))
+
+    # ------------------------------------------------------------ executors
+    def epipe_stage_enabled(self) -> bool:
+        """:5585-5598."""
+        c = self.cfg
+        if self.stage == "prefill":
+            return bool(c.epipe_prefill_enable)
+        if self.stage == "decode":
+            if c.planner_mode == "rs_prefetch":
+                return bool(c.epipe_enable and c.epipe_decode_rs_mode not in ("off", "disabled"))
+            return bool(c.epipe_enable)
+        return False
+
+    def execute(self, segments: Sequence[Segment]) -> str:
+        """Executor choice of ``_execute_local_recv_groups`` :13264-13357."""
+        if not segments:
+            return "empty"
+        c = self.cfg
+        result = None
+        if self.epipe_stage_enabled() and c.epipe_mode != "off":
+            rs_active = c.planner_mode == "rs_prefetch"
+            if self.stage == "decode" and rs_active and c.epipe_decode_rs_mode == "off":
+                result = None
+            elif self.stage == "decode" and rs_active and c.epipe_decode_rs_mode == "residual_scan":
+                result = self.epipe_rs_residual_scan(segments)
+            elif self.stage == "decode" and rs_active:
+                raise NotImplementedError("buffered / late_only / demand_only are not restated")
+            elif self.stage == "decode" and c.epipe_mode != "miss_triggered":
+                result = self.epipe_upfront_scan(segments)
+            elif c.epipe_mode == "upfront_scan":
+                result = self.epipe_upfront_scan(segments)
+            else:
+                raise NotImplementedError("miss_triggered is not restated")
+        if result is None:
+            for eid, _ in segments:  # ascending expert id, :13340-13357
+                self.compute(eid)
+            result = "plain"
+        return result
+
+    def contains_no_touch(self, eid: int) -> bool:
+        """:5815-5851."""
+        return self.extra.has(eid) or self.cache.has(eid)
+
+    def epipe_upfront_scan(self, segments: Sequence[Segment]) -> Optional[str]:
+        """:11867-12167."""
+        c = self.cfg
+        if not (c.epipe_enable if self.stage == "decode" else c.epipe_prefill_enable):
+            return None
+        ready = [s for s in segments if self.contains_no_touch(s[0])]
+        missing = [s for s in segments if not self.contains_no_touch(s[0])]
+        ready_items = sum(n for _, n in ready)
+        free = max(0, self.cache.capacity - len(self.cache.resident_ids()))
+        if len(ready) < c.epipe_min_ready_experts or ready_items < c.epipe_min_ready_items:
+            self._count("epipe_fallback_no_ready")
+            return None
+        if len(missing) < c.epipe_min_missing_experts:
+            self._count("epipe_fallback_no_missing")
+            return None
+        staged = missing[0][0]
+        can_insert = free > 0 and not (self.stage == "prefill" and not c.epipe_prefill_commit)
+        use_transient = not can_insert
+        if use_transient and not c.epipe_transient_staging:
+            self._count("epipe_fallback_cache_full_no_temp")
+            return None
+        self.trace.append(("h2d", "epipe", staged))
+        order = list(ready)
+        if c.epipe_sort_ready_by_work:
+            order.sort(key=lambda s: s[1], reverse=True)
+        for eid, _ in order:
+            self.compute(eid)
+        self.trace.append(("wait", staged))
+        self.trace.append(("miss", staged))
+        if self.stage != "prefill":
+            self.on_demand_access(staged)
+        if can_insert:
+            if len(self.cache.resident_ids()) < self.cache.capacity:
+                if self.stage == "prefill":
+                    self.on_demand_access(staged)
+                self.cache_put_guarded(staged)
+            else:
+                use_transient = True
+        if use_transient and self.stage == "prefill":
+            self.extra.put(staged, ("w", staged))
+        self.compute(staged, have_payload=True)
+        for eid, _ in missing[1:]:
+            self.compute(eid)
+        return "epipe_upfront"
+
+    def pending_prefetch_event(self, eid: int) -> bool:
+        """:11636-11650: True while the copy is in flight; a finished one is retired."""
+        if eid not in self.events:
+            return False
+        if self.copy_done(eid):
+            del self.events[eid]
+            self._count("prefetch_complete_before_use")
+            self._count("prefetch_completed")
+            return False
+        return True
+
+    def demand_gate_can_open(self) -> bool:
+        """:5880-5893 (the exposed-stall threshold is zero by default, so only the force flag opens it)."""
+        return bool(self.cfg.epipe_rs_handle_demand_miss and self.cfg.epipe_rs_force_demand_stage)
+
+    def _residual_present(self, segments: Sequence[Segment]) -> bool:
+        for eid, _ in segments:
+            if eid in self.events and self.cfg.epipe_rs_handle_late_prefetch and not self.copy_done(eid):
+                return True
+            if self.demand_gate_can_open() and not self.contains_no_touch(eid):
+                return True
+        return False
+
+    def _maybe_skip_gate(self, segments: Sequence[Segment]) -> bool:
+        """:12228-12254."""
+        c = self.cfg
+        if not c.epipe_rs_rolling_gate:
+            return False
+        if self.gate_skip > 0:
+            if self._residual_present(segments):
+                self.gate_skip = 0
+                return False
+            self.gate_skip -= 1
+            return True
+        self.gate_calls += 1
+        if self.gate_calls >= c.epipe_rs_gate_window and self.gate_triggers < c.epipe_rs_gate_min_triggers:
+            self.gate_calls = self.gate_triggers = 0
+            self.gate_skip = int(c.epipe_rs_gate_skip_steps)
+            if self.gate_skip > 0:
+                self.gate_skip -= 1
+                return True
+        if self.gate_calls >= c.epipe_rs_gate_window:
+            self.gate_calls = self.gate_triggers = 0
+        return False
+
+    def epipe_rs_residual_scan(self, segments: Sequence[Segment]) -> Optional[str]:
+        """:12169-12512."""
+        c = self.cfg
+        if self.stage != "decode" or c.planner_mode != "rs_prefetch" or not c.epipe_enable:
+            return None
+        if self._maybe_skip_gate(segments):
+            return None
+        ready: List[int] = []
+        late: List[int] = []
+        dem: List[int] = []
+        for i, (eid, _) in enumerate(segments):
+            pending = self.pending_prefetch_event(eid)
+            cached = self.contains_no_touch(eid)
+            if cached and not pending:
+                ready.append(i)
+            elif cached and pending and c.epipe_rs_handle_late_prefetch:
+                late.append(i)
+            elif not cached and c.epipe_rs_handle_demand_miss and self.demand_gate_can_open():
+                dem.append(i)
+        ready_items = sum(segments[i][1] for i in ready)
+        if len(ready) < c.epipe_rs_min_buffer_groups or ready_items < c.epipe_rs_min_buffer_items:
+            return None
+        residual, kind = None, ""
+        if late:
+            residual, kind = late[0], "late"
+        elif dem and c.epipe_rs_handle_demand_miss and ready_items >= c.epipe_rs_min_buffer_items \
+                and self.demand_gate_can_open():
+            residual, kind = dem[0], "demand"
+        if residual is None:
+            return None
+        reid = segments[residual][0]
+        cover = [i for i in ready if i != residual]
+        if len(cover) < c.epipe_rs_min_buffer_groups:
+            return None
+        if c.epipe_rs_rolling_gate:
+            self.gate_triggers += 1
+
+        def compute_ready(indices: Sequence[int]) -> None:
+            for i in indices:
+                eid = segments[i][0]
+                if self.cache.get(eid) is None:
+                    self.compute(eid)
+                else:
+                    self.record_cached_use(eid, wait=False)
+                    self.compute(eid, have_payload=True)
+
+        done = set()
+        if kind == "late":
+            if self.cache.get(reid) is None:
+                return None
+            compute_ready(cover)
+            done.update(cover)
+            self.maybe_wait_prefetch(reid)
+            self.record_cached_use(reid, wait=False)
+            self.compute(reid, have_payload=True)
+            done.add(residual)
+        else:
+            self.trace.append(("h2d", "epipe", reid))
+            compute_ready(cover)
+            done.update(cover)
+            self.trace.append(("wait", reid))
+            self.trace.append(("miss", reid))
+            self.on_demand_access(reid)
+            free = max(0, self.cache.capacity - len(self.cache.resident_ids()))
+            if c.epipe_rs_demand_commit and c.epipe_deferred_lru_commit and (free > 0 or not c.epipe_no_evict):
+                self.cache_put_guarded(reid)
+            self.compute(reid, have_payload=True)
+            done.add(residual)
+        for i, (eid, _) in enumerate(segments):
+            if i not in done:
+                self.compute(eid)
+        if c.epipe_rs_rolling_gate and self.gate_skip > 0:
+            self.gate_skip = 0
+        return "epipe_rs_residual_scan"
+
+    # ------------------------------------------------------------ RS prefetch
+    def effective_top_m(self) -> int:
+        return max(0, int(self.cfg.prefetch_top_m))
+
+    def predict_topk(self) -> int:
+        """:10888-10901."""
+        if self.cfg.pred_topk is not None:
+            return max(1, min(int(self.cfg.pred_topk), self.num_experts))
+        return max(self.top_k, min(self.num_experts, self.effective_top_m()))
+
+    def finalize_prev_group_prefetch(self) -> None:
+        """:9598-9635."""
+        for eid in list(self.events):
+            if self.copy_done(eid):
+                self._count("prefetch_completed")
+                del self.events[eid]
+        self._count("prefetch_wasted", len(self.prefetched - self.used))
+        self.cache.unpin_all()
+        self.prefetched.clear()
+        self.used.clear()
+        self.cycle_key = None
+
+    def begin_cycle(self, key) -> None:
+        """:9637-9649."""
+        if self.cycle_key == key:
+            return
+        self.finalize_prev_group_prefetch()
+        self.cycle_key = key
+
+    def prefetch_protect_ids(self) -> Set[int]:
+        """:9651-9665."""
+        if self.cfg.protect_mode in ("minimal", "current_next", "current-next"):
+            protect = set(self.used)
+        else:
+            protect = set(self.prefetched) | set(self.used)
+        protect |= self._protect_ttl()
+        r = int(self.cfg.recent_protect_steps)
+        if r > 0 and self.phase == "decode" and self.call_id >= 0:
+            for eid, last in self.last_used.items():
+                if self.call_id - last <= r:
+                    protect.add(eid)
+        return protect
+
+    def prefetch_budget(self, key) -> int:
+        """:9785-9810 with :9754-9771."""
+        top_m = self.effective_top_m()
+        if self.cfg.planner_mode != "rs_prefetch" or top_m <= 0:
+            return 0
+        self.begin_cycle(key)
+        protect = self.prefetch_protect_ids()
+        room = self.cache.prefetch_free_slots()
+        if self.cfg.allow_active_replace:
+            room += len(self.cache.evictable_prefetch_ids(protect))
+        return max(0, min(max(0, top_m - len(self.prefetched)), room))
+
+    @staticmethod
+    def score_map(flat_ids: Sequence[int], flat_probs: Sequence[float]) -> Dict[int, float]:
+        """:10040-10107 at world size 1 (every expert is local)."""
+        raw: Dict[int, float] = {}
+        occ: Dict[int, int] = {}
+        top: Dict[int, float] = {}
+        for eid, w in zip(flat_ids, flat_probs):
+            eid, w = int(eid), float(w)
+            raw[eid] = raw.get(eid, 0.0) + w
+            occ[eid] = occ.get(eid, 0) + 1
+            top[eid] = max(top.get(eid, 0.0), w)
+        out: Dict[int, float] = {}
+        for eid, s in raw.items():
+            out[eid] = float(s)
+        for eid in list(out):
+            boost = 1.0 + 0.15 * float(max(occ.get(eid, 1) - 1, 0))
+            out[eid] = out[eid] * boost + 0.05 * float(top.get(eid, 0.0))
+        return out
+
+    def resident_keep_bias(self, eid: int) -> float:
+        """:10031-10038 (plain LRU has no hot tier)."""
+        bias = 0.02 * float(min(self.freq.get(int(eid), 0), 16))
+        if int(eid) in self.prefetched:
+            bias += 0.10
+        return float(bias)
+
+    def pick_victims_by_low_value(self, scores: Dict[int, float], protect: Set[int]) -> List[int]:
+        """:10135-10142."""
+        ranked = []
+        for pos, eid in enumerate(self.cache.evictable_prefetch_ids(protect)):
+            ranked.append((float(scores.get(int(eid), 0.0)) + self.resident_keep_bias(int(eid)), pos, int(eid)))
+        ranked.sort(key=lambda x: (x[0], x[1]))
+        return [e for _, _, e in ranked]
+
+    def build_plan(self, scores: Dict[int, float], protect: Set[int], budget: int):
+        """:10144-10262."""
+        c = self.cfg
+        if budget <= 0 or len(scores) == 0:
+            return []
+        min_score, adv, margin = c.min_candidate_score, c.replace_advantage, c.replace_margin
+        if c.rs_policy in ("cache_safe", "cache-safe", "benefit_gate", "benefit-gate"):
+            min_score = max(min_score, c.cache_safe_min_score)
+            adv = max(adv, c.cache_safe_replace_advantage)
+            margin = max(margin, c.cache_safe_replace_margin)
+        cands = []
+        for eid, sc in scores.items():
+            if self.cache.has(int(eid)):
+                continue
+            if float(sc) < min_score:
+                continue
+            cands.append((float(sc), int(eid)))
+        if not cands:
+            return []
+        cands.sort(key=lambda x: x[0], reverse=True)
+        free = self.cache.prefetch_free_slots()
+        victims = self.pick_victims_by_low_value(scores, protect)
+        plan = []
+        cpos = 0
+        for _ in range(min(int(free), int(budget), len(cands))):
+            plan.append((cands[cpos][1], None))
+            cpos += 1
+        remaining = int(budget) - len(plan)
+        if remaining <= 0 or not c.allow_active_replace:
+            return plan
+        vpos = 0
+        while cpos < len(cands) and vpos < len(victims) and remaining > 0:
+            cs, ce = cands[cpos]
+            v = victims[vpos]
+            vs = float(scores.get(v, 0.0)) + self.resident_keep_bias(v)
+            if cs >= vs * margin or (cs - vs) >= adv:
+                plan.append((ce, v))
+                remaining -= 1
+                cpos += 1
+                vpos += 1
+            else:
+                break
+        return plan
+
+    def admit_plan(self, plan) -> None:
+        """:10433-10527."""
+        if not plan:
+            return
+        self._count("prefetch_issued", len(plan))
+        protect = self.prefetch_protect_ids()
+        for eid, victim in plan:
+            eid = int(eid)
+            if self.cache.has(eid):
+                payload = self.cache.get(eid)
+                if not self.cache.admit_prefetch(eid, payload, protect_ids=protect, preferred_victim=victim):
+                    continue
+                self.prefetched.add(eid)
+                protect.add(eid)
+                self._count("prefetch_admitted")
+                continue
+            if victim is not None:  # :10011-10026
+                if victim in self.events:
+                    del self.events[victim]
+                    if self.cfg.wait_before_evict:
+                        self.trace.append(("wait_prefetch_lane", victim))
+                self.cache.discard(victim)
+                self.prefetched.discard(victim)
+                self.used.discard(victim)
+            self.trace.append(("h2d", "prefetch", eid))
+            if not self.cache.admit_prefetch(eid, ("w", eid), protect_ids=protect, preferred_victim=victim):
+                continue
+            self.events[eid] = 1
+            self.prefetched.add(eid)
+            protect.add(eid)
+            if self.cfg.protect_mode in ("minimal", "current_next", "current-next"):
+                self.cache.unpin(eid)
+            self._count("prefetch_admitted")
+
+    def schedule_prefetch(self, flat_ids, flat_probs, budget: int):
+        """:10996-11010 with :10413-10431."""
+        protect = self.prefetch_protect_ids()
+        plan = self.build_plan(self.score_map(flat_ids, flat_probs), protect, budget)
+        if plan:
+            self.trace.append(("plan", tuple(plan)))
+        self.admit_plan(plan)
+        return plan
+
+    def reset_for_new_request(self, clear_expert_cache: bool = False, clear_cache_metadata: bool = True) -> None:
+        """:6097-6147."""
+        self.events.clear()
+        self.prefetched.clear()
+        self.used.clear()
+        self.freq.clear()
+        self.last_used.clear()
+        self.cycle_key = None
+        if clear_expert_cache:
+            self.cache.clear()
+            self.extra.clear()
+        elif clear_cache_metadata:
+            self.cache.reset_request_metadata(unpin=True)

@@ -1,0 +1,53 @@
+"""CPU oracle of the RS predictor and of candidate selection.  TEST INFRASTRUCTURE ONLY:
+only ``tests/``, ``__graft_entry__.smoke()`` and ``bench.py``'s ``cpu_baseline`` leg may
+import this.
+
+``routing_scout_forward`` restates ``RoutingScoutMLP.forward`` in eval mode
+(utils/eval_core.py:3402-3417: Linear, BatchNorm1d with running statistics, ReLU, Dropout
+as identity, Linear, Softmax) in numpy float32.  Pinned by closed form against
+``torch.nn`` layers with the same parameters (tests/test_residency.py).
+
+``select_candidates`` restates utils/rs_staging.py:97-118, the staging adapter's scoring
+(the same formula as utils/eval_core.py:10104-10106).  Pinned by the reference's own
+known-answer tests, tests/test_rs_staging.py:147-150 and :308-312.
+"""
+from __future__ import annotations
+
+from typing import Dict, Iterable, List, Optional, Sequence, Set
+
+import numpy as np
+
+
+def routing_scout_forward(x: np.ndarray, w1, b1, bn_weight, bn_bias, bn_mean, bn_var, w2, b2,
+                          eps: float = 1e-5) -> np.ndarray:
+    h = x.astype(np.float32) @ np.asarray(w1, np.float32).T + np.asarray(b1, np.float32)
+    h = (h - bn_mean) / np.sqrt(np.asarray(bn_var, np.float32) + eps) * bn_weight + bn_bias
+    h = np.maximum(h, 0.0)
+    z = h @ np.asarray(w2, np.float32).T + np.asarray(b2, np.float32)
+    z = z - z.max(axis=-1, keepdims=True)
+    e = np.exp(z)
+    return (e / e.sum(axis=-1, keepdims=True)).astype(np.float32)
+
+
+def select_candidates(ids: Sequence[int], weights: Sequence[float], *, allowed: Set[int], resident: Set[int],
+                      minimum: float, budget: int, diagnostics: Optional[Dict[str, int]] = None) -> List[int]:
+    total: Dict[int, float] = {}
+    seen: Dict[int, int] = {}
+    best: Dict[int, float] = {}
+    skipped_nonlocal = skipped_resident = 0
+    for eid, w in zip(ids, weights):
+        eid, w = int(eid), float(w)
+        if eid not in allowed:
+            skipped_nonlocal += 1
+        elif eid in resident:
+            skipped_resident += 1
+        else:
+            total[eid] = total.get(eid, 0.0) + w
+            seen[eid] = seen.get(eid, 0) + 1
+            best[eid] = max(best.get(eid, 0.0), w)
+    score = {e: s * (1 + 0.15 * (seen[e] - 1)) + 0.05 * best[e] for e, s in total.items()}
+    if diagnostics is not None:
+        diagnostics.update(nonlocal_entries=skipped_nonlocal, resident_entries=skipped_resident, scored=len(score),
+                           below_threshold=sum(1 for v in score.values() if v < minimum))
+    ranked = sorted(score, key=score.get, reverse=True)
+    return [e for e in ranked if score[e] >= minimum][:budget]

@@ -150,7 +150,7 @@ class _HipBackend(Backend):
     def event_done(self, event) -> bool:
         return event.query()
 
-    def wait_event(self, event, lane: str) -> None:
+    def wait_event(self, event, lane: str, ordering: bool = False) -> None:
         event.wait(self._stream(lane))
 
     def run_segments(self, segments: Sequence[Tuple[int, int]]) -> None:

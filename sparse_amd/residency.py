@@ -155,8 +155,9 @@ class Backend:
     def event_done(self, event: Any) -> bool:
         raise NotImplementedError
 
-    def wait_event(self, event: Any, lane: str) -> None:
-        """Make ``lane`` wait for ``event`` (never blocks the host)."""
+    def wait_event(self, event: Any, lane: str, ordering: bool = False) -> None:
+        """Make ``lane`` wait for ``event`` (never blocks the host).  ``ordering`` marks waits
+        that only protect the reuse of a slot, as opposed to waits the policy itself asks for."""
         raise NotImplementedError
 
     def run_segments(self, segments: Sequence[Tuple[int, int]]) -> None:
@@ -241,10 +242,10 @@ class LayerResidency:
     def _upload(self, eid: int, slot: int, lane: str) -> Any:
         fence = self._slot_fence.pop(slot, None)
         if fence is not None and lane != "compute":
-            self.backend.wait_event(fence, lane)
+            self.backend.wait_event(fence, lane, True)
         prev = self._slot_upload.get(slot)
         if prev is not None and prev[1] != lane:
-            self.backend.wait_event(prev[0], lane)
+            self.backend.wait_event(prev[0], lane, True)
         ev = self.backend.upload(int(eid), int(slot), lane)
         self._slot_upload[slot] = (ev, lane)
         return ev
@@ -849,7 +850,7 @@ class LayerResidency:
         """Reference :6097-6147."""
         self.metrics.prefetch_completed_count += len(self.prefetch_events)
         for ev in self.prefetch_events.values():
-            self.backend.wait_event(ev, "compute")  # nothing may read a slot before its copy lands
+            self.backend.wait_event(ev, "compute", True)  # nothing may read a slot before its copy lands
         self.prefetch_events.clear()
         self.prefetched_ids.clear()
         self.prefetch_used_ids.clear()

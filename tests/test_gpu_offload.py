@@ -1,0 +1,181 @@
+"""GPU tests of the offloaded path: HBM expert cache fed from pinned host memory, RS
+prefetch on a side stream, EPIPE readiness-ordered execution.
+
+For every method switch the layer outputs must equal the all-resident block bit for bit
+(residency changes where weights come from and in which order experts run, never the
+values), and the cache event sequence, the prefetch plans and the final LRU order must
+equal the CPU oracle driven with the same routing and the same predictor top-k."""
+import pytest
+import torch
+
+from oracle.ref_layer import RefConfig, RefLayer
+
+pytestmark = pytest.mark.gpu
+
+SHAPE = dict(family="qwen_shared", hidden=512, num_experts=12, inter=256, top_k=4, shared_inter=384, num_layers=3)
+
+
+def _stack(device, method, capacity, top_m, offload, seed0=0, **overrides):
+    from sparse_amd.block import DistributedSparseMoeBlock
+    from sparse_amd.context import DistEnv, Metrics, SparseContext
+    from sparse_amd.methods import method_settings, residency_config
+    from sparse_amd.rs import random_init_bank
+    from sparse_amd.synthetic import make_mlp_block
+    SparseContext.reset()
+    metrics = Metrics()
+    metrics.events = []
+    kw = method_settings(method)["kwargs"]
+    blocks = []
+    for layer in range(SHAPE["num_layers"]):
+        mlp = make_mlp_block(SHAPE, dtype=torch.bfloat16, seed=seed0 + layer)
+        cfg = residency_config(method, capacity, top_m, **overrides) if offload == "cpu" else None
+        blocks.append(DistributedSparseMoeBlock(
+            layer, mlp, None, DistEnv(0, 1, 0, device), num_layers=SHAPE["num_layers"],
+            num_experts=SHAPE["num_experts"], top_k=SHAPE["top_k"], dtype=torch.bfloat16, expert_offload=offload,
+            expert_cache=capacity, planner_mode=kw["planner_mode"] if offload == "cpu" else "none",
+            prefetch_top_m=top_m, placement_mode=kw["placement_mode"], metrics=metrics, residency_config=cfg))
+    if offload == "cpu" and kw["planner_mode"] == "rs_prefetch":
+        SparseContext.set_rs_bank(random_init_bank(SHAPE["num_layers"], SHAPE["hidden"], SHAPE["num_experts"],
+                                                   hidden_dim=64, seed=5, device=device))
+    return blocks, metrics
+
+
+def _run(blocks, device, steps, T, record=None, sync_prefetch=False, prefill_first=False):
+    from sparse_amd.block import _SideStreams
+    from sparse_amd.context import SparseContext
+    from sparse_amd.synthetic import make_hidden
+    outs = []
+    if record is not None:
+        for blk in blocks:
+            res = blk.residency
+            orig = res.execute
+
+            def wrapped(segments, _orig=orig, _l=blk.layer_idx):
+                record.append(("exec", _l, list(segments), SparseContext.current_phase, SparseContext.runtime_call_id))
+                name = _orig(segments)
+                record.append(("executor", _l, name))
+                return name
+            res.execute = wrapped
+
+            def hook(layer_idx, ids, probs, budget, plan):
+                record.append(("rs", layer_idx, list(ids), list(probs), int(budget), [tuple(p) for p in plan]))
+                if sync_prefetch:
+                    _SideStreams.get().prefetch.synchronize()
+            blk._rs_plan_hook = hook
+    for step in range(steps):
+        prefill = prefill_first and step == 0
+        SparseContext.current_phase = "prefill" if prefill else "decode"
+        SparseContext.begin_runtime_call(step)
+        n = 40 if prefill else T
+        x = make_hidden(n, SHAPE["hidden"], torch.bfloat16, seed=1000 + step).to(device)
+        hid = x.view(1, n, -1) if prefill else x.view(n, 1, -1)
+        for blk in blocks:
+            out, _logits = blk(hid)
+            outs.append(out.clone())
+    torch.cuda.synchronize()
+    return outs
+
+
+def _replay_oracle(record, cfg, capacity):
+    names = [n for n in vars(RefConfig()) if hasattr(cfg, n)]
+    rc = {n: getattr(cfg, n) for n in names}
+    lays = [RefLayer(l, SHAPE["num_experts"], SHAPE["top_k"], RefConfig(**rc)) for l in range(SHAPE["num_layers"])]
+    plans, executors = [], []
+    pending_rs = None
+    for item in record:
+        if item[0] == "rs":
+            pending_rs = item
+        elif item[0] == "exec":
+            _, l, segments, phase, call = item
+            # the source layer's RS step for layer l+1 happens inside layer l's forward, before
+            # layer l executes; budget / cycle bookkeeping runs even when no plan is recorded
+            if cfg.planner_mode == "rs_prefetch" and l + 1 < len(lays) and phase == "decode":
+                tgt = lays[l + 1]
+                tgt.phase, tgt.call_id = phase, call
+                budget = tgt.prefetch_budget(("next_layer_rs", phase, call, l, l + 1))
+                if budget > 0:
+                    assert pending_rs is not None and pending_rs[1] == l and pending_rs[4] == budget
+                    plan = tgt.schedule_prefetch(pending_rs[2], pending_rs[3], budget)
+                    assert [tuple(p) for p in plan] == pending_rs[5], "prefetch plan differs"
+                    plans.append(plan)
+                else:
+                    assert pending_rs is None
+            pending_rs = None
+            lay = lays[l]
+            lay.phase, lay.call_id, lay.stage = phase, call, phase
+            executors.append(lay.execute(segments))
+    return lays, plans, executors
+
+
+@pytest.mark.parametrize("method,overrides,prefill_first", [
+    ("rr", {}, False), ("rs", {}, False), ("epipe", {}, False), ("rs-epipe", {}, False), ("sparse", {}, False),
+    ("rs", dict(formal_thresholds=False), False),
+    ("epipe", dict(epipe_prefill_enable=True), True),
+])
+def test_offloaded_methods_match_resident_values_and_oracle_events(device, method, overrides, prefill_first):
+    from sparse_amd.methods import residency_config
+    capacity, top_m, steps, T = 4, 3, 16, 4
+    ref_blocks, _ = _stack(device, "rr", capacity, top_m, "gpu")
+    want = _run(ref_blocks, device, steps, T, prefill_first=prefill_first)
+    blocks, metrics = _stack(device, method, capacity, top_m, "cpu", **overrides)
+    record = []
+    got = _run(blocks, device, steps, T, record=record, sync_prefetch=True, prefill_first=prefill_first)
+    assert len(got) == len(want)
+    for i, (a, b) in enumerate(zip(got, want)):
+        assert torch.equal(a, b), f"output {i} differs from the all-resident block"
+
+    cfg = residency_config(method, capacity, top_m, **overrides)
+    lays, plans, executors = _replay_oracle(record, cfg, capacity)
+    assert executors == [r[2] for r in record if r[0] == "executor"]
+    for l, lay in enumerate(lays):
+        want_events = [t for t in lay.trace if t[0] in ("hit", "prefetch_hit", "miss")]
+        got_events = [(k, e) for k, ll, e in metrics.events if ll == l]
+        assert got_events == want_events, f"layer {l}: cache events differ from the oracle"
+        assert blocks[l].residency.cache.resident_ids() == lay.cache.resident_ids()
+    misses = sum(1 for k, _l, _e in metrics.events if k == "miss")
+    assert metrics.cache_miss_count == misses and misses > 0
+    assert metrics.demand_h2d_bytes == misses * blocks[0].arena.expert_bytes
+    if cfg.planner_mode == "rs_prefetch":
+        assert metrics.prefetch_admitted_count > 0 and metrics.prefetch_h2d_bytes > 0
+        assert any(k == "prefetch_hit" for k, _l, _e in metrics.events) or method == "rs"
+    if method in ("epipe", "rs-epipe", "sparse"):
+        assert any(n.startswith("epipe") for n in executors)
+
+
+def test_values_do_not_depend_on_copy_timing(device):
+    """Without forcing prefetch completion the late / ready classification may vary from run
+    to run; outputs still equal the resident block."""
+    capacity, top_m, steps, T = 4, 3, 12, 4
+    ref_blocks, _ = _stack(device, "rr", capacity, top_m, "gpu")
+    want = _run(ref_blocks, device, steps, T)
+    for method in ("rs", "rs-epipe"):
+        blocks, metrics = _stack(device, method, capacity, top_m, "cpu")
+        got = _run(blocks, device, steps, T)
+        for a, b in zip(got, want):
+            assert torch.equal(a, b)
+        total = metrics.cache_hit_count + metrics.prefetch_hit_count + metrics.cache_miss_count
+        assert total == len(metrics.events) > 0
+
+
+def test_zero_and_tiny_capacity_and_request_reset(device):
+    from sparse_amd.block import DistributedSparseMoeBlock
+    steps, T = 6, 4
+    ref_blocks, _ = _stack(device, "rr", 4, 2, "gpu")
+    want = _run(ref_blocks, device, steps, T)
+    for capacity in (0, 1):
+        blocks, metrics = _stack(device, "rr", capacity, 2, "cpu")
+        got = _run(blocks, device, steps, T)
+        for a, b in zip(got, want):
+            assert torch.equal(a, b)
+        if capacity == 0:
+            assert metrics.cache_hit_count == 0 and metrics.cache_miss_count == len(metrics.events)
+    blocks, metrics = _stack(device, "rs", 4, 2, "cpu")
+    _run(blocks, device, steps, T)
+    for blk in blocks:
+        blk.reset_runtime_state_for_new_request(clear_expert_cache=True)
+        assert blk.residency.cache.resident_ids() == [] and not blk.residency.prefetch_events
+        assert len(blk.residency._free_slots) == blk.residency.num_slots
+    DistributedSparseMoeBlock.clear_all_expert_caches()
+    got = _run(blocks, device, steps, T)
+    for a, b in zip(got, want):
+        assert torch.equal(a, b)

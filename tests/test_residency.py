@@ -1,0 +1,406 @@
+"""Residency state machine: oracle (``oracle/ref_layer.py``) against the reference's known
+answers and golden planner vectors, and the product (``sparse_amd/residency.py``) against
+the oracle on long random traces for every method switch.  Runs on the CPU: the product's
+device services are replaced by a recording backend that also checks slot safety."""
+import json
+import random
+from pathlib import Path
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import ref_rs
+from oracle.ref_layer import RefConfig, RefLayer
+from sparse_amd.context import Metrics
+from sparse_amd.methods import METHODS, method_settings, residency_config
+from sparse_amd.residency import Backend, LayerResidency, ResidencyConfig
+
+GOLDEN = Path(__file__).resolve().parent / "golden"
+
+
+# ----------------------------------------------------------------------------- fake device
+class FakeEvent:
+    def __init__(self, kind, eid=None):
+        self.kind, self.eid = kind, eid
+
+
+class RecordingBackend(Backend):
+    """Records device effects and asserts the physical invariants of the slot pool."""
+
+    def __init__(self, copy_done=None):
+        self.trace = []
+        self.slot_content = {}
+        self.copy_done = copy_done or (lambda eid: True)
+
+    def upload(self, eid, slot, lane):
+        self.trace.append(("h2d", lane, eid))
+        self.slot_content[slot] = eid
+        return FakeEvent("copy", eid)
+
+    def event_done(self, event):
+        return True if event.kind == "fence" else bool(self.copy_done(event.eid))
+
+    def wait_event(self, event, lane, ordering=False):
+        if ordering:
+            self.trace.append(("order_wait", lane, event.eid))
+        elif event.kind == "copy":
+            self.trace.append(("wait" if lane == "compute" else "wait_%s_lane" % lane, event.eid))
+
+    def run_segments(self, segments):
+        seen = set()
+        for eid, slot in segments:
+            assert self.slot_content.get(slot) == eid, f"slot {slot} holds {self.slot_content.get(slot)}, not {eid}"
+            assert slot not in seen, "two segments of one batch share a slot"
+            seen.add(slot)
+            self.trace.append(("compute", eid))
+
+    def fence(self):
+        return FakeEvent("fence")
+
+
+def product_layer(cfg: ResidencyConfig, E=16, K=2, copy_done=None, layer=0):
+    m = Metrics()
+    m.events = []
+    be = RecordingBackend(copy_done)
+    return LayerResidency(layer, E, K, cfg, be, m, expert_bytes=100), be, m
+
+
+def to_ref_config(cfg: ResidencyConfig) -> RefConfig:
+    names = [n for n in vars(RefConfig()) if hasattr(cfg, n)]
+    return RefConfig(**{n: getattr(cfg, n) for n in names})
+
+
+def split(trace):
+    events = [t for t in trace if t[0] in ("hit", "prefetch_hit", "miss")]
+    h2d = [t for t in trace if t[0] == "h2d"]
+    compute = [t[1] for t in trace if t[0] == "compute"]
+    waits = [t for t in trace if t[0] == "wait"]
+    return events, h2d, compute, waits
+
+
+# ----------------------------------------------------------------------------- scoring known answers
+def test_select_candidates_known_answers_of_the_reference():
+    # reference tests/test_rs_staging.py:147-150
+    assert ref_rs.select_candidates([0, 8, 8, 9, 12], [.9, .1, .1, 1., .15], allowed={0, 8, 12}, resident={0},
+                                    minimum=.2, budget=2) == [8]
+    # reference tests/test_rs_staging.py:308-312
+    diag = {}
+    assert ref_rs.select_candidates([0, 1, 8], [.9, .9, .01], allowed={0, 8}, resident={0}, minimum=.2, budget=2,
+                                    diagnostics=diag) == []
+    assert diag == dict(nonlocal_entries=1, resident_entries=1, scored=1, below_threshold=1)
+
+
+@pytest.mark.parametrize("impl", [RefLayer.score_map, LayerResidency.score_map])
+def test_score_map_formula(impl):
+    ids, w = [0, 8, 8, 9, 12], [.9, .1, .1, 1., .15]
+    s = impl(ids, w)
+    assert list(s) == [0, 8, 9, 12]                      # first-seen order
+    assert s[8] == pytest.approx((.1 + .1) * 1.15 + .05 * .1)
+    assert s[12] == pytest.approx(.15 + .05 * .15)
+    assert s[9] == pytest.approx(1.05)
+    # agrees with the staging adapter's selection on the same data
+    chosen = [e for e in sorted(s, key=s.get, reverse=True) if e in {8, 12} and s[e] >= .2][:2]
+    assert chosen == ref_rs.select_candidates(ids, w, allowed={0, 8, 12}, resident={0}, minimum=.2, budget=2)
+    # brute force on random data
+    rng = random.Random(3)
+    for _ in range(50):
+        n = rng.randrange(1, 40)
+        ids = [rng.randrange(10) for _ in range(n)]
+        w = [rng.random() for _ in range(n)]
+        s = impl(ids, w)
+        for e in set(ids):
+            ws = [x for i, x in zip(ids, w) if i == e]
+            assert s[e] == pytest.approx(sum(ws) * (1 + .15 * (len(ws) - 1)) + .05 * max(ws), rel=1e-12)
+
+
+# ----------------------------------------------------------------------------- golden planner vectors
+def _load_plan_cases():
+    return json.loads((GOLDEN / "rs_plan.json").read_text())
+
+
+def _setup_case(case, which):
+    kw = dict(capacity=case["capacity"], planner_mode="rs_prefetch", prefetch_top_m=8, rs_policy=case["policy"],
+              min_candidate_score=case["thresholds"][0], replace_advantage=case["thresholds"][1],
+              replace_margin=case["thresholds"][2])
+    if which == "oracle":
+        lay = RefLayer(1, case["E"], 4, RefConfig(**kw))
+        cache, freq, pre = lay.cache, lay.freq, lay.prefetched
+    else:
+        lay, _be, _m = product_layer(ResidencyConfig(**kw), E=case["E"], K=4, layer=1)
+        cache, freq, pre = lay.cache, lay.access_freq, lay.prefetched_ids
+    for e in case["residents"]:
+        cache.put(e, ("w", e) if which == "oracle" else 0, pinned=e in case["pinned"])
+    freq.update({int(k): int(v) for k, v in case["freq"]})
+    pre.update(case["prefetched"])
+    return lay
+
+
+@pytest.mark.parametrize("which", ["oracle", "product"])
+def test_planner_matches_golden_vectors_of_the_reference(which):
+    cases = _load_plan_cases()
+    assert len(cases) >= 100
+    nontrivial = 0
+    for case in cases:
+        lay = _setup_case(case, which)
+        score = lay.score_map(case["topi"], case["topv"])
+        assert [[k, v] for k, v in score.items()] == case["score"]       # same floats, same order
+        protect = set(case["protect"])
+        if which == "oracle":
+            assert lay.pick_victims_by_low_value(score, protect) == case["victims"]
+        plan = lay.build_plan(score, protect, case["budget"])
+        assert [[e, v] for e, v in plan] == case["plan"]
+        nontrivial += any(v is not None for _e, v in plan)
+        # invariants
+        assert len(plan) <= case["budget"]
+        assert all(not lay.cache.has(e) for e, _ in plan)
+        assert all(v is None or (v not in protect and v in case["residents"] and v not in case["pinned"])
+                   for _, v in plan)
+    assert nontrivial > 20
+
+
+# ----------------------------------------------------------------------------- predictor
+def test_routing_scout_forward_closed_form():
+    from sparse_amd.rs import RoutingScoutMLP
+    torch.manual_seed(0)
+    m = RoutingScoutMLP(32, 10, hidden_dim=16).eval()
+    bn = m.mlp[1]
+    bn.running_mean.uniform_(-1, 1)
+    bn.running_var.uniform_(0.5, 2.0)
+    x = torch.randn(5, 32)
+    with torch.no_grad():
+        want = m(x).numpy()
+    got = ref_rs.routing_scout_forward(
+        x.numpy(), m.mlp[0].weight.detach().numpy(), m.mlp[0].bias.detach().numpy(), bn.weight.detach().numpy(),
+        bn.bias.detach().numpy(), bn.running_mean.numpy(), bn.running_var.numpy(), m.mlp[4].weight.detach().numpy(),
+        m.mlp[4].bias.detach().numpy())
+    np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(got.sum(-1), 1.0, rtol=1e-5)
+    assert sorted(m.state_dict()) == sorted(
+        ["mlp.0.weight", "mlp.0.bias", "mlp.1.weight", "mlp.1.bias", "mlp.1.running_mean", "mlp.1.running_var",
+         "mlp.1.num_batches_tracked", "mlp.4.weight", "mlp.4.bias"])
+
+
+# ----------------------------------------------------------------------------- demand path
+def test_inflight_prefetch_hit_waits_once_and_does_not_reload():
+    """Restates reference tests/test_rs_staging.py:74-92 for both implementations."""
+    for which in ("oracle", "product"):
+        cfg = dict(capacity=4, planner_mode="rs_prefetch", prefetch_top_m=2)
+        if which == "oracle":
+            lay = RefLayer(0, 16, 2, RefConfig(**cfg), copy_done=lambda e: False)
+            trace = lay.trace
+        else:
+            lay, be, m = product_layer(ResidencyConfig(**cfg), copy_done=lambda e: False)
+        lay.phase, lay.call_id, lay.stage = "decode", 0, "decode"
+        assert lay.prefetch_budget(("k", 0)) == 2
+        lay.schedule_prefetch([8], [0.9], 2)
+        lay.execute([(8, 1)])
+        if which == "product":
+            trace = [(k, e) for k, _l, e in m.events] + be.trace
+        events, h2d, compute, waits = split(trace)
+        assert events == [("prefetch_hit", 8)]
+        assert h2d == [("h2d", "prefetch", 8)]        # no second load
+        assert waits == [("wait", 8)]                 # exactly one stream wait, never a host sync
+        assert compute == [8]
+        assert lay.cache.resident_ids() == [8]
+
+
+# ----------------------------------------------------------------------------- random traces, all methods
+class RoutingModel:
+    """Seeded routing with skewed popularity and an optional noisy predictor."""
+
+    def __init__(self, E, K, T, seed):
+        self.E, self.K, self.T = E, K, T
+        self.rng = random.Random(seed)
+        self.weights = [1.0 / (r + 1) ** 1.1 for r in range(E)]
+        self.rng.shuffle(self.weights)
+
+    def route(self):
+        counts = {}
+        for _ in range(self.T):
+            picked = set()
+            while len(picked) < self.K:
+                picked.add(self.rng.choices(range(self.E), self.weights)[0])
+            for e in picked:
+                counts[e] = counts.get(e, 0) + 1
+        return sorted(counts.items())
+
+    def predict(self, next_segments, pred_k):
+        ids, probs = [], []
+        truth = [e for e, _ in next_segments]
+        for _ in range(self.T):
+            row = set()
+            while len(row) < pred_k:
+                if truth and self.rng.random() < 0.6:
+                    row.add(self.rng.choice(truth))
+                else:
+                    row.add(self.rng.randrange(self.E))
+            p = sorted((self.rng.random() for _ in row), reverse=True)
+            s = sum(p)
+            for e, v in zip(row, p):
+                ids.append(e)
+                probs.append(float(torch.tensor(v / s).to(torch.bfloat16)))
+        return ids, probs
+
+
+def run_trace(method, which, *, steps=60, layers=3, E=16, K=2, T=4, capacity=4, top_m=3, seed=0, late_rate=0.0,
+              prefill_first=False, overrides=None, formal=True):
+    cfg = residency_config(method, capacity, top_m, formal_thresholds=formal, **(overrides or {}))
+    late_rng = random.Random(seed + 99)
+    late = {}
+
+    def copy_done(layer):
+        def fn(eid):
+            key = (layer, eid)
+            if key not in late:
+                late[key] = late_rng.random() >= late_rate
+            done = late[key]
+            late[key] = True          # a second query finds the copy finished
+            return done
+        return fn
+
+    lays, backs, mets = [], [], []
+    for l in range(layers):
+        if which == "oracle":
+            lays.append(RefLayer(l, E, K, to_ref_config(cfg), copy_done=copy_done(l)))
+        else:
+            lay, be, m = product_layer(cfg, E=E, K=K, copy_done=copy_done(l), layer=l)
+            lays.append(lay)
+            backs.append(be)
+            mets.append(m)
+    model = RoutingModel(E, K, T, seed)
+    executors = []
+    for step in range(steps):
+        phase = "prefill" if (prefill_first and step == 0) else "decode"
+        routes = [model.route() for _ in range(layers)]
+        preds = [model.predict(routes[l + 1], lays[l + 1].predict_topk()) if l + 1 < layers else None
+                 for l in range(layers)]
+        for l in range(layers):
+            if cfg.planner_mode == "rs_prefetch" and l + 1 < layers and phase == "decode":
+                tgt = lays[l + 1]
+                tgt.phase, tgt.call_id = phase, step
+                budget = tgt.prefetch_budget(("next_layer_rs", phase, step, l, l + 1))
+                if budget > 0:
+                    tgt.schedule_prefetch(preds[l][0], preds[l][1], budget)
+            lay = lays[l]
+            lay.phase, lay.call_id, lay.stage = phase, step, phase
+            executors.append(lay.execute(routes[l]))
+    out = []
+    for l in range(layers):
+        if which == "oracle":
+            trace = lays[l].trace
+            events, h2d, compute, waits = split(trace)
+            plans = [list(t[1]) for t in trace if t[0] == "plan"]
+        else:
+            events = [(k, e) for k, _l, e in mets[l].events]
+            _ev, h2d, compute, waits = split(backs[l].trace)
+            plans = None
+        out.append(dict(events=events, h2d=h2d, compute=compute, waits=waits, residents=lays[l].cache.resident_ids(),
+                        plans=plans))
+    return out, executors
+
+
+METHOD_CASES = [
+    ("rr", {}), ("rs", {}), ("epipe", {}), ("rs-epipe", {}), ("sparse", {}),
+    ("rs-epipe", dict(late_rate=0.5)), ("rs", dict(formal=False)), ("rs-epipe", dict(formal=False, late_rate=0.3)),
+    ("epipe", dict(prefill_first=True, overrides=dict(epipe_prefill_enable=True))),
+    ("rr", dict(capacity=1)), ("rr", dict(capacity=0)), ("epipe", dict(capacity=2, T=8)),
+    ("rs", dict(capacity=15, E=60, K=4, T=8, top_m=8)), ("rs-epipe", dict(capacity=15, E=60, K=4, T=8, top_m=8)),
+    ("epipe", dict(overrides=dict(epipe_sort_ready_by_work=True))),
+    ("epipe", dict(prefill_first=True, overrides=dict(epipe_prefill_enable=True, epipe_prefill_extra_cache_slots=2,
+                                                      epipe_prefill_commit=False))),
+]
+
+
+@pytest.mark.parametrize("method,kw", METHOD_CASES)
+def test_product_reproduces_the_oracle_event_for_event(method, kw):
+    for seed in range(3):
+        want, ex_o = run_trace(method, "oracle", seed=seed, **kw)
+        got, ex_p = run_trace(method, "product", seed=seed, **kw)
+        assert ex_o == ex_p
+        for l, (w, g) in enumerate(zip(want, got)):
+            assert g["events"] == w["events"], f"layer {l}: cache events differ"
+            assert g["h2d"] == w["h2d"], f"layer {l}: H2D sequence differs"
+            assert g["compute"] == w["compute"], f"layer {l}: execution order differs"
+            assert g["waits"] == w["waits"], f"layer {l}: stream waits differ"
+            assert g["residents"] == w["residents"], f"layer {l}: final LRU order differs"
+    if method in ("epipe", "rs-epipe", "sparse"):
+        assert any(e.startswith("epipe") for e in ex_o), "EPIPE never triggered in this trace"
+
+
+def test_invariants_of_every_method():
+    for method in METHODS:
+        if method.startswith("executor") or method.startswith("scp"):
+            continue
+        res, _ex = run_trace(method, "oracle", seed=11, steps=40)
+        rr, _ = run_trace("rr", "oracle", seed=11, steps=40)
+        for l, r in enumerate(res):
+            # every routed segment is computed exactly once, whatever the order
+            assert sorted(r["compute"]) == sorted(rr[l]["compute"])
+            n_miss = sum(1 for k, _ in r["events"] if k == "miss")
+            n_demand_h2d = sum(1 for _, lane, _e in r["h2d"] if lane in ("compute", "epipe"))
+            assert n_miss == n_demand_h2d                    # one copy per miss, staged experts included
+            assert len(r["events"]) == len(r["compute"])     # one cache event per executed segment
+    # rr is textbook LRU
+    from collections import OrderedDict
+    model = OrderedDict()
+    lay = RefLayer(0, 16, 2, RefConfig(capacity=4))
+    m = RoutingModel(16, 2, 4, 5)
+    for step in range(50):
+        segs = m.route()
+        lay.phase, lay.call_id, lay.stage = "decode", step, "decode"
+        before = len(lay.trace)
+        lay.execute(segs)
+        ev = [t for t in lay.trace[before:] if t[0] in ("hit", "miss")]
+        for (kind, eid), (e, _n) in zip(ev, segs):
+            assert eid == e and kind == ("hit" if e in model else "miss")
+            if e in model:
+                model.move_to_end(e)
+            else:
+                model[e] = 1
+                if len(model) > 4:
+                    model.popitem(last=False)
+        assert lay.cache.resident_ids() == list(model)
+
+
+def test_method_table_matches_the_reference_launcher():
+    # scripts/run/run_case.sh:85-138
+    assert METHODS["rr"] == ("none", False, "off", "unique_mask", "round_robin")
+    assert METHODS["rs"] == ("rs_prefetch", False, "off", "unique_mask", "round_robin")
+    assert METHODS["epipe"] == ("none", True, "off", "sorted_segment", "round_robin")
+    assert METHODS["rs-epipe"] == ("rs_prefetch", True, "residual_scan", "sorted_segment", "round_robin")
+    assert METHODS["sparse"] == ("rs_prefetch", True, "residual_scan", "sorted_segment", "scp_ep")
+    s = method_settings("sparse")
+    assert s["kwargs"]["planner_mode"] == "rs_prefetch" and s["kwargs"]["expert_offload"] == "cpu"
+    assert s["env"]["SPARSE_EPIPE_RS_FORCE_DEMAND_STAGE"] == "1" and s["env"]["SPARSE_EPIPE_PREFILL_ENABLE"] == "0"
+    assert method_settings("rr")["env"]["SPARSE_PREFETCH_ALLOW_ACTIVE_REPLACE"] == "0"
+    with pytest.raises(ValueError):
+        method_settings("nope")
+    cfg = residency_config("rs-epipe", 8, 2)
+    assert (cfg.min_candidate_score, cfg.replace_advantage, cfg.replace_margin) == (0.04, 0.08, 1.20)
+    assert cfg.recent_protect_steps == 1 and cfg.epipe_decode_rs_mode == "residual_scan"
+
+
+def test_rolling_gate_skips_after_a_quiet_window():
+    for which in ("oracle", "product"):
+        cfg = residency_config("rs-epipe", 4, 2)
+        if which == "oracle":
+            lay = RefLayer(0, 16, 2, to_ref_config(cfg))
+        else:
+            lay, _be, _m = product_layer(cfg)
+        for e in (1, 2, 3):
+            lay.cache.put(e, ("w", e) if which == "oracle" else e)
+            if which == "product":
+                lay._slot_of[e] = e
+                lay.backend.slot_content[e] = e
+                lay._free_slots.remove(e)
+        names = []
+        for step in range(30):
+            lay.phase, lay.call_id, lay.stage = "decode", step, "decode"
+            names.append(lay.execute([(1, 1), (2, 1)]))     # everything resident: never a residual
+        assert set(names) == {"plain"}
+        skip = lay.gate_skip if which == "oracle" else lay._gate_skip_remaining
+        calls = lay.gate_calls if which == "oracle" else lay._gate_calls
+        # the 16th call fills the window and is the first of 8 skipped calls (steps 15..22);
+        # the remaining 7 calls (steps 23..29) are counted again
+        assert (skip, calls) == (0, 7)
