@@ -213,6 +213,7 @@ def main():
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--no-extra", action="store_true", help="skip batch 1/32 decode and the prefill workload")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--only-prefill", action="store_true", help="run just the prefill workload (for profiling)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -226,6 +227,9 @@ def main():
     device = torch.device("cuda:0")
     dtype = torch.bfloat16
 
+    if args.only_prefill:
+        print(json.dumps(prefill_workload(DEEPSEEK, 4096, max(2, args.steps), args.warmup, dtype, device)))
+        return
     blocks = build_stack(QWEN, dtype, device)
     main_res = decode_workload(blocks, QWEN, 8, args.steps, args.warmup, dtype, device, not args.no_graph)
     extra = {}

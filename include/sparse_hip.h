@@ -174,8 +174,11 @@ int sparse_hip_route_decode(const void* x_dev, const void* wg_dev, const void* w
  * streamed once.  `_prefill` is the MFMA grouped-GEMM path for any T (bf16), and the
  * tiled FMA path for fp32.  Both produce the same rows up to fp32 summation order.
  * x [T,H]; topv [T,K] in dtype; inter_ws [T*K, I] and parts [T*K, H] in dtype.
- * H % 64 == 0 and I % 64 == 0.
+ * H % 64 == 0 and I % 64 == 0.  `_prefill` also takes `tile_ws_dev`, a workspace of
+ * sparse_hip_prefill_ws_bytes(T, K, segs->n, H, I) bytes in which a one-workgroup kernel
+ * lays out which tile every workgroup owns (segment lengths are only known on the device).
  */
+size_t sparse_hip_prefill_ws_bytes(int T, int K, int num_segments, int H, int I);
 int sparse_hip_grouped_swiglu_decode(const sparse_hip_experts* experts, const void* x_dev,
                                      const void* topv_dev, const int32_t* perm_dev,
                                      const int32_t* seg_offsets_dev,
@@ -185,7 +188,8 @@ int sparse_hip_grouped_swiglu_prefill(const sparse_hip_experts* experts, const v
                                       const void* topv_dev, const int32_t* perm_dev,
                                       const int32_t* seg_offsets_dev,
                                       const sparse_hip_seglist* segs, int T, int K,
-                                      void* inter_ws_dev, void* parts_dev, void* stream);
+                                      void* inter_ws_dev, void* parts_dev, void* tile_ws_dev,
+                                      void* stream);
 
 /* ---- A8: shared expert ----------------------------------------------------- */
 

@@ -13,7 +13,8 @@ int decode_fused_bf16(const sparse_hip_experts*, const void*, const void*, const
                       const sparse_hip_seglist*, int, int, void*, void*, const void*, const void*, const void*,
                       const void*, int, void*, void*, hipStream_t);
 int prefill_routed_bf16(const sparse_hip_experts*, const void*, const void*, const int32_t*, const int32_t*,
-                        const sparse_hip_seglist*, int, int, void*, void*, hipStream_t);
+                        const sparse_hip_seglist*, int, int, void*, void*, void*, hipStream_t);
+size_t prefill_ws_bytes(int, int, int, int, int);
 int prefill_shared_bf16(const void*, const void*, const void*, const void*, const void*, int, int, int, void*,
                         void*, hipStream_t);
 template <typename T>
@@ -67,6 +68,11 @@ using namespace sparse;
 
 extern "C" {
 
+size_t sparse_hip_prefill_ws_bytes(int T, int K, int num_segments, int H, int I) {
+  if (T <= 0 || K <= 0 || num_segments < 0 || H <= 0 || I <= 0) return 0;
+  return prefill_ws_bytes(T, K, num_segments, H, I);
+}
+
 int sparse_hip_grouped_swiglu_decode(const sparse_hip_experts* experts, const void* x_dev, const void* topv_dev,
                                      const int32_t* perm_dev, const int32_t* seg_offsets_dev,
                                      const sparse_hip_seglist* segs, int T, int K, void* inter_ws_dev,
@@ -88,15 +94,18 @@ int sparse_hip_grouped_swiglu_decode(const sparse_hip_experts* experts, const vo
 int sparse_hip_grouped_swiglu_prefill(const sparse_hip_experts* experts, const void* x_dev, const void* topv_dev,
                                       const int32_t* perm_dev, const int32_t* seg_offsets_dev,
                                       const sparse_hip_seglist* segs, int T, int K, void* inter_ws_dev,
-                                      void* parts_dev, void* stream) {
+                                      void* parts_dev, void* tile_ws_dev, void* stream) {
   int rc = check_routed("grouped_swiglu_prefill", experts, x_dev, topv_dev, perm_dev, seg_offsets_dev, segs, T,
                         K, inter_ws_dev, parts_dev);
   if (rc != SPARSE_HIP_OK) return rc;
   if (segs->n == 0) return SPARSE_HIP_OK;
   hipStream_t st = as_stream(stream);
-  if (experts->dtype == SPARSE_HIP_BF16)
+  if (experts->dtype == SPARSE_HIP_BF16) {
+    SP_REQUIRE(tile_ws_dev != nullptr && (reinterpret_cast<uintptr_t>(tile_ws_dev) & 15) == 0,
+               "grouped_swiglu_prefill: tile workspace is NULL or not 16-byte aligned");
     return prefill_routed_bf16(experts, x_dev, topv_dev, perm_dev, seg_offsets_dev, segs, T, K, inter_ws_dev,
-                               parts_dev, st);
+                               parts_dev, tile_ws_dev, st);
+  }
   return tiled_routed<float>(experts, x_dev, topv_dev, perm_dev, seg_offsets_dev, segs, T, K, inter_ws_dev,
                              parts_dev, st);
 }

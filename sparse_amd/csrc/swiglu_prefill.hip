@@ -2,17 +2,24 @@
 //
 // C[p, n] = sum_k A[p, k] * W[n, k] per expert segment.  A workgroup (4 waves) owns a
 // 128-row x 256-weight-row tile; wave w owns all 128 rows and 64 of the weight rows
-// (four by two 32x32x16 MFMA tiles, 128 accumulator registers), which keeps LDS reads at
-// 6 fragments per 8 MFMAs.  For the gate/up projection the 256 weight rows are 128 gate
-// rows and the 128 matching up rows, and a wave's two column tiles are the gate and
-// the up tile of the same 32 neurons, so SiLU(gate)*up is a lane-local epilogue.
-// Tiles go HBM -> registers -> LDS in 64-wide k slabs (one LDS buffer, the next slab
-// is prefetched into registers while the current one is multiplied); LDS rows are
-// padded to 144 bytes so 16-byte fragment reads are bank-conflict free.
+// (four by two 32x32x16 MFMA tiles, 128 accumulator registers).  For the gate/up
+// projection the 256 weight rows are 128 gate rows and the 128 matching up rows, and a
+// wave's two column tiles are the gate and the up tile of the same 32 neurons, so
+// SiLU(gate)*up is a lane-local epilogue.
 //
-// Block ids are dealt to the eight XCDs round-robin by the hardware; the kernel
-// re-maps them so that an XCD works through whole experts, m-tiles of one weight tile
-// adjacent in time, which keeps a weight tile in that XCD's L2 while it is reused.
+// The two operands take different roads.  Activation rows are shared by the four waves:
+// they go HBM/L2 -> registers -> LDS in 64-wide k slabs, two LDS buffers, one barrier per
+// slab, rows padded to 144 bytes so 16-byte fragment reads are bank-conflict free.
+// Weight rows are private to a wave: they go HBM/L2 -> registers directly in MFMA
+// B-operand order, which is exactly the order the tiled layout stores them in (a wave
+// load is four 256-byte runs), one slab ahead of the multiply.  LDS thus carries a third
+// of the bytes of a both-operands-through-LDS design, which is what bounds this shape.
+//
+// Which tile a workgroup owns is read from a map built by a one-workgroup kernel before
+// the launch (segment lengths are only known on the device).  Block ids are dealt to the
+// eight XCDs round-robin by the hardware; the map index is re-derived so that an XCD
+// works through whole experts, m-tiles of one weight tile adjacent in time, which keeps a
+// weight tile in that XCD's L2 while it is reused.
 //
 // MFMA 32x32x16 bf16 operand layout (lane l, c = l & 31, g = l >> 5):
 //   A: row c, k = g*8 .. g*8+7     B: column c, k = g*8 .. g*8+7
@@ -27,89 +34,119 @@ constexpr int kPfBK = 64;         // k slab
 constexpr int kPfThreads = 256;
 constexpr int kPfRowBytes = kPfBK * 2 + 16;  // padded LDS row
 constexpr int kPfLdsA = kPfBM * kPfRowBytes;
-constexpr int kPfLdsB = kPfBR * kPfRowBytes;
 constexpr int kPfXcds = 8;
+
+struct PfTile {
+  int32_t slot;  // weight slot of the segment's expert
+  int32_t r0;    // first permuted row of the tile
+  int32_t rows;  // rows in the tile (0: idle workgroup)
+  int32_t bn;    // column tile
+};
 
 struct PrefillArgs {
   const uint16_t* slab;
   uint64_t slot_stride;  // elements
   uint64_t mat_offset;   // elements
   uint64_t mat2_offset;  // elements
-  const int32_t* expert_slot;
   const int32_t* perm;
-  const int32_t* seg_offsets;
   const uint16_t* topv;
   const uint16_t* act;
   uint16_t* out;
+  const PfTile* map;   // routed: one entry per workgroup
   int32_t topk;
   int32_t Kdim;
   int32_t Ndim;       // output columns (neurons for gate-up, hidden for down)
   int32_t ntiles_n;
-  int32_t max_mtiles;
   int32_t shared;
   int32_t T;
   const uint16_t* w_s;
   const uint16_t* w2_s;
   const uint16_t* gate_s;
+};
+
+struct PfMapArgs {
+  const int32_t* expert_slot;
+  const int32_t* seg_offsets;
+  PfTile* map_gu;
+  PfTile* map_dn;
+  int32_t ntiles_gu, ntiles_dn;
+  int32_t cap_gu, cap_dn;  // entries in each map
   sparse_hip_seglist segs;
 };
 
+// One workgroup: segment s -> its m-tile count, exclusive scan, then every (segment,
+// column tile, m-tile) triple in that order; the rest of each map is marked idle.
+__global__ __launch_bounds__(256) void prefill_tile_map_kernel(const PfMapArgs a) {
+  __shared__ int32_t s_scan[SPARSE_HIP_MAX_EXPERTS];
+  __shared__ int32_t s_slot[SPARSE_HIP_MAX_EXPERTS];
+  __shared__ int32_t s_r0[SPARSE_HIP_MAX_EXPERTS];
+  __shared__ int32_t s_rows[SPARSE_HIP_MAX_EXPERTS];
+  const int tid = threadIdx.x;
+  int nseg = a.segs.n;
+  if (a.segs.eids_dev != nullptr) nseg = min(nseg, a.segs.count_dev[0]);
+  int mt = 0;
+  if (tid < nseg) {
+    const int e = (a.segs.eids_dev != nullptr) ? a.segs.eids_dev[tid] : a.segs.eids[tid];
+    const int b = a.seg_offsets[e], m = a.seg_offsets[e + 1] - b;
+    mt = (m + kPfBM - 1) / kPfBM;
+    s_slot[tid] = (a.segs.eids_dev != nullptr) ? a.expert_slot[e] : a.segs.slots[tid];
+    s_r0[tid] = b;
+    s_rows[tid] = m;
+  }
+  s_scan[tid] = mt;
+  __syncthreads();
+  for (int off = 1; off < 256; off <<= 1) {
+    const int v = (tid >= off) ? s_scan[tid - off] : 0;
+    __syncthreads();
+    s_scan[tid] += v;
+    __syncthreads();
+  }
+  const int total_mt = s_scan[255];
+#pragma unroll
+  for (int which = 0; which < 2; ++which) {
+    PfTile* map = which == 0 ? a.map_gu : a.map_dn;
+    const int nt = which == 0 ? a.ntiles_gu : a.ntiles_dn;
+    const int cap = which == 0 ? a.cap_gu : a.cap_dn;
+    if (tid < nseg && mt > 0) {
+      const int base = (s_scan[tid] - mt) * nt;
+      for (int bn = 0; bn < nt; ++bn)
+        for (int bm = 0; bm < mt; ++bm) {
+          const int idx = base + bn * mt + bm;
+          if (idx < cap)
+            map[idx] = PfTile{s_slot[tid], s_r0[tid] + bm * kPfBM, min(kPfBM, s_rows[tid] - bm * kPfBM), bn};
+        }
+    }
+    for (int idx = total_mt * nt + tid; idx < cap; idx += 256) map[idx] = PfTile{0, 0, 0, 0};
+  }
+}
+
 template <bool kGateUp>
 __global__ __launch_bounds__(kPfThreads, 2) void prefill_ffn_kernel(const PrefillArgs a) {
-  __shared__ __attribute__((aligned(16))) uint8_t lds[kPfLdsA + kPfLdsB];
+  __shared__ __attribute__((aligned(16))) uint8_t lds[2][kPfLdsA];
   __shared__ float s_scale[kPfBM];
-  __shared__ int32_t s_seg[5];  // eid, first row, rows, n-tile, slot
 
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63;
   const int fc = lane & 31, fg = lane >> 5;
 
-  // ---- XCD-aware tile lookup -------------------------------------------------
-  if (tid == 0) {
-    const int nblk = gridDim.x;
-    const int per_xcd = (nblk + kPfXcds - 1) / kPfXcds;
-    const int logical = (blockIdx.x % kPfXcds) * per_xcd + blockIdx.x / kPfXcds;
-    int eid = -1, r0 = 0, M = 0, bn = 0, slot_id = 0;
-    if (a.shared) {
-      // n-tile major, m fastest
-      const int mt = (a.T + kPfBM - 1) / kPfBM;
-      if (logical < mt * a.ntiles_n) {
-        bn = logical / mt;
-        const int bm = logical - bn * mt;
-        eid = 0;
-        r0 = bm * kPfBM;
-        M = min(kPfBM, a.T - r0);
-      }
-    } else {
-      int nseg = a.segs.n;
-      if (a.segs.eids_dev != nullptr) nseg = min(nseg, a.segs.count_dev[0]);
-      int left = logical;
-      for (int s = 0; s < nseg; ++s) {
-        const int e = (a.segs.eids_dev != nullptr) ? a.segs.eids_dev[s] : a.segs.eids[s];
-        const int b = a.seg_offsets[e], m = a.seg_offsets[e + 1] - b;
-        const int mt = (m + kPfBM - 1) / kPfBM;
-        const int nt = mt * a.ntiles_n;
-        if (left < nt) {
-          bn = left / mt;
-          const int bm = left - bn * mt;
-          eid = e;
-          slot_id = (a.segs.eids_dev != nullptr) ? a.expert_slot[e] : a.segs.slots[s];
-          r0 = b + bm * kPfBM;
-          M = min(kPfBM, m - bm * kPfBM);
-          break;
-        }
-        left -= nt;
-      }
-    }
-    s_seg[0] = eid;
-    s_seg[1] = r0;
-    s_seg[2] = M;
-    s_seg[3] = bn;
-    s_seg[4] = slot_id;
+  // ---- which tile (XCD-aware order) ----------------------------------------------
+  const int per_xcd = gridDim.x / kPfXcds;
+  const int logical = (blockIdx.x % kPfXcds) * per_xcd + blockIdx.x / kPfXcds;
+  int slot_id = 0, r0, M, bn;
+  if (a.shared) {
+    const int mt = (a.T + kPfBM - 1) / kPfBM;
+    if (logical >= mt * a.ntiles_n) return;
+    bn = logical / mt;
+    r0 = (logical - bn * mt) * kPfBM;
+    M = min(kPfBM, a.T - r0);
+  } else {
+    const PfTile tile = a.map[logical];
+    if (tile.rows <= 0) return;
+    slot_id = tile.slot;
+    r0 = tile.r0;
+    M = tile.rows;
+    bn = tile.bn;
   }
-  __syncthreads();
-  const int eid = s_seg[0], r0 = s_seg[1], M = s_seg[2], bn = s_seg[3];
-  if (eid < 0) return;
 
   const int Kdim = a.Kdim, Ndim = a.Ndim;
   const uint16_t *w0, *w1 = nullptr;
@@ -117,12 +154,11 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_ffn_kernel(const Prefil
     w0 = a.w_s;
     w1 = a.w2_s;
   } else {
-    const uint16_t* slot = a.slab + static_cast<uint64_t>(s_seg[4]) * a.slot_stride;
+    const uint16_t* slot = a.slab + static_cast<uint64_t>(slot_id) * a.slot_stride;
     w0 = slot + a.mat_offset;
     w1 = slot + a.mat2_offset;
   }
-  // first output column of this tile
-  const int n0 = bn * (kGateUp ? kPfBR / 2 : kPfBR);
+  const int n0 = bn * (kGateUp ? kPfBR / 2 : kPfBR);  // first output column of this tile
 
   // per-row epilogue scale (down projection only)
   if (!kGateUp && tid < kPfBM) {
@@ -138,44 +174,31 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_ffn_kernel(const Prefil
     s_scale[tid] = sc;
   }
 
-  // ---- loader mapping: 32 rows x 8 sixteen-byte chunks per pass ---------------
+  // ---- activation loader: 32 rows x 8 sixteen-byte chunks per pass, 4 passes --------
   const int lrow = tid >> 3, lchunk = tid & 7;
   const uint16_t* aptr[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int m = min(lrow + 32 * i, M - 1);
     const int p = r0 + m;
-    size_t row;
-    if (a.shared || !kGateUp) {
-      row = static_cast<size_t>(p);
-    } else {
-      row = static_cast<size_t>(a.perm[p] / a.topk);
-    }
+    const size_t row = (a.shared || !kGateUp) ? static_cast<size_t>(p) : static_cast<size_t>(a.perm[p] / a.topk);
     aptr[i] = a.act + row * Kdim + lchunk * 8;
   }
-  // Weight rows are tiled (16-row groups, 2 KB blocks of 64 k in MFMA lane order): a pass
-  // of the workgroup copies two whole blocks, 128 sixteen-byte units each, so global reads
-  // are 2 KB runs; unit u = h*64 + q*16 + r is row r, k = q*16 + h*8 .. +7 of its block.
-  const int bu = tid & 127, bgrp = tid >> 7;
-  const int br = bu & 15, bq = (bu >> 4) & 3, bh = bu >> 6;
-  const uint16_t* bptr[8];
-#pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const int g = 2 * i + bgrp;  // 16-row group inside the 256-row weight tile
-    const uint16_t* base;
-    int n;
-    if (kGateUp) {
-      base = (g < 8) ? w0 : w1;
-      n = n0 + (g & 7) * 16;
-    } else {
-      base = w0;
-      n = n0 + g * 16;
-    }
-    n = min(n, Ndim - 16);
-    bptr[i] = base + static_cast<size_t>(n >> 4) * 16 * Kdim + bu * 8;
-  }
-  const int lds_wr_b = (bgrp * 16 + br) * kPfRowBytes + (bq * 2 + bh) * 16;
   const int lds_wr = lrow * kPfRowBytes + lchunk * 16;
+
+  // ---- weight fragments straight from the tiled layout ------------------------------
+  // lane = (kh, gsel, r16): row r16 of 16-row group gsel of the wave's 32 rows, k half kh.
+  // In a 2 KB block of 64 k, the 16 bytes of (k step s, half kh, row r16) sit at element
+  // kh*512 + (s*16 + r16)*8, so k inside step s is s*16 + kh*8 + j: the MFMA's own order.
+  const int r16 = lane & 15, gsel = (lane >> 4) & 1, kh = lane >> 5;
+  const uint16_t* bptr[2];
+#pragma unroll
+  for (int ni = 0; ni < 2; ++ni) {
+    const uint16_t* base = (kGateUp && ni == 1) ? w1 : w0;
+    int n = kGateUp ? (n0 + wave * 32) : (n0 + wave * 64 + ni * 32);
+    n = min(n + gsel * 16, Ndim - 16);
+    bptr[ni] = base + static_cast<size_t>(n >> 4) * 16 * Kdim + kh * 512 + r16 * 8;
+  }
 
   f32x16 acc[4][2];
 #pragma unroll
@@ -185,52 +208,54 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_ffn_kernel(const Prefil
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[mi][ni][v] = 0.f;
 
-  u32x4 ra[4], rb[8];
+  u32x4 ra[4];
+  bf16x8 bcur[2][4], bnxt[2][4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) ra[i] = *reinterpret_cast<const u32x4*>(aptr[i]);
 #pragma unroll
-  for (int i = 0; i < 8; ++i) rb[i] = *reinterpret_cast<const u32x4*>(bptr[i]);
-
-  // fragment read offsets
-  const int a_rd = fc * kPfRowBytes + fg * 16;
-  int b_rd[2];
+  for (int ni = 0; ni < 2; ++ni)
 #pragma unroll
-  for (int ni = 0; ni < 2; ++ni) {
-    const int row = kGateUp ? (ni * (kPfBR / 2) + wave * 32 + fc) : (wave * 64 + ni * 32 + fc);
-    b_rd[ni] = kPfLdsA + row * kPfRowBytes + fg * 16;
-  }
+    for (int s = 0; s < 4; ++s) bcur[ni][s] = *reinterpret_cast<const bf16x8*>(bptr[ni] + s * 128);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(&lds[0][lds_wr + i * 32 * kPfRowBytes]) = ra[i];
+  __syncthreads();
 
+  const int a_rd = fc * kPfRowBytes + fg * 16;
   const int nk = Kdim / kPfBK;
   for (int kt = 0; kt < nk; ++kt) {
-    __syncthreads();  // previous slab fully consumed
+    const bool more = kt + 1 < nk;
+    if (more) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-      *reinterpret_cast<u32x4*>(lds + lds_wr + i * 32 * kPfRowBytes) = ra[i];
+      for (int i = 0; i < 4; ++i) ra[i] = *reinterpret_cast<const u32x4*>(aptr[i] + (kt + 1) * kPfBK);
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
-      *reinterpret_cast<u32x4*>(lds + kPfLdsA + lds_wr_b + i * 32 * kPfRowBytes) = rb[i];
-    __syncthreads();
-    if (kt + 1 < nk) {
-      const int ko = (kt + 1) * kPfBK;
+      for (int ni = 0; ni < 2; ++ni)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) ra[i] = *reinterpret_cast<const u32x4*>(aptr[i] + ko);
-#pragma unroll
-      for (int i = 0; i < 8; ++i) rb[i] = *reinterpret_cast<const u32x4*>(bptr[i] + (kt + 1) * 1024);
+        for (int s = 0; s < 4; ++s)
+          bnxt[ni][s] = *reinterpret_cast<const bf16x8*>(bptr[ni] + static_cast<size_t>(kt + 1) * 1024 + s * 128);
     }
+    const uint8_t* la = lds[kt & 1];
 #pragma unroll
-    for (int ks = 0; ks < kPfBK / 16; ++ks) {
-      bf16x8 fa[4], fb[2];
+    for (int s = 0; s < 4; ++s) {
+      bf16x8 fa[4];
 #pragma unroll
       for (int mi = 0; mi < 4; ++mi)
-        fa[mi] = *reinterpret_cast<const bf16x8*>(lds + a_rd + mi * 32 * kPfRowBytes + ks * 32);
-#pragma unroll
-      for (int ni = 0; ni < 2; ++ni) fb[ni] = *reinterpret_cast<const bf16x8*>(lds + b_rd[ni] + ks * 32);
+        fa[mi] = *reinterpret_cast<const bf16x8*>(la + a_rd + mi * 32 * kPfRowBytes + s * 32);
 #pragma unroll
       for (int mi = 0; mi < 4; ++mi)
 #pragma unroll
         for (int ni = 0; ni < 2; ++ni)
-          acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[mi], fb[ni], acc[mi][ni], 0, 0, 0);
+          acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[mi], bcur[ni][s], acc[mi][ni], 0, 0, 0);
     }
+    if (more) {
+      uint8_t* lw = lds[(kt + 1) & 1];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(lw + lds_wr + i * 32 * kPfRowBytes) = ra[i];
+#pragma unroll
+      for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+        for (int s = 0; s < 4; ++s) bcur[ni][s] = bnxt[ni][s];
+    }
+    __syncthreads();
   }
 
   // ---- epilogue ----------------------------------------------------------------
@@ -264,10 +289,8 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_ffn_kernel(const Prefil
 }
 
 template <bool kGateUp>
-static int launch_prefill(PrefillArgs& a, hipStream_t st) {
-  const int cols_per_tile = kGateUp ? kPfBR / 2 : kPfBR;
-  a.ntiles_n = (a.Ndim + cols_per_tile - 1) / cols_per_tile;
-  int64_t grid = static_cast<int64_t>(a.ntiles_n) * a.max_mtiles;
+static int launch_prefill(PrefillArgs& a, int max_mtiles, hipStream_t st) {
+  int64_t grid = static_cast<int64_t>(a.ntiles_n) * max_mtiles;
   grid = (grid + kPfXcds - 1) / kPfXcds * kPfXcds;
   if (grid == 0) return SPARSE_HIP_OK;
   SP_REQUIRE(grid < (1ll << 31), "prefill_ffn: grid too large");
@@ -278,36 +301,67 @@ static int launch_prefill(PrefillArgs& a, hipStream_t st) {
   return SPARSE_HIP_OK;
 }
 
+static inline int pf_max_mtiles(int Ttok, int K, int nseg) { return (Ttok * K + kPfBM - 1) / kPfBM + nseg; }
+static inline int64_t pf_round8(int64_t v) { return (v + kPfXcds - 1) / kPfXcds * kPfXcds; }
+
+size_t prefill_ws_bytes(int Ttok, int K, int nseg, int H, int I) {
+  const int64_t mt = pf_max_mtiles(Ttok, K, nseg);
+  const int64_t gu = pf_round8(mt * ((I + kPfBR / 2 - 1) / (kPfBR / 2)));
+  const int64_t dn = pf_round8(mt * ((H + kPfBR - 1) / kPfBR));
+  return static_cast<size_t>(gu + dn) * sizeof(PfTile);
+}
+
 int prefill_routed_bf16(const sparse_hip_experts* ex, const void* x, const void* topv, const int32_t* perm,
                         const int32_t* seg_offsets, const sparse_hip_seglist* segs, int Ttok, int K,
-                        void* inter_ws, void* parts, hipStream_t st) {
+                        void* inter_ws, void* parts, void* tile_ws, hipStream_t st) {
   const uint64_t H = ex->hidden, I = ex->inter;
+  const int mt = pf_max_mtiles(Ttok, K, segs->n);
+  const int nt_gu = static_cast<int>((I + kPfBR / 2 - 1) / (kPfBR / 2));
+  const int nt_dn = static_cast<int>((H + kPfBR - 1) / kPfBR);
+  const int cap_gu = static_cast<int>(pf_round8(static_cast<int64_t>(mt) * nt_gu));
+  const int cap_dn = static_cast<int>(pf_round8(static_cast<int64_t>(mt) * nt_dn));
+  PfTile* map_gu = static_cast<PfTile*>(tile_ws);
+  PfTile* map_dn = map_gu + cap_gu;
+  {
+    PfMapArgs m = {};
+    m.expert_slot = ex->expert_slot_dev;
+    m.seg_offsets = seg_offsets;
+    m.map_gu = map_gu;
+    m.map_dn = map_dn;
+    m.ntiles_gu = nt_gu;
+    m.ntiles_dn = nt_dn;
+    m.cap_gu = cap_gu;
+    m.cap_dn = cap_dn;
+    m.segs = *segs;
+    hipLaunchKernelGGL(prefill_tile_map_kernel, dim3(1), dim3(256), 0, st, m);
+    SP_LAUNCH_CHECK("prefill_tile_map_kernel");
+  }
   PrefillArgs a = {};
   a.slab = static_cast<const uint16_t*>(ex->slab_dev);
   a.slot_stride = ex->slot_stride / 2;
-  a.expert_slot = ex->expert_slot_dev;
   a.perm = perm;
-  a.seg_offsets = seg_offsets;
   a.topk = K;
   a.T = Ttok;
-  a.segs = *segs;
-  a.max_mtiles = (Ttok * K + kPfBM - 1) / kPfBM + segs->n;
   a.mat_offset = 0;
   a.mat2_offset = I * H;
   a.act = static_cast<const uint16_t*>(x);
   a.out = static_cast<uint16_t*>(inter_ws);
+  a.map = map_gu;
   a.Kdim = static_cast<int32_t>(H);
   a.Ndim = static_cast<int32_t>(I);
-  int rc = launch_prefill<true>(a, st);
+  a.ntiles_n = nt_gu;
+  int rc = launch_prefill<true>(a, mt, st);
   if (rc != SPARSE_HIP_OK) return rc;
   a.mat_offset = 2 * I * H;
   a.mat2_offset = 0;
   a.topv = static_cast<const uint16_t*>(topv);
   a.act = static_cast<const uint16_t*>(inter_ws);
   a.out = static_cast<uint16_t*>(parts);
+  a.map = map_dn;
   a.Kdim = static_cast<int32_t>(I);
   a.Ndim = static_cast<int32_t>(H);
-  return launch_prefill<false>(a, st);
+  a.ntiles_n = nt_dn;
+  return launch_prefill<false>(a, mt, st);
 }
 
 int prefill_shared_bf16(const void* x, const void* gate_w, const void* up_w, const void* down_w,
@@ -317,14 +371,15 @@ int prefill_shared_bf16(const void* x, const void* gate_w, const void* up_w, con
   a.shared = 1;
   a.T = Ttok;
   a.topk = 1;
-  a.max_mtiles = (Ttok + kPfBM - 1) / kPfBM;
+  const int mt = (Ttok + kPfBM - 1) / kPfBM;
   a.w_s = static_cast<const uint16_t*>(gate_w);
   a.w2_s = static_cast<const uint16_t*>(up_w);
   a.act = static_cast<const uint16_t*>(x);
   a.out = static_cast<uint16_t*>(inter_ws);
   a.Kdim = H;
   a.Ndim = Is;
-  int rc = launch_prefill<true>(a, st);
+  a.ntiles_n = (Is + kPfBR / 2 - 1) / (kPfBR / 2);
+  int rc = launch_prefill<true>(a, mt, st);
   if (rc != SPARSE_HIP_OK) return rc;
   a.w_s = static_cast<const uint16_t*>(down_w);
   a.w2_s = nullptr;
@@ -333,7 +388,8 @@ int prefill_shared_bf16(const void* x, const void* gate_w, const void* up_w, con
   a.out = static_cast<uint16_t*>(shared_out);
   a.Kdim = Is;
   a.Ndim = H;
-  return launch_prefill<false>(a, st);
+  a.ntiles_n = (H + kPfBR - 1) / kPfBR;
+  return launch_prefill<false>(a, mt, st);
 }
 
 }  // namespace sparse

@@ -180,7 +180,8 @@ def seglist_host(eids: Sequence[int], slots: Optional[Sequence[int]] = None) -> 
 
 
 def grouped_swiglu(experts: Experts, x: torch.Tensor, topv: torch.Tensor, perm: Permutation, segs: SegList,
-                   inter_ws: torch.Tensor, parts: torch.Tensor, *, decode: Optional[bool] = None) -> None:
+                   inter_ws: torch.Tensor, parts: torch.Tensor, *, decode: Optional[bool] = None,
+                   tile_ws: Optional[torch.Tensor] = None) -> None:
     """Routed-expert FFN over the segments in ``segs``; rows land in ``parts`` (permuted order)."""
     lib = _lib.load()
     T, H = x.shape
@@ -192,10 +193,33 @@ def grouped_swiglu(experts: Experts, x: torch.Tensor, topv: torch.Tensor, perm: 
     if H != experts.hidden:
         raise ValueError(f"x has hidden {H}, the expert slab has {experts.hidden}")
     use_decode = (T <= DECODE_MAX_TOKENS) if decode is None else bool(decode)
-    fn = lib.sparse_hip_grouped_swiglu_decode if use_decode else lib.sparse_hip_grouped_swiglu_prefill
-    rc = fn(C.byref(experts), _ptr(x), _ptr(topv), _ptr(perm.perm), _ptr(perm.seg_offsets), C.byref(segs), T, K,
-            _ptr(inter_ws), _ptr(parts), _stream())
-    _lib.check(rc, "sparse_hip_grouped_swiglu_" + ("decode" if use_decode else "prefill"))
+    if use_decode:
+        rc = lib.sparse_hip_grouped_swiglu_decode(C.byref(experts), _ptr(x), _ptr(topv), _ptr(perm.perm),
+                                                  _ptr(perm.seg_offsets), C.byref(segs), T, K, _ptr(inter_ws),
+                                                  _ptr(parts), _stream())
+        _lib.check(rc, "sparse_hip_grouped_swiglu_decode")
+        return
+    if tile_ws is None:
+        tile_ws = prefill_tile_ws(T, K, experts.num_experts, H, experts.inter, x.device)
+    rc = lib.sparse_hip_grouped_swiglu_prefill(C.byref(experts), _ptr(x), _ptr(topv), _ptr(perm.perm),
+                                               _ptr(perm.seg_offsets), C.byref(segs), T, K, _ptr(inter_ws),
+                                               _ptr(parts), _ptr(tile_ws), _stream())
+    _lib.check(rc, "sparse_hip_grouped_swiglu_prefill")
+
+
+_TILE_WS = {}
+
+
+def prefill_tile_ws(T: int, K: int, num_segments: int, hidden: int, inter: int, device) -> torch.Tensor:
+    """Tile-map workspace of the prefill kernels, cached per shape (launches on one stream
+    reuse it in order)."""
+    key = (T, K, num_segments, hidden, inter, str(device))
+    ws = _TILE_WS.get(key)
+    if ws is None:
+        nbytes = _lib.load().sparse_hip_prefill_ws_bytes(T, K, num_segments, hidden, inter)
+        ws = torch.empty((max(16, nbytes),), device=device, dtype=torch.uint8)
+        _TILE_WS[key] = ws
+    return ws
 
 
 def shared_expert(x: torch.Tensor, gate_w: torch.Tensor, up_w: torch.Tensor, down_w: torch.Tensor,
