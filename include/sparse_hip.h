@@ -146,11 +146,14 @@ int sparse_hip_permute_build(const int64_t* topi_dev, int T, int K, int E, int32
 /*
  * Decode fast path: sparse_hip_router_logits + sparse_hip_gate_topk +
  * sparse_hip_permute_build in ONE launch for T <= SPARSE_HIP_DECODE_MAX_TOKENS (topv is
- * written in `dtype`).  Each workgroup computes one column of the logits; the workgroup
- * that finishes last (counted in `counter_dev` behind a device-scope fence) does the
- * top-k and the permutation.  `counter_dev` is one int32 that must be zero before the
- * first call; every call leaves it zero.  Same outputs, bit for bit, as the three
- * separate calls (utils/eval_core.py:9519-9595, :14728-14730, :13240-13262).
+ * written in `dtype`).  Each workgroup computes one token's logits and its top-k; the
+ * workgroup that finishes last (counted in `counter_dev` behind a device-scope fence)
+ * builds the permutation.  `counter_dev` is one int32 that must be zero before the
+ * first call; every call leaves it zero.  The logits may differ from
+ * sparse_hip_router_logits' in the last fp32 bit before rounding (another summation
+ * order); top-k and permutation are, bit for bit, what sparse_hip_gate_topk and
+ * sparse_hip_permute_build return for the logits written here
+ * (utils/eval_core.py:9519-9595, :14728-14730, :13240-13262).
  */
 int sparse_hip_route_decode(const void* x_dev, const void* wg_dev, const void* wsg_dev, int dtype,
                             int logits_dtype, int T, int H, int E, int K, int renorm, void* logits_dev,

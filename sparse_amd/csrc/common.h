@@ -93,15 +93,47 @@ __device__ __forceinline__ float silu_f32(float v) { return v / (1.0f + expf(-v)
 __device__ __forceinline__ float sigmoid_f32(float v) { return 1.0f / (1.0f + expf(-v)); }
 
 // ---- wavefront (64 lanes) reductions ---------------------------------------
+// Data-parallel-primitive moves instead of LDS permutes: four shifts inside each row of
+// 16 lanes leave the row total in its lane 15, two row broadcasts carry the totals up to
+// lane 63, and a read of lane 63 hands the result to every lane.  All 64 lanes must be
+// active.  A lane whose source falls outside its row, or whose row is masked off, gets
+// `identity`.
+template <int kCtrl, int kRowMask>
+__device__ __forceinline__ float dpp_move(float identity, float v) {
+  return __int_as_float(
+      __builtin_amdgcn_update_dpp(__float_as_int(identity), __float_as_int(v), kCtrl, kRowMask, 0xf, false));
+}
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
-  return v;
+  v += dpp_move<0x111, 0xf>(0.f, v);  // row_shr:1
+  v += dpp_move<0x112, 0xf>(0.f, v);  // row_shr:2
+  v += dpp_move<0x114, 0xf>(0.f, v);  // row_shr:4
+  v += dpp_move<0x118, 0xf>(0.f, v);  // row_shr:8
+  v += dpp_move<0x142, 0xa>(0.f, v);  // row_bcast:15 into rows 1 and 3
+  v += dpp_move<0x143, 0xc>(0.f, v);  // row_bcast:31 into rows 2 and 3
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
+}
+template <int kCtrl, int kRowMask>
+__device__ __forceinline__ int dpp_move_int(int identity, int v) {
+  return __builtin_amdgcn_update_dpp(identity, v, kCtrl, kRowMask, 0xf, false);
+}
+__device__ __forceinline__ int wave_min_int(int v) {
+  constexpr int kMax = 0x7fffffff;
+  v = min(v, dpp_move_int<0x111, 0xf>(kMax, v));
+  v = min(v, dpp_move_int<0x112, 0xf>(kMax, v));
+  v = min(v, dpp_move_int<0x114, 0xf>(kMax, v));
+  v = min(v, dpp_move_int<0x118, 0xf>(kMax, v));
+  v = min(v, dpp_move_int<0x142, 0xa>(kMax, v));
+  v = min(v, dpp_move_int<0x143, 0xc>(kMax, v));
+  return __builtin_amdgcn_readlane(v, 63);
 }
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
-  return v;
+  v = fmaxf(v, dpp_move<0x111, 0xf>(-INFINITY, v));
+  v = fmaxf(v, dpp_move<0x112, 0xf>(-INFINITY, v));
+  v = fmaxf(v, dpp_move<0x114, 0xf>(-INFINITY, v));
+  v = fmaxf(v, dpp_move<0x118, 0xf>(-INFINITY, v));
+  v = fmaxf(v, dpp_move<0x142, 0xa>(-INFINITY, v));
+  v = fmaxf(v, dpp_move<0x143, 0xc>(-INFINITY, v));
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
 }
 
 }  // namespace sparse

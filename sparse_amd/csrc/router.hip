@@ -13,22 +13,37 @@ namespace sparse {
 constexpr int kRouterThreads = 256;
 constexpr int kRouterTokTile = 32;
 
+// Eight consecutive elements as they sit in memory, and their widening to fp32.
 template <typename T>
-__device__ __forceinline__ void load8(const T* p, float (&v)[8]);
+struct Raw8;
 template <>
-__device__ __forceinline__ void load8<float>(const float* p, float (&v)[8]) {
-  const float4 a = *reinterpret_cast<const float4*>(p);
-  const float4 b = *reinterpret_cast<const float4*>(p + 4);
-  v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
-  v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
-}
+struct Raw8<float> {
+  float4 a, b;
+  __device__ __forceinline__ void load(const float* p) {
+    a = *reinterpret_cast<const float4*>(p);
+    b = *reinterpret_cast<const float4*>(p + 4);
+  }
+  __device__ __forceinline__ void widen(float (&v)[8]) const {
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+    v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+  }
+};
 template <>
-__device__ __forceinline__ void load8<uint16_t>(const uint16_t* p, float (&v)[8]) {
-  const u32x4 a = *reinterpret_cast<const u32x4*>(p);
-  v[0] = __uint_as_float(a.x << 16); v[1] = __uint_as_float(a.x & 0xffff0000u);
-  v[2] = __uint_as_float(a.y << 16); v[3] = __uint_as_float(a.y & 0xffff0000u);
-  v[4] = __uint_as_float(a.z << 16); v[5] = __uint_as_float(a.z & 0xffff0000u);
-  v[6] = __uint_as_float(a.w << 16); v[7] = __uint_as_float(a.w & 0xffff0000u);
+struct Raw8<uint16_t> {
+  u32x4 a;
+  __device__ __forceinline__ void load(const uint16_t* p) { a = *reinterpret_cast<const u32x4*>(p); }
+  __device__ __forceinline__ void widen(float (&v)[8]) const {
+    v[0] = __uint_as_float(a.x << 16); v[1] = __uint_as_float(a.x & 0xffff0000u);
+    v[2] = __uint_as_float(a.y << 16); v[3] = __uint_as_float(a.y & 0xffff0000u);
+    v[4] = __uint_as_float(a.z << 16); v[5] = __uint_as_float(a.z & 0xffff0000u);
+    v[6] = __uint_as_float(a.w << 16); v[7] = __uint_as_float(a.w & 0xffff0000u);
+  }
+};
+template <typename T>
+__device__ __forceinline__ void load8(const T* p, float (&v)[8]) {
+  Raw8<T> r;
+  r.load(p);
+  r.widen(v);
 }
 
 // Dot products of one weight row with up to 32 token rows; the workgroup's result for
@@ -89,8 +104,9 @@ __global__ __launch_bounds__(kRouterThreads) void router_logits_kernel(
 
 // ---------------------------------------------------------------------------
 // Fused softmax(fp32) + top-k of one token by one wavefront; lane l holds experts
-// l, l+64, l+128, l+192.  Selection runs K rounds of a wave-wide arg-max whose
-// order is (probability descending, expert id ascending).
+// l, l+64, l+128, l+192.  Selection runs K rounds of a wave-wide arg-max whose order is
+// (probability descending, expert id ascending): the largest probability first, then
+// the lowest id among the lanes that hold it.  All cross-lane steps are DPP reductions.
 // ---------------------------------------------------------------------------
 constexpr int kTopkWaves = 4;
 constexpr int kTopkNV = SPARSE_HIP_MAX_EXPERTS / 64;
@@ -103,8 +119,11 @@ __device__ __forceinline__ void topk_token(const TL* __restrict__ row, int E, in
 #pragma unroll
   for (int j = 0; j < kTopkNV; ++j) {
     const int e = lane + 64 * j;
-    p[j] = (e < E) ? Elem<TL>::load(row + e) : -INFINITY;
-    m = fmaxf(m, p[j]);
+    p[j] = -INFINITY;
+    if (64 * j < E) {  // uniform: whole groups of 64 experts that do not exist cost nothing
+      p[j] = (e < E) ? Elem<TL>::load(row + e) : -INFINITY;
+      m = fmaxf(m, p[j]);
+    }
   }
   m = wave_max(m);
   float s = 0.f;
@@ -129,32 +148,24 @@ __device__ __forceinline__ void topk_token(const TL* __restrict__ row, int E, in
     int bi = 0x7fffffff;
 #pragma unroll
     for (int j = 0; j < kTopkNV; ++j) {
-      const int e = lane + 64 * j;
-      if (p[j] > bv) {  // ascending j == ascending id, so strict > keeps the lower id
+      if (64 * j < E && p[j] > bv) {  // ascending j == ascending id, so strict > keeps the lower id
         bv = p[j];
-        bi = e;
+        bi = lane + 64 * j;
       }
     }
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
-      const float ov = __shfl_xor(bv, off, 64);
-      const int oi = __shfl_xor(bi, off, 64);
-      if (ov > bv || (ov == bv && oi < bi)) {
-        bv = ov;
-        bi = oi;
-      }
-    }
+    const float wv = wave_max(bv);
+    const int wi = wave_min_int(bv == wv ? bi : 0x7fffffff);
     // every lane now holds the winner; its owner retires it
-    if ((bi & 63) == lane) {
+    if ((wi & 63) == lane) {
 #pragma unroll
       for (int j = 0; j < kTopkNV; ++j)
-        if ((bi >> 6) == j) p[j] = -1.f;
+        if ((wi >> 6) == j) p[j] = -1.f;
     }
     if (lane == r) {
-      sel_v = bv;
-      sel_i = bi;
+      sel_v = wv;
+      sel_i = wi;
     }
-    sum_sel += bv;
+    sum_sel += wv;
   }
   if (lane < K) {
     float v = sel_v;
@@ -175,10 +186,13 @@ __global__ __launch_bounds__(kTopkWaves * 64) void gate_topk_kernel(
 }
 
 // ---------------------------------------------------------------------------
-// Decode router in one launch (T <= 32).  Workgroup e computes logits[:, e] (workgroup E
-// the shared gate); the workgroup that finishes last -- counted with a device atomic
-// behind a fence -- runs softmax/top-k for every token and the single-block
-// permutation, then puts the counter back to zero for the next launch.
+// Decode router in one launch (T <= 32).  Workgroup t owns token t: its 16 wavefronts
+// compute the token's E logits (and the shared gate), four weight rows per wavefront at
+// a time with the activation chunk shared between them, the values meet in LDS and
+// wavefront 0 runs softmax/top-k on them -- so no workgroup waits for another up to
+// here.  The workgroup that finishes last (a device atomic behind a fence) builds the
+// permutation of all T*K items from one 32-bit token mask per expert and puts the
+// counter back to zero for the next launch.
 // ---------------------------------------------------------------------------
 struct RouteArgs {
   const void* x;
@@ -197,44 +211,154 @@ struct RouteArgs {
   int32_t T, H, E, K, renorm;
 };
 
-template <typename T, typename TL>
-__global__ __launch_bounds__(kRouterThreads) void route_decode_kernel(const RouteArgs a) {
-  const int row = blockIdx.x;
-  const T* x = static_cast<const T*>(a.x);
-  const T* w = (row < a.E) ? static_cast<const T*>(a.wg) + static_cast<size_t>(row) * a.H
-                           : static_cast<const T*>(a.wsg);
-  TL* logits = static_cast<TL*>(a.logits);
-  T* shared_gate = static_cast<T*>(a.shared_gate);
-  const int E = a.E;
-  router_row_dots<T>(x, w, 0, a.T, a.H, [&](int t, float s) {
-    if (row < E) {
-      Elem<TL>::store(logits + static_cast<size_t>(t) * E + row, s);
-    } else {
-      Elem<T>::store(shared_gate + t, s);
-    }
-  });
+constexpr int kRouteThreads = 1024;
+constexpr int kRouteWaves = kRouteThreads / 64;
+constexpr int kRouteRowsPerWave = 4;
 
-  __shared__ int s_last;
-  __threadfence();  // this block's logits are visible device-wide before it is counted
+// Stable bucketing of T*K items (T <= 32) by expert id, run by one 1024-thread block.
+// A token picks an expert at most once, so bit t of mask[e] says "token t chose e" and
+// the rank of item (t, k) inside its segment is the popcount of the bits below t.
+__device__ __forceinline__ void permute_small_block(const int64_t* __restrict__ topi, int T, int K, int E,
+                                                    int32_t* __restrict__ perm, int32_t* __restrict__ inv_perm,
+                                                    int32_t* __restrict__ seg_offsets,
+                                                    int32_t* __restrict__ active_eids,
+                                                    int32_t* __restrict__ n_active) {
+  __shared__ __attribute__((aligned(16))) uint32_t mask[SPARSE_HIP_MAX_EXPERTS];
+  __shared__ int32_t base[SPARSE_HIP_MAX_EXPERTS];
+  const int tid = threadIdx.x;
+  if (tid < SPARSE_HIP_MAX_EXPERTS) mask[tid] = 0u;
   __syncthreads();
-  if (threadIdx.x == 0) {
-    const int prev = atomicAdd(a.counter, 1);
-    s_last = (prev == static_cast<int>(gridDim.x) - 1);
+  const int n = T * K;
+  int e = -1, t = 0;
+  if (tid < n) {
+    const int64_t ev = topi[tid];
+    t = tid / K;
+    if (ev >= 0 && ev < E) {
+      e = static_cast<int>(ev);
+      atomicOr(&mask[e], 1u << t);
+    }
   }
   __syncthreads();
-  if (!s_last) return;
-  __threadfence();
-  if (threadIdx.x == 0) a.counter[0] = 0;
-
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  for (int t = wave; t < a.T; t += kRouterThreads / 64)
-    topk_token<TL, T>(logits + static_cast<size_t>(t) * E, E, a.K, a.renorm,
-                      static_cast<T*>(a.topv) + static_cast<size_t>(t) * a.K, a.topi + static_cast<size_t>(t) * a.K,
-                      lane);
-  __threadfence_block();
+  if (tid < E) {  // every thread reads the same mask words at a time: LDS broadcasts
+    int32_t off = 0, act = 0;
+    for (int e0 = 0; e0 < E; e0 += 16) {  // words past E are zero
+      uint4 m4[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) m4[q] = *reinterpret_cast<const uint4*>(&mask[e0 + 4 * q]);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const uint32_t w[4] = {m4[q].x, m4[q].y, m4[q].z, m4[q].w};
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          const int32_t cnt = __popc(w[c]);
+          if (e0 + 4 * q + c < tid) {
+            off += cnt;
+            act += cnt > 0;
+          }
+        }
+      }
+    }
+    const int32_t mine = __popc(mask[tid]);
+    base[tid] = off;
+    seg_offsets[tid] = off;
+    if (mine > 0) active_eids[act] = tid;
+    if (tid == E - 1) {
+      seg_offsets[E] = off + mine;
+      n_active[0] = act + (mine > 0);
+    }
+  }
   __syncthreads();
-  permute_scatter_block<true>(a.topi, a.T, a.K, E, nullptr, 0, 1, a.perm, a.inv_perm, a.seg_offsets,
-                              a.active_eids, a.n_active);
+  if (e >= 0) {
+    const int32_t pos = base[e] + __popc(mask[e] & ((1u << t) - 1u));
+    perm[pos] = tid;
+    inv_perm[tid] = pos;
+  }
+}
+
+template <typename T, typename TL>
+__global__ __launch_bounds__(kRouteThreads) void route_decode_kernel(const RouteArgs a) {
+  __shared__ float s_logit[SPARSE_HIP_MAX_EXPERTS];
+  __shared__ int s_last;
+  constexpr int kSweeps = sizeof(T) == 2 ? 4 : 1;  // 16-byte loads in flight per row: 4 (bf16), 2 (fp32)
+  const int t = blockIdx.x;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int E = a.E, H = a.H;
+  const int R = E + (a.wsg != nullptr ? 1 : 0);  // row E is the shared-expert gate vector
+  const T* x = static_cast<const T*>(a.x) + static_cast<size_t>(t) * H;
+  const T* wg = static_cast<const T*>(a.wg);
+  TL* logits = static_cast<TL*>(a.logits) + static_cast<size_t>(t) * E;
+
+  for (int r0 = 0; r0 < R; r0 += kRouteWaves * kRouteRowsPerWave) {
+    const T* wrow[kRouteRowsPerWave];
+    float acc[kRouteRowsPerWave];
+#pragma unroll
+    for (int j = 0; j < kRouteRowsPerWave; ++j) {
+      const int r = r0 + wave + kRouteWaves * j;
+      wrow[j] = (r < E) ? wg + static_cast<size_t>(r) * H
+                        : (r == E && a.wsg != nullptr ? static_cast<const T*>(a.wsg) : wg);
+      acc[j] = 0.f;
+    }
+    for (int hh = 0; hh < H; hh += kSweeps * 512) {
+      Raw8<T> rx[kSweeps], rw[kSweeps][kRouteRowsPerWave];
+      bool ok[kSweeps];
+#pragma unroll
+      for (int sw = 0; sw < kSweeps; ++sw) {
+        const int h = hh + sw * 512 + lane * 8;
+        ok[sw] = h < H;
+        const int hc = ok[sw] ? h : 0;
+        rx[sw].load(x + hc);
+#pragma unroll
+        for (int j = 0; j < kRouteRowsPerWave; ++j) rw[sw][j].load(wrow[j] + hc);
+      }
+      __builtin_amdgcn_sched_barrier(0);  // every load of the span is in flight before the first use
+#pragma unroll
+      for (int sw = 0; sw < kSweeps; ++sw) {
+        float xv[8];
+        rx[sw].widen(xv);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) xv[i] = ok[sw] ? xv[i] : 0.f;
+#pragma unroll
+        for (int j = 0; j < kRouteRowsPerWave; ++j) {
+          float wv[8];
+          rw[sw][j].widen(wv);
+#pragma unroll
+          for (int i = 0; i < 8; ++i) acc[j] = fmaf(xv[i], wv[i], acc[j]);
+        }
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < kRouteRowsPerWave; ++j) {
+      const int r = r0 + wave + kRouteWaves * j;
+      const float s = wave_sum(acc[j]);
+      if (lane == 0) {
+        if (r < E) {
+          Elem<TL>::store(logits + r, s);
+          s_logit[r] = Elem<TL>::round(s);
+        } else if (r == E && a.wsg != nullptr) {
+          Elem<T>::store(static_cast<T*>(a.shared_gate) + t, s);
+        }
+      }
+    }
+  }
+  __syncthreads();
+  if (wave == 0)
+    topk_token<float, T>(s_logit, E, a.K, a.renorm, static_cast<T*>(a.topv) + static_cast<size_t>(t) * a.K,
+                         a.topi + static_cast<size_t>(t) * a.K, lane);
+  if (gridDim.x > 1) {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");  // this token's top-k is visible before it is counted
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      const int prev = atomicAdd(a.counter, 1);
+      s_last = (prev == static_cast<int>(gridDim.x) - 1);
+    }
+    __syncthreads();
+    if (!s_last) return;
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    if (threadIdx.x == 0) a.counter[0] = 0;
+  } else {
+    __syncthreads();
+  }
+  permute_small_block(a.topi, a.T, a.K, E, a.perm, a.inv_perm, a.seg_offsets, a.active_eids, a.n_active);
 }
 
 template <typename T, typename TL>
@@ -262,9 +386,8 @@ static int launch_gate_topk(const void* logits, int Ttok, int E, int K, int reno
 
 template <typename T, typename TL>
 static int launch_route_decode(const RouteArgs& a, hipStream_t st) {
-  const int grid = a.E + (a.wsg != nullptr ? 1 : 0);
   ProfScope prof(SPARSE_HIP_K_ROUTE_DECODE, st);
-  hipLaunchKernelGGL((route_decode_kernel<T, TL>), dim3(grid), dim3(kRouterThreads), 0, st, a);
+  hipLaunchKernelGGL((route_decode_kernel<T, TL>), dim3(a.T), dim3(kRouteThreads), 0, st, a);
   SP_LAUNCH_CHECK("route_decode_kernel");
   return SPARSE_HIP_OK;
 }

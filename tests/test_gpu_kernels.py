@@ -122,8 +122,10 @@ def test_router_logits(device, dtype, T):
                                        (torch.float32, torch.float32)])
 @pytest.mark.parametrize("T", [1, 8, 32])
 def test_route_decode_equals_the_three_separate_calls(device, dtype, ldt, T):
-    """The single-launch decode router must reproduce router_logits + gate_topk +
-    permute_build bit for bit, call after call (its counter goes back to zero)."""
+    """The single-launch decode router: its logits agree with router_logits up to the
+    summation order, and its top-k and permutation are bit for bit what gate_topk and
+    permute_build return for the logits it wrote, call after call (its counter goes back
+    to zero)."""
     ops = _ops()
     E, K, H = 60, 4, 2048
     layer = make_layer(H, E, 64, K, Is=64, shared_gate=True, dtype=dtype, seed=7)
@@ -132,22 +134,58 @@ def test_route_decode_equals_the_three_separate_calls(device, dtype, ldt, T):
     for rep in range(3):
         x = make_hidden(T, H, dtype, seed=100 + rep).to(device)
         logits_a, sg_a = ops.router_logits(x, wg, wsg, logits_dtype=ldt)
-        topv_a, topi_a = ops.gate_topk(logits_a, K, out_dtype=dtype)
-        perm_a = ops.permute_build(topi_a, E)
         logits_b = torch.empty_like(logits_a)
         sg_b = torch.empty_like(sg_a)
-        topv_b, topi_b = torch.empty_like(topv_a), torch.empty_like(topi_a)
+        topv_b = torch.empty(T, K, dtype=dtype, device=device)
+        topi_b = torch.empty(T, K, dtype=torch.int64, device=device)
         perm_b = ops.Permutation(T, K, E, device)
         ops.route_decode(x, wg, wsg, K, False, logits_b, sg_b, topv_b, topi_b, perm_b, counter)
         torch.cuda.synchronize()
         assert int(counter.item()) == 0
-        assert torch.equal(logits_a, logits_b) and torch.equal(sg_a, sg_b)
+        # one bf16 ulp where the rounding boundary falls between two summation orders
+        tol = dict(rtol=8e-3, atol=1e-6) if ldt == torch.bfloat16 else dict(rtol=1e-5, atol=1e-6)
+        torch.testing.assert_close(logits_b.float(), logits_a.float(), **tol)
+        tol = dict(rtol=8e-3, atol=1e-6) if dtype == torch.bfloat16 else dict(rtol=1e-5, atol=1e-6)
+        torch.testing.assert_close(sg_b.float(), sg_a.float(), **tol)
+        topv_a, topi_a = ops.gate_topk(logits_b, K, out_dtype=dtype)
+        perm_a = ops.permute_build(topi_a, E)
+        torch.cuda.synchronize()
         assert torch.equal(topv_a, topv_b) and torch.equal(topi_a, topi_b)
         n = int(perm_a.n_active.item())
         assert n == int(perm_b.n_active.item())
         for name in ("perm", "inv_perm", "seg_offsets"):
             assert torch.equal(getattr(perm_a, name), getattr(perm_b, name)), name
         assert torch.equal(perm_a.active_eids[:n], perm_b.active_eids[:n])
+
+
+@pytest.mark.parametrize("T,E,K", [(1, 4, 4), (32, 256, 16), (7, 64, 6), (32, 60, 1)])
+def test_route_decode_shapes_against_oracle(device, T, E, K):
+    """Corner shapes of the decode router (K == E, the largest E and K, K == 1) against the
+    CPU oracle: indices exact wherever the top-k boundary is not a rounding tie."""
+    ops = _ops()
+    H = 512
+    dtype = torch.float32
+    layer = make_layer(H, E, 64, K, Is=64, shared_gate=False, dtype=dtype, seed=11)
+    wg = layer["gate_w"].to(device)
+    x = make_hidden(T, H, dtype, seed=5).to(device)
+    logits = torch.empty(T, E, dtype=dtype, device=device)
+    topv = torch.empty(T, K, dtype=dtype, device=device)
+    topi = torch.empty(T, K, dtype=torch.int64, device=device)
+    perm = ops.Permutation(T, K, E, device)
+    counter = torch.zeros(1, dtype=torch.int32, device=device)
+    ops.route_decode(x, wg, None, K, False, logits, None, topv, topi, perm, counter)
+    torch.cuda.synchronize()
+    ref_v, ref_i, ref_logits = ref_moe.routing_router(x.cpu(), layer["gate_w"], K, False)
+    torch.testing.assert_close(logits.cpu(), ref_logits, rtol=1e-5, atol=1e-5)
+    safe = _boundary_safe(ref_logits, K)
+    assert torch.equal(topi.cpu()[safe], ref_i[safe])
+    torch.testing.assert_close(topv.cpu()[safe], ref_v[safe], rtol=1e-5, atol=1e-6)
+    p_perm, p_inv, p_off, p_active = ref_permute.permute_build(topi.cpu().numpy(), E)
+    assert np.array_equal(perm.perm.cpu().numpy(), p_perm)
+    assert np.array_equal(perm.inv_perm.cpu().numpy(), p_inv)
+    assert np.array_equal(perm.seg_offsets.cpu().numpy(), p_off)
+    n = int(perm.n_active.item())
+    assert n == p_active.size and np.array_equal(perm.active_eids.cpu().numpy()[:n], p_active)
 
 
 # ------------------------------------------------------------------ permute
