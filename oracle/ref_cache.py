@@ -7,7 +7,7 @@ Restates ``ExpertWeightCache`` (utils/eval_core.py:3669-3881) and
 ``EpipePrefillExtraCache`` (:3884-3950) with a plain Python list as the recency order
 (index 0 = least recently used), so that it shares no data structure with the product.
 
-Pinned by (tests/test_oracle_cache.py):
+Pinned by (tests/test_cache.py):
   - the reference's own known-answer cases: access moves an entry to the MRU end and a
     staged-but-unused expert changes nothing (tests/test_rs_staging.py:60-66), eviction
     victim is the oldest entry and ``resident_ids()`` lists oldest first (:152-180), all 64
@@ -17,7 +17,7 @@ Pinned by (tests/test_oracle_cache.py):
   - textbook LRU by brute force (an OrderedDict model) on random traces without pins,
     and the 4-class victim rule on hand-built pinned / protected / transient states;
   - golden traces written by running the reference's own class (extracted from its
-    source, tests/golden/make_cache_golden.py) on random operation sequences.
+    source, tests/golden/make_residency_golden.py) on random operation sequences.
 """
 from __future__ import annotations
 

@@ -17,7 +17,7 @@ are recorded in ``trace`` as tuples:
 Copy completion is not modelled by time: ``copy_done(eid)`` (a callable given by the
 test, default "always complete") answers ``event.query()``.
 
-Pinned by (tests/test_oracle_residency.py and tests/golden/):
+Pinned by (tests/test_residency.py and tests/golden/):
   score map          the reference's known-answer tests of the same formula through
                      ``select_candidates`` (tests/test_rs_staging.py:147-150, :308-312)
                      and golden vectors from the reference's own

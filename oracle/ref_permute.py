@@ -6,7 +6,7 @@ import this.  Restates utils/eval_core.py:14728-14730 (flat index f = t*K + k),
 (``out[order] = out_sorted``).  The reference's ``argsort`` is not ``stable=True``; the
 permutation is therefore defined here by the stable rule, order (expert id, f).
 
-Pinned by (tests/test_oracle_permute.py): a brute-force O(n^2) rank computation on small
+Pinned by (tests/test_oracle_moe.py): a brute-force O(n^2) rank computation on small
 inputs, ``perm`` being a permutation, ``inv_perm[perm[p]] == p``, segment offsets equal to
 the exclusive prefix sum of ``bincount``, sortedness of ``topi.flat[perm]``.
 """
