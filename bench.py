@@ -20,6 +20,7 @@ shared MLP 2816, 26 layers) with its MFMA roofline.
 from __future__ import annotations
 
 import argparse
+import gc
 import json
 import os
 import sys
@@ -176,6 +177,167 @@ def prefill_workload(shape, tokens, steps, warmup, dtype, device):
     return out
 
 
+def build_offload_stack(shape, dtype, device, method, capacity, top_m, rs_kind="random", offload="cpu",
+                        **overrides):
+    """A stack whose routing is skewed (Zipf popularity + co-activating clusters of 4) and whose
+    routed experts live in pinned host memory behind an HBM cache of ``capacity`` slots."""
+    from sparse_amd.block import DistributedSparseMoeBlock
+    from sparse_amd.context import DistEnv, Metrics, SparseContext
+    from sparse_amd.methods import method_settings, residency_config
+    from sparse_amd.rs import informed_bank, random_init_bank
+    from sparse_amd.synthetic import add_routing_structure, make_mlp_block
+    SparseContext.reset()
+    metrics = Metrics()
+    metrics.time_copies = True
+    kw = method_settings(method)["kwargs"]
+    env = DistEnv(0, 1, 0, device)
+    blocks, gates, structure = [], [], None
+    for layer in range(shape["num_layers"]):
+        mlp = make_mlp_block(shape, dtype=dtype, seed=layer, device=device, fused=True)
+        structure = add_routing_structure(mlp, shape["num_experts"], seed=layer)
+        gates.append(mlp.gate.weight.detach().clone() if layer > 0 else None)
+        cfg = residency_config(method, capacity, top_m, **overrides) if offload == "cpu" else None
+        blocks.append(DistributedSparseMoeBlock(
+            layer, mlp, None, env, num_layers=shape["num_layers"], num_experts=shape["num_experts"],
+            top_k=shape["top_k"], dtype=dtype, expert_offload=offload, expert_cache=capacity,
+            planner_mode=kw["planner_mode"] if offload == "cpu" else "none", prefetch_top_m=top_m,
+            placement_mode=kw["placement_mode"], metrics=metrics, residency_config=cfg))
+        del mlp
+    if offload == "cpu" and kw["planner_mode"] == "rs_prefetch":
+        if rs_kind == "informed":
+            bank = informed_bank(gates, hidden_dim=512, device=device)
+        else:
+            bank = random_init_bank(shape["num_layers"], shape["hidden"], shape["num_experts"], hidden_dim=512,
+                                    seed=0, device=device)
+        SparseContext.set_rs_bank(bank)
+    return blocks, metrics, structure
+
+
+def release_stack():
+    """Drop a stack the caller has let go of: the layer registry and the block <-> backend
+    cycle keep it alive until a collection, and with it its HBM slab and pinned arena."""
+    from sparse_amd.block import _Workspace
+    from sparse_amd.context import SparseContext
+    SparseContext.reset()
+    _Workspace._cache.clear()
+    gc.collect()
+    torch.cuda.empty_cache()
+
+
+def run_phase_steps(blocks, inputs, phase, first_call=0):
+    """Drive the stack as the reference's decode loop does: phase and call id before every
+    pass over the layers.  Returns the wall time with the device drained on both sides."""
+    from sparse_amd.context import SparseContext
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i, x in enumerate(inputs):
+        SparseContext.current_phase = phase
+        SparseContext.begin_runtime_call(first_call + i)
+        for blk in blocks:
+            blk(x)
+    torch.cuda.synchronize()
+    return time.perf_counter() - t0
+
+
+def offload_report(metrics, blocks, wall, n_steps, tokens_per_step, resident_ms):
+    lanes = dict(metrics.harvest_timings())
+    counts = dict(metrics.timings_n)
+    eb = blocks[0].arena.expert_bytes
+    demand_bytes, pf_bytes = metrics.demand_h2d_bytes, metrics.prefetch_h2d_bytes
+    total_bytes = demand_bytes + pf_bytes
+    n_copies = total_bytes // eb
+    timed_n = sum(counts.values())
+    timed_ms = sum(lanes.values())
+    # only the first 100 000 copies carry an event pair; scale lane times to all copies
+    scale = n_copies / timed_n if timed_n else 0.0
+    accesses = metrics.cache_hit_count + metrics.prefetch_hit_count + metrics.cache_miss_count
+    ms_step = wall / n_steps * 1e3
+    return dict(
+        ms_per_step=ms_step, tokens_per_s=tokens_per_step * n_steps / wall,
+        ratio_to_resident=ms_step / resident_ms if resident_ms else None,
+        hit_rate=metrics.hit_rate(), accesses=accesses, misses=metrics.cache_miss_count,
+        prefetch_hits=metrics.prefetch_hit_count, prefetch_admitted=metrics.prefetch_admitted_count,
+        prefetch_wasted=metrics.prefetch_wasted_count,
+        h2d_gb=total_bytes / 1e9, demand_h2d_gb=demand_bytes / 1e9, prefetch_h2d_gb=pf_bytes / 1e9,
+        copies=int(n_copies), copies_timed=int(timed_n),
+        # copies on the compute lane are the exposed stall (the reference's demand-H2D window)
+        exposed_demand_copy_ms_per_step=lanes.get("compute_h2d_ms", 0.0) * scale / n_steps,
+        side_copy_ms_per_step=(lanes.get("prefetch_h2d_ms", 0.0) + lanes.get("epipe_h2d_ms", 0.0)) * scale / n_steps,
+        stall_ms_per_step=max(0.0, ms_step - resident_ms) if resident_ms else None,
+        # one copy's bytes over its own event-pair time (copies on two lanes share the link)
+        h2d_gbps_per_copy=timed_n * eb / (timed_ms / 1e3) / 1e9 if timed_ms else 0.0,
+        h2d_gbps_over_wall=total_bytes / wall / 1e9,
+        expert_bytes=eb,
+    )
+
+
+def cached_decode_workload(dtype, device, steps, batch=8, capacity=15, top_m=8):
+    """BASELINE configs[3]: Qwen shape, HBM cache of 25 % of each layer's experts, the rest in
+    pinned host memory, skewed co-activating routing, rr vs rs (random-init predictor, as the
+    config says, and a predictor that reproduces the next layer's router)."""
+    from sparse_amd.block import _Workspace
+    from sparse_amd.synthetic import QWEN, make_structured_hidden
+    shape = QWEN
+    n_clusters = shape["num_experts"] // 4
+    out = {"steps": steps, "batch": batch, "capacity": capacity, "experts": shape["num_experts"], "top_m": top_m}
+
+    def inputs_for(structure):
+        return [make_structured_hidden(batch, shape["hidden"], n_clusters, structure["cluster_prob"], dtype,
+                                       seed=5000 + i, device=device).view(batch, 1, -1) for i in range(steps)]
+
+    blocks, _m, structure = build_offload_stack(shape, dtype, device, "rr", capacity, top_m, offload="gpu")
+    inputs = inputs_for(structure)
+    run_phase_steps(blocks, inputs[:8], "decode")
+    wall = run_phase_steps(blocks, inputs, "decode")
+    resident_ms = wall / steps * 1e3
+    out["resident_eager_ms_per_step"] = resident_ms
+    del blocks
+    release_stack()
+    for name, method, rs_kind in (("rr", "rr", "random"), ("rs_random_init", "rs", "random"),
+                                  ("rs_informed", "rs", "informed"), ("rs-epipe_informed", "rs-epipe", "informed")):
+        blocks, metrics, _ = build_offload_stack(shape, dtype, device, method, capacity, top_m, rs_kind=rs_kind)
+        wall = run_phase_steps(blocks, inputs, "decode")   # cold cache, all steps timed
+        out[name] = offload_report(metrics, blocks, wall, steps, batch, resident_ms)
+        del blocks, metrics
+        release_stack()
+    return out
+
+
+def epipe_prefill_workload(dtype, device, tokens=4096, chunk=2048, capacity=19, top_m=8):
+    """BASELINE configs[4]: DeepSeek shape, 4096-token prefill as two 2048-token prefill-phase
+    calls, HBM cache of 30 % of the routed experts, rr vs rs-epipe vs sparse with the EPIPE
+    prefill stage on."""
+    from sparse_amd.block import _Workspace
+    from sparse_amd.synthetic import DEEPSEEK, make_structured_hidden
+    shape = DEEPSEEK
+    n_clusters = shape["num_experts"] // 4
+    n_chunks = tokens // chunk
+    out = {"tokens": tokens, "chunk": chunk, "capacity": capacity, "experts": shape["num_experts"]}
+
+    def inputs_for(structure, seed0):
+        return [make_structured_hidden(chunk, shape["hidden"], n_clusters, structure["cluster_prob"], dtype,
+                                       seed=seed0 + i, device=device).view(1, chunk, -1) for i in range(n_chunks)]
+
+    blocks, _m, structure = build_offload_stack(shape, dtype, device, "rr", capacity, top_m, offload="gpu")
+    warm, inputs = inputs_for(structure, 7000), inputs_for(structure, 7100)
+    run_phase_steps(blocks, warm, "prefill")
+    wall = run_phase_steps(blocks, inputs, "prefill")
+    resident_ms = wall * 1e3
+    out["resident_ms_per_request"] = resident_ms
+    del blocks
+    release_stack()
+    for method in ("rr", "rs-epipe", "sparse"):
+        blocks, metrics, _ = build_offload_stack(shape, dtype, device, method, capacity, top_m, rs_kind="informed",
+                                                 epipe_prefill_enable=True)
+        wall = run_phase_steps(blocks, inputs, "prefill")   # cold cache
+        rep = offload_report(metrics, blocks, wall, 1, tokens, resident_ms)
+        rep["ms_per_request"] = rep.pop("ms_per_step")
+        out[method] = rep
+        del blocks, metrics
+        release_stack()
+    return out
+
+
 def cpu_baseline(shape, batch, dtype, device, budget_s=12.0):
     """The CPU oracle of one layer of the same workload on this box's host cores."""
     from oracle import ref_moe
@@ -214,6 +376,10 @@ def main():
     ap.add_argument("--no-extra", action="store_true", help="skip batch 1/32 decode and the prefill workload")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--only-prefill", action="store_true", help="run just the prefill workload (for profiling)")
+    ap.add_argument("--cached-decode", type=int, default=0, metavar="STEPS",
+                    help="run just the expert-cache decode comparison (rr vs rs) for STEPS decode steps")
+    ap.add_argument("--epipe-prefill", action="store_true",
+                    help="run just the readiness-aware chunked prefill comparison (rr vs rs-epipe vs sparse)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -229,6 +395,12 @@ def main():
 
     if args.only_prefill:
         print(json.dumps(prefill_workload(DEEPSEEK, 4096, max(2, args.steps), args.warmup, dtype, device)))
+        return
+    if args.cached_decode:
+        print(json.dumps({"cached_decode_qwen": cached_decode_workload(dtype, device, args.cached_decode)}))
+        return
+    if args.epipe_prefill:
+        print(json.dumps({"epipe_prefill_deepseek": epipe_prefill_workload(dtype, device)}))
         return
     blocks = build_stack(QWEN, dtype, device)
     main_res = decode_workload(blocks, QWEN, 8, args.steps, args.warmup, dtype, device, not args.no_graph)

@@ -143,8 +143,16 @@ class _HipBackend(Backend):
     def upload(self, eid: int, slot: int, lane: str):
         blk = self.block
         ev = self.rings[lane].take()
+        stream = self._stream(lane)
+        timed = blk.metrics.time_copies and len(blk.metrics.pending_events) < 100000
+        if timed:
+            start, end = ops.Event(timing=True), ops.Event(timing=True)
+            start.record(stream)
         ops.expert_upload_async(blk.slab.slot_ptr(slot), blk.arena.host_ptr(eid), blk.arena.expert_bytes,
-                                self._stream(lane), ev)
+                                stream, ev)
+        if timed:
+            end.record(stream)
+            blk.metrics.pending_events.append((start, end, f"{lane}_h2d_ms", blk.layer_idx))
         return ev
 
     def event_done(self, event) -> bool:

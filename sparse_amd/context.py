@@ -44,9 +44,12 @@ class Metrics:
     counters: Dict[str, float] = field(default_factory=dict)
     # (kind, layer, expert) in issue order: kind in hit | prefetch_hit | miss
     events: Optional[List[Tuple[str, int, int]]] = None
+    # when set, every expert upload is bracketed by a timing event pair on its lane
+    time_copies: bool = False
     # deferred timing: (start_event, end_event, tag, layer)
     pending_events: List[Tuple[Any, Any, str, int]] = field(default_factory=list)
     timings_ms: Dict[str, float] = field(default_factory=dict)
+    timings_n: Dict[str, int] = field(default_factory=dict)
 
     def bump(self, name: str, value: float = 1) -> None:
         self.counters[name] = self.counters.get(name, 0) + value
@@ -59,6 +62,7 @@ class Metrics:
         """Read deferred event pairs (call after a device synchronisation)."""
         for start, end, tag, _layer in self.pending_events:
             self.timings_ms[tag] = self.timings_ms.get(tag, 0.0) + start.elapsed_ms(end)
+            self.timings_n[tag] = self.timings_n.get(tag, 0) + 1
         self.pending_events.clear()
         return self.timings_ms
 

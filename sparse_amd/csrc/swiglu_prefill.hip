@@ -35,6 +35,10 @@ constexpr int kPfThreads = 256;
 constexpr int kPfRowBytes = kPfBK * 2 + 16;  // padded LDS row
 constexpr int kPfLdsA = kPfBM * kPfRowBytes;
 constexpr int kPfXcds = 8;
+// Scheduling fence that vector/scalar ALU and LDS instructions may cross but global loads and MFMAs may
+// not: it keeps every prefetch where the loop puts it (the compiler otherwise sinks the
+// loads to the end of the slab, right in front of their first use).
+constexpr int kPfSchedMask = 0x2 | 0x4 | 0x80 | 0x100 | 0x200;
 
 struct PfTile {
   int32_t slot;  // weight slot of the segment's expert
@@ -208,31 +212,30 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_ffn_kernel(const Prefil
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[mi][ni][v] = 0.f;
 
-  u32x4 ra[4];
-  bf16x8 bcur[2][4], bnxt[2][4];
+  bf16x8 ra[4];
+  bf16x8 bfrag[2][4];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) ra[i] = *reinterpret_cast<const u32x4*>(aptr[i]);
+  for (int i = 0; i < 4; ++i) ra[i] = *reinterpret_cast<const bf16x8*>(aptr[i]);
 #pragma unroll
   for (int ni = 0; ni < 2; ++ni)
 #pragma unroll
-    for (int s = 0; s < 4; ++s) bcur[ni][s] = *reinterpret_cast<const bf16x8*>(bptr[ni] + s * 128);
+    for (int s = 0; s < 4; ++s) bfrag[ni][s] = *reinterpret_cast<const bf16x8*>(bptr[ni] + s * 128);
 #pragma unroll
-  for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(&lds[0][lds_wr + i * 32 * kPfRowBytes]) = ra[i];
+  for (int i = 0; i < 4; ++i) *reinterpret_cast<bf16x8*>(&lds[0][lds_wr + i * 32 * kPfRowBytes]) = ra[i];
   __syncthreads();
 
+  // Slab kt is multiplied while slab kt+1 is fetched: the activation rows into registers
+  // (stored to the other LDS buffer at the end of the slab), the weight fragments of k step s
+  // into the very registers step s has just finished with, so a fragment is a full slab of
+  // MFMA work ahead of its use and no second fragment buffer exists.  The last slab
+  // refetches itself instead of branching, which keeps the body straight-line.
   const int a_rd = fc * kPfRowBytes + fg * 16;
   const int nk = Kdim / kPfBK;
   for (int kt = 0; kt < nk; ++kt) {
-    const bool more = kt + 1 < nk;
-    if (more) {
+    const int ktn = min(kt + 1, nk - 1);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) ra[i] = *reinterpret_cast<const u32x4*>(aptr[i] + (kt + 1) * kPfBK);
-#pragma unroll
-      for (int ni = 0; ni < 2; ++ni)
-#pragma unroll
-        for (int s = 0; s < 4; ++s)
-          bnxt[ni][s] = *reinterpret_cast<const bf16x8*>(bptr[ni] + static_cast<size_t>(kt + 1) * 1024 + s * 128);
-    }
+    for (int i = 0; i < 4; ++i) ra[i] = *reinterpret_cast<const bf16x8*>(aptr[i] + ktn * kPfBK);
+    __builtin_amdgcn_sched_barrier(kPfSchedMask);
     const uint8_t* la = lds[kt & 1];
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
@@ -244,17 +247,16 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_ffn_kernel(const Prefil
       for (int mi = 0; mi < 4; ++mi)
 #pragma unroll
         for (int ni = 0; ni < 2; ++ni)
-          acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[mi], bcur[ni][s], acc[mi][ni], 0, 0, 0);
-    }
-    if (more) {
-      uint8_t* lw = lds[(kt + 1) & 1];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(lw + lds_wr + i * 32 * kPfRowBytes) = ra[i];
+          acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[mi], bfrag[ni][s], acc[mi][ni], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(kPfSchedMask);
 #pragma unroll
       for (int ni = 0; ni < 2; ++ni)
-#pragma unroll
-        for (int s = 0; s < 4; ++s) bcur[ni][s] = bnxt[ni][s];
+        bfrag[ni][s] = *reinterpret_cast<const bf16x8*>(bptr[ni] + static_cast<size_t>(ktn) * 1024 + s * 128);
+      __builtin_amdgcn_sched_barrier(kPfSchedMask);
     }
+    uint8_t* lw = lds[(kt + 1) & 1];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) *reinterpret_cast<bf16x8*>(lw + lds_wr + i * 32 * kPfRowBytes) = ra[i];
     __syncthreads();
   }
 

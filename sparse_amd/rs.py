@@ -57,3 +57,40 @@ def load_rs_payload(path: str, device: Optional[torch.device] = None) -> nn.Modu
     module.load_state_dict(state)
     module.eval()
     return module.to(device) if device is not None else module
+
+
+def informed_bank(gate_weights: List[Optional[torch.Tensor]], hidden_dim: int = 512,
+                  device: Optional[torch.device] = None) -> List[Optional[nn.Module]]:
+    """Predictors that reproduce a given router: entry l is built from ``gate_weights[l]``
+    ([E,H], the gate of layer l) so that ``RS_l(x) = softmax(gate_l x)``.  The hidden layer
+    holds +gate and -gate rows (ReLU(a) - ReLU(-a) = a), BatchNorm is the identity in eval
+    mode.  Useful where every layer of a synthetic stack reads the same hidden state, so the
+    next layer's routing is predictable from the current layer's input."""
+    bank: List[Optional[nn.Module]] = []
+    for gw in gate_weights:
+        if gw is None:
+            bank.append(None)
+            continue
+        E, H = gw.shape
+        if 2 * E > hidden_dim:
+            raise ValueError("hidden_dim must be at least twice the number of experts")
+        module = RoutingScoutMLP(H, E, hidden_dim=hidden_dim).eval()
+        lin1, bn, lin2 = module.mlp[0], module.mlp[1], module.mlp[4]
+        with torch.no_grad():
+            lin1.weight.zero_()
+            lin1.bias.zero_()
+            lin1.weight[:E] = gw.float().cpu()
+            lin1.weight[E:2 * E] = -gw.float().cpu()
+            bn.weight.fill_(1.0)
+            bn.bias.zero_()
+            bn.running_mean.zero_()
+            bn.running_var.fill_(1.0)
+            lin2.weight.zero_()
+            lin2.bias.zero_()
+            idx = torch.arange(E)
+            lin2.weight[idx, idx] = 1.0
+            lin2.weight[idx, E + idx] = -1.0
+        for p in module.parameters():
+            p.requires_grad_(False)
+        bank.append(module.to(device) if device is not None else module)
+    return bank

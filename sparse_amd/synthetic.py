@@ -58,12 +58,56 @@ def make_hidden(tokens: int, hidden: int, dtype: torch.dtype = torch.bfloat16, s
     return torch.randn(tokens, hidden, generator=g, device=dev, dtype=torch.float32).to(dtype)
 
 
-def zipf_coactivation_bias(num_experts: int, seed: int = 0, s: float = 1.1, cluster: int = 4,
-                           scale: float = 1.0) -> torch.Tensor:
-    """Per-expert logit bias making expert popularity follow Zipf(s) over a seeded
-    permutation of the experts: bias_e = scale * log(rank_e ** -s), rank 1 = most popular."""
+# ---- skewed, co-activating routing -------------------------------------------------
+# The router is a bias-free Linear, so structure is put into the data: a few reserved
+# hidden dimensions carry control values and the matching gate columns turn them into logit
+# offsets.  Dimension 0 holds a constant and gate column 0 the per-expert popularity bias;
+# dimension 1+c is raised for tokens that activate cluster c and gate column 1+c lifts the
+# experts of that cluster together.
+ROUTING_CONST = 4.0
+
+
+def routing_structure(num_experts: int, seed: int = 0, s: float = 1.1, cluster: int = 4):
+    """(bias[E], clusters[C][cluster], cluster_prob[C]) for one layer: popularity Zipf(s)
+    over a seeded permutation; consecutive popularity ranks form a cluster."""
     g = torch.Generator().manual_seed(int(seed))
-    order = torch.randperm(num_experts, generator=g)
+    order = torch.randperm(num_experts, generator=g)          # order[r] = expert of rank r+1
     rank = torch.empty(num_experts, dtype=torch.float32)
     rank[order] = torch.arange(1, num_experts + 1, dtype=torch.float32)
-    return scale * (-s) * torch.log(rank)
+    bias = (-s) * torch.log(rank)
+    n_clusters = num_experts // cluster
+    clusters = order[: n_clusters * cluster].reshape(n_clusters, cluster)
+    weight = torch.exp(bias)[clusters].sum(dim=1)
+    return bias, clusters, weight / weight.sum()
+
+
+def add_routing_structure(mlp_block, num_experts: int, seed: int = 0, s: float = 1.1, cluster: int = 4,
+                          boost: float = 5.0):
+    """Write the popularity bias and the cluster columns into ``mlp_block.gate.weight`` (in
+    place) and return the structure for ``make_structured_hidden``."""
+    bias, clusters, prob = routing_structure(num_experts, seed, s, cluster)
+    w = mlp_block.gate.weight
+    n_clusters = clusters.shape[0]
+    if w.shape[1] < 1 + n_clusters:
+        raise ValueError("hidden size too small for the reserved routing dimensions")
+    w[:, : 1 + n_clusters] = 0
+    w[:, 0] = (bias / ROUTING_CONST).to(w.dtype).to(w.device)
+    for c in range(n_clusters):
+        w[clusters[c].to(w.device), 1 + c] = boost / ROUTING_CONST
+    return dict(bias=bias, clusters=clusters, cluster_prob=prob)
+
+
+def make_structured_hidden(tokens: int, hidden: int, n_clusters: int, cluster_prob: torch.Tensor,
+                           dtype: torch.dtype = torch.bfloat16, seed: int = 1000, device="cpu", p: float = 0.6):
+    """Hidden states ~N(0,1) whose reserved dimensions say which cluster (if any, with
+    probability ``p``) each token activates.  All layers of a synthetic stack read the same
+    hidden state, so one cluster draw per token serves every layer's own cluster table."""
+    x = make_hidden(tokens, hidden, torch.float32, seed, device)
+    g = torch.Generator().manual_seed(int(seed) + 77)
+    active = torch.rand(tokens, generator=g) < p
+    which = torch.multinomial(cluster_prob, tokens, replacement=True, generator=g)
+    ctrl = torch.zeros(tokens, 1 + n_clusters)
+    ctrl[:, 0] = ROUTING_CONST
+    ctrl[torch.arange(tokens)[active], 1 + which[active]] = ROUTING_CONST
+    x[:, : 1 + n_clusters] = ctrl.to(x.device)
+    return x.to(dtype)

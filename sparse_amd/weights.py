@@ -10,9 +10,12 @@ All-resident layers use ``E`` slots with the identity slot table; cached layers 
 """
 from __future__ import annotations
 
+import ctypes
 from typing import Optional, Sequence, Tuple
 
 import torch
+
+from . import ops
 
 ExpertWeights = Tuple[torch.Tensor, torch.Tensor, torch.Tensor]
 
@@ -60,10 +63,30 @@ class HostExpertArena:
                  pin: bool = True) -> None:
         self.hidden, self.inter, self.dtype = hidden, inter, dtype
         self.num_experts = len(experts)
-        self.rows = torch.empty((self.num_experts, expert_numel(hidden, inter)), dtype=dtype, pin_memory=pin)
+        numel = expert_numel(hidden, inter)
+        self._pinned_ptr = None
+        if pin:
+            # hipHostMalloc of the exact size: torch's pinned allocator rounds every block up
+            # to a power of two, which nearly doubles a 1.1 GB layer
+            esize = torch.empty((), dtype=dtype).element_size()
+            nbytes = self.num_experts * numel * esize
+            self._pinned_ptr = ops.host_alloc(nbytes)
+            buf = (ctypes.c_uint8 * nbytes).from_address(self._pinned_ptr)
+            self.rows = torch.frombuffer(buf, dtype=torch.uint8).view(dtype).view(self.num_experts, numel)
+        else:
+            self.rows = torch.empty((self.num_experts, numel), dtype=dtype)
         for e, w in enumerate(experts):
             pack_expert_into(self.rows[e], tuple(t.to(dtype) for t in w), hidden, inter)
         self.expert_bytes = self.rows[0].numel() * self.rows.element_size()
+
+    def __del__(self) -> None:
+        ptr, self._pinned_ptr = getattr(self, "_pinned_ptr", None), None
+        if ptr:
+            self.rows = None
+            try:
+                ops.host_free(ptr)
+            except Exception:
+                pass
 
     def host_ptr(self, eid: int) -> int:
         return self.rows[eid].data_ptr()
