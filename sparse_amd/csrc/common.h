@@ -57,12 +57,17 @@ struct __attribute__((aligned(16))) u32x4 {
 };
 
 // ---- bf16 <-> fp32 ----------------------------------------------------------
-// Round-to-nearest-even, the rounding torch applies when it stores fp32 into bf16.
+// Round-to-nearest-even, the rounding torch applies when it stores fp32 into bf16; gfx950
+// converts in hardware (v_cvt_pk_bf16_f32).
 __device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return 0x7fc0;  // NaN
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return static_cast<uint16_t>(u >> 16);
+  return __builtin_bit_cast(uint16_t, static_cast<__bf16>(f));
+}
+// Two values at once, `lo` in bits 0..15.
+__device__ __forceinline__ uint32_t f32x2_to_bf16x2_bits(float lo, float hi) {
+  typedef __attribute__((__vector_size__(2 * sizeof(float)))) float f32x2_t;
+  typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2_t;
+  const f32x2_t v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
 }
 __device__ __forceinline__ float bf16_bits_to_f32(uint16_t b) {
   return __uint_as_float(static_cast<uint32_t>(b) << 16);
@@ -88,8 +93,12 @@ struct Elem<uint16_t> {
   __device__ static __forceinline__ float round(float v) { return round_bf16(v); }
 };
 
-// SiLU and sigmoid evaluated in fp32, as ATen does for reduced-precision inputs.
-__device__ __forceinline__ float silu_f32(float v) { return v / (1.0f + expf(-v)); }
+// SiLU and sigmoid evaluated in fp32, as ATen does for reduced-precision inputs.  SiLU runs
+// once per intermediate element, so it uses the hardware exp2 and reciprocal (a few fp32
+// ulp, far below the bf16 rounding that follows).
+__device__ __forceinline__ float silu_f32(float v) {
+  return v * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.44269504088896341f * v));
+}
 __device__ __forceinline__ float sigmoid_f32(float v) { return 1.0f / (1.0f + expf(-v)); }
 
 // ---- wavefront (64 lanes) reductions ---------------------------------------

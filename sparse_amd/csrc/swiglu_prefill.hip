@@ -24,6 +24,8 @@
 // MFMA 32x32x16 bf16 operand layout (lane l, c = l & 31, g = l >> 5):
 //   A: row c, k = g*8 .. g*8+7     B: column c, k = g*8 .. g*8+7
 //   D: column c, rows 8*i + 4*g + j for register 4*i + j
+// The weights are passed as A and the activations as B, so D is the transposed output
+// tile: a lane owns one activation row and runs of four consecutive output columns.
 #include "common.h"
 
 namespace sparse {
@@ -247,7 +249,7 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_ffn_kernel(const Prefil
       for (int mi = 0; mi < 4; ++mi)
 #pragma unroll
         for (int ni = 0; ni < 2; ++ni)
-          acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[mi], bfrag[ni][s], acc[mi][ni], 0, 0, 0);
+          acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfrag[ni][s], fa[mi], acc[mi][ni], 0, 0, 0);
       __builtin_amdgcn_sched_barrier(kPfSchedMask);
 #pragma unroll
       for (int ni = 0; ni < 2; ++ni)
@@ -261,31 +263,51 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_ffn_kernel(const Prefil
   }
 
   // ---- epilogue ----------------------------------------------------------------
+  // The product was formed as W * X^T, so a lane holds one row m (= 32*mi + fc) and, per
+  // accumulator quad i, four consecutive output columns 8*i + 4*fg + j: eight bytes of
+  // bf16 that go to the wave's private staging area in LDS (free now: every wave is past
+  // the last barrier of the k loop) as one write.  The area holds a 128-row x 32-column
+  // tile, rows of 64 bytes with the 16-byte chunks swizzled by row; it is read back a row
+  // quarter per lane and stored with 16-byte writes, 64 contiguous bytes per row.
+  uint8_t* st = &lds[0][0] + wave * (kPfBM * 64);
+  float sc[4];
 #pragma unroll
-  for (int mi = 0; mi < 4; ++mi) {
+  for (int mi = 0; mi < 4; ++mi) sc[mi] = kGateUp ? 1.f : s_scale[mi * 32 + fc];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+  for (int pass = 0; pass < (kGateUp ? 1 : 2); ++pass) {
+    if (pass) __syncthreads();  // staging rows are reused
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int m = mi * 32 + 8 * i + 4 * fg + j;
-        if (m >= M) continue;
-        const size_t p = static_cast<size_t>(r0 + m);
-        if (kGateUp) {
-          const int n = n0 + wave * 32 + fc;
-          if (n < Ndim) {
+    for (int mi = 0; mi < 4; ++mi) {
+      const int m = mi * 32 + fc;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float v[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          if (kGateUp) {
             const float g = round_bf16(acc[mi][0][4 * i + j]);
             const float u = round_bf16(acc[mi][1][4 * i + j]);
-            a.out[p * Ndim + n] = f32_to_bf16_bits(round_bf16(silu_f32(g)) * u);
-          }
-        } else {
-          const float sc = s_scale[m];
-#pragma unroll
-          for (int ni = 0; ni < 2; ++ni) {
-            const int n = n0 + wave * 64 + ni * 32 + fc;
-            if (n < Ndim) a.out[p * Ndim + n] = f32_to_bf16_bits(round_bf16(acc[mi][ni][4 * i + j]) * sc);
+            v[j] = round_bf16(silu_f32(g)) * u;
+          } else {
+            v[j] = round_bf16(acc[mi][pass][4 * i + j]) * sc[mi];
           }
         }
+        uint2 pk;
+        pk.x = f32x2_to_bf16x2_bits(v[0], v[1]);
+        pk.y = f32x2_to_bf16x2_bits(v[2], v[3]);
+        const int chunk = i ^ ((m >> 1) & 3);
+        *reinterpret_cast<uint2*>(st + m * 64 + chunk * 16 + fg * 8) = pk;
       }
+    }
+    __syncthreads();
+    const int ncol0 = kGateUp ? (n0 + wave * 32) : (n0 + wave * 64 + pass * 32);
+#pragma unroll
+    for (int it = 0; it < 8; ++it) {
+      const int m = it * 16 + (lane >> 2), q = lane & 3;
+      const uint4 val = *reinterpret_cast<const uint4*>(st + m * 64 + (q ^ ((m >> 1) & 3)) * 16);
+      const int n = ncol0 + q * 8;
+      if (m < M && n + 8 <= Ndim)
+        *reinterpret_cast<uint4*>(a.out + static_cast<size_t>(r0 + m) * Ndim + n) = val;
     }
   }
 }
