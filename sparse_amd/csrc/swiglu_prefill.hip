@@ -8,8 +8,9 @@
 // SiLU(gate)*up is a lane-local epilogue.
 //
 // The two operands take different roads.  Activation rows are shared by the four waves:
-// they go HBM/L2 -> registers -> LDS in 64-wide k slabs, two LDS buffers, one barrier per
-// slab, rows padded to 144 bytes so 16-byte fragment reads are bank-conflict free.
+// they go HBM/L2 -> LDS directly (no register hop) in 64-wide k slabs, three LDS buffers,
+// two slabs ahead of the multiply, one barrier per slab, chunks swizzled by row so that
+// 16-byte fragment reads are bank-conflict free.
 // Weight rows are private to a wave: they go HBM/L2 -> registers directly in MFMA
 // B-operand order, which is exactly the order the tiled layout stores them in (a wave
 // load is four 256-byte runs), one slab ahead of the multiply.  LDS thus carries a third
@@ -26,6 +27,8 @@
 //   D: column c, rows 8*i + 4*g + j for register 4*i + j
 // The weights are passed as A and the activations as B, so D is the transposed output
 // tile: a lane owns one activation row and runs of four consecutive output columns.
+#include <type_traits>
+
 #include "common.h"
 
 namespace sparse {
@@ -34,8 +37,9 @@ constexpr int kPfBM = 128;        // rows per tile
 constexpr int kPfBR = 256;        // weight rows per tile
 constexpr int kPfBK = 64;         // k slab
 constexpr int kPfThreads = 256;
-constexpr int kPfRowBytes = kPfBK * 2 + 16;  // padded LDS row
+constexpr int kPfRowBytes = kPfBK * 2;  // LDS row of one k slab (16-byte chunks swizzled by row)
 constexpr int kPfLdsA = kPfBM * kPfRowBytes;
+constexpr int kPfStages = 3;            // activation slabs resident in LDS
 constexpr int kPfXcds = 8;
 // Scheduling fence that vector/scalar ALU and LDS instructions may cross but global loads and MFMAs may
 // not: it keeps every prefetch where the loop puts it (the compiler otherwise sinks the
@@ -58,7 +62,8 @@ struct PrefillArgs {
   const uint16_t* topv;
   const uint16_t* act;
   uint16_t* out;
-  const PfTile* map;   // routed: one entry per workgroup
+  const PfTile* map;      // routed: one entry per tile
+  const int32_t* total;   // routed: number of tiles in the map
   int32_t topk;
   int32_t Kdim;
   int32_t Ndim;       // output columns (neurons for gate-up, hidden for down)
@@ -75,6 +80,7 @@ struct PfMapArgs {
   const int32_t* seg_offsets;
   PfTile* map_gu;
   PfTile* map_dn;
+  int32_t* totals;  // [0] gate/up tiles, [1] down tiles
   int32_t ntiles_gu, ntiles_dn;
   int32_t cap_gu, cap_dn;  // entries in each map
   sparse_hip_seglist segs;
@@ -123,12 +129,13 @@ __global__ __launch_bounds__(256) void prefill_tile_map_kernel(const PfMapArgs a
         }
     }
     for (int idx = total_mt * nt + tid; idx < cap; idx += 256) map[idx] = PfTile{0, 0, 0, 0};
+    if (tid == 0) a.totals[which] = total_mt * nt;
   }
 }
 
 template <bool kGateUp>
 __global__ __launch_bounds__(kPfThreads, 2) void prefill_ffn_kernel(const PrefillArgs a) {
-  __shared__ __attribute__((aligned(16))) uint8_t lds[2][kPfLdsA];
+  __shared__ __attribute__((aligned(1024))) uint8_t lds[kPfStages][kPfLdsA];
   __shared__ float s_scale[kPfBM];
 
   const int tid = threadIdx.x;
@@ -136,12 +143,17 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_ffn_kernel(const Prefil
   const int fc = lane & 31, fg = lane >> 5;
 
   // ---- which tile (XCD-aware order) ----------------------------------------------
-  const int per_xcd = gridDim.x / kPfXcds;
-  const int logical = (blockIdx.x % kPfXcds) * per_xcd + blockIdx.x / kPfXcds;
+  // The real tile count is split evenly over the XCDs (the grid is sized for the worst
+  // case, and the idle remainder must not fall on one XCD).
   int slot_id = 0, r0, M, bn;
+  const int mt_s = (a.T + kPfBM - 1) / kPfBM;
+  const int total = a.shared ? mt_s * a.ntiles_n : a.total[0];
+  const int per_xcd = (total + kPfXcds - 1) / kPfXcds;
+  const int in_xcd = blockIdx.x / kPfXcds;
+  const int logical = (blockIdx.x % kPfXcds) * per_xcd + in_xcd;
+  if (in_xcd >= per_xcd || logical >= total) return;
   if (a.shared) {
-    const int mt = (a.T + kPfBM - 1) / kPfBM;
-    if (logical >= mt * a.ntiles_n) return;
+    const int mt = mt_s;
     bn = logical / mt;
     r0 = (logical - bn * mt) * kPfBM;
     M = min(kPfBM, a.T - r0);
@@ -180,17 +192,34 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_ffn_kernel(const Prefil
     s_scale[tid] = sc;
   }
 
-  // ---- activation loader: 32 rows x 8 sixteen-byte chunks per pass, 4 passes --------
-  const int lrow = tid >> 3, lchunk = tid & 7;
-  const uint16_t* aptr[4];
+  // ---- activation loader: global -> LDS without passing through registers ----------
+  // One wave instruction moves 64 sixteen-byte pieces to 1 KB of consecutive LDS (lane l
+  // lands at byte 16*l), i.e. eight 128-byte rows of the slab; the lane chooses which
+  // piece of which row it fetches.  Row r keeps its chunk j at position j ^ f(r) with
+  // f(r) = ((r >> 1) & 7) ^ ((r & 1) << 2), which spreads the 16-byte fragment reads of
+  // 8 and of 16 consecutive rows over all banks.  Wave w owns rows 32w .. 32w+31.
+  const uint16_t* dptr[4];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int m = min(lrow + 32 * i, M - 1);
-    const int p = r0 + m;
-    const size_t row = (a.shared || !kGateUp) ? static_cast<size_t>(p) : static_cast<size_t>(a.perm[p] / a.topk);
-    aptr[i] = a.act + row * Kdim + lchunk * 8;
+  for (int it = 0; it < 4; ++it) {
+    const int row = wave * 32 + it * 8 + (lane >> 3);
+    const int p = r0 + min(row, M - 1);
+    const size_t grow = (a.shared || !kGateUp) ? static_cast<size_t>(p) : static_cast<size_t>(a.perm[p] / a.topk);
+    const int f = ((row >> 1) & 7) ^ ((row & 1) << 2);
+    dptr[it] = a.act + grow * Kdim + (((lane & 7) ^ f) << 3);
   }
-  const int lds_wr = lrow * kPfRowBytes + lchunk * 16;
+  // Issued as inline assembly: the compiler would otherwise make every barrier wait for all
+  // outstanding vector memory operations because one of them writes LDS, which is exactly
+  // the prefetch distance this loop exists for.  Completion is awaited by count below.
+  const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
+      (__attribute__((address_space(3))) uint8_t*)(&lds[0][0])));
+  auto stage_slab = [&](int slab, int buf) {
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+      const uint16_t* g = dptr[it] + slab * kPfBK;
+      const uint32_t dst = __builtin_amdgcn_readfirstlane(lds_base + buf * kPfLdsA + (wave * 4 + it) * 1024);
+      asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(dst) : "memory", "m0");
+    }
+  };
 
   // ---- weight fragments straight from the tiled layout ------------------------------
   // lane = (kh, gsel, r16): row r16 of 16-row group gsel of the wave's 32 rows, k half kh.
@@ -214,53 +243,70 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_ffn_kernel(const Prefil
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[mi][ni][v] = 0.f;
 
-  bf16x8 ra[4];
-  bf16x8 bfrag[2][4];
+  // Pipeline: while slab kt is multiplied, the activation rows of slab kt+2 travel to the
+  // third LDS buffer and the weight fragments of slab kt+2 to the registers step s has just
+  // finished with (two fragment sets, used alternately), so every operand is requested two
+  // slabs of MFMA work before its use -- enough bytes in flight to cover an HBM miss.
+  // Vector memory operations retire in order, so "the copies of slab kt+1 have landed" is a
+  // count of the younger operations: the 8 fragment loads of slab kt-1's steps, the 4 copies
+  // of slab kt+2 and the 8 fragment loads of slab kt's steps -- vmcnt(20) -- and the
+  // scheduling fences keep exactly that order.  Slabs past the end refetch the last one
+  // instead of branching.
+  constexpr int kWaitVm20 = 0x4F74, kWaitVm0 = 0x0F70;  // s_waitcnt vmcnt(n), other counters untouched
+  const int nk = Kdim / kPfBK;
+  bf16x8 bfrag[2][2][4];
+  stage_slab(0, 0);
+  stage_slab(min(1, nk - 1), 1);
+  __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-  for (int i = 0; i < 4; ++i) ra[i] = *reinterpret_cast<const bf16x8*>(aptr[i]);
+  for (int st = 0; st < 2; ++st)
 #pragma unroll
-  for (int ni = 0; ni < 2; ++ni)
+    for (int ni = 0; ni < 2; ++ni)
 #pragma unroll
-    for (int s = 0; s < 4; ++s) bfrag[ni][s] = *reinterpret_cast<const bf16x8*>(bptr[ni] + s * 128);
-#pragma unroll
-  for (int i = 0; i < 4; ++i) *reinterpret_cast<bf16x8*>(&lds[0][lds_wr + i * 32 * kPfRowBytes]) = ra[i];
+      for (int s = 0; s < 4; ++s)
+        bfrag[st][ni][s] =
+            *reinterpret_cast<const bf16x8*>(bptr[ni] + static_cast<size_t>(min(st, nk - 1)) * 1024 + s * 128);
+  __builtin_amdgcn_sched_barrier(0);
+  __builtin_amdgcn_s_waitcnt(kWaitVm20);
   __syncthreads();
 
-  // Slab kt is multiplied while slab kt+1 is fetched: the activation rows into registers
-  // (stored to the other LDS buffer at the end of the slab), the weight fragments of k step s
-  // into the very registers step s has just finished with, so a fragment is a full slab of
-  // MFMA work ahead of its use and no second fragment buffer exists.  The last slab
-  // refetches itself instead of branching, which keeps the body straight-line.
-  const int a_rd = fc * kPfRowBytes + fg * 16;
-  const int nk = Kdim / kPfBK;
-  for (int kt = 0; kt < nk; ++kt) {
-    const int ktn = min(kt + 1, nk - 1);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) ra[i] = *reinterpret_cast<const bf16x8*>(aptr[i] + ktn * kPfBK);
+  const int fsw = ((fc >> 1) & 7) ^ ((fc & 1) << 2);
+  const int a_row = fc * kPfRowBytes, a_x = (fg ^ fsw) << 4;
+  int cur = 0, nxt2 = 2;  // buffer of slab kt, buffer of slab kt+2
+  auto slab = [&](auto stage_c, int kt) {
+    constexpr int st = decltype(stage_c)::value;
+    const int kt2 = min(kt + 2, nk - 1);
+    stage_slab(kt2, nxt2);
     __builtin_amdgcn_sched_barrier(kPfSchedMask);
-    const uint8_t* la = lds[kt & 1];
+    const uint8_t* la = lds[cur] + a_row;
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
       bf16x8 fa[4];
 #pragma unroll
       for (int mi = 0; mi < 4; ++mi)
-        fa[mi] = *reinterpret_cast<const bf16x8*>(la + a_rd + mi * 32 * kPfRowBytes + s * 32);
+        fa[mi] = *reinterpret_cast<const bf16x8*>(la + mi * 32 * kPfRowBytes + (a_x ^ (s << 5)));
 #pragma unroll
       for (int mi = 0; mi < 4; ++mi)
 #pragma unroll
         for (int ni = 0; ni < 2; ++ni)
-          acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfrag[ni][s], fa[mi], acc[mi][ni], 0, 0, 0);
+          acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfrag[st][ni][s], fa[mi], acc[mi][ni], 0, 0, 0);
       __builtin_amdgcn_sched_barrier(kPfSchedMask);
 #pragma unroll
       for (int ni = 0; ni < 2; ++ni)
-        bfrag[ni][s] = *reinterpret_cast<const bf16x8*>(bptr[ni] + static_cast<size_t>(ktn) * 1024 + s * 128);
+        bfrag[st][ni][s] = *reinterpret_cast<const bf16x8*>(bptr[ni] + static_cast<size_t>(kt2) * 1024 + s * 128);
       __builtin_amdgcn_sched_barrier(kPfSchedMask);
     }
-    uint8_t* lw = lds[(kt + 1) & 1];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) *reinterpret_cast<bf16x8*>(lw + lds_wr + i * 32 * kPfRowBytes) = ra[i];
+    __builtin_amdgcn_s_waitcnt(kWaitVm20);
     __syncthreads();
+    cur = (cur == kPfStages - 1) ? 0 : cur + 1;
+    nxt2 = (nxt2 == kPfStages - 1) ? 0 : nxt2 + 1;
+  };
+  for (int kt = 0; kt < nk; kt += 2) {
+    slab(std::integral_constant<int, 0>{}, kt);
+    if (kt + 1 < nk) slab(std::integral_constant<int, 1>{}, kt + 1);
   }
+  __builtin_amdgcn_s_waitcnt(kWaitVm0);  // no copy may land in LDS after the epilogue starts to reuse it
+  __syncthreads();
 
   // ---- epilogue ----------------------------------------------------------------
   // The product was formed as W * X^T, so a lane holds one row m (= 32*mi + fc) and, per
@@ -332,7 +378,7 @@ size_t prefill_ws_bytes(int Ttok, int K, int nseg, int H, int I) {
   const int64_t mt = pf_max_mtiles(Ttok, K, nseg);
   const int64_t gu = pf_round8(mt * ((I + kPfBR / 2 - 1) / (kPfBR / 2)));
   const int64_t dn = pf_round8(mt * ((H + kPfBR - 1) / kPfBR));
-  return static_cast<size_t>(gu + dn) * sizeof(PfTile);
+  return static_cast<size_t>(gu + dn + 1) * sizeof(PfTile);  // one leading entry holds the two totals
 }
 
 int prefill_routed_bf16(const sparse_hip_experts* ex, const void* x, const void* topv, const int32_t* perm,
@@ -344,7 +390,8 @@ int prefill_routed_bf16(const sparse_hip_experts* ex, const void* x, const void*
   const int nt_dn = static_cast<int>((H + kPfBR - 1) / kPfBR);
   const int cap_gu = static_cast<int>(pf_round8(static_cast<int64_t>(mt) * nt_gu));
   const int cap_dn = static_cast<int>(pf_round8(static_cast<int64_t>(mt) * nt_dn));
-  PfTile* map_gu = static_cast<PfTile*>(tile_ws);
+  int32_t* totals = static_cast<int32_t*>(tile_ws);
+  PfTile* map_gu = static_cast<PfTile*>(tile_ws) + 1;
   PfTile* map_dn = map_gu + cap_gu;
   {
     PfMapArgs m = {};
@@ -352,6 +399,7 @@ int prefill_routed_bf16(const sparse_hip_experts* ex, const void* x, const void*
     m.seg_offsets = seg_offsets;
     m.map_gu = map_gu;
     m.map_dn = map_dn;
+    m.totals = totals;
     m.ntiles_gu = nt_gu;
     m.ntiles_dn = nt_dn;
     m.cap_gu = cap_gu;
@@ -371,6 +419,7 @@ int prefill_routed_bf16(const sparse_hip_experts* ex, const void* x, const void*
   a.act = static_cast<const uint16_t*>(x);
   a.out = static_cast<uint16_t*>(inter_ws);
   a.map = map_gu;
+  a.total = totals;
   a.Kdim = static_cast<int32_t>(H);
   a.Ndim = static_cast<int32_t>(I);
   a.ntiles_n = nt_gu;
@@ -382,6 +431,7 @@ int prefill_routed_bf16(const sparse_hip_experts* ex, const void* x, const void*
   a.act = static_cast<const uint16_t*>(inter_ws);
   a.out = static_cast<uint16_t*>(parts);
   a.map = map_dn;
+  a.total = totals + 1;
   a.Kdim = static_cast<int32_t>(I);
   a.Ndim = static_cast<int32_t>(H);
   a.ntiles_n = nt_dn;
