@@ -103,6 +103,77 @@ __global__ __launch_bounds__(kRouterThreads) void router_logits_kernel(
 }
 
 // ---------------------------------------------------------------------------
+// Prefill-size router logits (bf16): one workgroup per 16 tokens, the four wavefronts
+// split H.  A wavefront multiplies its 16 x (H/4) slice of x with 64 gate rows at a time
+// (four 16x16x32 MFMA tiles; x rows are the A operand, gate rows the B operand, both read
+// from global memory in operand order: lane (r = l & 15, q = l >> 4) holds row r,
+// k = q*8 .. q*8+7), the four partial tiles meet in LDS and are summed in wavefront order.
+// Row E (when present) is the shared-expert gate vector.  Needs H % 512 == 0.
+// ---------------------------------------------------------------------------
+constexpr int kRlTok = 16;
+constexpr int kRlRows = 64;   // gate rows per pass
+constexpr int kRlPad = 65;    // LDS row stride in floats
+
+template <typename TL>
+__global__ __launch_bounds__(256) void router_logits_mfma_kernel(
+    const uint16_t* __restrict__ x, const uint16_t* __restrict__ wg, const uint16_t* __restrict__ wsg, int Ttok,
+    int H, int E, TL* __restrict__ logits, uint16_t* __restrict__ shared_gate) {
+  __shared__ float part[4][kRlTok][kRlPad];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int r = lane & 15, q = lane >> 4;
+  const int t0 = blockIdx.x * kRlTok;
+  const int R = E + (wsg != nullptr ? 1 : 0);
+  const int kspan = H / 4, kbeg = wave * kspan;
+  const uint16_t* xrow = x + static_cast<size_t>(min(t0 + r, Ttok - 1)) * H + kbeg + q * 8;
+
+  for (int row0 = 0; row0 < R; row0 += kRlRows) {
+    const uint16_t* wrow[4];
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt) {
+      const int row = row0 + nt * 16 + r;
+      wrow[nt] = (row < E ? wg + static_cast<size_t>(row) * H : (row == E && wsg != nullptr ? wsg : wg)) + kbeg + q * 8;
+    }
+    f32x4 acc[4];
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt) acc[nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int k0 = 0; k0 < kspan; k0 += 128) {
+      bf16x8 av[4], bv[4][4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        av[u] = *reinterpret_cast<const bf16x8*>(xrow + k0 + u * 32);
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt) bv[u][nt] = *reinterpret_cast<const bf16x8*>(wrow[nt] + k0 + u * 32);
+      }
+      __builtin_amdgcn_sched_barrier(0);  // all 20 loads of the span in flight before the first MFMA
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt)
+          acc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[u], bv[u][nt], acc[nt], 0, 0, 0);
+    }
+    // D: lane holds gate row (column) nt*16 + r for tokens q*4 .. q*4+3
+    if (row0 > 0) __syncthreads();
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) part[wave][q * 4 + v][nt * 16 + r] = acc[nt][v];
+    __syncthreads();
+    for (int i = tid; i < kRlTok * kRlRows; i += 256) {
+      const int tok = i >> 6, col = i & 63;
+      const int row = row0 + col, t = t0 + tok;
+      if (t < Ttok && row < R) {
+        const float sum = ((part[0][tok][col] + part[1][tok][col]) + part[2][tok][col]) + part[3][tok][col];
+        if (row < E) {
+          Elem<TL>::store(logits + static_cast<size_t>(t) * E + row, sum);
+        } else {
+          shared_gate[t] = f32_to_bf16_bits(sum);
+        }
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
 // Fused softmax(fp32) + top-k of one token by one wavefront; lane l holds experts
 // l, l+64, l+128, l+192.  Selection runs K rounds of a wave-wide arg-max whose order is
 // (probability descending, expert id ascending): the largest probability first, then
@@ -364,6 +435,17 @@ __global__ __launch_bounds__(kRouteThreads) void route_decode_kernel(const Route
 template <typename T, typename TL>
 static int launch_router_logits(const void* x, const void* wg, const void* wsg, int Ttok, int H, int E,
                                 void* logits, void* shared_gate, hipStream_t st) {
+  if constexpr (sizeof(T) == 2) {
+    if (Ttok >= 64 && H % 512 == 0) {
+      ProfScope prof(SPARSE_HIP_K_ROUTER_LOGITS, st);
+      hipLaunchKernelGGL((router_logits_mfma_kernel<TL>), dim3((Ttok + kRlTok - 1) / kRlTok), dim3(256), 0, st,
+                         static_cast<const uint16_t*>(x), static_cast<const uint16_t*>(wg),
+                         static_cast<const uint16_t*>(wsg), Ttok, H, E, static_cast<TL*>(logits),
+                         static_cast<uint16_t*>(shared_gate));
+      SP_LAUNCH_CHECK("router_logits_mfma_kernel");
+      return SPARSE_HIP_OK;
+    }
+  }
   dim3 grid(E + (wsg != nullptr ? 1 : 0), (Ttok + kRouterTokTile - 1) / kRouterTokTile);
   ProfScope prof(SPARSE_HIP_K_ROUTER_LOGITS, st);
   hipLaunchKernelGGL((router_logits_kernel<T, TL>), grid, dim3(kRouterThreads), 0, st,
