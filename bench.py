@@ -338,6 +338,21 @@ def epipe_prefill_workload(dtype, device, tokens=4096, chunk=2048, capacity=19, 
     return out
 
 
+def measured_traffic_ratio(kernel="decode_gateup"):
+    """HBM bytes per launch over algorithmic bytes per launch for the dominant kernel, as
+    measured with hardware counters (two profiler runs, scaled by a plain copy) and recorded
+    in the committed summary; None when there is no summary."""
+    path = os.path.join(ROOT, "profiles", "decode_b8_qwen_hbm_traffic.txt")
+    try:
+        for line in open(path):
+            parts = line.split()
+            if len(parts) == 3 and parts[0] == "traffic_over_algorithmic" and parts[1] == kernel:
+                return float(parts[2])
+    except OSError:
+        pass
+    return None
+
+
 def cpu_baseline(shape, batch, dtype, device, budget_s=12.0):
     """The CPU oracle of one layer of the same workload on this box's host cores."""
     from oracle import ref_moe
@@ -376,6 +391,8 @@ def main():
     ap.add_argument("--no-extra", action="store_true", help="skip batch 1/32 decode and the prefill workload")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--only-prefill", action="store_true", help="run just the prefill workload (for profiling)")
+    ap.add_argument("--calib-copy", action="store_true",
+                    help="also launch a 256 MiB plain copy kernel a few times (yardstick for --pmc byte counters)")
     ap.add_argument("--cached-decode", type=int, default=0, metavar="STEPS",
                     help="run just the expert-cache decode comparison (rr vs rs) for STEPS decode steps")
     ap.add_argument("--epipe-prefill", action="store_true",
@@ -402,6 +419,14 @@ def main():
     if args.epipe_prefill:
         print(json.dumps({"epipe_prefill_deepseek": epipe_prefill_workload(dtype, device)}))
         return
+    if args.calib_copy:
+        from sparse_amd import ops
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=device).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(4):
+            ops.calib_copy(src, dst)
+        torch.cuda.synchronize()
+        del src, dst
     blocks = build_stack(QWEN, dtype, device)
     main_res = decode_workload(blocks, QWEN, 8, args.steps, args.warmup, dtype, device, not args.no_graph)
     extra = {}
@@ -419,6 +444,7 @@ def main():
     cpu = None if args.no_cpu_baseline else cpu_baseline(QWEN, 8, dtype, device)
 
     gu = main_res["gateup"]
+    ratio = measured_traffic_ratio()
     line = {
         "metric": "MoE-layer tokens/s (decode b=8, prefill 4k) + % of MFMA/HBM/H2D roofline",
         "value": main_res["tokens_per_s"],
@@ -441,7 +467,11 @@ def main():
         },
         "roofline": {
             "bound": "hbm", "achieved": gu["gbps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-            "frac": gu["gbps"] / HBM_PEAK_GBPS, "traffic": None, "kernel": gu["kernel"],
+            "frac": gu["gbps"] / HBM_PEAK_GBPS,
+            # counter-measured HBM bytes per launch: the ratio recorded in profiles/ (FETCH_SIZE +
+            # WRITE_SIZE runs scaled by a plain copy) applied to this run's algorithmic bytes
+            "traffic": (gu["bytes_per_launch"] * ratio) if ratio else None,
+            "traffic_over_algorithmic": ratio, "kernel": gu["kernel"],
             "bytes_per_launch": gu["bytes_per_launch"], "avg_launch_us": gu["avg_us"], "launches": gu["launches"],
             "mean_distinct_experts": main_res["mean_distinct_experts"],
         },

@@ -333,6 +333,15 @@ def host_free(ptr: int) -> None:
 
 
 # --------------------------------------------------------------------------- measurement
+def calib_copy(src: torch.Tensor, dst: torch.Tensor) -> None:
+    """Plain device copy of a known size: the yardstick the hardware byte counters of a
+    profiler run are scaled with."""
+    _need(src, "src")
+    _need(dst, "dst", src.dtype, tuple(src.shape))
+    nbytes = src.numel() * src.element_size()
+    _lib.check(_lib.load().sparse_hip_calib_copy(_ptr(src), _ptr(dst), nbytes, _stream()), "sparse_hip_calib_copy")
+
+
 def profile_enable(on: bool) -> None:
     _lib.check(_lib.load().sparse_hip_profile_enable(int(bool(on))), "sparse_hip_profile_enable")
 
