@@ -13,9 +13,12 @@ the HBM roofline of the dominant kernel (the fused gate/up projection), measured
 events in an instrumented eager pass over the same steps, and a CPU baseline: the CPU
 oracle of the same layer timed on the host cores of this box on a bounded sample.
 
-Extra workloads (reported under "extra"): decode at batch 1 and 32, and the
+Extra workloads (reported under "extra"): decode at batch 1 and 32, the
 DeepSeek-V2-Lite-shaped 4096-token prefill (hidden 2048, 64 experts x 1408, top-6,
-shared MLP 2816, 26 layers) with its MFMA roofline.
+shared MLP 2816, 26 layers) with its MFMA roofline, and the two offloaded configurations
+(expert-cache decode rr vs rs, readiness-aware chunked prefill rr vs rs-epipe vs sparse)
+with hit rates, stall and host-link rates; ``--cached-decode N`` / ``--epipe-prefill`` run
+those two alone at full length.
 """
 from __future__ import annotations
 
@@ -441,6 +444,16 @@ def main():
     if not args.no_extra:
         extra["prefill_4k_deepseek"] = prefill_workload(DEEPSEEK, 4096, max(2, min(10, args.steps // 10)), 1, dtype,
                                                         device)
+    if not args.no_extra:
+        # the offloaded configurations, shortened (64 decode steps from a cold cache); a failure
+        # here (e.g. no pinned memory to be had) must not cost the main line
+        for name, leg in (("cached_decode_qwen", lambda: cached_decode_workload(dtype, device, 64)),
+                          ("epipe_prefill_deepseek", lambda: epipe_prefill_workload(dtype, device))):
+            try:
+                extra[name] = leg()
+            except Exception as exc:  # noqa: BLE001
+                extra[name] = {"error": repr(exc)[:300]}
+            release_stack()
     cpu = None if args.no_cpu_baseline else cpu_baseline(QWEN, 8, dtype, device)
 
     gu = main_res["gateup"]
