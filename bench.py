@@ -297,10 +297,31 @@ def cached_decode_workload(dtype, device, steps, batch=8, capacity=15, top_m=8):
     del blocks
     release_stack()
     for name, method, rs_kind in (("rr", "rr", "random"), ("rs_random_init", "rs", "random"),
-                                  ("rs_informed", "rs", "informed"), ("rs-epipe_informed", "rs-epipe", "informed")):
-        blocks, metrics, _ = build_offload_stack(shape, dtype, device, method, capacity, top_m, rs_kind=rs_kind)
+                                  ("rs_informed", "rs", "informed"), ("rs-epipe_informed", "rs-epipe", "informed"),
+                                  ("rs-epipe_staged_informed", "rs-epipe", "informed")):
+        staged = "staged" in name
+        kw = dict(staging_pool_slots=4) if staged else {}
+        blocks, metrics, _ = build_offload_stack(shape, dtype, device, method, capacity, top_m, rs_kind=rs_kind,
+                                                 **kw)
+        engine = None
+        if staged:
+            # the bounded staging engine instead of the in-line planner: graph-captured predictor,
+            # worker-thread publication into a per-layer pool of 4 slots
+            from sparse_amd.context import SparseContext
+            from sparse_amd.staging import BoundedRS
+            engine = BoundedRS(slots=4)
+            engine.prepare({b.layer_idx: b for b in blocks}, SparseContext.rs_bank, batch=batch, dtype=dtype)
+            engine.enabled = True
+            SparseContext.staging = engine
+            engine.begin(name)
         wall = run_phase_steps(blocks, inputs, "decode")   # cold cache, all steps timed
         out[name] = offload_report(metrics, blocks, wall, steps, batch, resident_ms)
+        if engine is not None:
+            st = engine.finish()
+            engine.shutdown()
+            out[name]["staging"] = {k: st[k] for k in ("predictions", "issued", "used", "wasted", "retained",
+                                                        "skipped_slots", "closed_before_publish")}
+            del engine
         del blocks, metrics
         release_stack()
     return out

@@ -420,7 +420,18 @@ class DistributedSparseMoeBlock(nn.Module):
             logits = torch.empty((0, self.num_experts), device=x.device, dtype=self.logits_dtype)
             return hidden_states if self._return_tensor_only_mlp() else (hidden_states, logits)
         ws = self._workspace(T)
-        rs_job = self._rs_begin(x, S, ws)
+        staging = SparseContext.staging
+        staged = (staging is not None and self.residency is not None and staging.handles(self, S))
+        if staged:
+            # bounded staging engine: the prediction for layer l+1 leaves on a side stream and
+            # is never joined; this layer's own staged copies are exposed at the executor
+            self.residency.staging = staging
+            staging.predict(self, x, int(SparseContext.runtime_call_id))
+            rs_job = None
+        else:
+            if self.residency is not None:
+                self.residency.staging = None
+            rs_job = self._rs_begin(x, S, ws)
 
         logits = self._route(x, ws)
         shared_gate = ws.shared_gate if self.shared_gate_weight is not None else None
@@ -446,7 +457,13 @@ class DistributedSparseMoeBlock(nn.Module):
             res.phase, res.call_id = str(SparseContext.current_phase), int(SparseContext.runtime_call_id)
             res.stage = self._current_stage(S)
             self._backend.bind(x, ws)
-            self.last_executor = res.execute(segments)
+            if staged:
+                staging.activate_at_demand(self, int(SparseContext.runtime_call_id))
+            try:
+                self.last_executor = res.execute(segments)
+            finally:
+                if staged:
+                    staging.release(self)
         if self.residency is None and rs_job is not None:
             torch.cuda.current_stream().synchronize()
             self._rs_finish(rs_job, ws)

@@ -80,6 +80,7 @@ class SparseContext:
     rs_bank_source_layers: List[int] = []
     routing_cache: Dict[int, Tuple[torch.Tensor, torch.Tensor]] = {}
     prefill_scp_transient_demoted_for_decode: bool = False
+    staging: Optional[Any] = None          # bounded RS staging engine (sparse_amd.staging.BoundedRS)
 
     @classmethod
     def register_layer_block(cls, layer_idx: int, block: Any) -> None:
@@ -114,3 +115,4 @@ class SparseContext:
         cls.rs_bank_source_layers = []
         cls.routing_cache = {}
         cls.prefill_scp_transient_demoted_for_decode = False
+        cls.staging = None

@@ -51,6 +51,7 @@ class ResidencyConfig:
 
     capacity: int = 10
     staging_slots: int = 4
+    staging_pool_slots: int = 0            # slots reserved for the bounded RS staging engine
     planner_mode: str = "none"            # none | rs_prefetch
     prefetch_top_m: int = 4
     pred_topk: Optional[int] = None        # SPARSE_RS_PREFETCH_PRED_TOPK
@@ -188,7 +189,11 @@ class LayerResidency:
         self.extra_cache = EpipePrefillExtraCache(int(config.epipe_prefill_extra_cache_slots))
         self.num_slots = max(0, int(config.capacity)) + max(1, int(config.staging_slots)) + \
             max(0, int(config.epipe_prefill_extra_cache_slots))
+        # slots of the bounded RS staging pool sit after the ordinary ones and never enter the free list
+        self._pool_slots: List[int] = list(range(self.num_slots, self.num_slots + max(0, int(config.staging_pool_slots))))
         self._free_slots: List[int] = list(range(self.num_slots - 1, -1, -1))
+        self.num_slots += len(self._pool_slots)
+        self.staging: Any = None   # the BoundedRS engine while a request runs with it enabled
         self._retired: List[int] = []           # evicted, still read by the pending batch
         self._pending: List[Tuple[int, int]] = []  # (eid, slot) not launched yet
         self._pending_slots: Set[int] = set()
@@ -220,6 +225,8 @@ class LayerResidency:
             m.prefetch_hit_count += 1
         else:
             m.cache_miss_count += 1
+            if self.staging is not None and self.stage == "decode":
+                self.staging.note_demand_miss(self)
         if m.events is not None:
             m.events.append((kind, self.layer_idx, int(eid)))
 
@@ -375,7 +382,13 @@ class LayerResidency:
             if self.stage == "decode" and rs_active and mode == "off":
                 name = None
             elif self.stage == "decode" and rs_active and mode == "residual_scan":
-                name = self._epipe_rs_residual_scan(segments)
+                if self.staging is not None:
+                    # staged experts are classified like cached ones by the upfront scan
+                    # (utils/rs_overlap.py:474-479)
+                    self.staging.stats["unified_epipe_calls"] += 1
+                    name = self._epipe_upfront_scan(segments)
+                else:
+                    name = self._epipe_rs_residual_scan(segments)
             elif self.stage == "decode" and rs_active:
                 raise NotImplementedError(
                     f"SPARSE_EPIPE_DECODE_RS_MODE={mode} is not built; use off or residual_scan")
@@ -650,6 +663,48 @@ class LayerResidency:
         return self._demand_gate_can_open()
 
     # ------------------------------------------------------------------ RS prefetch
+    # ---- bounded RS staging (utils/rs_overlap.py) -------------------------------------
+    def claim_staging_pool(self, n: int) -> List[int]:
+        """Slot ids reserved for the staging engine (``staging_pool_slots`` of the config)."""
+        if n > len(self._pool_slots):
+            raise ValueError(
+                f"layer {self.layer_idx}: {n} staging pool slots asked, {len(self._pool_slots)} reserved "
+                "(set ResidencyConfig.staging_pool_slots before the block is built)")
+        return list(self._pool_slots[:n])
+
+    def min_candidate_score(self) -> float:
+        """``_prefetch_min_candidate_score`` with the cache-safe floor (reference :4954-4972)."""
+        score = float(self.cfg.min_candidate_score)
+        if self.cfg.rs_policy in ("cache_safe", "cache-safe", "benefit_gate", "benefit-gate"):
+            score = max(score, float(self.cfg.cache_safe_min_score))
+        return score
+
+    def adopt_staged(self, eid: int, slot: int, event: Any) -> Tuple[Optional[int], bool]:
+        """Admit a staged expert that this call really used into the LRU, keeping its bytes
+        where they are: ``slot`` becomes the cache's, and the slot handed back -- the evicted
+        resident's (``recycled``) or a free one -- becomes the pool's
+        (``_retain_used``, utils/rs_overlap.py:352-381).  ``(None, False)`` if the cache did
+        not take the expert."""
+        resident = getattr(self.cache, "resident", self.cache)
+        if resident.capacity <= 0:
+            return None, False
+        self._on_demand_access(eid)
+        protect = self._protect_with_fallback(eid)
+        resident.put(int(eid), int(slot), pinned=False, protect_ids=protect)
+        if not resident.has(eid):
+            return None, False
+        self._slot_of[int(eid)] = int(slot)
+        self._slot_upload[int(slot)] = (event, "staging")
+        evicted = [e for e in self._slot_of if not resident.has(e)]
+        assert len(evicted) <= 1, "Only a layer-local plain LRU is supported"
+        if evicted:
+            self.prefetch_events.pop(evicted[0], None)
+            replacement, recycled = self._slot_of.pop(evicted[0]), True
+        else:
+            replacement, recycled = self._acquire_slot(), False
+        self._pool_slots[self._pool_slots.index(int(slot))] = replacement
+        return replacement, recycled
+
     def effective_top_m(self) -> int:
         return max(0, int(self.cfg.prefetch_top_m))
 
@@ -868,5 +923,6 @@ class LayerResidency:
         self.cache.clear()
         self.extra_cache.clear()
         self._slot_of.clear()
-        self._free_slots = list(range(self.num_slots - 1, -1, -1))
+        pool = set(self._pool_slots)
+        self._free_slots = [s for s in range(self.num_slots - 1, -1, -1) if s not in pool]
         self._retired = []

@@ -179,3 +179,80 @@ def test_zero_and_tiny_capacity_and_request_reset(device):
     got = _run(blocks, device, steps, T)
     for a, b in zip(got, want):
         assert torch.equal(a, b)
+
+
+def _staged_stack(device, capacity, top_m, pool_slots, method="rs-epipe"):
+    """Offloaded stack with pool slots for the bounded staging engine and predictors that
+    reproduce the next layer's router (every layer reads the same hidden state here)."""
+    from sparse_amd.block import DistributedSparseMoeBlock
+    from sparse_amd.context import DistEnv, Metrics, SparseContext
+    from sparse_amd.methods import method_settings, residency_config
+    from sparse_amd.rs import informed_bank
+    from sparse_amd.synthetic import make_mlp_block
+    SparseContext.reset()
+    metrics = Metrics()
+    metrics.events = []
+    kw = method_settings(method)["kwargs"]
+    blocks, gates = {}, []
+    for layer in range(SHAPE["num_layers"]):
+        mlp = make_mlp_block(SHAPE, dtype=torch.bfloat16, seed=layer)
+        gates.append(mlp.gate.weight.detach().clone() if layer > 0 else None)
+        cfg = residency_config(method, capacity, top_m, staging_pool_slots=pool_slots, formal_thresholds=False)
+        blocks[layer] = DistributedSparseMoeBlock(
+            layer, mlp, None, DistEnv(0, 1, 0, device), num_layers=SHAPE["num_layers"],
+            num_experts=SHAPE["num_experts"], top_k=SHAPE["top_k"], dtype=torch.bfloat16, expert_offload="cpu",
+            expert_cache=capacity, planner_mode=kw["planner_mode"], prefetch_top_m=top_m,
+            placement_mode=kw["placement_mode"], metrics=metrics, residency_config=cfg)
+    bank = informed_bank(gates, hidden_dim=64, device=device)
+    SparseContext.set_rs_bank(bank)
+    return blocks, metrics, bank
+
+
+def test_bounded_staging_engine_decode(device):
+    """The staging engine changes where weights come from, never the values: outputs equal
+    the all-resident block bit for bit; staged experts that were used are admitted to the
+    LRU by slot exchange; wrong forecasts leave the LRU untouched; the request drains."""
+    from sparse_amd.context import SparseContext
+    from sparse_amd.staging import BoundedRS
+    capacity, top_m, steps, T = 4, 2, 24, 4
+    ref_blocks, _ = _stack(device, "rr", capacity, top_m, "gpu")
+    want = _run(ref_blocks, device, steps, T)
+    blocks, metrics, bank = _staged_stack(device, capacity, top_m, pool_slots=4)
+    engine = BoundedRS(slots=4)
+    engine.prepare(blocks, bank, batch=T, dtype=torch.bfloat16)
+    engine.enabled = True
+    SparseContext.staging = engine
+    engine.begin("test")
+    got = _run(list(blocks.values()), device, steps, T)
+    stats = engine.finish()
+    assert len(got) == len(want)
+    for i, (a, b) in enumerate(zip(got, want)):
+        assert torch.equal(a, b), f"output {i} differs from the all-resident block"
+    assert stats["predictions"] > 0 and stats["issued"] > 0
+    assert stats["used"] + stats["wasted"] == stats["issued"]
+    assert stats["used"] > 0 and stats["retained"] > 0
+    assert stats["retained"] == stats["recycled_payloads"] + stats["allocated_replacements"]
+    assert stats["unified_epipe_calls"] > 0
+    assert metrics.prefetch_hit_count >= stats["used"] > 0
+    assert metrics.prefetch_h2d_bytes == stats["issued"] * blocks[0].arena.expert_bytes
+    for layer, blk in blocks.items():
+        res = blk.residency
+        assert res.cache is blk._cache and not hasattr(res.cache, "staged")      # views are gone
+        slots = [res._slot_of[e] for e in res.cache.resident_ids()]
+        pool = [s["payload"] for s in engine.slots[layer]]
+        assert len(set(slots)) == len(slots) and not set(slots) & set(pool)       # no slot has two owners
+        assert sorted(pool) == sorted(res._pool_slots) and not set(pool) & set(res._free_slots)
+        assert all(not s["busy"] for s in engine.slots[layer])
+    # a second request on the same engine, then the ordinary planner again
+    engine.begin("again")
+    got2 = _run(list(blocks.values()), device, 6, T)
+    stats2 = engine.finish()
+    assert stats2["predictions"] > 0 and stats2["case"] == "again"
+    engine.enabled = False
+    SparseContext.staging = None
+    for a, b in zip(got2, want[: len(got2)]):
+        assert torch.equal(a, b)
+    got3 = _run(list(blocks.values()), device, 6, T)
+    for a, b in zip(got3, want[: len(got3)]):
+        assert torch.equal(a, b)
+    engine.shutdown()
