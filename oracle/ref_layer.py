@@ -41,7 +41,8 @@ from __future__ import annotations
 
 from typing import Any, Callable, Dict, List, Optional, Sequence, Set, Tuple
 
-from .ref_cache import RefEpipePrefillExtraCache, RefExpertWeightCache
+from .ref_cache import (RefEpipePrefillExtraCache, RefExpertWeightCache, RefTieredExpertWeightCache,
+                        ref_tiered_capacity_split)
 
 Segment = Tuple[int, int]  # (expert id, rows)
 
@@ -51,6 +52,9 @@ class RefConfig:
 
     def __init__(self, **kw: Any) -> None:
         self.capacity = 10
+        self.cache_policy = "lru"            # lru | tiered (:4843-4899)
+        self.prefetch_reserved = 0
+        self.prefetch_extra_capacity = 0
         self.planner_mode = "none"
         self.prefetch_top_m = 4
         self.pred_topk: Optional[int] = None
@@ -99,7 +103,13 @@ class RefLayer:
     def __init__(self, layer_idx: int, num_experts: int, top_k: int, cfg: RefConfig,
                  copy_done: Optional[Callable[[int], bool]] = None) -> None:
         self.layer_idx, self.num_experts, self.top_k, self.cfg = layer_idx, num_experts, top_k, cfg
-        self.cache = RefExpertWeightCache(cfg.capacity)
+        self.cache = None
+        if cfg.cache_policy == "tiered":
+            total, hot, reserved = ref_tiered_capacity_split(cfg.capacity, cfg.planner_mode == "rs_prefetch",
+                                                              cfg.prefetch_reserved, cfg.prefetch_extra_capacity)
+            self.cache = RefTieredExpertWeightCache(total, hot, reserved) if hot > 0 else RefExpertWeightCache(total)
+        else:
+            self.cache = RefExpertWeightCache(cfg.capacity)
         self.extra = RefEpipePrefillExtraCache(cfg.epipe_prefill_extra_cache_slots)
         self.copy_done = copy_done or (lambda eid: True)
         self.prefetched: Set[int] = set()        # _prefetched_ids_this_group
@@ -141,7 +151,8 @@ class RefLayer:
         resident = set(self.cache.resident_ids())
         if resident and resident.issubset(protect):
             protect = set()
-        self.cache.put(eid, ("w", eid), pinned=False, protect_ids=protect)
+        prefer_hot = int(self.freq.get(eid, 0)) >= 2   # _should_prefer_hot, :11223-11232
+        self.cache.put(eid, ("w", eid), pinned=False, prefer_hot=prefer_hot, protect_ids=protect)
 
     def maybe_wait_prefetch(self, eid: int) -> None:
         """:11176-11210."""
@@ -239,7 +250,8 @@ class RefLayer:
             self._count("epipe_fallback_no_missing")
             return None
         staged = missing[0][0]
-        can_insert = free > 0 and not (self.stage == "prefill" and not c.epipe_prefill_commit)
+        can_insert = (free > 0 and c.cache_policy != "tiered"
+                      and not (self.stage == "prefill" and not c.epipe_prefill_commit))   # :11964-11969
         use_transient = not can_insert
         if use_transient and not c.epipe_transient_staging:
             self._count("epipe_fallback_cache_full_no_temp")

@@ -248,8 +248,8 @@ class DistributedSparseMoeBlock(nn.Module):
         self.cache_policy = str(cache_policy).lower()
         if self.cache_policy not in ("lru", "lfu", "tiered"):
             raise ValueError(f"cache_policy must be lru|lfu|tiered, got {self.cache_policy}")
-        if self.cache_policy != "lru":
-            raise NotImplementedError(f"cache_policy={self.cache_policy} is not built; formal runs use lru")
+        if self.cache_policy == "lfu":
+            raise NotImplementedError("cache_policy=lfu is not built; use lru or tiered")
         if self.dtype not in (torch.bfloat16, torch.float32):
             raise ValueError(f"dtype must be bfloat16 or float32, got {self.dtype}")
         self.rs_group = int(rs_group)
@@ -296,6 +296,10 @@ class DistributedSparseMoeBlock(nn.Module):
             cfg = residency_config if residency_config is not None else ResidencyConfig.from_env(
                 capacity=int(expert_cache), planner_mode=self.planner_mode, prefetch_top_m=int(prefetch_top_m))
             cfg.capacity = int(expert_cache) if residency_config is None else cfg.capacity
+            if residency_config is None:
+                cfg.cache_policy = self.cache_policy
+            elif cfg.cache_policy != self.cache_policy and self.cache_policy != "lru":
+                cfg.cache_policy = self.cache_policy
             self.arena = HostExpertArena(expert_weights, H, I, self.dtype, pin=True)
             self._backend = _HipBackend(self)
             self.residency = LayerResidency(self.layer_idx, E, self.top_k, cfg, self._backend, self.metrics,

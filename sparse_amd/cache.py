@@ -267,3 +267,304 @@ class EpipePrefillExtraCache:
 
     def resident_nbytes(self) -> int:
         return sum(n for _, n in self._entries.values())
+
+
+class _Tier:
+    """One recency-ordered tier of the tiered cache (oldest first)."""
+
+    def __init__(self) -> None:
+        self.entries: Dict[int, CacheEntry] = {}
+
+    def __contains__(self, eid: int) -> bool:
+        return eid in self.entries
+
+    def __len__(self) -> int:
+        return len(self.entries)
+
+    def get(self, eid: int) -> Optional[CacheEntry]:
+        return self.entries.get(eid)
+
+    def to_mru(self, eid: int, entry: Optional[CacheEntry] = None) -> CacheEntry:
+        """(Re)insert ``eid`` as the most recently used entry."""
+        old = self.entries.pop(eid, None)
+        entry = entry if entry is not None else old
+        self.entries[eid] = entry
+        return entry
+
+    def to_lru(self, eid: int, entry: CacheEntry) -> None:
+        rest = self.entries
+        rest.pop(eid, None)
+        self.entries = {eid: entry}
+        self.entries.update(rest)
+
+    def pop(self, eid: int) -> Optional[CacheEntry]:
+        return self.entries.pop(eid, None)
+
+    def first(self, ok) -> Optional[int]:
+        for eid, entry in self.entries.items():
+            if ok(eid, entry):
+                return eid
+        return None
+
+
+class TieredExpertWeightCache:
+    """Hot / transient-demand / transient-prefetch tiers (reference :3953-4338,
+    ``--cache-policy tiered``).  Hot residents are never replaced by speculation; prefetch
+    fills its reserved area first, then replaces unpinned speculative residents, then spills
+    into the transient-demand tier.  Same methods, recency order and victim choice as the
+    reference, so identical operation sequences give identical contents."""
+
+    def __init__(self, capacity: int, hot_capacity: int, prefetch_reserved: int = 1) -> None:
+        self.capacity = int(capacity)
+        self.hot_capacity = max(0, min(int(hot_capacity), self.capacity))
+        self.transient_capacity = max(0, self.capacity - self.hot_capacity)
+        self.transient_prefetch_capacity = (
+            max(0, min(int(prefetch_reserved), self.transient_capacity)) if self.transient_capacity > 0 else 0)
+        self.transient_demand_capacity = max(0, self.transient_capacity - self.transient_prefetch_capacity)
+        self._hot, self._demand, self._prefetch = _Tier(), _Tier(), _Tier()
+        self._last_evicted_transient = False
+
+    def _tiers(self) -> Tuple[_Tier, _Tier, _Tier]:
+        return self._hot, self._demand, self._prefetch
+
+    def _find(self, eid: int) -> Tuple[Optional[_Tier], Optional[CacheEntry]]:
+        for tier in self._tiers():
+            entry = tier.get(eid)
+            if entry is not None:
+                return tier, entry
+        return None, None
+
+    # ---- eviction -------------------------------------------------------------
+    def _shrink(self, tier: _Tier, capacity: int, protect_ids: Optional[Set[int]]) -> Optional[int]:
+        """Evict from ``tier`` down to ``capacity``; the four victim classes of the plain
+        cache, in the same priority (:3978-4013).  Returns the last evicted id."""
+        protect = protect_ids or set()
+        evicted: Optional[int] = None
+        transient = False
+        while len(tier) > int(capacity):
+            victim = tier.first(lambda e, v: not v.pinned and int(e) not in protect and v.prefill_scp_transient)
+            if victim is None:
+                victim = tier.first(lambda e, v: not v.pinned and int(e) not in protect)
+            if victim is None:
+                victim = tier.first(lambda e, v: not v.pinned and v.prefill_scp_transient)
+            if victim is None:
+                victim = tier.first(lambda e, v: not v.pinned)
+            if victim is None:
+                victim = next(iter(tier.entries))
+            transient = bool(tier.pop(victim).prefill_scp_transient)
+            evicted = int(victim)
+        self._last_evicted_transient = transient
+        return evicted
+
+    def _insert_hot(self, eid: int, weights, protect_ids: Optional[Set[int]] = None) -> Optional[int]:
+        """:4021-4048: enter the hot tier; overflow demotes the oldest unprotected hot entry
+        to the transient-demand tier, which may evict in turn."""
+        if self.hot_capacity <= 0:
+            return self.put(eid, weights, pinned=False, prefer_hot=False, protect_ids=protect_ids)
+        self._demand.pop(eid)
+        self._prefetch.pop(eid)
+        self._hot.to_mru(eid, CacheEntry(weights, pinned=False, hot=True))
+        protect = protect_ids or set()
+        evicted: Optional[int] = None
+        while len(self._hot) > self.hot_capacity:
+            demote = self._hot.first(lambda e, v: not v.pinned and int(e) not in protect)
+            if demote is None:
+                demote = self._hot.first(lambda e, v: not v.pinned)
+            if demote is None:
+                demote = next(iter(self._hot.entries))
+            old = self._hot.pop(demote)
+            self._demand.to_mru(demote, CacheEntry(old.payload, pinned=False, hot=False,
+                                                   prefill_scp_transient=old.prefill_scp_transient))
+            evicted = self._shrink(self._demand, self.transient_demand_capacity, protect_ids)
+        return evicted
+
+    # ---- lookups ------------------------------------------------------------------
+    def get(self, expert_id: int):
+        tier, entry = self._find(expert_id)
+        if entry is None:
+            return None
+        tier.to_mru(expert_id)
+        return entry.payload
+
+    def peek(self, expert_id: int):
+        _tier, entry = self._find(int(expert_id))
+        return entry.payload if entry is not None else None
+
+    def has(self, expert_id: int) -> bool:
+        return any(expert_id in tier for tier in self._tiers())
+
+    def resident_ids(self) -> List[int]:
+        return [eid for tier in self._tiers() for eid in tier.entries]
+
+    def __len__(self) -> int:
+        return sum(len(tier) for tier in self._tiers())
+
+    def discard(self, expert_id: int) -> bool:
+        expert_id = int(expert_id)
+        return any([tier.pop(expert_id) is not None for tier in self._tiers()])
+
+    def unpin_all(self) -> None:
+        for tier in (self._prefetch, self._demand):
+            for entry in tier.entries.values():
+                entry.pinned = False
+
+    def unpin(self, expert_id: int) -> None:
+        for tier in (self._prefetch, self._demand):
+            entry = tier.get(expert_id)
+            if entry is not None:
+                entry.pinned = False
+
+    def clear(self) -> None:
+        for tier in self._tiers():
+            tier.entries.clear()
+        self._last_evicted_transient = False
+
+    def promote_hot(self, expert_id: int) -> None:
+        if expert_id in self._hot:
+            self._hot.to_mru(expert_id)
+            return
+        entry = self._demand.get(expert_id) or self._prefetch.get(expert_id)
+        if entry is not None:
+            self._insert_hot(expert_id, entry.payload)
+
+    def evictable_prefetch_ids(self, protect_ids: Optional[Set[int]] = None) -> List[int]:
+        protect = protect_ids or set()
+        return [int(e) for tier in (self._prefetch, self._demand) for e, v in tier.entries.items()
+                if not v.pinned and e not in protect]
+
+    def prefetch_free_slots(self) -> int:
+        """Only the reserved speculative area counts as free (:4145-4150)."""
+        return max(0, self.transient_prefetch_capacity - len(self._prefetch))
+
+    # ---- insertion -------------------------------------------------------------------
+    def put(self, expert_id: int, weights, pinned: bool = False, prefer_hot: bool = False,
+            protect_ids: Optional[Set[int]] = None, prefill_scp_transient: bool = False) -> Optional[int]:
+        """:4152-4202.  Pinned insertions go to the speculative tier, others to transient
+        demand, ``prefer_hot`` straight to the hot tier."""
+        if self.capacity <= 0:
+            return None
+        if prefer_hot and self.hot_capacity > 0:
+            return self._insert_hot(expert_id, weights, protect_ids=protect_ids)
+        entry = self._hot.get(expert_id)
+        if entry is not None:
+            entry.payload = weights
+            self._hot.to_mru(expert_id)
+            return None
+        entry = self._demand.get(expert_id)
+        if entry is not None:
+            entry.payload = weights
+            entry.pinned = entry.pinned or bool(pinned)
+            entry.prefill_scp_transient = bool(entry.prefill_scp_transient or prefill_scp_transient)
+            self._demand.to_mru(expert_id)
+            return None
+        entry = self._prefetch.get(expert_id)
+        if entry is not None:
+            entry.payload = weights
+            entry.pinned = entry.pinned or bool(pinned)
+            entry.prefill_scp_transient = bool(entry.prefill_scp_transient or prefill_scp_transient)
+            self._prefetch.to_mru(expert_id)
+            return self._shrink(self._prefetch, self.transient_prefetch_capacity, protect_ids)
+        fresh = CacheEntry(weights, pinned=bool(pinned), hot=False, prefill_scp_transient=bool(prefill_scp_transient))
+        if pinned:
+            self._prefetch.to_mru(expert_id, fresh)
+            return self._shrink(self._prefetch, self.transient_prefetch_capacity, protect_ids)
+        self._demand.to_mru(expert_id, fresh)
+        return self._shrink(self._demand, self.transient_demand_capacity, protect_ids)
+
+    def admit_prefetch(self, expert_id: int, weights, *, protect_ids: Optional[Set[int]] = None,
+                       preferred_victim: Optional[int] = None) -> bool:
+        """:4204-4270."""
+        if self.capacity <= 0:
+            return False
+        if expert_id in self._hot:
+            self._hot.to_mru(expert_id)
+            return True
+        for tier in (self._demand, self._prefetch):
+            entry = tier.get(expert_id)
+            if entry is not None:
+                entry.payload = weights
+                entry.pinned = True
+                tier.to_mru(expert_id)
+                return True
+        protect = protect_ids or set()
+        victim_hint = int(preferred_victim) if preferred_victim is not None else None
+
+        def place(tier: _Tier) -> bool:
+            tier.to_mru(expert_id, CacheEntry(weights, pinned=True, hot=False))
+            return True
+
+        for tier, room in ((self._prefetch, self.transient_prefetch_capacity),
+                           (self._demand, self.transient_demand_capacity)):
+            if len(tier) < room:
+                return place(tier)
+            victims = [e for e, v in tier.entries.items() if e not in protect and not v.pinned]
+            if victims:
+                tier.pop(victim_hint if victim_hint in victims else int(victims[0]))
+                return place(tier)
+        return False
+
+    # ---- prefill placement transients, request boundaries -----------------------------
+    def is_prefill_scp_transient(self, expert_id: int) -> bool:
+        _tier, entry = self._find(int(expert_id))
+        return bool(entry is not None and entry.prefill_scp_transient)
+
+    def last_evicted_was_prefill_scp_transient(self) -> bool:
+        return bool(self._last_evicted_transient)
+
+    def clear_prefill_scp_transient(self, expert_id: int) -> bool:
+        _tier, entry = self._find(int(expert_id))
+        if entry is not None and entry.prefill_scp_transient:
+            entry.prefill_scp_transient = False
+            return True
+        return False
+
+    def prefill_scp_transient_ids(self) -> List[int]:
+        return [int(e) for tier in self._tiers() for e, v in tier.entries.items() if v.prefill_scp_transient]
+
+    def reset_request_metadata(self, *, unpin: bool = True, demote_hot: bool = False) -> None:
+        if unpin:
+            self.unpin_all()
+        if demote_hot and len(self._hot):
+            for eid, entry in list(self._hot.entries.items()):
+                self._demand.to_mru(int(eid), CacheEntry(entry.payload, pinned=False, hot=False))
+            self._hot.entries.clear()
+            self._shrink(self._demand, self.transient_demand_capacity, set())
+
+    def demote_prefill_scp_transients(self) -> int:
+        ids = self.prefill_scp_transient_ids()
+        for eid in ids:
+            entry = self._hot.pop(eid) or self._prefetch.pop(eid) or self._demand.get(eid)
+            entry.hot = False
+            entry.pinned = False
+            self._demand.to_lru(eid, entry)
+        if ids:
+            self._shrink(self._demand, self.transient_demand_capacity, set())
+        return len(ids)
+
+    def occupancy(self) -> Dict[str, int]:
+        return {"capacity": self.capacity, "resident": len(self), "hot": len(self._hot),
+                "transient_demand": len(self._demand), "transient_prefetch": len(self._prefetch),
+                "prefill_scp_transient": len(self.prefill_scp_transient_ids())}
+
+
+def tiered_capacity_split(expert_cache: int, prefetch_enabled: bool, prefetch_reserved: int = 0,
+                          prefetch_extra_capacity: int = 0) -> Tuple[int, int, int]:
+    """``(total_capacity, hot_capacity, prefetch_reserved)`` of a ``--cache-policy tiered``
+    layer (reference :4843-4890).  ``hot_capacity == 0`` means "use the plain LRU"."""
+    base = int(expert_cache)
+    extra = max(0, int(prefetch_extra_capacity)) if prefetch_enabled else 0
+    total = base + extra
+    if base <= 1:
+        return total, 0, 0
+    if base >= 12:
+        transient = 4
+    elif base >= 8:
+        transient = 3
+    else:
+        transient = max(2, base // 3)
+    transient = min(transient, max(1, base - 1))
+    reserved = max(0, int(prefetch_reserved)) if prefetch_enabled else 0
+    if reserved > 0 and extra <= 0:
+        transient = min(max(1, base - 1), transient + reserved)
+    reserved = min(reserved, max(0, transient))
+    return total, max(1, base - transient), reserved

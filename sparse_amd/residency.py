@@ -20,7 +20,7 @@ import os
 from dataclasses import dataclass, field
 from typing import Any, Callable, Dict, List, Optional, Sequence, Set, Tuple
 
-from .cache import EpipePrefillExtraCache, ExpertWeightCache
+from .cache import TieredExpertWeightCache, tiered_capacity_split, EpipePrefillExtraCache, ExpertWeightCache
 from .context import Metrics
 
 Segment = Tuple[int, int]  # (expert id, routed rows)
@@ -52,6 +52,9 @@ class ResidencyConfig:
     capacity: int = 10
     staging_slots: int = 4
     staging_pool_slots: int = 0            # slots reserved for the bounded RS staging engine
+    cache_policy: str = "lru"              # lru | tiered (--cache-policy)
+    prefetch_reserved: int = 0             # SPARSE_PREFETCH_RESERVED (tiered only)
+    prefetch_extra_capacity: int = 0       # SPARSE_PREFETCH_EXTRA_CAPACITY (tiered only)
     planner_mode: str = "none"            # none | rs_prefetch
     prefetch_top_m: int = 4
     pred_topk: Optional[int] = None        # SPARSE_RS_PREFETCH_PRED_TOPK
@@ -100,6 +103,8 @@ class ResidencyConfig:
     def from_env(cls, **overrides) -> "ResidencyConfig":
         c = cls()
         c.staging_slots = max(1, _env_int("SPARSE_HIP_STAGING_SLOTS", c.staging_slots))
+        c.prefetch_reserved = max(0, _env_int("SPARSE_PREFETCH_RESERVED", 0))
+        c.prefetch_extra_capacity = max(0, _env_int("SPARSE_PREFETCH_EXTRA_CAPACITY", 0))
         raw = os.environ.get("SPARSE_RS_PREFETCH_PRED_TOPK", "").strip()
         c.pred_topk = int(raw) if raw else None
         c.rs_policy = str(os.environ.get("SPARSE_RS_PREFETCH_POLICY", "default") or "default").strip().lower()
@@ -185,9 +190,21 @@ class LayerResidency:
         self.backend = backend
         self.metrics = metrics if metrics is not None else Metrics()
         self.expert_bytes = int(expert_bytes)
-        self.cache = ExpertWeightCache(int(config.capacity))
+        total_capacity = int(config.capacity)
+        self.cache: Any = None
+        if str(config.cache_policy) == "tiered":
+            # hot / transient-demand / transient-prefetch split of the constructor (reference :4843-4899)
+            total_capacity, hot, reserved = tiered_capacity_split(
+                int(config.capacity), config.planner_mode == "rs_prefetch", int(config.prefetch_reserved),
+                int(config.prefetch_extra_capacity))
+            if hot > 0:
+                self.cache = TieredExpertWeightCache(total_capacity, hot_capacity=hot, prefetch_reserved=reserved)
+        elif str(config.cache_policy) != "lru":
+            raise NotImplementedError(f"cache_policy={config.cache_policy} is not built (lru | tiered)")
+        if self.cache is None:
+            self.cache = ExpertWeightCache(total_capacity)
         self.extra_cache = EpipePrefillExtraCache(int(config.epipe_prefill_extra_cache_slots))
-        self.num_slots = max(0, int(config.capacity)) + max(1, int(config.staging_slots)) + \
+        self.num_slots = max(0, total_capacity) + max(1, int(config.staging_slots)) + \
             max(0, int(config.epipe_prefill_extra_cache_slots))
         # slots of the bounded RS staging pool sit after the ordinary ones and never enter the free list
         self._pool_slots: List[int] = list(range(self.num_slots, self.num_slots + max(0, int(config.staging_pool_slots))))
@@ -301,6 +318,7 @@ class LayerResidency:
             self.last_used_decode_step[int(eid)] = int(self.call_id)
         if self.access_freq[eid] >= 2:
             self.cache.promote_hot(eid)
+            self._sync_slots()   # entering the hot tier of a tiered cache may push another expert out
 
     def _sync_slots(self) -> None:
         """Release the slot of every expert the cache no longer holds."""
@@ -318,8 +336,16 @@ class LayerResidency:
             self._retired.append(slot)
             return
         protect = self._protect_with_fallback(eid)
-        self.cache.put(int(eid), slot, pinned=False, protect_ids=protect)
-        self._slot_of[int(eid)] = slot
+        # a repeatedly used expert enters the hot tier of a tiered cache (reference :11223-11232)
+        prefer_hot = int(self.access_freq.get(int(eid), 0)) >= 2
+        self.cache.put(int(eid), slot, pinned=False, prefer_hot=prefer_hot, protect_ids=protect)
+        if self.cache.has(int(eid)):
+            self._slot_of[int(eid)] = slot
+        else:
+            # a full tier whose other entries are all pinned or protected gives the newcomer up at
+            # once: its slot then only lives until the batch that uses it is launched
+            self._pending_slots.add(slot)
+            self._retired.append(slot)
         self._sync_slots()
 
     def _record_cached_use(self, eid: int, wait_prefetch: bool) -> None:
@@ -330,6 +356,7 @@ class LayerResidency:
             self.prefetch_used_ids.add(eid)
             self.cache.unpin(eid)
             self.cache.promote_hot(eid)
+            self._sync_slots()
         else:
             self._event("hit", eid)
         if wait_prefetch:
@@ -450,7 +477,8 @@ class LayerResidency:
             self._fallback("epipe_fallback_no_missing")
             return None
         staged_eid = missing[0][0]
-        can_insert = free_cache_slots > 0 and not (stage == "prefill" and not cfg.epipe_prefill_commit)
+        can_insert = (free_cache_slots > 0 and cfg.cache_policy != "tiered"
+                      and not (stage == "prefill" and not cfg.epipe_prefill_commit))
         use_transient = not can_insert
         if use_transient:
             if not cfg.epipe_transient_staging:

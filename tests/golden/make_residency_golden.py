@@ -3,7 +3,9 @@
 
 Runs ONLY in the build container, where the reference checkout is mounted at
 /root/reference; the fixtures it writes (``cache_ops.json``, ``rs_plan.json``) are what the
-tests read, so nothing at test time touches the reference.
+tests read, so nothing at test time touches the reference.  ``tiered_ops.json`` holds the
+same kind of traces for ``TieredExpertWeightCache`` (utils/eval_core.py:3953-4338) and the
+capacity split of a tiered layer (:4843-4890).
 
 The reference's classes and methods are taken out of ``utils/eval_core.py`` by name with
 ``ast`` (the technique of the reference's own tests, tests/test_rs_staging.py:18-34) and
@@ -45,7 +47,8 @@ BLOCK_METHODS = (
 def extract():
     import torch
     tree = ast.parse(REF.read_text())
-    classes = [n for n in tree.body if isinstance(n, ast.ClassDef) and n.name in ("CacheEntry", "ExpertWeightCache")]
+    classes = [n for n in tree.body if isinstance(n, ast.ClassDef)
+               and n.name in ("CacheEntry", "ExpertWeightCache", "TieredExpertWeightCache")]
     block = next(n for n in tree.body if isinstance(n, ast.ClassDef) and n.name == "DistributedSparseMoeBlock")
     methods = [n for n in block.body if isinstance(n, ast.FunctionDef) and n.name in BLOCK_METHODS]
     future = ast.ImportFrom(module="__future__", names=[ast.alias(name="annotations")], level=0)
@@ -168,6 +171,84 @@ def plan_cases(ns, rng: random.Random, n_cases: int = 200):
     return cases
 
 
+def tiered_cases(ns, rng: random.Random, n_cases: int = 24, n_ops: int = 150):
+    """Random operation sequences on the reference's ``TieredExpertWeightCache``."""
+    cases = []
+    for case in range(n_cases):
+        cap = rng.choice([2, 3, 4, 6, 8, 12])
+        hot = rng.randrange(0, cap + 1)
+        reserved = rng.randrange(0, 3)
+        universe = rng.choice([8, 12, 20])
+        cache = ns["TieredExpertWeightCache"](cap, hot_capacity=hot, prefetch_reserved=reserved)
+        ops, results = [], []
+        for _ in range(n_ops):
+            op = rng.choices(["get", "put", "admit", "discard", "unpin", "unpin_all", "promote", "evictable", "has",
+                              "peek", "reset", "demote_transients", "clear_transient"],
+                             weights=[30, 30, 14, 4, 4, 2, 8, 5, 3, 3, 1, 2, 2])[0]
+            eid = rng.randrange(universe)
+            protect = sorted(rng.sample(range(universe), rng.randrange(0, 4))) if rng.random() < 0.4 else []
+            if op == "get":
+                r, rec = cache.get(eid), ["get", eid]
+            elif op == "put":
+                pinned, transient, hotp = rng.random() < 0.2, rng.random() < 0.15, rng.random() < 0.25
+                r = cache.put(eid, "w%d" % eid, pinned=pinned, prefer_hot=hotp, protect_ids=set(protect),
+                              prefill_scp_transient=transient)
+                rec = ["put", eid, pinned, transient, hotp, protect]
+            elif op == "admit":
+                victim = rng.randrange(universe) if rng.random() < 0.6 else None
+                r = cache.admit_prefetch(eid, "p%d" % eid, protect_ids=set(protect), preferred_victim=victim)
+                rec = ["admit", eid, victim, protect]
+            elif op == "discard":
+                r, rec = cache.discard(eid), ["discard", eid]
+            elif op == "unpin":
+                r, rec = cache.unpin(eid), ["unpin", eid]
+            elif op == "unpin_all":
+                r, rec = cache.unpin_all(), ["unpin_all"]
+            elif op == "promote":
+                r, rec = cache.promote_hot(eid), ["promote", eid]
+            elif op == "evictable":
+                r, rec = cache.evictable_prefetch_ids(set(protect)), ["evictable", protect]
+            elif op == "has":
+                r, rec = cache.has(eid), ["has", eid]
+            elif op == "peek":
+                r, rec = cache.peek(eid), ["peek", eid]
+            elif op == "reset":
+                demote = rng.random() < 0.5
+                r, rec = cache.reset_request_metadata(unpin=True, demote_hot=demote), ["reset", demote]
+            elif op == "demote_transients":
+                r, rec = cache.demote_prefill_scp_transients(), ["demote_transients"]
+            else:
+                r, rec = cache.clear_prefill_scp_transient(eid), ["clear_transient", eid]
+            ops.append(rec)
+            occ = cache.occupancy()
+            results.append([r, list(cache.resident_ids()), cache.prefetch_free_slots(),
+                            [occ["hot"], occ["transient_demand"], occ["transient_prefetch"], occ["prefill_scp_transient"]],
+                            bool(cache.last_evicted_was_prefill_scp_transient())])
+        cases.append(dict(capacity=cap, hot=hot, reserved=reserved, ops=ops, results=results))
+    return cases
+
+
+def split_cases():
+    """The capacity split of a tiered layer is inline code of the block's constructor
+    (utils/eval_core.py:4843-4890); those lines are run as they stand against a stub."""
+    lines = REF.read_text().splitlines()[4842:4890]
+    indent = len(lines[0]) - len(lines[0].lstrip())
+    body = "\n".join(line[indent:] if line.strip() else "" for line in lines)
+    code = compile(body, str(REF), "exec")
+    cases = []
+    for cache in range(0, 21):
+        for planner in ("none", "rs_prefetch"):
+            for reserved in (0, 1, 2, 5):
+                for extra in (0, 2):
+                    env = {"SPARSE_PREFETCH_RESERVED": str(reserved), "SPARSE_PREFETCH_EXTRA_CAPACITY": str(extra)}
+                    ns = dict(self=NS(planner_mode=planner), expert_cache=cache, os=NS(environ=env), int=int, max=max,
+                              min=min)
+                    exec(code, ns)
+                    cases.append([cache, planner == "rs_prefetch", reserved, extra,
+                                  [int(ns["total_capacity"]), int(ns["hot_capacity"]), int(ns["prefetch_reserved"])]])
+    return cases
+
+
 def main() -> None:
     if not REF.exists():
         sys.exit("the reference checkout is not mounted; fixtures are only written in the build container")
@@ -175,7 +256,8 @@ def main() -> None:
     rng = random.Random(20261125)
     (OUT / "cache_ops.json").write_text(json.dumps(cache_cases(ns, rng)))
     (OUT / "rs_plan.json").write_text(json.dumps(plan_cases(ns, rng)))
-    print("wrote", OUT / "cache_ops.json", OUT / "rs_plan.json")
+    (OUT / "tiered_ops.json").write_text(json.dumps(dict(ops=tiered_cases(ns, rng), split=split_cases())))
+    print("wrote", OUT / "cache_ops.json", OUT / "rs_plan.json", OUT / "tiered_ops.json")
 
 
 if __name__ == "__main__":

@@ -216,3 +216,104 @@ def test_product_and_oracle_agree_on_random_operations():
             assert a.resident_ids() == b.resident_ids()
             assert a.evictable_prefetch_ids(protect) == b.evictable_prefetch_ids(protect)
             assert a.prefill_scp_transient_ids() == b.prefill_scp_transient_ids()
+
+
+# ---------------------------------------------------------------------------- tiered cache
+def _tiered_impls():
+    from oracle.ref_cache import RefTieredExpertWeightCache
+    from sparse_amd.cache import TieredExpertWeightCache
+    return {"product": TieredExpertWeightCache, "oracle": RefTieredExpertWeightCache}
+
+
+def _tiered_counts(cache):
+    if hasattr(cache, "occupancy_counts"):
+        return cache.occupancy_counts()
+    occ = cache.occupancy()
+    return [occ["hot"], occ["transient_demand"], occ["transient_prefetch"], occ["prefill_scp_transient"]]
+
+
+def _tiered_flag(cache):
+    fn = getattr(cache, "last_evicted_was_prefill_scp_transient", None)
+    return bool(fn()) if fn is not None else bool(cache.last_evicted_transient)
+
+
+def _apply_tiered(cache, rec):
+    op = rec[0]
+    if op == "get":
+        return cache.get(rec[1])
+    if op == "put":
+        return cache.put(rec[1], "w%d" % rec[1], pinned=rec[2], prefer_hot=rec[4], protect_ids=set(rec[5]),
+                         prefill_scp_transient=rec[3])
+    if op == "admit":
+        return cache.admit_prefetch(rec[1], "p%d" % rec[1], protect_ids=set(rec[3]), preferred_victim=rec[2])
+    if op == "discard":
+        return cache.discard(rec[1])
+    if op == "unpin":
+        return cache.unpin(rec[1])
+    if op == "unpin_all":
+        return cache.unpin_all()
+    if op == "promote":
+        return cache.promote_hot(rec[1])
+    if op == "evictable":
+        return cache.evictable_prefetch_ids(set(rec[1]))
+    if op == "has":
+        return cache.has(rec[1])
+    if op == "peek":
+        return cache.peek(rec[1])
+    if op == "reset":
+        return cache.reset_request_metadata(unpin=True, demote_hot=rec[1])
+    if op == "demote_transients":
+        return cache.demote_prefill_scp_transients()
+    if op == "clear_transient":
+        return cache.clear_prefill_scp_transient(rec[1])
+    raise AssertionError(op)
+
+
+@pytest.mark.parametrize("impl", ["product", "oracle"])
+def test_tiered_cache_golden_traces_from_the_reference_class(impl):
+    """Every operation of every recorded sequence: return value, resident order (hot, then
+    transient demand, then transient prefetch), free speculative slots, tier occupancy and
+    the last-evicted flag equal what the reference's own class produced."""
+    import json
+    from pathlib import Path
+    data = json.loads((Path(__file__).parent / "golden" / "tiered_ops.json").read_text())
+    cls = _tiered_impls()[impl]
+    assert len(data["ops"]) >= 20
+    for case in data["ops"]:
+        cache = cls(case["capacity"], hot_capacity=case["hot"], prefetch_reserved=case["reserved"])
+        for step, (rec, want) in enumerate(zip(case["ops"], case["results"])):
+            got = _apply_tiered(cache, rec)
+            state = [got, list(cache.resident_ids()), cache.prefetch_free_slots(), _tiered_counts(cache),
+                     _tiered_flag(cache)]
+            assert state == want, (case["capacity"], case["hot"], case["reserved"], step, rec)
+
+
+def test_tiered_capacity_split_matches_the_reference_constructor():
+    import json
+    from pathlib import Path
+    from oracle.ref_cache import ref_tiered_capacity_split
+    from sparse_amd.cache import tiered_capacity_split
+    data = json.loads((Path(__file__).parent / "golden" / "tiered_ops.json").read_text())
+    assert len(data["split"]) > 300
+    for cache, planner, reserved, extra, want in data["split"]:
+        assert list(tiered_capacity_split(cache, planner, reserved, extra)) == want, (cache, planner, reserved, extra)
+        assert list(ref_tiered_capacity_split(cache, planner, reserved, extra)) == want
+
+
+def test_tiered_cache_speculation_never_displaces_hot_residents():
+    """Closed-form property of the design (:3954-3962): whatever is admitted by prefetch, an
+    expert in the hot tier stays resident and hot."""
+    import random
+    from sparse_amd.cache import TieredExpertWeightCache
+    rng = random.Random(5)
+    for _ in range(50):
+        cache = TieredExpertWeightCache(8, hot_capacity=4, prefetch_reserved=1)
+        hot = rng.sample(range(32), 4)
+        for eid in hot:
+            cache.put(eid, eid, prefer_hot=True)
+        for _ in range(60):
+            cache.admit_prefetch(rng.randrange(32, 64), "p", preferred_victim=rng.choice(hot))
+            if rng.random() < 0.3:
+                cache.unpin_all()
+        assert all(cache.has(eid) for eid in hot) and cache.occupancy()["hot"] == 4
+        assert len(cache) <= 8

@@ -111,6 +111,8 @@ def _replay_oracle(record, cfg, capacity):
     ("rr", {}, False), ("rs", {}, False), ("epipe", {}, False), ("rs-epipe", {}, False), ("sparse", {}, False),
     ("rs", dict(formal_thresholds=False), False),
     ("epipe", dict(epipe_prefill_enable=True), True),
+    ("rs", dict(cache_policy="tiered", prefetch_reserved=1, formal_thresholds=False), False),
+    ("rs-epipe", dict(cache_policy="tiered", prefetch_reserved=1, formal_thresholds=False), False),
 ])
 def test_offloaded_methods_match_resident_values_and_oracle_events(device, method, overrides, prefill_first):
     from sparse_amd.methods import residency_config

@@ -309,6 +309,14 @@ METHOD_CASES = [
     ("epipe", dict(overrides=dict(epipe_sort_ready_by_work=True))),
     ("epipe", dict(prefill_first=True, overrides=dict(epipe_prefill_enable=True, epipe_prefill_extra_cache_slots=2,
                                                       epipe_prefill_commit=False))),
+    # --cache-policy tiered: hot / transient tiers, prefetch into its reserved area first
+    ("rr", dict(capacity=8, E=24, T=8, overrides=dict(cache_policy="tiered"))),
+    ("rs", dict(capacity=8, E=24, T=8, top_m=4, overrides=dict(cache_policy="tiered", prefetch_reserved=1))),
+    ("rs", dict(capacity=12, E=60, K=4, T=8, top_m=8, formal=False,
+                overrides=dict(cache_policy="tiered", prefetch_reserved=2))),
+    ("epipe", dict(capacity=6, E=24, T=8, overrides=dict(cache_policy="tiered"))),
+    ("rs-epipe", dict(capacity=8, E=24, T=8, top_m=4, formal=False,
+                      overrides=dict(cache_policy="tiered", prefetch_reserved=1))),
 ]
 
 
