@@ -248,8 +248,6 @@ class DistributedSparseMoeBlock(nn.Module):
         self.cache_policy = str(cache_policy).lower()
         if self.cache_policy not in ("lru", "lfu", "tiered"):
             raise ValueError(f"cache_policy must be lru|lfu|tiered, got {self.cache_policy}")
-        if self.cache_policy == "lfu":
-            raise NotImplementedError("cache_policy=lfu is not built; use lru or tiered")
         if self.dtype not in (torch.bfloat16, torch.float32):
             raise ValueError(f"dtype must be bfloat16 or float32, got {self.dtype}")
         self.rs_group = int(rs_group)

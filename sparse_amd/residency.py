@@ -199,8 +199,10 @@ class LayerResidency:
                 int(config.prefetch_extra_capacity))
             if hot > 0:
                 self.cache = TieredExpertWeightCache(total_capacity, hot_capacity=hot, prefetch_reserved=reserved)
-        elif str(config.cache_policy) != "lru":
-            raise NotImplementedError(f"cache_policy={config.cache_policy} is not built (lru | tiered)")
+        elif str(config.cache_policy) not in ("lru", "lfu"):
+            # lfu shares the plain cache with lru (reference :4840-4841); it only lowers the
+            # prefer-hot threshold, which the plain cache ignores
+            raise ValueError(f"cache_policy must be lru|lfu|tiered, got {config.cache_policy}")
         if self.cache is None:
             self.cache = ExpertWeightCache(total_capacity)
         self.extra_cache = EpipePrefillExtraCache(int(config.epipe_prefill_extra_cache_slots))
