@@ -92,11 +92,14 @@ class SparseContext:
         cls.routing_cache = {}
 
     @classmethod
-    def set_rs_bank(cls, modules: List[Any]) -> None:
-        """``modules[l]`` (or None) is the predictor of layer l's experts from layer l-1."""
+    def set_rs_bank(cls, modules: List[Any], source_layers: Optional[List[int]] = None) -> None:
+        """``modules[l]`` (or None) is the predictor of layer l's experts from the input of
+        layer ``source_layers[l]`` (default l-1; a layer only prefetches for the next one
+        when that entry names it)."""
         cls.rs_bank = list(modules)
         cls.rs_bank_layout = "next_layer"
-        cls.rs_bank_source_layers = [l - 1 for l in range(len(modules))]
+        cls.rs_bank_source_layers = (
+            [int(s) for s in source_layers] if source_layers is not None else [l - 1 for l in range(len(modules))])
 
     @classmethod
     def finalize_prefetch_all(cls) -> None:

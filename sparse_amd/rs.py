@@ -8,7 +8,9 @@ in fp32 through PyTorch; only its top-k leaves the device.
 """
 from __future__ import annotations
 
-from typing import List, Optional
+import os
+import re
+from typing import Any, Dict, List, Optional, Tuple
 
 import torch
 from torch import nn
@@ -29,6 +31,37 @@ class RoutingScoutMLP(nn.Module):
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         return self.mlp(x.reshape(-1, x.shape[-1]))
+
+
+class _ResidualUnit(nn.Module):
+    def __init__(self, width: int, dropout: float) -> None:
+        super().__init__()
+        self.net = nn.Sequential(
+            nn.LayerNorm(width), nn.Linear(width, 2 * width), nn.GELU(), nn.Dropout(dropout),
+            nn.Linear(2 * width, width), nn.Dropout(dropout))
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return x + self.net(x)
+
+
+class RoutingScoutResidualMLP(nn.Module):
+    """The deeper predictor (``model_type = next_layer_residual_logits_rs``): LayerNorm +
+    Linear + GELU stem, pre-norm residual units twice as wide inside, LayerNorm, Linear head,
+    softmax.  Submodule names (``input``, ``blocks.N.net``, ``out_norm``, ``head``) follow
+    utils/eval_core.py:3419-3464 so that its checkpoints load by key."""
+
+    def __init__(self, input_dim: int, num_experts: int, hidden_dim: int = 1024, num_hidden_layers: int = 3,
+                 dropout: float = 0.05) -> None:
+        super().__init__()
+        self.input = nn.Sequential(nn.LayerNorm(input_dim), nn.Linear(input_dim, hidden_dim), nn.GELU(),
+                                   nn.Dropout(dropout))
+        self.blocks = nn.Sequential(*[_ResidualUnit(hidden_dim, dropout) for _ in range(max(0, int(num_hidden_layers)))])
+        self.out_norm = nn.LayerNorm(hidden_dim)
+        self.head = nn.Linear(hidden_dim, num_experts)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        h = self.blocks(self.input(x.reshape(-1, x.shape[-1])))
+        return torch.softmax(self.head(self.out_norm(h)), dim=-1)
 
 
 def random_init_bank(num_layers: int, hidden: int, num_experts: int, hidden_dim: int = 512, seed: int = 0,
@@ -94,3 +127,85 @@ def informed_bank(gate_weights: List[Optional[torch.Tensor]], hidden_dim: int = 
             p.requires_grad_(False)
         bank.append(module.to(device) if device is not None else module)
     return bank
+
+
+# ---- checkpoint directories -------------------------------------------------------------
+_CKPT_NAME = re.compile(r"(rs|cv)_l(\d+)_inL(-?\d+)\.pth")
+
+
+def _state_dict_of(payload: Any) -> Dict[str, torch.Tensor]:
+    if isinstance(payload, dict):
+        for key in ("state_dict", "model_state_dict"):
+            if isinstance(payload.get(key), dict):
+                return payload[key]
+        if payload and all(torch.is_tensor(v) for v in payload.values()):
+            return payload
+    raise RuntimeError(f"Cannot extract state_dict from payload type={type(payload)}")
+
+
+def module_from_payload(payload: Any, fallback_input_dim: int, fallback_num_experts: int) -> nn.Module:
+    """Build the predictor a checkpoint payload describes (utils/eval_core.py:3490-3550):
+    ``model_type`` picks the class, a bare state dict is a 1024-wide ``RoutingScoutMLP``.
+    Only predictors of routing probabilities read from the layer's hidden state are built;
+    cache-value checkpoints and the ``hidden_router_topk`` feature raise."""
+    meta = payload if isinstance(payload, dict) else {}
+    if meta.get("task", "") == "cache_value_rs":
+        raise NotImplementedError("cache_value_rs checkpoints are not supported")
+    feature = str(meta.get("feature_mode", "hidden"))
+    if feature != "hidden":
+        raise NotImplementedError(f"RS feature_mode {feature!r} is not supported")
+    kind = meta.get("model_type", "")
+    input_dim = int(meta.get("input_dim", fallback_input_dim))
+    num_experts = int(meta.get("num_experts", fallback_num_experts))
+    hidden_dim = int(meta.get("hidden_dim", 1024))
+    if kind == "next_layer_residual_logits_rs":
+        module: nn.Module = RoutingScoutResidualMLP(input_dim, num_experts, hidden_dim=hidden_dim,
+                                                    num_hidden_layers=int(meta.get("num_hidden_layers", 3)))
+    elif kind == "independent_light_logits_rs":
+        module = RoutingScoutMLP(input_dim, num_experts, hidden_dim=hidden_dim)
+    else:
+        module = RoutingScoutMLP(fallback_input_dim, fallback_num_experts, hidden_dim=1024)
+    module.load_state_dict(_state_dict_of(payload), strict=True)
+    return module
+
+
+def load_rs_bank(rs_dir: str, num_layers: int, hidden_dim: int, num_experts: int,
+                 device: Optional[torch.device] = None,
+                 require_complete: bool = True) -> Tuple[List[nn.Module], List[int], List[str]]:
+    """Load a directory of next-layer predictors, ``rs_l{L}_inL{L-1}.pth`` for target layer L
+    (utils/eval_core.py:3553-3658).  Returns ``(modules, source_layers, missing)`` with one
+    module per layer.  Layers below the first target present are never predicted, so their
+    absence is not an error and they get an untrained placeholder, as do other absent layers
+    when ``require_complete`` is false; with it true an absent layer raises.  Files are read
+    with ``weights_only=True``."""
+    names = {}
+    for name in sorted(os.listdir(rs_dir)):
+        m = _CKPT_NAME.fullmatch(name)
+        if m and int(m.group(2)) == int(m.group(3)) + 1:
+            names.setdefault(int(m.group(2)), {})[m.group(1)] = name
+    if not names:
+        raise NotImplementedError(f"{rs_dir} holds no next-layer predictors (rs_l{{L}}_inL{{L-1}}.pth)")
+    first_target = min(names)
+    modules: List[nn.Module] = []
+    sources: List[int] = []
+    missing: List[str] = []
+    for layer in range(int(num_layers)):
+        found = names.get(layer, {})
+        name = found.get("cv") or found.get("rs")
+        if name is None:
+            if layer >= first_target:
+                missing.append(f"[L{layer}] tried: cv_l{layer}_inL{layer - 1}.pth, rs_l{layer}_inL{layer - 1}.pth")
+            module: nn.Module = RoutingScoutMLP(hidden_dim, num_experts, hidden_dim=1024)
+            source = layer - 1
+        else:
+            payload = torch.load(os.path.join(rs_dir, name), map_location="cpu", weights_only=True)
+            module = module_from_payload(payload, hidden_dim, num_experts)
+            source = int(payload.get("source_layer", layer - 1)) if isinstance(payload, dict) else layer - 1
+        module = module.to(torch.float32).eval()
+        for p in module.parameters():
+            p.requires_grad_(False)
+        modules.append(module.to(device) if device is not None else module)
+        sources.append(source)
+    if require_complete and missing:
+        raise RuntimeError("RS checkpoint set incomplete:\n" + "\n".join(missing[:32]))
+    return modules, sources, missing
