@@ -30,9 +30,11 @@ Pinned by (tests/test_residency.py and tests/golden/):
   demand path        reference test tests/test_rs_staging.py:74-92 (in-flight prefetch hit:
                      exactly one wait, ``is_prefetch_hit``, no second load) restated;
                      textbook LRU replay.
-  EPIPE executors    parity unpinned against executed reference code: all four executors
-                     return None unless ``device.type == "cuda"`` (:11881, :12184), so they
-                     cannot run in a GPU-less container.  Pinned only by restatement plus
+  EPIPE executors    (upfront scan, RS residual scan, bounded ready buffer, miss-triggered
+                     look-ahead) parity unpinned against executed reference code: all four
+                     return None unless ``device.type == "cuda"`` (:11881, :12184, :12530,
+                     :12860), so they cannot run in a GPU-less container.  Pinned only by
+                     restatement, hand-made walk-throughs of each executor, and
                      invariants: every segment computed exactly once, the staged expert
                      counts exactly one miss, resident experts run before the wait,
                      outputs equal the plain path.
@@ -93,6 +95,15 @@ class RefConfig:
         self.epipe_rs_gate_min_triggers = 1
         self.epipe_rs_gate_skip_steps = 8
         self.epipe_prefill_extra_cache_slots = 0
+        self.epipe_prefill_mark_transient = True      # default follows the default prefill policy (:5012-5016)
+        self.epipe_promote_transient_on_decode_hit = True
+        self.epipe_rs_buffer_max_groups = 4
+        self.epipe_rs_buffer_max_items = 32
+        self.epipe_lookahead_experts = 4
+        self.epipe_lookahead_min_ready_items = 64
+        self.epipe_prefill_lookahead_min_ready_items = 256
+        self.epipe_decode_rs_commit = True
+        self.epipe_decode_no_rs_commit = True
         for k, v in kw.items():
             if not hasattr(self, k):
                 raise ValueError(f"unknown option {k}")
@@ -144,15 +155,19 @@ class RefLayer:
         if self.freq[eid] >= 2:
             self.cache.promote_hot(eid)
 
-    def cache_put_guarded(self, eid: int) -> None:
-        """:5985-6022 with :5940-5951."""
+    def cache_put_guarded(self, eid: int, transient: bool = False) -> None:
+        """:5985-6022 with :5940-5951.  ``transient`` is the ``prefill_scp_transient`` mark; at
+        world size 1 only EPIPE prefill commits set it (:12083-12089, :13103-13109)."""
         protect = self._protect_ttl()
         protect.discard(eid)
         resident = set(self.cache.resident_ids())
         if resident and resident.issubset(protect):
             protect = set()
         prefer_hot = int(self.freq.get(eid, 0)) >= 2   # _should_prefer_hot, :11223-11232
-        self.cache.put(eid, ("w", eid), pinned=False, prefer_hot=prefer_hot, protect_ids=protect)
+        self.cache.put(eid, ("w", eid), pinned=False, prefer_hot=prefer_hot, protect_ids=protect,
+                       prefill_scp_transient=bool(transient))
+        if transient:
+            self._count("prefill_scp_transient_load_count")
 
     def maybe_wait_prefetch(self, eid: int) -> None:
         """:11176-11210."""
@@ -164,7 +179,12 @@ class RefLayer:
             self._count("prefetch_completed")
 
     def record_cached_use(self, eid: int, wait: bool) -> None:
-        """:11395-11412 and :11652-11670."""
+        """:11395-11412 and :11652-11670; first the transient upgrade of :11324-11336."""
+        if (self.stage == "decode" and self.cfg.epipe_promote_transient_on_decode_hit
+                and self.cache.is_prefill_scp_transient(eid)):
+            self._count("prefill_scp_transient_hit_count")
+            if self.cache.clear_prefill_scp_transient(eid):
+                self._count("prefill_scp_transient_promote_count")
         if eid in self.prefetched:
             self.trace.append(("prefetch_hit", eid))
             self.used.add(eid)
@@ -216,14 +236,15 @@ class RefLayer:
                 result = None
             elif self.stage == "decode" and rs_active and c.epipe_decode_rs_mode == "residual_scan":
                 result = self.epipe_rs_residual_scan(segments)
-            elif self.stage == "decode" and rs_active:
-                raise NotImplementedError("buffered / late_only / demand_only are not restated")
-            elif self.stage == "decode" and c.epipe_mode != "miss_triggered":
+            elif self.stage == "decode" and rs_active and c.epipe_decode_rs_mode in (
+                    "buffered", "late_only", "demand_only"):
+                result = self.epipe_rs_buffered(segments)
+            elif self.stage == "decode" and not rs_active and c.epipe_mode != "miss_triggered":
                 result = self.epipe_upfront_scan(segments)
             elif c.epipe_mode == "upfront_scan":
                 result = self.epipe_upfront_scan(segments)
             else:
-                raise NotImplementedError("miss_triggered is not restated")
+                result = self.epipe_miss_triggered(segments)
         if result is None:
             for eid, _ in segments:  # ascending expert id, :13340-13357
                 self.compute(eid)
@@ -270,7 +291,7 @@ class RefLayer:
             if len(self.cache.resident_ids()) < self.cache.capacity:
                 if self.stage == "prefill":
                     self.on_demand_access(staged)
-                self.cache_put_guarded(staged)
+                self.cache_put_guarded(staged, transient=self.stage == "prefill" and c.epipe_prefill_mark_transient)
             else:
                 use_transient = True
         if use_transient and self.stage == "prefill":
@@ -293,11 +314,11 @@ class RefLayer:
 
     def demand_gate_can_open(self) -> bool:
         """:5880-5893 (the exposed-stall threshold is zero by default, so only the force flag opens it)."""
-        return bool(self.cfg.epipe_rs_handle_demand_miss and self.cfg.epipe_rs_force_demand_stage)
+        return bool(self._handle_demand() and self.cfg.epipe_rs_force_demand_stage)
 
     def _residual_present(self, segments: Sequence[Segment]) -> bool:
         for eid, _ in segments:
-            if eid in self.events and self.cfg.epipe_rs_handle_late_prefetch and not self.copy_done(eid):
+            if eid in self.events and self._handle_late() and not self.copy_done(eid):
                 return True
             if self.demand_gate_can_open() and not self.contains_no_touch(eid):
                 return True
@@ -399,6 +420,171 @@ class RefLayer:
         if c.epipe_rs_rolling_gate and self.gate_skip > 0:
             self.gate_skip = 0
         return "epipe_rs_residual_scan"
+
+    def _handle_late(self) -> bool:
+        """:4975-4984: ``demand_only`` switches the late-prefetch handling off."""
+        return bool(self.cfg.epipe_rs_handle_late_prefetch) and self.cfg.epipe_decode_rs_mode != "demand_only"
+
+    def _handle_demand(self) -> bool:
+        """``late_only`` switches the demand-miss handling off."""
+        return bool(self.cfg.epipe_rs_handle_demand_miss) and self.cfg.epipe_decode_rs_mode != "late_only"
+
+    def demand_gate_open(self, ready_items: int) -> bool:
+        """:5895-5907."""
+        if not self._handle_demand() or ready_items < self.cfg.epipe_rs_min_buffer_items:
+            return False
+        return self.demand_gate_can_open()
+
+    def epipe_rs_buffered(self, segments: Sequence[Segment]) -> Optional[str]:
+        """:12514-12843.  One pass in ascending expert id: resident experts collect in a
+        bounded buffer (their hits counted as they are seen), which is executed when it is
+        full and in any case before a segment that has to wait; a prefetch still in flight
+        is waited for only after the buffer ran; a miss is staged beside the buffer only in
+        the modes that handle demand misses."""
+        c = self.cfg
+        if self.stage != "decode" or c.planner_mode != "rs_prefetch" or not c.epipe_enable:
+            return None
+        handle_late, handle_demand = self._handle_late(), self._handle_demand()
+        if self._maybe_skip_gate(segments):
+            return None
+        buffered: List[int] = []
+        items = [0]
+        trigger_seen = False
+
+        def flush() -> None:
+            for e in buffered:
+                self.compute(e, have_payload=True)
+            buffered.clear()
+            items[0] = 0
+
+        def sufficient() -> bool:
+            return len(buffered) >= c.epipe_rs_min_buffer_groups and items[0] >= c.epipe_rs_min_buffer_items
+
+        for eid, rows in segments:
+            pending = self.pending_prefetch_event(eid)
+            if self.cache.get(eid) is not None:
+                if not pending:
+                    self.record_cached_use(eid, wait=False)
+                    buffered.append(eid)
+                    items[0] += rows
+                    if len(buffered) >= c.epipe_rs_buffer_max_groups or items[0] >= c.epipe_rs_buffer_max_items:
+                        flush()
+                    continue
+                if not handle_late:
+                    flush()
+                    self.record_cached_use(eid, wait=True)
+                    self.compute(eid, have_payload=True)
+                    continue
+                if c.epipe_rs_rolling_gate:
+                    self.gate_triggers += 1
+                trigger_seen = True
+                if not sufficient():
+                    flush()
+                    self.record_cached_use(eid, wait=True)
+                    self.compute(eid, have_payload=True)
+                    continue
+                flush()
+                self.maybe_wait_prefetch(eid)
+                self.record_cached_use(eid, wait=False)
+                self.compute(eid, have_payload=True)
+                continue
+            if not handle_demand:
+                flush()
+                self.compute(eid)
+                continue
+            if c.epipe_rs_rolling_gate:
+                self.gate_triggers += 1
+            trigger_seen = True
+            if not sufficient() or not self.demand_gate_open(items[0]):
+                flush()
+                self.compute(eid)
+                continue
+            self.trace.append(("h2d", "epipe", eid))
+            flush()
+            self.trace.append(("wait", eid))
+            self.trace.append(("miss", eid))
+            self.on_demand_access(eid)
+            free = max(0, self.cache.capacity - len(self.cache.resident_ids()))
+            if c.epipe_rs_demand_commit and c.epipe_deferred_lru_commit and (free > 0 or not c.epipe_no_evict):
+                self.cache_put_guarded(eid)
+            self.compute(eid, have_payload=True)
+        flush()
+        if trigger_seen and c.epipe_rs_rolling_gate and self.gate_skip > 0:
+            self.gate_skip = 0
+        return "epipe_rs_buffered"
+
+    def ready_payload_for_compute(self, eid: int) -> bool:
+        """:11672-11698: cache first (touching, counted as a hit, waiting a pending copy),
+        then the prefill side cache (touching, not counted)."""
+        if self.cache.get(eid) is not None:
+            self.record_cached_use(eid, wait=True)
+            return True
+        return self.extra.get(eid) is not None
+
+    def epipe_miss_triggered(self, segments: Sequence[Segment]) -> Optional[str]:
+        """:12845-13154.  Walk the segments in ascending expert id; at the first miss look
+        ahead a few segments for resident experts, stage the missing expert on the side
+        lane, run those resident experts meanwhile, then wait, count the miss and run it.
+        Later misses of the same call take the ordinary demand path."""
+        c = self.cfg
+        stage, rs_active = self.stage, c.planner_mode == "rs_prefetch"
+        if not (c.epipe_prefill_enable if stage == "prefill" else c.epipe_enable):
+            return None
+        if stage == "decode" and rs_active and c.epipe_decode_rs_mode == "off":
+            return None
+        if stage == "decode" and rs_active and c.epipe_decode_rs_mode == "buffered":
+            return self.epipe_rs_buffered(segments)
+        if stage == "decode" and rs_active and c.epipe_decode_rs_mode == "upfront_scan":
+            return self.epipe_upfront_scan(segments)
+        min_ready_items = (c.epipe_prefill_lookahead_min_ready_items if stage == "prefill"
+                           else c.epipe_lookahead_min_ready_items)
+        done: Set[int] = set()
+        staged_once = False
+        for i, (eid, _rows) in enumerate(segments):
+            if i in done:
+                continue
+            if self.ready_payload_for_compute(eid):
+                self.compute(eid, have_payload=True)
+                continue
+            if staged_once:
+                self.compute(eid)
+                continue
+            ahead = [j for j in range(i + 1, min(len(segments), i + 1 + int(c.epipe_lookahead_experts)))
+                     if j not in done and self.contains_no_touch(segments[j][0])]
+            ready_items = sum(segments[j][1] for j in ahead)
+            if not ahead:
+                self._count("epipe_fallback_no_ready_lookahead")
+                self.compute(eid)
+                continue
+            if ready_items < min_ready_items:
+                self._count("epipe_fallback_low_ready_items")
+                self.compute(eid)
+                continue
+            self.trace.append(("h2d", "epipe", eid))
+            for j in ahead:
+                self.compute(segments[j][0])
+                done.add(j)
+            self.trace.append(("wait", eid))
+            self.trace.append(("miss", eid))
+            if stage != "prefill":
+                self.on_demand_access(eid)
+            free = max(0, self.cache.capacity - len(self.cache.resident_ids()))
+            if stage == "prefill":
+                commit_allowed, mark = bool(c.epipe_prefill_commit), bool(c.epipe_prefill_mark_transient)
+            elif rs_active:
+                commit_allowed, mark = bool(c.epipe_decode_rs_commit) or free > 0, False
+            else:
+                commit_allowed, mark = bool(c.epipe_decode_no_rs_commit), False
+            insert = commit_allowed and c.epipe_deferred_lru_commit and (free > 0 or not c.epipe_no_evict)
+            if stage == "prefill" and insert:
+                self.on_demand_access(eid)
+            if insert:
+                self.cache_put_guarded(eid, transient=mark)
+            elif stage == "prefill":
+                self.extra.put(eid, ("w", eid))
+            self.compute(eid, have_payload=True)
+            staged_once = True
+        return "epipe_miss_triggered"
 
     # ------------------------------------------------------------ RS prefetch
     def effective_top_m(self) -> int:

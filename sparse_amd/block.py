@@ -242,6 +242,12 @@ class DistributedSparseMoeBlock(nn.Module):
             raise ValueError(
                 "expert_source=rs requires RS cache available, so routing_mode must be 'rs' "
                 "or planner_mode must be 'rs_prefetch'.")
+        # accepted by the reference, not built here: fail before any weight is touched
+        if self.exec_routing_mode == "rs" or self.expert_source == "rs":
+            raise NotImplementedError("routing_mode=rs / expert_source=rs (routing replay from RS) is not built")
+        if str(oracle_mode) != "none":
+            raise NotImplementedError(f"oracle_mode={oracle_mode} (record / replay traces) is not built")
+        self.oracle_mode = "none"
         self.expert_offload = str(expert_offload)
         if self.expert_offload not in ("cpu", "gpu"):
             raise ValueError(f"expert_offload must be cpu|gpu, got {self.expert_offload}")
@@ -497,8 +503,8 @@ class DistributedSparseMoeBlock(nn.Module):
 
     @classmethod
     def demote_prefill_scp_transients_for_decode(cls, metrics: Optional[Any] = None) -> None:
-        """Once per request, at the prefill -> decode boundary (:16565-16601).  At world
-        size 1 no entry is ever transient, so this only flips the request flag."""
+        """Once per request, at the prefill -> decode boundary (:16565-16601): entries that
+        EPIPE staged and committed during prefill go to the LRU end of their cache."""
         if SparseContext.prefill_scp_transient_demoted_for_decode:
             return
         resident = demoted = 0

@@ -44,6 +44,20 @@ def _env_float(name: str, default: float) -> float:
         return float(default)
 
 
+def normalize_decode_rs_mode(raw: Optional[str]) -> str:
+    """Spellings the reference accepts for ``SPARSE_EPIPE_DECODE_RS_MODE`` (:4942-4962)."""
+    mode = str(raw or "late_only").strip().lower() or "late_only"
+    if mode == "disabled":
+        return "off"
+    if mode == "late":
+        return "late_only"
+    if mode == "demand":
+        return "demand_only"
+    if mode in ("scan", "residual", "residual-scan", "buffered_scan", "buffered-scan"):
+        return "residual_scan"
+    return mode
+
+
 @dataclass
 class ResidencyConfig:
     """Knobs of the cache / prefetch / EPIPE machinery with the reference's defaults
@@ -96,6 +110,15 @@ class ResidencyConfig:
     epipe_rs_gate_min_triggers: int = 1
     epipe_rs_gate_skip_steps: int = 8
     epipe_prefill_extra_cache_slots: int = 0
+    epipe_prefill_mark_transient: bool = True     # staged prefill commits are first in line for eviction
+    epipe_promote_transient_on_decode_hit: bool = True
+    epipe_rs_buffer_max_groups: int = 4
+    epipe_rs_buffer_max_items: int = 32
+    epipe_lookahead_experts: int = 4
+    epipe_lookahead_min_ready_items: int = 64
+    epipe_prefill_lookahead_min_ready_items: int = 256
+    epipe_decode_rs_commit: bool = True
+    epipe_decode_no_rs_commit: bool = True
     # execution order for plain EP: unique_mask | full_mask | sorted_segment (same events)
     plain_ep_exec_mode: str = "unique_mask"
 
@@ -123,13 +146,27 @@ class ResidencyConfig:
         c.epipe_enable = _env_flag("SPARSE_EPIPE_ENABLE", "0")
         c.epipe_prefill_enable = _env_flag("SPARSE_EPIPE_PREFILL_ENABLE", "0")
         c.epipe_mode = str(os.environ.get("SPARSE_EPIPE_MODE", "upfront_scan") or "upfront_scan").strip().lower()
-        c.epipe_decode_rs_mode = str(
-            os.environ.get("SPARSE_EPIPE_DECODE_RS_MODE", "late_only") or "late_only").strip().lower()
+        c.epipe_decode_rs_mode = normalize_decode_rs_mode(os.environ.get(
+            "SPARSE_EPIPE_DECODE_RS_MODE", os.environ.get("SPARSE_EPIPE_DECODE_WITH_RS_MODE", "late_only")))
         c.epipe_no_evict = _env_flag("SPARSE_EPIPE_NO_EVICT", "1")
         c.epipe_transient_staging = _env_flag("SPARSE_EPIPE_TRANSIENT_STAGING", "1")
         c.epipe_max_staged_experts = _env_int("SPARSE_EPIPE_MAX_STAGED_EXPERTS", 1)
         c.epipe_sort_ready_by_work = _env_flag("SPARSE_EPIPE_SORT_READY_BY_WORK", "0")
-        c.epipe_prefill_commit = _env_flag("SPARSE_EPIPE_PREFILL_COMMIT", "1")
+        # the prefill policy sets the defaults of commit and transient mark (reference :5007-5016)
+        policy = str(os.environ.get("SPARSE_EPIPE_PREFILL_POLICY", "deferred_lru_commit")
+                     or "deferred_lru_commit").strip().lower()
+        commit_default = "1" if policy in ("deferred_lru_commit", "commit", "lru_commit") else "0"
+        c.epipe_prefill_commit = _env_flag("SPARSE_EPIPE_PREFILL_COMMIT", commit_default)
+        c.epipe_prefill_mark_transient = _env_flag("SPARSE_EPIPE_PREFILL_MARK_TRANSIENT", commit_default)
+        c.epipe_promote_transient_on_decode_hit = _env_flag("SPARSE_EPIPE_PROMOTE_TRANSIENT_ON_DECODE_HIT", "1")
+        c.epipe_rs_buffer_max_groups = max(1, _env_int("SPARSE_EPIPE_RS_BUFFER_MAX_GROUPS", 4))
+        c.epipe_rs_buffer_max_items = max(1, _env_int("SPARSE_EPIPE_RS_BUFFER_MAX_ITEMS", 32))
+        c.epipe_lookahead_experts = max(0, _env_int("SPARSE_EPIPE_LOOKAHEAD_EXPERTS", 4))
+        c.epipe_lookahead_min_ready_items = max(0, _env_int("SPARSE_EPIPE_LOOKAHEAD_MIN_READY_ITEMS", 64))
+        c.epipe_prefill_lookahead_min_ready_items = max(
+            0, _env_int("SPARSE_EPIPE_PREFILL_LOOKAHEAD_MIN_READY_ITEMS", 256))
+        c.epipe_decode_rs_commit = _env_flag("SPARSE_EPIPE_DECODE_RS_COMMIT", "1")
+        c.epipe_decode_no_rs_commit = _env_flag("SPARSE_EPIPE_DECODE_NO_RS_COMMIT", "1")
         c.epipe_rs_handle_late_prefetch = _env_flag("SPARSE_EPIPE_RS_HANDLE_LATE_PREFETCH", "1")
         c.epipe_rs_handle_demand_miss = _env_flag("SPARSE_EPIPE_RS_HANDLE_DEMAND_MISS", "0")
         c.epipe_rs_force_demand_stage = _env_flag("SPARSE_EPIPE_RS_FORCE_DEMAND_STAGE", "0")
@@ -330,8 +367,9 @@ class LayerResidency:
             self.prefetch_events.pop(eid, None)
             self._release_slot(self._slot_of.pop(eid))
 
-    def _cache_put(self, eid: int, slot: int) -> None:
-        """``_cache_put_guarded`` (reference :5985-6022) plus slot bookkeeping."""
+    def _cache_put(self, eid: int, slot: int, transient: bool = False) -> None:
+        """``_cache_put_guarded`` (reference :5985-6022) plus slot bookkeeping.  ``transient``
+        is the entry's ``prefill_scp_transient`` mark: such entries are evicted first."""
         if self.cache.capacity <= 0:
             # nothing is ever stored: the slot only lives until the batch is launched
             self._pending_slots.add(slot)
@@ -340,7 +378,10 @@ class LayerResidency:
         protect = self._protect_with_fallback(eid)
         # a repeatedly used expert enters the hot tier of a tiered cache (reference :11223-11232)
         prefer_hot = int(self.access_freq.get(int(eid), 0)) >= 2
-        self.cache.put(int(eid), slot, pinned=False, prefer_hot=prefer_hot, protect_ids=protect)
+        self.cache.put(int(eid), slot, pinned=False, prefer_hot=prefer_hot, protect_ids=protect,
+                       prefill_scp_transient=bool(transient))
+        if transient:
+            self.metrics.bump("prefill_scp_transient_load_count")
         if self.cache.has(int(eid)):
             self._slot_of[int(eid)] = slot
         else:
@@ -352,7 +393,13 @@ class LayerResidency:
 
     def _record_cached_use(self, eid: int, wait_prefetch: bool) -> None:
         """Hit accounting shared by the demand path and EPIPE (reference :11395-11412,
-        :11652-11670)."""
+        :11652-11670).  A decode hit on an entry staged during prefill makes it an ordinary
+        entry again (:11324-11336)."""
+        if (self.stage == "decode" and self.cfg.epipe_promote_transient_on_decode_hit
+                and self.cache.is_prefill_scp_transient(eid)):
+            self.metrics.bump("prefill_scp_transient_hit_count")
+            if self.cache.clear_prefill_scp_transient(eid):
+                self.metrics.bump("prefill_scp_transient_promote_count")
         if eid in self.prefetched_ids:
             self._event("prefetch_hit", eid)
             self.prefetch_used_ids.add(eid)
@@ -418,15 +465,14 @@ class LayerResidency:
                     name = self._epipe_upfront_scan(segments)
                 else:
                     name = self._epipe_rs_residual_scan(segments)
-            elif self.stage == "decode" and rs_active:
-                raise NotImplementedError(
-                    f"SPARSE_EPIPE_DECODE_RS_MODE={mode} is not built; use off or residual_scan")
-            elif self.stage == "decode" and self.cfg.epipe_mode != "miss_triggered":
+            elif self.stage == "decode" and rs_active and mode in ("buffered", "late_only", "demand_only"):
+                name = self._epipe_rs_buffered(segments)
+            elif self.stage == "decode" and not rs_active and self.cfg.epipe_mode != "miss_triggered":
                 name = self._epipe_upfront_scan(segments)
             elif self.cfg.epipe_mode == "upfront_scan":
                 name = self._epipe_upfront_scan(segments)
             else:
-                raise NotImplementedError("SPARSE_EPIPE_MODE=miss_triggered is not built")
+                name = self._epipe_miss_triggered(segments)
         if name is None:
             for eid, _rows in segments:
                 self._compute(eid)
@@ -512,7 +558,8 @@ class LayerResidency:
                 if stage == "prefill":
                     self._on_demand_access(staged_eid)
                 self._enqueue(staged_eid, slot)
-                self._cache_put(staged_eid, slot)
+                self._cache_put(staged_eid, slot,
+                                transient=stage == "prefill" and cfg.epipe_prefill_mark_transient)
                 m.bump("epipe_cache_insert_count")
                 kept = True
             else:
@@ -547,12 +594,20 @@ class LayerResidency:
 
     def _demand_gate_can_open(self) -> bool:
         """Reference :5880-5893; the exposed-stall threshold variant is not built."""
-        return bool(self.cfg.epipe_rs_handle_demand_miss and self.cfg.epipe_rs_force_demand_stage)
+        return bool(self._handle_demand() and self.cfg.epipe_rs_force_demand_stage)
+
+    def _handle_late(self) -> bool:
+        """``demand_only`` switches the handling of late prefetches off (reference :4975-4984)."""
+        return bool(self.cfg.epipe_rs_handle_late_prefetch) and self.cfg.epipe_decode_rs_mode != "demand_only"
+
+    def _handle_demand(self) -> bool:
+        """``late_only`` switches the staging of demand misses off."""
+        return bool(self.cfg.epipe_rs_handle_demand_miss) and self.cfg.epipe_decode_rs_mode != "late_only"
 
     def _residual_present(self, segments: Sequence[Segment]) -> bool:
         for eid, _rows in segments:
             ev = self.prefetch_events.get(eid)
-            if ev is not None and self.cfg.epipe_rs_handle_late_prefetch and not self.backend.event_done(ev):
+            if ev is not None and self._handle_late() and not self.backend.event_done(ev):
                 return True
             if self._demand_gate_can_open() and not self._contains_no_touch(eid):
                 return True
@@ -686,11 +741,216 @@ class LayerResidency:
 
     def _demand_gate_open(self, ready_items: int) -> bool:
         """Reference :5895-5907."""
-        if not self.cfg.epipe_rs_handle_demand_miss:
+        if not self._handle_demand():
             return False
         if ready_items < self.cfg.epipe_rs_min_buffer_items:
             return False
         return self._demand_gate_can_open()
+
+    def _stage_on_epipe_lane(self, eid: int) -> Tuple[int, Any]:
+        slot = self._acquire_slot()
+        return slot, self._upload(eid, slot, "epipe")
+
+    def _finish_staged(self, eid: int, slot: int, stage_event: Any, commit: bool, transient: bool = False,
+                       to_extra: bool = False) -> None:
+        """Wait a staged copy on the compute lane, queue the expert, and either commit its
+        slot to the cache, hand it to the prefill side cache, or let it go after the batch."""
+        m = self.metrics
+        self.backend.wait_event(stage_event, "compute")
+        m.demand_h2d_bytes += self.expert_bytes
+        self._enqueue(eid, slot)
+        kept = False
+        if commit and self.cache.capacity > 0:
+            self._cache_put(eid, slot, transient=transient)
+            m.bump("epipe_cache_insert_count")
+            kept = True
+        elif to_extra and self.extra_cache.capacity > 0:
+            old_extra = {e: self.extra_cache.peek(e) for e in self.extra_cache.resident_ids()}
+            kept, _upd, _ev = self.extra_cache.put(eid, slot, nbytes=self.expert_bytes)
+            for e, s_old in old_extra.items():
+                if not self.extra_cache.has(e) or (e == eid and s_old != slot):
+                    self._release_slot(s_old)
+        if not kept:
+            m.bump("epipe_transient_payload_count")
+            self._retired.append(slot)
+        m.bump("epipe_enabled_count")
+        m.bump("epipe_staged_missing_count")
+
+    # ---- EPIPE on top of RS prefetch: bounded ready buffer (reference :12514-12843) -----
+    def _epipe_rs_buffered(self, segments: Sequence[Segment]) -> Optional[str]:
+        """One pass in ascending expert id.  Resident experts are counted as hits when seen
+        and queued; the queue is launched before any segment that has to wait (a prefetch in
+        flight, a staged copy), so the wait only starts once the resident work is on the
+        device.  The reference also drains its buffer every ``max_groups`` / ``max_items``;
+        here that only closes a batch, which changes no order."""
+        cfg, m = self.cfg, self.metrics
+        if self.stage != "decode" or cfg.planner_mode != "rs_prefetch" or not cfg.epipe_enable:
+            return None
+        m.bump("epipe_rs_buffered_calls")
+        if self._maybe_skip_gate(segments):
+            return None
+        handle_late, handle_demand = self._handle_late(), self._handle_demand()
+        groups = items = 0
+        trigger_seen = False
+
+        def drain() -> None:
+            nonlocal groups, items
+            self.flush()
+            if groups:
+                m.bump("epipe_rs_buffer_flush_count")
+            groups = items = 0
+
+        def sufficient() -> bool:
+            return groups >= cfg.epipe_rs_min_buffer_groups and items >= cfg.epipe_rs_min_buffer_items
+
+        def trigger(kind: str) -> None:
+            nonlocal trigger_seen
+            m.bump("epipe_rs_trigger_count")
+            m.bump(kind)
+            if cfg.epipe_rs_rolling_gate:
+                self._gate_triggers += 1
+            trigger_seen = True
+
+        for eid, rows in segments:
+            pending = self._pending_prefetch_event(eid)
+            slot = self.cache.get(eid)
+            if slot is not None:
+                if pending is None:
+                    self._record_cached_use(eid, wait_prefetch=False)
+                    self._enqueue(eid, slot)
+                    groups += 1
+                    items += rows
+                    if groups >= cfg.epipe_rs_buffer_max_groups or items >= cfg.epipe_rs_buffer_max_items:
+                        groups = items = 0      # the reference's buffer starts over here
+                    continue
+                if not handle_late:
+                    drain()
+                    self._record_cached_use(eid, wait_prefetch=True)
+                    self._enqueue(eid, slot)
+                    continue
+                trigger("epipe_rs_late_prefetch_trigger_count")
+                if not sufficient():
+                    m.bump("epipe_rs_buffer_too_small_count")
+                    drain()
+                    self._record_cached_use(eid, wait_prefetch=True)
+                    self._enqueue(eid, slot)
+                    continue
+                drain()
+                self._maybe_wait_prefetch(eid)
+                self._record_cached_use(eid, wait_prefetch=False)
+                m.bump("epipe_enabled_count")
+                m.bump("epipe_rs_late_prefetch_overlap_count")
+                self._enqueue(eid, slot)
+                continue
+            if not handle_demand:
+                drain()
+                self._compute(eid)
+                continue
+            trigger("epipe_rs_demand_miss_trigger_count")
+            if not sufficient() or not self._demand_gate_open(items):
+                if not sufficient():
+                    m.bump("epipe_rs_buffer_too_small_count")
+                drain()
+                self._compute(eid)
+                continue
+            if not self._headroom_ok():
+                self._fallback("epipe_fallback_memory")
+                drain()
+                self._compute(eid)
+                continue
+            slot, stage_event = self._stage_on_epipe_lane(eid)
+            drain()
+            self._event("miss", eid)
+            self._on_demand_access(eid)
+            free_cache_slots = max(0, self.cache.capacity - len(self.cache))
+            commit = bool(cfg.epipe_rs_demand_commit and cfg.epipe_deferred_lru_commit
+                          and (free_cache_slots > 0 or not cfg.epipe_no_evict))
+            self._finish_staged(eid, slot, stage_event, commit)
+            m.bump("epipe_rs_demand_stage_count")
+        if trigger_seen and cfg.epipe_rs_rolling_gate and self._gate_skip_remaining > 0:
+            self._gate_skip_remaining = 0
+            m.bump("epipe_rs_gate_reenable_count")
+        if not trigger_seen:
+            m.bump("epipe_fallback_no_miss_trigger")
+        return "epipe_rs_buffered"
+
+    # ---- EPIPE, miss-triggered look-ahead (reference :12845-13154) -----------------------
+    def _ready_slot_for_compute(self, eid: int) -> Optional[int]:
+        """Reference :11672-11698: the cache first (touched, counted as a hit, a pending copy
+        waited for), then the prefill side cache (touched, not counted)."""
+        slot = self.cache.get(eid)
+        if slot is not None:
+            self._record_cached_use(eid, wait_prefetch=True)
+            return slot
+        return self.extra_cache.get(eid)
+
+    def _epipe_miss_triggered(self, segments: Sequence[Segment]) -> Optional[str]:
+        """Walk the segments in ascending expert id; at the first miss look a few segments
+        ahead for resident experts, stage the missing expert on the EPIPE lane, run those
+        resident experts meanwhile, then wait, count the miss and run it.  Later misses of
+        the call take the ordinary demand path."""
+        cfg, m = self.cfg, self.metrics
+        stage, rs_active = self.stage, cfg.planner_mode == "rs_prefetch"
+        if not (cfg.epipe_prefill_enable if stage == "prefill" else cfg.epipe_enable):
+            return None
+        mode = cfg.epipe_decode_rs_mode
+        if stage == "decode" and rs_active and mode == "off":
+            return None
+        if stage == "decode" and rs_active and mode == "buffered":
+            return self._epipe_rs_buffered(segments)
+        if stage == "decode" and rs_active and mode == "upfront_scan":
+            return self._epipe_upfront_scan(segments)
+        min_ready_items = (cfg.epipe_prefill_lookahead_min_ready_items if stage == "prefill"
+                           else cfg.epipe_lookahead_min_ready_items)
+        done: Set[int] = set()
+        staged_once = False
+        for i, (eid, _rows) in enumerate(segments):
+            if i in done:
+                continue
+            slot = self._ready_slot_for_compute(eid)
+            if slot is not None:
+                self._enqueue(eid, slot)
+                continue
+            if staged_once:
+                self._compute(eid)
+                continue
+            ahead = [j for j in range(i + 1, min(len(segments), i + 1 + int(cfg.epipe_lookahead_experts)))
+                     if j not in done and self._contains_no_touch(segments[j][0])]
+            ready_items = sum(segments[j][1] for j in ahead)
+            if not ahead:
+                self._fallback("epipe_fallback_no_ready_lookahead")
+                self._compute(eid)
+                continue
+            if ready_items < min_ready_items:
+                self._fallback("epipe_fallback_low_ready_items")
+                self._compute(eid)
+                continue
+            if not self._headroom_ok():
+                self._fallback("epipe_fallback_memory")
+                self._compute(eid)
+                continue
+            slot, stage_event = self._stage_on_epipe_lane(eid)
+            for j in ahead:
+                self._compute(segments[j][0])
+                done.add(j)
+            self.flush()   # everything queued so far runs while the copy lands
+            self._event("miss", eid)
+            if stage != "prefill":
+                self._on_demand_access(eid)
+            free_cache_slots = max(0, self.cache.capacity - len(self.cache))
+            if stage == "prefill":
+                commit_allowed, mark = bool(cfg.epipe_prefill_commit), bool(cfg.epipe_prefill_mark_transient)
+            elif rs_active:
+                commit_allowed, mark = bool(cfg.epipe_decode_rs_commit) or free_cache_slots > 0, False
+            else:
+                commit_allowed, mark = bool(cfg.epipe_decode_no_rs_commit), False
+            insert = bool(commit_allowed and cfg.epipe_deferred_lru_commit
+                          and (free_cache_slots > 0 or not cfg.epipe_no_evict))
+            if stage == "prefill" and insert:
+                self._on_demand_access(eid)
+            self._finish_staged(eid, slot, stage_event, insert, transient=mark, to_extra=stage == "prefill")
+            staged_once = True
+        return "epipe_miss_triggered"
 
     # ------------------------------------------------------------------ RS prefetch
     # ---- bounded RS staging (utils/rs_overlap.py) -------------------------------------

@@ -115,6 +115,11 @@ def test_constructor_rejects_bad_enums(device):
                dict(expert_source="rs")):
         with pytest.raises(ValueError):
             DistributedSparseMoeBlock(0, mlp, None, env, num_layers=1, num_experts=12, top_k=4, **kw)
+    # settings the reference accepts and this build does not
+    for kw in (dict(routing_mode="rs"), dict(expert_source="rs", planner_mode="rs_prefetch"),
+               dict(oracle_mode="replay")):
+        with pytest.raises(NotImplementedError):
+            DistributedSparseMoeBlock(0, mlp, None, env, num_layers=1, num_experts=12, top_k=4, **kw)
 
 
 def test_deepseek_full_size_4096_tokens_properties(device):

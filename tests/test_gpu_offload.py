@@ -113,6 +113,13 @@ def _replay_oracle(record, cfg, capacity):
     ("epipe", dict(epipe_prefill_enable=True), True),
     ("rs", dict(cache_policy="tiered", prefetch_reserved=1, formal_thresholds=False), False),
     ("rs-epipe", dict(cache_policy="tiered", prefetch_reserved=1, formal_thresholds=False), False),
+    # the other EPIPE executors: bounded ready buffer (the code default mode and with demand
+    # staging) and the miss-triggered look-ahead (decode, and prefill + decode)
+    ("rs-epipe", dict(epipe_decode_rs_mode="late_only"), False),
+    ("rs-epipe", dict(epipe_decode_rs_mode="buffered"), False),
+    ("epipe", dict(epipe_mode="miss_triggered", epipe_lookahead_min_ready_items=1), False),
+    ("epipe", dict(epipe_mode="miss_triggered", epipe_prefill_enable=True, epipe_lookahead_min_ready_items=1,
+                   epipe_prefill_lookahead_min_ready_items=1), True),
 ])
 def test_offloaded_methods_match_resident_values_and_oracle_events(device, method, overrides, prefill_first):
     from sparse_amd.methods import residency_config
@@ -150,8 +157,9 @@ def test_values_do_not_depend_on_copy_timing(device):
     capacity, top_m, steps, T = 4, 3, 12, 4
     ref_blocks, _ = _stack(device, "rr", capacity, top_m, "gpu")
     want = _run(ref_blocks, device, steps, T)
-    for method in ("rs", "rs-epipe"):
-        blocks, metrics = _stack(device, method, capacity, top_m, "cpu")
+    for method, overrides in (("rs", {}), ("rs-epipe", {}), ("rs-epipe", dict(epipe_decode_rs_mode="late_only")),
+                              ("rs-epipe", dict(epipe_decode_rs_mode="buffered"))):
+        blocks, metrics = _stack(device, method, capacity, top_m, "cpu", **overrides)
         got = _run(blocks, device, steps, T)
         for a, b in zip(got, want):
             assert torch.equal(a, b)

@@ -244,7 +244,7 @@ class RoutingModel:
 
 
 def run_trace(method, which, *, steps=60, layers=3, E=16, K=2, T=4, capacity=4, top_m=3, seed=0, late_rate=0.0,
-              prefill_first=False, overrides=None, formal=True):
+              prefill_first=False, prefill_steps=0, overrides=None, formal=True):
     cfg = residency_config(method, capacity, top_m, formal_thresholds=formal, **(overrides or {}))
     late_rng = random.Random(seed + 99)
     late = {}
@@ -270,8 +270,13 @@ def run_trace(method, which, *, steps=60, layers=3, E=16, K=2, T=4, capacity=4, 
             mets.append(m)
     model = RoutingModel(E, K, T, seed)
     executors = []
+    prefill_steps = max(int(prefill_steps), 1 if prefill_first else 0)
     for step in range(steps):
-        phase = "prefill" if (prefill_first and step == 0) else "decode"
+        phase = "prefill" if step < prefill_steps else "decode"
+        if prefill_steps and step == prefill_steps:
+            # the prefill -> decode boundary hook: entries staged during prefill go to the LRU end
+            for lay in lays:
+                lay.cache.demote_prefill_scp_transients()
         routes = [model.route() for _ in range(layers)]
         preds = [model.predict(routes[l + 1], lays[l + 1].predict_topk()) if l + 1 < layers else None
                  for l in range(layers)]
@@ -317,6 +322,31 @@ METHOD_CASES = [
     ("epipe", dict(capacity=6, E=24, T=8, overrides=dict(cache_policy="tiered"))),
     ("rs-epipe", dict(capacity=8, E=24, T=8, top_m=4, formal=False,
                       overrides=dict(cache_policy="tiered", prefetch_reserved=1))),
+    # several prefill calls: staged commits carry the transient mark and are evicted first
+    ("epipe", dict(prefill_steps=5, capacity=8, T=2, overrides=dict(epipe_prefill_enable=True))),
+    ("epipe", dict(prefill_steps=5, capacity=8, T=2,
+                   overrides=dict(epipe_prefill_enable=True, epipe_prefill_mark_transient=False))),
+    # bounded ready buffer: the code default (late_only), with demand staging, demand only
+    ("rs-epipe", dict(late_rate=0.5, overrides=dict(epipe_decode_rs_mode="late_only"))),
+    ("rs-epipe", dict(late_rate=0.3, formal=False, overrides=dict(epipe_decode_rs_mode="buffered"))),
+    ("rs-epipe", dict(late_rate=0.3, overrides=dict(epipe_decode_rs_mode="demand_only"))),
+    ("rs-epipe", dict(late_rate=0.4, capacity=15, E=60, K=4, T=8, top_m=8,
+                      overrides=dict(epipe_decode_rs_mode="buffered", epipe_rs_buffer_max_groups=2))),
+    ("rs-epipe", dict(late_rate=0.4, overrides=dict(epipe_decode_rs_mode="buffered", epipe_rs_min_buffer_groups=2,
+                                                    epipe_rs_min_buffer_items=3))),
+    # miss-triggered look-ahead: decode, decode with RS active, prefill with and without commit
+    ("epipe", dict(overrides=dict(epipe_mode="miss_triggered", epipe_lookahead_min_ready_items=1))),
+    ("epipe", dict(capacity=6, T=8, overrides=dict(epipe_mode="miss_triggered", epipe_lookahead_min_ready_items=4,
+                                                   epipe_lookahead_experts=2))),
+    ("rs-epipe", dict(late_rate=0.3, overrides=dict(epipe_mode="miss_triggered", epipe_decode_rs_mode="stream",
+                                                    epipe_lookahead_min_ready_items=1))),
+    ("epipe", dict(prefill_steps=4, capacity=6, T=8,
+                   overrides=dict(epipe_mode="miss_triggered", epipe_prefill_enable=True,
+                                  epipe_prefill_lookahead_min_ready_items=1, epipe_lookahead_min_ready_items=1))),
+    ("epipe", dict(prefill_steps=4, capacity=6, T=8,
+                   overrides=dict(epipe_mode="miss_triggered", epipe_prefill_enable=True, epipe_prefill_commit=False,
+                                  epipe_prefill_extra_cache_slots=2, epipe_prefill_lookahead_min_ready_items=1,
+                                  epipe_lookahead_min_ready_items=1))),
 ]
 
 
@@ -334,6 +364,113 @@ def test_product_reproduces_the_oracle_event_for_event(method, kw):
             assert g["residents"] == w["residents"], f"layer {l}: final LRU order differs"
     if method in ("epipe", "rs-epipe", "sparse"):
         assert any(e.startswith("epipe") for e in ex_o), "EPIPE never triggered in this trace"
+
+
+def test_transient_mark_of_prefill_commits_changes_later_evictions():
+    """An expert staged during prefill and committed to a free slot is the preferred victim
+    (reference :12083-12089 with :3770-3796) until a decode hit clears the mark: with the
+    mark switched off the same trace evicts differently."""
+    kw = dict(seed=0, prefill_steps=5, capacity=8, T=2)
+    marked, _ = run_trace("epipe", "oracle", overrides=dict(epipe_prefill_enable=True), **kw)
+    plain, _ = run_trace("epipe", "oracle",
+                         overrides=dict(epipe_prefill_enable=True, epipe_prefill_mark_transient=False), **kw)
+    assert any(a["events"] != b["events"] for a, b in zip(marked, plain))
+    # the mark is set on commits in prefill only, and a decode hit clears it
+    lay = RefLayer(0, 16, 2, RefConfig(capacity=4, epipe_enable=True, epipe_prefill_enable=True))
+    lay.phase, lay.call_id, lay.stage = "prefill", 0, "prefill"
+    lay.execute([(1, 3)])
+    assert lay.execute([(1, 2), (2, 2)]) == "epipe_upfront"
+    assert lay.cache.prefill_scp_transient_ids() == [2]
+    lay.phase, lay.call_id, lay.stage = "decode", 1, "decode"
+    lay.execute([(2, 1)])
+    assert lay.cache.prefill_scp_transient_ids() == [] and lay.counters["prefill_scp_transient_promote_count"] == 1
+
+
+def _walk(lay, stage, call, segments):
+    lay.phase, lay.call_id, lay.stage = stage, call, stage
+    before = len(lay.trace)
+    name = lay.execute(segments)
+    return name, lay.trace[before:]
+
+
+def test_buffered_executor_walkthrough():
+    """The bounded-buffer pass of the reference (:12514-12843) on a hand-made call: a resident
+    expert is counted at once and buffered; the expert whose prefetch is still in flight
+    triggers, the buffer runs first, only then the copy is waited for; the miss that follows
+    takes the demand path (``late_only`` never stages)."""
+    late = {4}
+    lay = RefLayer(1, 16, 2, RefConfig(capacity=4, planner_mode="rs_prefetch", epipe_enable=True,
+                                       epipe_decode_rs_mode="late_only"),
+                   copy_done=lambda eid: eid not in late)
+    lay.cache.put(2, ("w", 2))
+    lay.cache.admit_prefetch(4, ("w", 4))
+    lay.prefetched.add(4)
+    lay.events[4] = 1
+    name, trace = _walk(lay, "decode", 0, [(2, 3), (4, 1), (9, 2)])
+    assert name == "epipe_rs_buffered"
+    assert trace == [("hit", 2), ("compute", 2), ("wait", 4), ("prefetch_hit", 4), ("compute", 4),
+                     ("miss", 9), ("h2d", "compute", 9), ("compute", 9)]
+    # with demand staging the miss is copied on the side lane while the buffer runs
+    lay = RefLayer(1, 16, 2, RefConfig(capacity=4, planner_mode="rs_prefetch", epipe_enable=True,
+                                       epipe_decode_rs_mode="buffered", epipe_rs_handle_demand_miss=True,
+                                       epipe_rs_force_demand_stage=True))
+    lay.cache.put(2, ("w", 2))
+    lay.cache.put(3, ("w", 3))
+    name, trace = _walk(lay, "decode", 0, [(2, 1), (3, 1), (9, 2), (11, 1)])
+    assert trace == [("hit", 2), ("hit", 3), ("h2d", "epipe", 9), ("compute", 2), ("compute", 3), ("wait", 9),
+                     ("miss", 9), ("compute", 9),
+                     # nothing is buffered any more, so the second miss is not staged
+                     ("miss", 11), ("h2d", "compute", 11), ("compute", 11)]
+    assert lay.cache.resident_ids() == [2, 3, 9, 11]
+    # a full buffer runs at once: with max_groups=1 nothing is left to cover a late copy
+    lay = RefLayer(1, 16, 2, RefConfig(capacity=4, planner_mode="rs_prefetch", epipe_enable=True,
+                                       epipe_decode_rs_mode="late_only", epipe_rs_buffer_max_groups=1),
+                   copy_done=lambda eid: eid != 4)
+    lay.cache.put(2, ("w", 2))
+    lay.cache.admit_prefetch(4, ("w", 4))
+    lay.prefetched.add(4)
+    lay.events[4] = 1
+    _name, trace = _walk(lay, "decode", 0, [(2, 3), (4, 1)])
+    assert trace == [("hit", 2), ("compute", 2), ("prefetch_hit", 4), ("wait", 4), ("compute", 4)]
+
+
+def test_miss_triggered_executor_walkthrough():
+    """The look-ahead executor of the reference (:12845-13154): the first miss is staged on
+    the side lane while up to ``lookahead`` later resident experts run; a later miss of the
+    same call is an ordinary demand miss; with a full cache the staged expert is not kept."""
+    cfg = dict(capacity=2, epipe_enable=True, epipe_mode="miss_triggered", epipe_lookahead_min_ready_items=1)
+    lay = RefLayer(0, 16, 2, RefConfig(**cfg))
+    lay.cache.put(3, ("w", 3))
+    lay.cache.put(5, ("w", 5))
+    name, trace = _walk(lay, "decode", 0, [(1, 1), (3, 2), (5, 1), (7, 1)])
+    assert name == "epipe_miss_triggered"
+    assert trace == [("h2d", "epipe", 1), ("hit", 3), ("compute", 3), ("hit", 5), ("compute", 5), ("wait", 1),
+                     ("miss", 1), ("compute", 1), ("miss", 7), ("h2d", "compute", 7), ("compute", 7)]
+    assert lay.cache.resident_ids() == [5, 7]              # expert 1 was transient, 7 evicted 3
+    # look-ahead window of one segment: expert 5 is out of reach, too little work -> demand path
+    lay = RefLayer(0, 16, 2, RefConfig(**dict(cfg, epipe_lookahead_experts=1, epipe_lookahead_min_ready_items=3)))
+    lay.cache.put(3, ("w", 3))
+    lay.cache.put(5, ("w", 5))
+    _name, trace = _walk(lay, "decode", 0, [(1, 1), (3, 2), (5, 1)])
+    assert trace[:3] == [("miss", 1), ("h2d", "compute", 1), ("compute", 1)]
+    # loading expert 1 evicted expert 3 (capacity 2), whose own look-ahead is again too small
+    assert trace[3:6] == [("miss", 3), ("h2d", "compute", 3), ("compute", 3)]
+    assert lay.counters["epipe_fallback_low_ready_items"] == 2
+    # prefill: a free slot commits the staged expert with the transient mark
+    lay = RefLayer(0, 16, 2, RefConfig(**dict(cfg, capacity=3, epipe_prefill_enable=True,
+                                              epipe_prefill_lookahead_min_ready_items=1)))
+    lay.cache.put(3, ("w", 3))
+    _name, trace = _walk(lay, "prefill", 0, [(1, 4), (3, 4)])
+    assert trace == [("h2d", "epipe", 1), ("hit", 3), ("compute", 3), ("wait", 1), ("miss", 1), ("compute", 1)]
+    assert lay.cache.prefill_scp_transient_ids() == [1] and lay.freq[1] == 1
+
+
+def test_decode_rs_mode_spellings():
+    from sparse_amd.residency import normalize_decode_rs_mode
+    assert [normalize_decode_rs_mode(m) for m in
+            (None, "", "Disabled", "late", "demand", "scan", "residual-scan", "buffered_scan", "buffered", "off")] == \
+        ["late_only", "late_only", "off", "late_only", "demand_only", "residual_scan", "residual_scan",
+         "residual_scan", "buffered", "off"]
 
 
 def test_invariants_of_every_method():
