@@ -27,6 +27,7 @@ import gc
 import json
 import os
 import sys
+import tempfile
 import time
 
 import torch
@@ -294,15 +295,23 @@ def cached_decode_workload(dtype, device, steps, batch=8, capacity=15, top_m=8):
     wall = run_phase_steps(blocks, inputs, "decode")
     resident_ms = wall / steps * 1e3
     out["resident_eager_ms_per_step"] = resident_ms
+    # cost table for the cost-aware local policy, measured on this GPU with the resident layer 0
+    from sparse_amd.local_policy import CostProfile, install_lightweight_policies, measure_costs, write_profile
+    costs = measure_costs(blocks[0])
+    out["measured_costs"] = {k: round(v, 6) for k, v in costs.items()}
+    profile_path = os.path.join(tempfile.gettempdir(), f"sparse_costs_{os.getpid()}.json")
+    write_profile(profile_path, costs, calibrated=True, provenance="bench.py measure_costs on the running GPU")
     del blocks
     release_stack()
     for name, method, rs_kind in (("rr", "rr", "random"), ("rs_random_init", "rs", "random"),
                                   ("rs_informed", "rs", "informed"), ("rs-epipe_informed", "rs-epipe", "informed"),
+                                  ("rs-epipe_light_informed", "rs-epipe", "informed"),
                                   ("rs-epipe_staged_informed", "rs-epipe", "informed")):
         staged = "staged" in name
         kw = dict(staging_pool_slots=4) if staged else {}
         blocks, metrics, _ = build_offload_stack(shape, dtype, device, method, capacity, top_m, rs_kind=rs_kind,
                                                  **kw)
+        policies = install_lightweight_policies(CostProfile(profile_path, 1)) if "light" in name else []
         engine = None
         if staged:
             # the bounded staging engine instead of the in-line planner: graph-captured predictor,
@@ -316,6 +325,10 @@ def cached_decode_workload(dtype, device, steps, batch=8, capacity=15, top_m=8):
             engine.begin(name)
         wall = run_phase_steps(blocks, inputs, "decode")   # cold cache, all steps timed
         out[name] = offload_report(metrics, blocks, wall, steps, batch, resident_ms)
+        if policies:
+            out[name]["policy"] = {k: sum(p.stats[k] for p in policies)
+                                   for k in ("prefetch_calls", "candidate_scores", "feedback_updates",
+                                             "residual_calls")}
         if engine is not None:
             st = engine.finish()
             engine.shutdown()

@@ -43,6 +43,7 @@ from __future__ import annotations
 
 from typing import Any, Callable, Dict, List, Optional, Sequence, Set, Tuple
 
+from . import ref_policy
 from .ref_cache import (RefEpipePrefillExtraCache, RefExpertWeightCache, RefTieredExpertWeightCache,
                         ref_tiered_capacity_split)
 
@@ -133,6 +134,9 @@ class RefLayer:
         self.phase, self.call_id, self.stage = "none", -1, "decode"
         self.trace: List[Tuple] = []
         self.counters: Dict[str, int] = {}
+        # cost-aware local policy (utils/lightweight_policy.py), off unless a test sets it:
+        # dict(costs=..., expert_bytes=..., window_ms=0.0, ready_ms=0.0, feedback=True, prefetch=True)
+        self.policy: Optional[Dict[str, Any]] = None
 
     def _count(self, name: str, n: int = 1) -> None:
         self.counters[name] = self.counters.get(name, 0) + n
@@ -366,14 +370,21 @@ class RefLayer:
             elif not cached and c.epipe_rs_handle_demand_miss and self.demand_gate_can_open():
                 dem.append(i)
         ready_items = sum(segments[i][1] for i in ready)
+        pol = self.policy
+        if pol is not None and pol["feedback"]:                                  # :12322-12324
+            pol["ready_ms"] = ref_policy.compute_ms(pol["costs"], len(ready), ready_items)
         if len(ready) < c.epipe_rs_min_buffer_groups or ready_items < c.epipe_rs_min_buffer_items:
             return None
         residual, kind = None, ""
         if late:
             residual, kind = late[0], "late"
-        elif dem and c.epipe_rs_handle_demand_miss and ready_items >= c.epipe_rs_min_buffer_items \
-                and self.demand_gate_can_open():
+        elif dem and self.demand_gate_open(ready_items):
             residual, kind = dem[0], "demand"
+        if pol is not None and pol["feedback"]:                                  # :12342-12348
+            stageable = dem if self.demand_gate_open(ready_items) else []
+            cands = [(i, segments[i][0], "late") for i in late] + [(i, segments[i][0], "demand") for i in stageable]
+            chosen = ref_policy.choose_residual(pol["costs"], pol["expert_bytes"], len(ready), ready_items, cands)
+            residual, kind = chosen if chosen is not None else (None, "")
         if residual is None:
             return None
         reid = segments[residual][0]
@@ -756,7 +767,13 @@ class RefLayer:
     def schedule_prefetch(self, flat_ids, flat_probs, budget: int):
         """:10996-11010 with :10413-10431."""
         protect = self.prefetch_protect_ids()
-        plan = self.build_plan(self.score_map(flat_ids, flat_probs), protect, budget)
+        scores = self.score_map(flat_ids, flat_probs)
+        pol = self.policy
+        if pol is not None and pol["prefetch"] and self.phase == "decode":      # :10428-10430
+            scores = ref_policy.adjusted_scores(pol["costs"], pol["expert_bytes"], scores,
+                                                set(self.cache.resident_ids()), pol["window_ms"], pol["ready_ms"],
+                                                pol["feedback"])
+        plan = self.build_plan(scores, protect, budget)
         if plan:
             self.trace.append(("plan", tuple(plan)))
         self.admit_plan(plan)
@@ -764,6 +781,8 @@ class RefLayer:
 
     def reset_for_new_request(self, clear_expert_cache: bool = False, clear_cache_metadata: bool = True) -> None:
         """:6097-6147."""
+        if self.policy is not None:
+            self.policy["ready_ms"] = self.policy["window_ms"] = 0.0
         self.events.clear()
         self.prefetched.clear()
         self.used.clear()

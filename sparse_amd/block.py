@@ -386,6 +386,12 @@ class DistributedSparseMoeBlock(nn.Module):
         budget = tres.prefetch_budget(key)
         if budget <= 0:
             return None
+        if tres.light_policy is not None:
+            # time a copy issued now has before its layer runs: this layer's routed compute
+            # plus the next attention (reference :10993-10996)
+            policy = tres.light_policy
+            here = policy.profile.cost(self.rank, self.layer_idx)
+            policy.window_ms = here.compute(self.top_k, int(x.shape[0]) * self.top_k) + policy.cost.attention
         pred = SparseContext.rs_bank[target](x.float()).to(torch.float32)
         self.metrics.rs_next_layer_pred_calls += 1
         self.metrics.rs_mlp_calls += 1

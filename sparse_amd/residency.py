@@ -250,6 +250,7 @@ class LayerResidency:
         self._free_slots: List[int] = list(range(self.num_slots - 1, -1, -1))
         self.num_slots += len(self._pool_slots)
         self.staging: Any = None   # the BoundedRS engine while a request runs with it enabled
+        self.light_policy: Optional[Any] = None     # sparse_amd.local_policy.LocalPolicy, when installed
         self._retired: List[int] = []           # evicted, still read by the pending batch
         self._pending: List[Tuple[int, int]] = []  # (eid, slot) not launched yet
         self._pending_slots: Set[int] = set()
@@ -659,6 +660,9 @@ class LayerResidency:
             elif (not cached) and cfg.epipe_rs_handle_demand_miss and self._demand_gate_can_open():
                 demand_idx.append(i)
         ready_items = sum(segments[i][1] for i in ready_idx)
+        policy = self.light_policy
+        if policy is not None:
+            policy.observe_ready(len(ready_idx), ready_items)
         if len(ready_idx) < cfg.epipe_rs_min_buffer_groups or ready_items < cfg.epipe_rs_min_buffer_items:
             m.bump("epipe_rs_residual_scan_no_ready_count")
             return None
@@ -668,6 +672,13 @@ class LayerResidency:
             residual, kind = late_idx[0], "late"
         elif demand_idx and self._demand_gate_open(ready_items):
             residual, kind = demand_idx[0], "demand"
+        if policy is not None and policy.feedback:
+            # cost-aware choice among all candidates, late ones first (reference :12342-12348)
+            stageable = demand_idx if self._demand_gate_open(ready_items) else []
+            candidates = [(i, segments[i][0], "late") for i in late_idx]
+            candidates.extend((i, segments[i][0], "demand") for i in stageable)
+            chosen = policy.residual(len(ready_idx), ready_items, candidates)
+            residual, kind = chosen if chosen is not None else (None, "")
         if residual is None:
             m.bump("epipe_fallback_no_miss_trigger")
             return None
@@ -1186,13 +1197,18 @@ class LayerResidency:
         """Plan and admit from the predictor's flattened ``[T, pred_k]`` top-k
         (reference :10996-11010, :10413-10431)."""
         protect = self.prefetch_protect_ids()
-        plan = self.build_plan(self.score_map(flat_ids, flat_probs), protect, int(budget))
+        scores = self.score_map(flat_ids, flat_probs)
+        if self.light_policy is not None and self.phase == "decode":     # reference :10428-10430
+            scores = self.light_policy.scores(scores, set(self.cache.resident_ids()))
+        plan = self.build_plan(scores, protect, int(budget))
         self.admit_plan(plan)
         return plan
 
     # ------------------------------------------------------------------ lifecycle
     def reset_for_new_request(self, *, clear_expert_cache: bool = False, clear_cache_metadata: bool = True) -> None:
         """Reference :6097-6147."""
+        if self.light_policy is not None:
+            self.light_policy.reset()
         self.metrics.prefetch_completed_count += len(self.prefetch_events)
         for ev in self.prefetch_events.values():
             self.backend.wait_event(ev, "compute", True)  # nothing may read a slot before its copy lands

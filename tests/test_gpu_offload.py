@@ -266,3 +266,37 @@ def test_bounded_staging_engine_decode(device):
     for a, b in zip(got3, want[: len(got3)]):
         assert torch.equal(a, b)
     engine.shutdown()
+
+
+def test_cost_aware_local_policy_on_the_device(device, tmp_path):
+    """Costs measured on this GPU, written as a profile, installed on an rs-epipe stack:
+    values stay those of the resident block, the policy is consulted, and a stack that is
+    not RS-prefetching refuses it."""
+    from sparse_amd.local_policy import (COST_FIELDS, CostProfile, install_lightweight_policies, measure_costs,
+                                         write_profile)
+    capacity, top_m, steps, T = 4, 3, 12, 4
+    ref_blocks, _ = _stack(device, "rr", capacity, top_m, "gpu")
+    costs = measure_costs(ref_blocks[0], batches=(1, 2, 4, 8), repeats=5)
+    assert set(costs) == set(COST_FIELDS)
+    assert costs["h2d_bytes_per_ms"] > 1e6 and costs["h2d_latency_ms"] >= 0     # > 1 GB/s over the link
+    assert costs["expert_ms"] >= 0 and costs["item_ms"] >= 0 and costs["expert_ms"] + costs["item_ms"] > 0
+    with pytest.raises(ValueError):
+        blocks, _ = _stack(device, "rr", capacity, top_m, "cpu")
+        measure_costs(blocks[0])
+    want = _run(ref_blocks, device, steps, T)
+    path = tmp_path / "costs.json"
+    write_profile(path, costs, calibrated=True, provenance="measured in the test")
+    blocks, metrics = _stack(device, "rs-epipe", capacity, top_m, "cpu")
+    policies = install_lightweight_policies(CostProfile(path, 1))
+    assert len(policies) == len(blocks) and blocks[1].residency.light_policy is policies[1]
+    got = _run(blocks, device, steps, T)
+    for a, b in zip(got, want):
+        assert torch.equal(a, b)
+    assert sum(p.stats["prefetch_calls"] for p in policies) > 0
+    assert sum(p.stats["feedback_updates"] for p in policies) > 0
+    assert policies[1].window_ms > 0
+    blocks[0].reset_runtime_state_for_new_request(clear_expert_cache=True)
+    assert policies[0].stats["prefetch_calls"] == 0 and policies[0].ready_ms == 0
+    _stack(device, "rr", capacity, top_m, "cpu")
+    with pytest.raises(ValueError):
+        install_lightweight_policies(CostProfile(path, 1))

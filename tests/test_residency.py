@@ -244,7 +244,7 @@ class RoutingModel:
 
 
 def run_trace(method, which, *, steps=60, layers=3, E=16, K=2, T=4, capacity=4, top_m=3, seed=0, late_rate=0.0,
-              prefill_first=False, prefill_steps=0, overrides=None, formal=True):
+              prefill_first=False, prefill_steps=0, overrides=None, formal=True, policy_costs=None):
     cfg = residency_config(method, capacity, top_m, formal_thresholds=formal, **(overrides or {}))
     late_rng = random.Random(seed + 99)
     late = {}
@@ -268,6 +268,23 @@ def run_trace(method, which, *, steps=60, layers=3, E=16, K=2, T=4, capacity=4, 
             lays.append(lay)
             backs.append(be)
             mets.append(m)
+    if policy_costs is not None:
+        # the cost-aware local policy on every layer: the product's class, the oracle's plain state
+        import json
+        import tempfile
+        from sparse_amd.local_policy import CostProfile, LocalPolicy
+        sizes = {e: 100.0 + 40.0 * (e % 5) for e in range(E)}
+        with tempfile.TemporaryDirectory() as d:
+            path = Path(d) / "costs.json"
+            path.write_text(json.dumps(dict(schema_version=1, world_size=1, calibrated=False,
+                                            rank_defaults=policy_costs)))
+            profile = CostProfile(path, 1)
+        for l, lay in enumerate(lays):
+            if which == "oracle":
+                lay.policy = dict(costs=dict(policy_costs), expert_bytes=sizes, window_ms=0.0, ready_ms=0.0,
+                                  feedback=True, prefetch=True)
+            else:
+                lay.light_policy = LocalPolicy(profile, 0, l, sizes, ())
     model = RoutingModel(E, K, T, seed)
     executors = []
     prefill_steps = max(int(prefill_steps), 1 if prefill_first else 0)
@@ -286,6 +303,14 @@ def run_trace(method, which, *, steps=60, layers=3, E=16, K=2, T=4, capacity=4, 
                 tgt.phase, tgt.call_id = phase, step
                 budget = tgt.prefetch_budget(("next_layer_rs", phase, step, l, l + 1))
                 if budget > 0:
+                    if policy_costs is not None:
+                        # what the source layer's forward sets before planning (reference :10993-10996)
+                        window = (policy_costs["expert_ms"] * K + policy_costs["item_ms"] * T * K
+                                  + policy_costs["next_attention_ms"])
+                        if which == "oracle":
+                            tgt.policy["window_ms"] = window
+                        else:
+                            tgt.light_policy.window_ms = window
                     tgt.schedule_prefetch(preds[l][0], preds[l][1], budget)
             lay = lays[l]
             lay.phase, lay.call_id, lay.stage = phase, step, phase
@@ -384,6 +409,32 @@ def test_transient_mark_of_prefill_commits_changes_later_evictions():
     lay.phase, lay.call_id, lay.stage = "decode", 1, "decode"
     lay.execute([(2, 1)])
     assert lay.cache.prefill_scp_transient_ids() == [] and lay.counters["prefill_scp_transient_promote_count"] == 1
+
+
+POLICY_COSTS = dict(h2d_bytes_per_ms=100.0, h2d_latency_ms=0.1, expert_ms=0.3, item_ms=0.05, next_attention_ms=0.4,
+                    split_overhead_ms=0.5)
+
+
+@pytest.mark.parametrize("method,kw", [
+    ("rs", {}), ("rs-epipe", dict(late_rate=0.4)), ("sparse", dict(late_rate=0.3, T=8, capacity=6)),
+    ("rs-epipe", dict(late_rate=0.5, capacity=15, E=60, K=4, T=8, top_m=8)),
+])
+def test_local_policy_through_the_layer_state_machine(method, kw):
+    """With the cost-aware policy installed the product still follows the oracle event for
+    event, and where the residual scan runs the policy does change decisions (plans or
+    residual choices) on these traces."""
+    changed = False
+    for seed in range(3):
+        want, ex_o = run_trace(method, "oracle", seed=seed, policy_costs=POLICY_COSTS, **kw)
+        got, ex_p = run_trace(method, "product", seed=seed, policy_costs=POLICY_COSTS, **kw)
+        base, ex_b = run_trace(method, "oracle", seed=seed, **kw)
+        assert ex_o == ex_p
+        for w, g in zip(want, got):
+            for key in ("events", "h2d", "compute", "waits", "residents"):
+                assert g[key] == w[key], key
+        changed = changed or ex_b != ex_o or any(b["h2d"] != w["h2d"] for b, w in zip(base, want))
+    # without the residual scan nothing ever reports covered time, and the discount is then 1
+    assert changed == (method != "rs"), "the policy changed decisions" if method == "rs" else "never changed one"
 
 
 def _walk(lay, stage, call, segments):
