@@ -404,19 +404,28 @@ def cpu_baseline(shape, batch, dtype, device, budget_s=12.0):
     shared = (sh.gate_proj.weight.cpu(), sh.up_proj.weight.cpu(), sh.down_proj.weight.cpu())
     gate_w, sgw = mlp.gate.weight.cpu(), mlp.shared_expert_gate.weight.cpu().reshape(-1)
     del mlp
-    n = 0
-    t0 = time.perf_counter()
-    while True:
-        x = make_hidden(batch, shape["hidden"], dtype, seed=1000 + n)
-        ref_moe.moe_forward(x, gate_w, experts, shape["top_k"], shared, sgw)
-        n += 1
-        dt = time.perf_counter() - t0
-        if dt > budget_s or n >= 200:
-            break
-    per_layer = dt / n
-    return dict(value=batch / (per_layer * shape["num_layers"]), unit="tokens/s", cores=cores, kind="port",
-                sample=f"{n} decode layer-calls (batch {batch}, 1 of {shape['num_layers']} layers, bf16) of the "
-                       f"CPU oracle in {dt:.1f} s, scaled linearly to {shape['num_layers']} layers")
+
+    def run(threads, budget):
+        torch.set_num_threads(threads)
+        n = 0
+        t0 = time.perf_counter()
+        while True:
+            x = make_hidden(batch, shape["hidden"], dtype, seed=1000 + n)
+            ref_moe.moe_forward(x, gate_w, experts, shape["top_k"], shared, sgw)
+            n += 1
+            dt = time.perf_counter() - t0
+            if dt > budget or n >= 200:
+                return n, dt
+
+    n, dt = run(cores, budget_s * 0.6)
+    n1, dt1 = run(1, budget_s * 0.4)      # the reference serves with OMP_NUM_THREADS=1 (run_case.sh:229)
+    torch.set_num_threads(cores)
+    layers = shape["num_layers"]
+    return dict(value=batch / (dt / n * layers), unit="tokens/s", cores=cores, kind="port",
+                value_1_thread=batch / (dt1 / n1 * layers),
+                sample=f"{n} decode layer-calls (batch {batch}, 1 of {layers} layers, bf16) of the CPU oracle in "
+                       f"{dt:.1f} s on {cores} threads, and {n1} in {dt1:.1f} s on 1 thread, each scaled linearly "
+                       f"to {layers} layers")
 
 
 def main():

@@ -26,6 +26,8 @@ How each function is pinned (see tests/test_oracle_moe.py):
                             invariance, equality with execute_sorted_segments+combine.
   combine_expert_outputs    brute force on tiny inputs, order sensitivity in bf16.
   shared_expert_forward     closed form.
+  rs_routing                closed form on hand-made probabilities (top-k of a known row,
+                            renormalised sum, log / -1e9 pseudo logits), brute-force top-k.
 """
 from __future__ import annotations
 
@@ -167,6 +169,28 @@ def shared_expert_forward(x: torch.Tensor, shared: Optional[ExpertWeights],
     if shared_gate_w is not None:
         out = torch.sigmoid(F.linear(x, shared_gate_w.reshape(1, -1))) * out
     return out
+
+
+def rs_routing(pred: torch.Tensor, top_k: int, dtype: torch.dtype, norm_topk_prob: bool = False,
+               eps: float = 1e-12):
+    """Routing replayed from a predictor's probabilities ``pred [T,E]`` instead of the router
+    (``expert_source="rs"``): top-k of the prediction (:10971-10983), optional renormalisation,
+    weights in the activation dtype, and pseudo logits that hold ``log(clamp(w, eps))`` at the
+    chosen experts and -1e9 elsewhere (:11137-11155)."""
+    topv, topi = topk_lower_id_first(pred.float(), top_k)
+    if norm_topk_prob:
+        topv = topv / topv.sum(dim=-1, keepdim=True).clamp_min(1e-12)
+    w = topv.to(dtype)
+    logits = torch.full((pred.shape[0], pred.shape[1]), -1e9, dtype=torch.float32)
+    logits.scatter_(1, topi, torch.log(w.float().clamp_min(eps)))
+    return w, topi, logits
+
+
+def moe_forward_routed(x: torch.Tensor, topv: torch.Tensor, topi: torch.Tensor, experts: Sequence[ExpertWeights],
+                       shared: Optional[ExpertWeights] = None,
+                       shared_gate_w: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``forward`` with the routing given (:16488, :16520-16526)."""
+    return experts_world1_exact(x, topi, topv, experts) + shared_expert_forward(x, shared, shared_gate_w)
 
 
 def moe_forward(x: torch.Tensor, gate_w: torch.Tensor, experts: Sequence[ExpertWeights], top_k: int,

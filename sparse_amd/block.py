@@ -243,8 +243,6 @@ class DistributedSparseMoeBlock(nn.Module):
                 "expert_source=rs requires RS cache available, so routing_mode must be 'rs' "
                 "or planner_mode must be 'rs_prefetch'.")
         # accepted by the reference, not built here: fail before any weight is touched
-        if self.exec_routing_mode == "rs" or self.expert_source == "rs":
-            raise NotImplementedError("routing_mode=rs / expert_source=rs (routing replay from RS) is not built")
         if str(oracle_mode) != "none":
             raise NotImplementedError(f"oracle_mode={oracle_mode} (record / replay traces) is not built")
         self.oracle_mode = "none"
@@ -257,6 +255,7 @@ class DistributedSparseMoeBlock(nn.Module):
         if self.dtype not in (torch.bfloat16, torch.float32):
             raise ValueError(f"dtype must be bfloat16 or float32, got {self.dtype}")
         self.rs_group = int(rs_group)
+        self.rs_prob_to_logit_eps = float(rs_prob_to_logit_eps)
         self.prefetch_top_m = int(prefetch_top_m)
         self.metrics = metrics if metrics is not None else Metrics()
 
@@ -351,6 +350,26 @@ class DistributedSparseMoeBlock(nn.Module):
         ops.permute_build(ws.topi, self.num_experts, out=ws.perm)
         return logits
 
+    def _route_from_cache(self, x: torch.Tensor, ws: _Workspace) -> torch.Tensor:
+        """``expert_source="rs"``: execute with the weights and indices the previous layer's
+        predictor left in ``SparseContext.routing_cache`` (:11118-11155).  Returns pseudo
+        logits: log of the replayed weight at the chosen experts, -1e9 elsewhere."""
+        w, idx = SparseContext.routing_cache[self.layer_idx]
+        T = int(x.shape[0])
+        if tuple(idx.shape) != (T, self.top_k) or tuple(w.shape) != (T, self.top_k):
+            raise NotImplementedError(
+                f"RS routing replay with {tuple(idx.shape)} predictions for top_k={self.top_k} is not built")
+        ws.topv.copy_(w.to(self.dtype))
+        ws.topi.copy_(idx)
+        ops.permute_build(ws.topi, self.num_experts, out=ws.perm)
+        if self.shared_gate_weight is not None:
+            # the shared expert's gate comes out of the router-logits kernel; the logits are unused
+            ops.router_logits(x, self.gate_weight, self.shared_gate_weight, self.logits_dtype,
+                              shared_gate_out=ws.shared_gate)
+        logits = torch.full((T, self.num_experts), -1e9, device=x.device, dtype=torch.float32)
+        logits.scatter_(1, ws.topi, ws.topv.float().clamp_min(self.rs_prob_to_logit_eps).log())
+        return logits
+
     def _routing_router(self, x: torch.Tensor):
         """``(topv, topi, router_logits)`` like the reference's method (:9502-9595)."""
         ws = self._workspace(int(x.shape[0]))
@@ -364,7 +383,8 @@ class DistributedSparseMoeBlock(nn.Module):
     def _rs_begin(self, x: torch.Tensor, seq_len: int, ws: _Workspace):
         """Device half of ``_compute_and_schedule_next_layer_rs`` (:10916-11010): budget on
         the host, predictor + top-k on the device, async copy of the top-k to the host."""
-        if self.planner_mode != "rs_prefetch" or SparseContext.rs_bank is None:
+        for_routing = self.expert_source == "rs" or self.exec_routing_mode == "rs"
+        if (self.planner_mode != "rs_prefetch" and not for_routing) or SparseContext.rs_bank is None:
             return None
         if SparseContext.rs_bank_layout != "next_layer":
             return None
@@ -375,18 +395,20 @@ class DistributedSparseMoeBlock(nn.Module):
         if target >= len(src) or int(src[target]) != self.layer_idx:
             return None
         tblk = SparseContext.layer_blocks.get(target)
-        if tblk is None or tblk.residency is None or target >= len(SparseContext.rs_bank):
+        if tblk is None or target >= len(SparseContext.rs_bank):
             return None
         tres = tblk.residency
-        if int(seq_len) != 1 and not tres.cfg.rs_prefetch_prefill:
+        if int(seq_len) != 1 and not (tres is not None and tres.cfg.rs_prefetch_prefill):
             return None
-        tres.phase, tres.call_id = str(SparseContext.current_phase), int(SparseContext.runtime_call_id)
-        key = ("next_layer_rs", str(SparseContext.current_phase), int(SparseContext.runtime_call_id),
-               self.layer_idx, target)
-        budget = tres.prefetch_budget(key)
-        if budget <= 0:
+        budget = 0
+        if self.planner_mode == "rs_prefetch" and tres is not None:
+            tres.phase, tres.call_id = str(SparseContext.current_phase), int(SparseContext.runtime_call_id)
+            key = ("next_layer_rs", str(SparseContext.current_phase), int(SparseContext.runtime_call_id),
+                   self.layer_idx, target)
+            budget = tres.prefetch_budget(key)
+        if budget <= 0 and not for_routing:
             return None
-        if tres.light_policy is not None:
+        if tres is not None and tres.light_policy is not None:
             # time a copy issued now has before its layer runs: this layer's routed compute
             # plus the next attention (reference :10993-10996)
             policy = tres.light_policy
@@ -395,6 +417,16 @@ class DistributedSparseMoeBlock(nn.Module):
         pred = SparseContext.rs_bank[target](x.float()).to(torch.float32)
         self.metrics.rs_next_layer_pred_calls += 1
         self.metrics.rs_mlp_calls += 1
+        if for_routing:
+            # the next layer may execute with this prediction instead of its router (:10971-10983)
+            raw = os.environ.get("SPARSE_RS_EXEC_TOPK", "").strip()
+            exec_topk = max(1, min(int(raw) if raw else self.top_k, int(pred.shape[-1])))
+            route_v, route_i = torch.topk(pred, k=exec_topk, dim=-1)
+            if self.norm_topk_prob:
+                route_v = route_v / route_v.sum(dim=-1, keepdim=True).clamp_min(1e-12)
+            SparseContext.routing_cache[target] = (route_v.to(x.dtype), route_i.to(torch.long))
+        if self.planner_mode != "rs_prefetch" or tres is None or budget <= 0:
+            return None
         pred_k = min(int(pred.shape[-1]), int(tres.predict_topk()))
         topv, topi = torch.topk(pred, k=pred_k, dim=-1)
         if self.norm_topk_prob:
@@ -447,7 +479,11 @@ class DistributedSparseMoeBlock(nn.Module):
                 self.residency.staging = None
             rs_job = self._rs_begin(x, S, ws)
 
-        logits = self._route(x, ws)
+        if self.expert_source == "rs" and self.layer_idx in SparseContext.routing_cache:
+            logits = self._route_from_cache(x, ws)
+        else:
+            # also the first layer and prefill of an RS-routed run (:11128-11136)
+            logits = self._route(x, ws)
         shared_gate = ws.shared_gate if self.shared_gate_weight is not None else None
         fused = (self.residency is None and self.shared_weights is not None and self.dtype == torch.bfloat16
                  and T <= ops.DECODE_MAX_TOKENS)

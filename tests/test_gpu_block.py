@@ -116,8 +116,7 @@ def test_constructor_rejects_bad_enums(device):
         with pytest.raises(ValueError):
             DistributedSparseMoeBlock(0, mlp, None, env, num_layers=1, num_experts=12, top_k=4, **kw)
     # settings the reference accepts and this build does not
-    for kw in (dict(routing_mode="rs"), dict(expert_source="rs", planner_mode="rs_prefetch"),
-               dict(oracle_mode="replay")):
+    for kw in (dict(oracle_mode="replay"), dict(oracle_mode="record")):
         with pytest.raises(NotImplementedError):
             DistributedSparseMoeBlock(0, mlp, None, env, num_layers=1, num_experts=12, top_k=4, **kw)
 
@@ -180,3 +179,61 @@ def test_prefill_with_empty_and_tiny_segments(device):
     torch.testing.assert_close(out.float(), ref_out.float(), **BF16_TOL)
     # identical tokens give identical rows
     assert torch.equal(out[0], out[299]) and torch.equal(out[301], out[429])
+
+
+@pytest.mark.parametrize("dtype,offload", [(torch.float32, "gpu"), (torch.bfloat16, "gpu"), (torch.bfloat16, "cpu")])
+def test_expert_source_rs_executes_the_predicted_routing(device, dtype, offload):
+    """``expert_source="rs"``: layer l's predictor leaves (weights, ids) for layer l+1, which
+    then executes them instead of its own router; layer 0 and prefill calls use the router
+    (reference :11118-11155, :10971-10983).  Checked against the oracle fed with the
+    device's own prediction."""
+    from sparse_amd.block import DistributedSparseMoeBlock
+    from sparse_amd.context import DistEnv, SparseContext
+    from sparse_amd.rs import random_init_bank
+    from sparse_amd.synthetic import make_hidden, make_mlp_block
+    shape, T, L = SMALL_Q, 6, 3
+    SparseContext.reset()
+    mlps = [make_mlp_block(shape, dtype=dtype, seed=20 + l) for l in range(L)]
+    kw = dict(expert_offload=offload, expert_cache=4, planner_mode="rs_prefetch", prefetch_top_m=3) \
+        if offload == "cpu" else dict(expert_offload="gpu", routing_mode="rs")
+    blocks = [DistributedSparseMoeBlock(l, mlps[l], None, DistEnv(0, 1, 0, device), num_layers=L,
+                                        num_experts=shape["num_experts"], top_k=shape["top_k"], dtype=dtype,
+                                        expert_source="rs", **kw) for l in range(L)]
+    SparseContext.set_rs_bank(random_init_bank(L, shape["hidden"], shape["num_experts"], hidden_dim=32, seed=1,
+                                               device=device))
+    tol = BF16_TOL if dtype == torch.bfloat16 else F32_TOL
+    for call, phase in enumerate(["prefill", "decode", "decode"]):
+        SparseContext.current_phase = phase
+        SparseContext.begin_runtime_call(call)
+        x = make_hidden(T, shape["hidden"], dtype, seed=300 + call)
+        hid = (x.view(1, T, -1) if phase == "prefill" else x.view(T, 1, -1)).to(device)
+        for l, blk in enumerate(blocks):
+            replay = phase == "decode" and l > 0
+            assert (l in SparseContext.routing_cache) == replay
+            if replay:
+                w_dev, i_dev = (t.cpu() for t in SparseContext.routing_cache[l])
+            out, logits = blk(hid)
+            torch.cuda.synchronize()
+            lay = oracle_layer(mlps[l])
+            xin = hid.view(T, -1).cpu()
+            ws = blk._workspace(T)
+            if replay:
+                assert torch.equal(ws.topi.cpu(), i_dev) and torch.equal(ws.topv.cpu(), w_dev)
+                # the prediction itself: the oracle's top-k of the device's probabilities
+                pred = SparseContext.rs_bank[l](prev_in.to(device).float()).cpu()
+                w_ref, i_ref, logits_ref = ref_moe.rs_routing(pred, shape["top_k"], dtype)
+                assert torch.equal(i_ref, i_dev)
+                torch.testing.assert_close(w_ref.float(), w_dev.float(), rtol=1e-2, atol=1e-6)
+                assert logits.dtype == torch.float32
+                torch.testing.assert_close(logits.cpu(), ref_moe.rs_routing(pred, shape["top_k"], dtype)[2],
+                                           rtol=1e-2, atol=1e-2)
+                want = ref_moe.moe_forward_routed(xin, w_dev, i_dev, lay["experts"], lay["shared"],
+                                                  lay["shared_gate_w"])
+            else:
+                want, _, ref_topi, _ = ref_moe.moe_forward(
+                    xin, lay["gate_w"], lay["experts"], shape["top_k"], lay["shared"], lay["shared_gate_w"],
+                    router_logits=logits.cpu())
+                assert torch.equal(ws.topi.cpu(), ref_topi)
+            torch.testing.assert_close(out.view(T, -1).cpu().float(), want.float(), **tol)
+            prev_in = xin
+            hid = out

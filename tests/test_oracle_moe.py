@@ -4,6 +4,8 @@ sign or index or a transposed operand fails here rather than hiding in a GPU com
 import itertools
 
 import numpy as np
+import math
+
 import pytest
 import torch
 import torch.nn.functional as F
@@ -207,3 +209,35 @@ def test_permute_brute_force_and_invariants():
     topi = torch.tensor([[3, 1], [1, 0], [3, 2]])
     perm, _, _, _ = ref_permute.permute_build(topi.numpy(), 4)
     assert perm.tolist() == torch.argsort(topi.reshape(-1), stable=True).tolist()
+
+
+def test_rs_routing_closed_form():
+    """Routing replayed from predictor probabilities: a hand-made row and brute force."""
+    pred = torch.tensor([[.05, .4, .1, .3, .15], [.2, .2, .5, .05, .05]])
+    w, idx, logits = ref_moe.rs_routing(pred, 2, torch.float32)
+    assert idx.tolist() == [[1, 3], [2, 0]]                       # tie between experts 0 and 1: lower id
+    torch.testing.assert_close(w, torch.tensor([[.4, .3], [.5, .2]]))
+    assert logits[0, 1].item() == pytest.approx(math.log(.4), rel=1e-6)
+    assert logits[0, 0].item() == -1e9 and logits.dtype == torch.float32
+    w, _, _ = ref_moe.rs_routing(pred, 2, torch.float32, norm_topk_prob=True)
+    torch.testing.assert_close(w, torch.tensor([[.4 / .7, .3 / .7], [.5 / .7, .2 / .7]]))
+    wb, _, lb = ref_moe.rs_routing(pred, 2, torch.bfloat16)
+    assert wb.dtype == torch.bfloat16
+    assert lb[0, 3].item() == pytest.approx(math.log(float(torch.tensor(.3).bfloat16())), rel=1e-6)
+    # a zero probability is clamped before the log
+    _, _, lz = ref_moe.rs_routing(torch.tensor([[1., 0., 0.]]), 2, torch.float32, eps=1e-12)
+    assert lz[0, 1].item() == pytest.approx(math.log(1e-12), rel=1e-6)
+    g = torch.Generator().manual_seed(3)
+    pred = torch.softmax(torch.randn(20, 9, generator=g), -1)
+    w, idx, _ = ref_moe.rs_routing(pred, 3, torch.float32)
+    for t in range(20):
+        want = sorted(range(9), key=lambda e: (-pred[t, e].item(), e))[:3]
+        assert idx[t].tolist() == want
+    # given routing: same as routing by a gate that produces those logits
+    H, E, I = 16, 6, 8
+    x = torch.randn(5, H, generator=g)
+    experts = [(torch.randn(I, H, generator=g) * .1, torch.randn(I, H, generator=g) * .1,
+                torch.randn(H, I, generator=g) * .1) for _ in range(E)]
+    gate_w = torch.randn(E, H, generator=g)
+    out, topv, topi, _ = ref_moe.moe_forward(x, gate_w, experts, 2)
+    torch.testing.assert_close(ref_moe.moe_forward_routed(x, topv, topi, experts), out)
