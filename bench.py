@@ -414,7 +414,7 @@ def cpu_baseline(shape, batch, dtype, device, budget_s=12.0):
             ref_moe.moe_forward(x, gate_w, experts, shape["top_k"], shared, sgw)
             n += 1
             dt = time.perf_counter() - t0
-            if dt > budget or n >= 200:
+            if dt > budget or n >= 5000:
                 return n, dt
 
     n, dt = run(cores, budget_s * 0.6)
