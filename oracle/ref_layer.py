@@ -96,6 +96,10 @@ class RefConfig:
         self.epipe_rs_gate_min_triggers = 1
         self.epipe_rs_gate_skip_steps = 8
         self.epipe_prefill_extra_cache_slots = 0
+        self.epipe_prefill_extra_cache_decode_read = True
+        self.epipe_prefill_extra_cache_clear_at_decode = False
+        self.epipe_prefill_extra_cache_persist_requests = False
+        self.epipe_prefill_extra_cache_max_mb = 128.0
         self.epipe_prefill_mark_transient = True      # default follows the default prefill policy (:5012-5016)
         self.epipe_promote_transient_on_decode_hit = True
         self.epipe_rs_buffer_max_groups = 4
@@ -123,6 +127,7 @@ class RefLayer:
         else:
             self.cache = RefExpertWeightCache(cfg.capacity)
         self.extra = RefEpipePrefillExtraCache(cfg.epipe_prefill_extra_cache_slots)
+        self.expert_bytes = 0                    # size of one expert for the side cache's byte guard
         self.copy_done = copy_done or (lambda eid: True)
         self.prefetched: Set[int] = set()        # _prefetched_ids_this_group
         self.used: Set[int] = set()              # _prefetch_used_ids_this_group
@@ -204,12 +209,47 @@ class RefLayer:
         if self.cache.get(eid) is not None:
             self.record_cached_use(eid, wait=True)
             return
-        if self.extra.get(eid) is not None:
+        if self.extra_get(eid):
             return
         self.trace.append(("miss", eid))
         self.trace.append(("h2d", "compute", eid))
         self.on_demand_access(eid)
         self.cache_put_guarded(eid)
+
+    # ---- prefill side cache (:5637-5720) -----------------------------------------------
+    def extra_enabled(self) -> bool:
+        return self.extra.capacity > 0 and bool(self.cfg.epipe_prefill_enable)
+
+    def _extra_readable(self) -> bool:
+        return self.extra_enabled() and not (self.stage == "decode"
+                                             and not self.cfg.epipe_prefill_extra_cache_decode_read)
+
+    def extra_get(self, eid: int) -> bool:
+        """A payload found in the side cache counts as an ordinary hit (:5687-5704)."""
+        if not self._extra_readable() or self.extra.get(eid) is None:
+            return False
+        self.trace.append(("hit", eid))
+        self._count("epipe_prefill_extra_cache_hit_count")
+        return True
+
+    def extra_store(self, eid: int) -> bool:
+        """:5647-5685: prefill only, bounded by slots and by bytes."""
+        if self.stage != "prefill" or not self.extra_enabled():
+            return False
+        max_bytes = int(float(self.cfg.epipe_prefill_extra_cache_max_mb) * 1024.0 * 1024.0)
+        if max_bytes > 0 and not self.extra.has(eid) and self.extra.resident_nbytes() + self.expert_bytes > max_bytes:
+            self._count("epipe_prefill_extra_cache_no_room_count")
+            return False
+        ok, _updated, _evicted = self.extra.put(eid, ("w", eid), nbytes=self.expert_bytes)
+        return bool(ok)
+
+    def decode_boundary(self) -> int:
+        """Per-layer part of the prefill -> decode hooks (:16565-16640): transients to the LRU
+        end, the side cache dropped only when asked to.  Returns the demoted count."""
+        demoted = self.cache.demote_prefill_scp_transients()
+        if self.cfg.epipe_prefill_extra_cache_clear_at_decode:
+            self.extra.clear()
+        return demoted
 
     def compute(self, eid: int, have_payload: bool = False) -> None:
         if not have_payload:
@@ -257,7 +297,7 @@ class RefLayer:
 
     def contains_no_touch(self, eid: int) -> bool:
         """:5815-5851."""
-        return self.extra.has(eid) or self.cache.has(eid)
+        return (self._extra_readable() and self.extra.has(eid)) or self.cache.has(eid)
 
     def epipe_upfront_scan(self, segments: Sequence[Segment]) -> Optional[str]:
         """:11867-12167."""
@@ -299,7 +339,7 @@ class RefLayer:
             else:
                 use_transient = True
         if use_transient and self.stage == "prefill":
-            self.extra.put(staged, ("w", staged))
+            self.extra_store(staged)
         self.compute(staged, have_payload=True)
         for eid, _ in missing[1:]:
             self.compute(eid)
@@ -530,7 +570,7 @@ class RefLayer:
         if self.cache.get(eid) is not None:
             self.record_cached_use(eid, wait=True)
             return True
-        return self.extra.get(eid) is not None
+        return self.extra_get(eid)
 
     def epipe_miss_triggered(self, segments: Sequence[Segment]) -> Optional[str]:
         """:12845-13154.  Walk the segments in ascending expert id; at the first miss look
@@ -592,7 +632,7 @@ class RefLayer:
             if insert:
                 self.cache_put_guarded(eid, transient=mark)
             elif stage == "prefill":
-                self.extra.put(eid, ("w", eid))
+                self.extra_store(eid)
             self.compute(eid, have_payload=True)
             staged_once = True
         return "epipe_miss_triggered"
@@ -791,6 +831,7 @@ class RefLayer:
         self.cycle_key = None
         if clear_expert_cache:
             self.cache.clear()
-            self.extra.clear()
         elif clear_cache_metadata:
             self.cache.reset_request_metadata(unpin=True)
+        if clear_expert_cache or not self.cfg.epipe_prefill_extra_cache_persist_requests:     # :6146-6147
+            self.extra.clear()

@@ -34,6 +34,15 @@ def _is_silu(fn: Any) -> bool:
     return fn is None or fn is F.silu or isinstance(fn, nn.SiLU) or getattr(fn, "__name__", "") == "silu"
 
 
+def _bump(metrics: Any, name: str, value: int) -> None:
+    """Add to a counter of either metrics flavour: this package's ``Metrics`` or any object
+    with plain integer attributes, as the reference's harness passes."""
+    if hasattr(metrics, "bump"):
+        metrics.bump(name, value)
+    else:
+        setattr(metrics, name, int(getattr(metrics, name, 0)) + int(value))
+
+
 def _mlp_weights(mod: Any) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     return mod.gate_proj.weight.detach(), mod.up_proj.weight.detach(), mod.down_proj.weight.detach()
 
@@ -545,31 +554,60 @@ class DistributedSparseMoeBlock(nn.Module):
 
     @classmethod
     def demote_prefill_scp_transients_for_decode(cls, metrics: Optional[Any] = None) -> None:
-        """Once per request, at the prefill -> decode boundary (:16565-16601): entries that
+        """Once per request, at the prefill -> decode boundary (:16629-16653): entries that
         EPIPE staged and committed during prefill go to the LRU end of their cache."""
         if SparseContext.prefill_scp_transient_demoted_for_decode:
             return
         resident = demoted = 0
-        for blk in SparseContext.layer_blocks.values():
+        for blk in list(SparseContext.layer_blocks.values()):
             cache = getattr(blk, "_cache", None)
             if cache is None:
                 continue
             resident += len(cache.prefill_scp_transient_ids())
             demoted += int(cache.demote_prefill_scp_transients())
         if metrics is not None:
-            metrics.bump("prefill_scp_transient_resident_at_decode_start", resident)
-            metrics.bump("prefill_scp_transient_demote_count", demoted)
+            _bump(metrics, "prefill_scp_transient_resident_at_decode_start", resident)
+            _bump(metrics, "prefill_scp_transient_demote_count", demoted)
+            _bump(metrics, "epipe_prefill_transient_demote_count", demoted)
         SparseContext.prefill_scp_transient_demoted_for_decode = True
 
     @classmethod
+    def record_prefill_scp_transient_decode_end(cls, metrics: Optional[Any] = None) -> None:
+        """Transient entries still resident when decoding ends (:16655-16667)."""
+        if metrics is None:
+            return
+        left = 0
+        for blk in list(SparseContext.layer_blocks.values()):
+            cache = getattr(blk, "_cache", None)
+            if cache is not None:
+                left += len(cache.prefill_scp_transient_ids())
+        _bump(metrics, "prefill_scp_transient_resident_at_decode_end", left)
+
+    @classmethod
     def handle_epipe_prefill_extra_cache_decode_boundary(cls, metrics: Optional[Any] = None) -> None:
-        """Drop prefill-staged payloads before decode (:16603-16640)."""
-        for blk in SparseContext.layer_blocks.values():
-            res = blk.residency
-            if res is None or res.extra_cache.capacity <= 0:
+        """Count the payloads the prefill side caches hold at the boundary and drop them only
+        where ``SPARSE_EPIPE_PREFILL_EXTRA_CACHE_CLEAR_AT_DECODE`` asks for it (:16591-16610);
+        by default decode keeps reading them."""
+        held = cleared = 0
+        for blk in list(SparseContext.layer_blocks.values()):
+            res = getattr(blk, "residency", None)
+            if res is None:
                 continue
-            for eid in res.extra_cache.resident_ids():
-                res._release_slot(res.extra_cache.peek(eid))
-            n = res.extra_cache.clear()
-            if metrics is not None:
-                metrics.bump("epipe_prefill_extra_cache_cleared", n)
+            held += res.extra_cache.resident_count()
+            if res.cfg.epipe_prefill_extra_cache_clear_at_decode:
+                res.flush()
+                cleared += res.clear_extra_cache()
+        if metrics is not None:
+            _bump(metrics, "epipe_prefill_extra_cache_resident_at_decode_start", held)
+            if cleared > 0:
+                _bump(metrics, "epipe_prefill_extra_cache_evict_count", cleared)
+
+    @classmethod
+    def record_epipe_prefill_extra_cache_decode_end(cls, metrics: Optional[Any] = None) -> None:
+        """:16612-16627."""
+        if metrics is None:
+            return
+        held = sum(blk.residency.extra_cache.resident_count() for blk in list(SparseContext.layer_blocks.values())
+                   if getattr(blk, "residency", None) is not None)
+        _bump(metrics, "epipe_prefill_extra_cache_resident_count", held)
+        _bump(metrics, "epipe_prefill_extra_cache_resident_at_decode_end", held)

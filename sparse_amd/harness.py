@@ -149,6 +149,8 @@ def greedy_decode(model: Any, input_ids: torch.Tensor, attention_mask: Optional[
         past = out.past_key_values
         cur = torch.argmax(out.logits[:, -1, :], dim=-1, keepdim=True)
         generated.append(cur)
+    DistributedSparseMoeBlock.record_prefill_scp_transient_decode_end(metrics)
+    DistributedSparseMoeBlock.record_epipe_prefill_extra_cache_decode_end(metrics)
     SparseContext.current_phase = "none"
     if metrics is not None:
         metrics.timings_ms["wall_prefill"] = metrics.timings_ms.get("wall_prefill", 0.0) + prefill_ms

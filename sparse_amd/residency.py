@@ -110,6 +110,10 @@ class ResidencyConfig:
     epipe_rs_gate_min_triggers: int = 1
     epipe_rs_gate_skip_steps: int = 8
     epipe_prefill_extra_cache_slots: int = 0
+    epipe_prefill_extra_cache_decode_read: bool = True
+    epipe_prefill_extra_cache_clear_at_decode: bool = False
+    epipe_prefill_extra_cache_persist_requests: bool = False
+    epipe_prefill_extra_cache_max_mb: float = 128.0
     epipe_prefill_mark_transient: bool = True     # staged prefill commits are first in line for eviction
     epipe_promote_transient_on_decode_hit: bool = True
     epipe_rs_buffer_max_groups: int = 4
@@ -177,6 +181,11 @@ class ResidencyConfig:
         c.epipe_rs_gate_min_triggers = _env_int("SPARSE_EPIPE_RS_GATE_MIN_TRIGGERS", 1)
         c.epipe_rs_gate_skip_steps = _env_int("SPARSE_EPIPE_RS_GATE_SKIP_STEPS", 8)
         c.epipe_prefill_extra_cache_slots = _env_int("SPARSE_EPIPE_PREFILL_EXTRA_CACHE_SLOTS", 0)
+        c.epipe_prefill_extra_cache_decode_read = _env_flag("SPARSE_EPIPE_PREFILL_EXTRA_CACHE_DECODE_READ", "1")
+        c.epipe_prefill_extra_cache_clear_at_decode = _env_flag("SPARSE_EPIPE_PREFILL_EXTRA_CACHE_CLEAR_AT_DECODE", "0")
+        c.epipe_prefill_extra_cache_persist_requests = _env_flag(
+            "SPARSE_EPIPE_PREFILL_EXTRA_CACHE_PERSIST_REQUESTS", "0")
+        c.epipe_prefill_extra_cache_max_mb = max(0.0, _env_float("SPARSE_EPIPE_PREFILL_EXTRA_CACHE_MAX_MB", 128.0))
         c.plain_ep_exec_mode = str(
             os.environ.get("SPARSE_PLAIN_EP_EXEC_MODE", "unique_mask") or "unique_mask").strip().lower()
         for k, v in overrides.items():
@@ -428,7 +437,7 @@ class LayerResidency:
         if slot is not None:
             self._record_cached_use(eid, wait_prefetch=True)
             return slot
-        extra = self.extra_cache.get(eid)
+        extra = self._extra_get(eid)
         if extra is not None:
             return extra
         self._event("miss", eid)
@@ -438,6 +447,47 @@ class LayerResidency:
         self._on_demand_access(eid)
         self._cache_put(eid, slot)
         return slot
+
+    # ---- prefill side cache (reference :5637-5720) ------------------------------------
+    def _extra_enabled(self) -> bool:
+        return self.extra_cache.capacity > 0 and bool(self.cfg.epipe_prefill_enable)
+
+    def _extra_readable(self) -> bool:
+        return self._extra_enabled() and not (self.stage == "decode"
+                                              and not self.cfg.epipe_prefill_extra_cache_decode_read)
+
+    def _extra_get(self, eid: int) -> Optional[int]:
+        """Slot of an expert staged during prefill; finding it counts as an ordinary hit."""
+        if not self._extra_readable():
+            return None
+        slot = self.extra_cache.get(eid)
+        if slot is not None:
+            self._event("hit", eid)
+            self.metrics.bump("epipe_prefill_extra_cache_hit_count")
+        return slot
+
+    def _extra_store(self, eid: int, slot: int) -> bool:
+        """Keep a staged payload for later prefill / decode calls: prefill only, bounded by
+        slots and by bytes (reference :5647-5685).  Slots of entries it pushes out return to
+        the pool."""
+        if self.stage != "prefill" or not self._extra_enabled():
+            return False
+        max_bytes = int(float(self.cfg.epipe_prefill_extra_cache_max_mb) * 1024.0 * 1024.0)
+        if (max_bytes > 0 and not self.extra_cache.has(eid)
+                and self.extra_cache.resident_nbytes() + self.expert_bytes > max_bytes):
+            self.metrics.bump("epipe_prefill_extra_cache_no_room_count")
+            return False
+        before = {e: self.extra_cache.peek(e) for e in self.extra_cache.resident_ids()}
+        kept, _updated, _evicted = self.extra_cache.put(eid, slot, nbytes=self.expert_bytes)
+        for e, s_old in before.items():
+            if not self.extra_cache.has(e) or (e == eid and s_old != slot):
+                self._release_slot(s_old)
+        return bool(kept)
+
+    def clear_extra_cache(self) -> int:
+        for eid in self.extra_cache.resident_ids():
+            self._release_slot(self.extra_cache.peek(eid))
+        return self.extra_cache.clear()
 
     def _compute(self, eid: int, slot: Optional[int] = None) -> None:
         """Queue expert ``eid`` for execution, loading it on demand when no slot is given."""
@@ -493,7 +543,7 @@ class LayerResidency:
 
     def _contains_no_touch(self, eid: int) -> bool:
         """Reference :5815-5851."""
-        return self.extra_cache.has(eid) or self.cache.has(eid)
+        return (self._extra_readable() and self.extra_cache.has(eid)) or self.cache.has(eid)
 
     def _headroom_ok(self) -> bool:
         """A transient needs a slot that no cache entry owns."""
@@ -567,12 +617,8 @@ class LayerResidency:
                 use_transient = True
         if not kept:
             self._enqueue(staged_eid, slot)
-            if use_transient and stage == "prefill" and self.extra_cache.capacity > 0:
-                old_extra = {e: self.extra_cache.peek(e) for e in self.extra_cache.resident_ids()}
-                kept, _upd, _ev = self.extra_cache.put(staged_eid, slot, nbytes=self.expert_bytes)
-                for e, s_old in old_extra.items():
-                    if not self.extra_cache.has(e) or (e == staged_eid and s_old != slot):
-                        self._release_slot(s_old)
+            if use_transient and stage == "prefill":
+                kept = self._extra_store(staged_eid, slot)
             if not kept:
                 m.bump("epipe_transient_payload_count")
                 self._retired.append(slot)  # back to the pool once this batch is launched
@@ -775,12 +821,8 @@ class LayerResidency:
             self._cache_put(eid, slot, transient=transient)
             m.bump("epipe_cache_insert_count")
             kept = True
-        elif to_extra and self.extra_cache.capacity > 0:
-            old_extra = {e: self.extra_cache.peek(e) for e in self.extra_cache.resident_ids()}
-            kept, _upd, _ev = self.extra_cache.put(eid, slot, nbytes=self.expert_bytes)
-            for e, s_old in old_extra.items():
-                if not self.extra_cache.has(e) or (e == eid and s_old != slot):
-                    self._release_slot(s_old)
+        elif to_extra:
+            kept = self._extra_store(eid, slot)
         if not kept:
             m.bump("epipe_transient_payload_count")
             self._retired.append(slot)
@@ -893,7 +935,7 @@ class LayerResidency:
         if slot is not None:
             self._record_cached_use(eid, wait_prefetch=True)
             return slot
-        return self.extra_cache.get(eid)
+        return self._extra_get(eid)
 
     def _epipe_miss_triggered(self, segments: Sequence[Segment]) -> Optional[str]:
         """Walk the segments in ascending expert id; at the first miss look a few segments
@@ -1222,6 +1264,9 @@ class LayerResidency:
             self.clear()
         elif clear_cache_metadata:
             self.cache.reset_request_metadata(unpin=True)
+        if not clear_expert_cache and not self.cfg.epipe_prefill_extra_cache_persist_requests:
+            self.flush()
+            self.clear_extra_cache()       # reference :6146-6147
 
     def clear(self) -> None:
         """Drop every resident expert; all slots return to the pool."""
