@@ -31,13 +31,18 @@ Pinned by (tests/test_residency.py and tests/golden/):
                      exactly one wait, ``is_prefetch_hit``, no second load) restated;
                      textbook LRU replay.
   EPIPE executors    (upfront scan, RS residual scan, bounded ready buffer, miss-triggered
-                     look-ahead) parity unpinned against executed reference code: all four
-                     return None unless ``device.type == "cuda"`` (:11881, :12184, :12530,
-                     :12860), so they cannot run in a GPU-less container.  Pinned only by
-                     restatement, hand-made walk-throughs of each executor, and
-                     invariants: every segment computed exactly once, the staged expert
-                     counts exactly one miss, resident experts run before the wait,
-                     outputs equal the plain path.
+  and the whole      look-ahead) golden traces recorded from the reference's own methods
+  state machine      (tests/golden/make_layer_golden.py -> layer_traces.json): the methods are
+                     taken out of the reference source with ``ast`` and run as written
+                     against recording stand-ins for streams, events and weights, because
+                     they refuse to run without a CUDA device (:11881, :12184, :12530,
+                     :12860).  37 cases cover every method switch, late prefetch copies,
+                     prefill commits / side cache / transient marks, the tiered cache,
+                     request resets and the local policy; tests/test_layer_golden.py
+                     replays them through this oracle and through the product.  Hand-made
+                     walk-throughs and invariants (every segment computed exactly once, the
+                     staged expert counts exactly one miss, resident experts run before the
+                     wait) stay in tests/test_residency.py.
 """
 from __future__ import annotations
 

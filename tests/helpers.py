@@ -50,3 +50,11 @@ def oracle_layer(mlp_block):
         shared_gate_w=cpu(sg.weight).reshape(-1) if sg is not None else None,
         family="qwen_shared" if hasattr(mlp_block, "shared_expert") else "deepseek_shared",
     )
+
+
+def copy_is_late(seed: int, layer: int, step: int, eid: int, rate: float) -> bool:
+    """Whether the prefetch copy of expert ``eid`` admitted at ``step`` into ``layer`` is still
+    in flight the first time anyone asks (a pure function of its arguments, so that traces
+    recorded from different implementations agree on it whatever order they ask in)."""
+    import zlib
+    return (zlib.crc32(f"{seed}:{layer}:{step}:{eid}".encode()) % 10000) < int(rate * 10000)
