@@ -11,7 +11,8 @@ Pinned by (tests/test_staging.py): the reference's own known-answer tests, resta
 tests/test_rs_staging.py:60-66 (a wrong forecast neither evicts nor reorders), :94-99
 (a resident hit has precedence over a staged shadow), :134-145 (all 64 access sequences
 over two residents), :152-180 (first-use order of staged experts).  Candidate selection
-is ``oracle/ref_rs.select_candidates``.
+is ``oracle/ref_rs.select_candidates``.  Both are also checked against vectors recorded from
+the reference's own modules (tests/golden/make_staging_golden.py, tests/test_staging_golden.py).
 """
 from __future__ import annotations
 
