@@ -26,6 +26,10 @@ How each function is pinned (see tests/test_oracle_moe.py):
                             invariance, equality with execute_sorted_segments+combine.
   combine_expert_outputs    brute force on tiny inputs, order sensitivity in bf16.
   shared_expert_forward     closed form.
+  every function above      bit-for-bit equality on the CPU with vectors recorded from the
+                            reference's own functions, taken out of its source and run on
+                            small fp32 and bf16 inputs (tests/golden/make_moe_golden.py,
+                            tests/test_moe_golden.py).
   rs_routing                closed form on hand-made probabilities (top-k of a known row,
                             renormalised sum, log / -1e9 pseudo logits), brute-force top-k.
 """
@@ -122,20 +126,23 @@ def combine_expert_outputs(parts: torch.Tensor, expert_ids: torch.Tensor) -> tor
 
 def execute_sorted_segments(x: torch.Tensor, idx: torch.Tensor, w: torch.Tensor,
                             experts: Sequence[ExpertWeights],
-                            order: Optional[Sequence[int]] = None) -> torch.Tensor:
+                            order: Optional[Sequence[int]] = None, stable: bool = True) -> torch.Tensor:
     """World-size-1 form of the EP executor: token x K expansion (:14728-14730), sort by
     expert id and contiguous segments (:13240-13262), per-segment SwiGLU times route
     weight (:13340-13357, :11700-11765), un-permute (:13359-13360), then
     ``combine_expert_outputs`` (:14861-14863).  ``order`` optionally gives the expert
     execution order (EPIPE changes the order, never the values).  The sort is the stable
-    one; the reference's ``argsort`` leaves ties unspecified and only row order inside a
-    segment depends on it."""
+    one by default; the reference's plain ``argsort`` leaves the order of equal ids
+    unspecified, and only row order inside a segment depends on it.  ``stable=False`` makes
+    the very call the reference makes: on the CPU a row's fp32 result can depend on its
+    position inside the segment's matrix product in the last bit, so bit-for-bit comparison
+    with vectors recorded from the reference needs the same row order."""
     T, H = x.shape
     K = idx.shape[1]
     expanded = x.unsqueeze(1).expand(-1, K, -1).reshape(-1, H)
     flat_i = idx.reshape(-1).to(torch.long)
     flat_w = w.reshape(-1).to(expanded.dtype)
-    perm = torch.argsort(flat_i, stable=True)
+    perm = torch.argsort(flat_i, stable=True) if stable else torch.argsort(flat_i)
     sorted_i = flat_i[perm]
     hidden_sorted = expanded[perm]
     w_sorted = flat_w[perm]

@@ -58,3 +58,25 @@ def copy_is_late(seed: int, layer: int, step: int, eid: int, rate: float) -> boo
     recorded from different implementations agree on it whatever order they ask in)."""
     import zlib
     return (zlib.crc32(f"{seed}:{layer}:{step}:{eid}".encode()) % 10000) < int(rate * 10000)
+
+
+def seeded_moe_layer(shape, T, dtype, seed, shared_gate=True, std=0.25):
+    """Inputs of one small layer call, a pure function of its arguments: ``shape`` is
+    ``(H, E, I, K, Is)``.  Used where a fixture stores only outputs: the script that records
+    them and the test that replays them both build the inputs here; ``checksum`` guards
+    against the generator ever producing other numbers."""
+    H, E, I, _K, Is = shape
+    g = torch.Generator().manual_seed(seed)
+
+    def w(*dims):
+        return (torch.randn(*dims, generator=g) * std).to(dtype)
+
+    out = dict(x=torch.randn(T, H, generator=g).to(dtype), gate_w=w(E, H),
+               experts=[(w(I, H), w(I, H), w(H, I)) for _ in range(E)],
+               shared=(w(Is, H), w(Is, H), w(H, Is)) if Is else None,
+               shared_gate_w=w(H) if (Is and shared_gate) else None)
+    total = out["x"].double().abs().sum() + out["gate_w"].double().abs().sum()
+    for triple in out["experts"] + ([out["shared"]] if Is else []):
+        total = total + sum(t.double().abs().sum() for t in triple)
+    out["checksum"] = float(total)
+    return out
