@@ -12,6 +12,7 @@ any causal LM with the Hugging Face call convention (``input_ids``, ``attention_
 """
 from __future__ import annotations
 
+import os
 import time
 from typing import Any, Iterable, List, Optional
 
@@ -102,10 +103,24 @@ def begin_request(*, clear_expert_cache: bool = True, clear_cache_metadata: bool
                                                 clear_cache_metadata=clear_cache_metadata)
 
 
+def _env_flag(name: str, default: str) -> bool:
+    return str(os.environ.get(name, default)).strip().lower() not in ("", "0", "false", "no", "off")
+
+
+def _demote_at_boundary() -> bool:
+    """The reference's switch for the transient demotion and its end-of-decode count
+    (:18530-18531, :18588-18589); on unless both variables say otherwise."""
+    return (_env_flag("SPARSE_SCP_TRANSIENT_PREFILL_CACHE", "0")
+            or _env_flag("SPARSE_EPIPE_DECODE_DEMOTE_PREFILL_TRANSIENT", "1"))
+
+
 def prefill_decode_boundary(metrics: Optional[Metrics] = None) -> None:
-    """Hooks between the prefill pass and the first decode step (:18514-18518)."""
-    DistributedSparseMoeBlock.demote_prefill_scp_transients_for_decode(metrics)
+    """Hooks between the prefill pass and the first decode step (:18530-18537)."""
+    if _demote_at_boundary():
+        DistributedSparseMoeBlock.demote_prefill_scp_transients_for_decode(metrics)
     DistributedSparseMoeBlock.handle_epipe_prefill_extra_cache_decode_boundary(metrics)
+    if _env_flag("SPARSE_SCP_CLEAR_CACHE_BEFORE_DECODE", "0"):
+        DistributedSparseMoeBlock.clear_all_expert_caches()
 
 
 @torch.no_grad()
@@ -149,7 +164,8 @@ def greedy_decode(model: Any, input_ids: torch.Tensor, attention_mask: Optional[
         past = out.past_key_values
         cur = torch.argmax(out.logits[:, -1, :], dim=-1, keepdim=True)
         generated.append(cur)
-    DistributedSparseMoeBlock.record_prefill_scp_transient_decode_end(metrics)
+    if _demote_at_boundary():
+        DistributedSparseMoeBlock.record_prefill_scp_transient_decode_end(metrics)
     DistributedSparseMoeBlock.record_epipe_prefill_extra_cache_decode_end(metrics)
     SparseContext.current_phase = "none"
     if metrics is not None:

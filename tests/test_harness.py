@@ -140,3 +140,66 @@ def test_payload_variants():
                              "state_dict": plain.state_dict()}, 8, 5)
     with pytest.raises(RuntimeError):
         module_from_payload([1, 2, 3], 8, 5)
+
+
+# ---- the reference's generation loop, recorded ------------------------------------------
+PROTOCOL = __import__("json").loads((__import__("pathlib").Path(__file__).resolve().parent / "golden" /
+                                     "decode_protocol.json").read_text())
+
+
+@pytest.mark.parametrize("rec", PROTOCOL, ids=[f"tokens{r['max_new_tokens']}-{len(r['env'])}env" for r in PROTOCOL])
+def test_greedy_decode_follows_the_recorded_sequence_of_the_reference(rec, monkeypatch):
+    """``tests/golden/decode_protocol.json`` holds what the reference's own
+    ``greedy_decode_profiled`` did with a toy LM (written by
+    ``tests/golden/make_protocol_golden.py``): phases, call ids, model calls and boundary hooks
+    in order, and the generated ids."""
+    from sparse_amd.block import DistributedSparseMoeBlock
+    for name in ("SPARSE_SCP_TRANSIENT_PREFILL_CACHE", "SPARSE_EPIPE_DECODE_DEMOTE_PREFILL_TRANSIENT",
+                 "SPARSE_SCP_CLEAR_CACHE_BEFORE_DECODE"):
+        monkeypatch.delenv(name, raising=False)
+    for name, value in rec["env"].items():
+        monkeypatch.setenv(name, value)
+    SparseContext.reset()
+    log = []
+    for hook in ("demote_prefill_scp_transients_for_decode", "handle_epipe_prefill_extra_cache_decode_boundary",
+                 "record_prefill_scp_transient_decode_end", "record_epipe_prefill_extra_cache_decode_end",
+                 "clear_all_expert_caches"):
+        monkeypatch.setattr(DistributedSparseMoeBlock, hook,
+                            classmethod(lambda cls, *a, _n=hook, **k: log.append(["hook", _n])))
+    begin = SparseContext.begin_runtime_call.__func__
+    monkeypatch.setattr(SparseContext, "begin_runtime_call",
+                        classmethod(lambda cls, call_id: (log.append(["begin_runtime_call", int(call_id)]),
+                                                          begin(cls, call_id))[1]))
+    model = ToyCausalLM(50, 16, [_Plain(), _Plain()])
+    forward = model.forward
+
+    def logged(input_ids, attention_mask=None, use_cache=True, past_key_values=None, return_dict=True):
+        log.append(["phase", SparseContext.current_phase])
+        log.append(["model", list(input_ids.shape), None if attention_mask is None else int(attention_mask.shape[1]),
+                    past_key_values is not None])
+        return forward(input_ids, attention_mask=attention_mask, use_cache=use_cache,
+                       past_key_values=past_key_values, return_dict=return_dict)
+
+    model.forward = logged
+    ids = torch.tensor(rec["input_ids"])
+    out = harness.greedy_decode(model, ids, torch.ones_like(ids), rec["max_new_tokens"])
+    assert out.tolist() == rec["output_ids"]
+
+    def normal(entries):
+        """One entry per model call, carrying the phase and call id in force, and the hooks."""
+        seq, phase, call = [], None, None
+        for e in entries:
+            if e[0] == "phase":
+                phase = e[1]
+            elif e[0] == "begin_runtime_call":
+                call = e[1]
+            elif e[0] == "model":
+                seq.append(["model", phase, call, *e[1:]])
+            else:
+                seq.append(e)
+        return seq, phase
+
+    want, want_phase = normal(rec["log"])
+    got, _ = normal(log)
+    assert got == want
+    assert SparseContext.current_phase == want_phase == "none"
