@@ -125,6 +125,12 @@ class ResidencyConfig:
     epipe_decode_no_rs_commit: bool = True
     # execution order for plain EP: unique_mask | full_mask | sorted_segment (same events)
     plain_ep_exec_mode: str = "unique_mask"
+    # The reference's forward reaches the EPIPE executors only through its expert-parallel
+    # paths; a single process (world size 1) runs the plain ascending loop whatever the EPIPE
+    # switches say (utils/eval_core.py:16520-16526).  This build treats the one GPU as an
+    # expert-parallel rank that owns every expert, so EPIPE applies; set this to get the
+    # reference's single-process behaviour instead.
+    world1_exact: bool = False
 
     @classmethod
     def from_env(cls, **overrides) -> "ResidencyConfig":
@@ -188,6 +194,7 @@ class ResidencyConfig:
         c.epipe_prefill_extra_cache_max_mb = max(0.0, _env_float("SPARSE_EPIPE_PREFILL_EXTRA_CACHE_MAX_MB", 128.0))
         c.plain_ep_exec_mode = str(
             os.environ.get("SPARSE_PLAIN_EP_EXEC_MODE", "unique_mask") or "unique_mask").strip().lower()
+        c.world1_exact = _env_flag("SPARSE_HIP_WORLD1_EXACT", "0")
         for k, v in overrides.items():
             if not hasattr(c, k):
                 raise ValueError(f"unknown residency option {k}")
@@ -503,7 +510,7 @@ class LayerResidency:
         if not segments:
             return "empty"
         name = None
-        if self._epipe_stage_enabled() and self.cfg.epipe_mode != "off":
+        if self._epipe_stage_enabled() and self.cfg.epipe_mode != "off" and not self.cfg.world1_exact:
             rs_active = self.cfg.planner_mode == "rs_prefetch"
             mode = self.cfg.epipe_decode_rs_mode
             if self.stage == "decode" and rs_active and mode == "off":

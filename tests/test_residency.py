@@ -516,6 +516,17 @@ def test_miss_triggered_executor_walkthrough():
     assert lay.cache.prefill_scp_transient_ids() == [1] and lay.freq[1] == 1
 
 
+def test_world1_exact_runs_the_plain_loop_whatever_the_epipe_switches_say():
+    """The reference's single-process forward never reaches the EPIPE executors
+    (utils/eval_core.py:16520-16526); with ``world1_exact`` the product does the same, and its
+    events are those of the same method without EPIPE."""
+    got, ex = run_trace("rs-epipe", "product", seed=3, late_rate=0.4, overrides=dict(world1_exact=True))
+    want, ex_rs = run_trace("rs", "product", seed=3, late_rate=0.4)
+    assert set(ex) == {"plain"} == set(ex_rs)
+    for g, w in zip(got, want):
+        assert g["events"] == w["events"] and g["compute"] == w["compute"] and g["h2d"] == w["h2d"]
+
+
 def test_decode_rs_mode_spellings():
     from sparse_amd.residency import normalize_decode_rs_mode
     assert [normalize_decode_rs_mode(m) for m in
