@@ -51,3 +51,18 @@ def select_candidates(ids: Sequence[int], weights: Sequence[float], *, allowed: 
                            below_threshold=sum(1 for v in score.values() if v < minimum))
     ranked = sorted(score, key=score.get, reverse=True)
     return [e for e in ranked if score[e] >= minimum][:budget]
+
+
+def plan_inputs(pred, pred_k: int, norm_topk_prob: bool, dtype):
+    """Flattened ``[T * pred_k]`` expert ids and probabilities the planner scans, from a dense
+    predictor output (utils/eval_core.py:10985-10996): per token the ``pred_k`` largest
+    probabilities in descending order (lower id first among equals), optionally renormalised,
+    rounded to the activation dtype.  Plain Python lists of ints and floats."""
+    import torch
+    pred = torch.as_tensor(pred, dtype=torch.float32)
+    k = min(int(pred.shape[-1]), int(pred_k))
+    order = torch.sort(pred, dim=-1, descending=True, stable=True)
+    vals, ids = order.values[:, :k], order.indices[:, :k]
+    if norm_topk_prob:
+        vals = vals / vals.sum(dim=-1, keepdim=True).clamp_min(1e-12)
+    return ids.reshape(-1).tolist(), vals.to(dtype).to(torch.float32).reshape(-1).tolist()

@@ -27,6 +27,7 @@ from torch import nn
 from . import ops
 from .context import DistEnv, Metrics, SparseContext
 from .residency import Backend, LayerResidency, ResidencyConfig
+from .rs import topk_for_planning
 from .weights import ExpertSlab, HostExpertArena, tile_weight
 
 
@@ -436,13 +437,10 @@ class DistributedSparseMoeBlock(nn.Module):
             SparseContext.routing_cache[target] = (route_v.to(x.dtype), route_i.to(torch.long))
         if self.planner_mode != "rs_prefetch" or tres is None or budget <= 0:
             return None
-        pred_k = min(int(pred.shape[-1]), int(tres.predict_topk()))
-        topv, topi = torch.topk(pred, k=pred_k, dim=-1)
-        if self.norm_topk_prob:
-            topv = topv / topv.sum(dim=-1, keepdim=True).clamp_min(1e-12)
-        T = int(x.shape[0])
+        topi, topv = topk_for_planning(pred, tres.predict_topk(), self.norm_topk_prob, x.dtype)
+        T, pred_k = int(topi.shape[0]), int(topi.shape[1])
         ws.host_rs_topi[:T * pred_k].view(T, pred_k).copy_(topi, non_blocking=True)
-        ws.host_rs_topv[:T * pred_k].view(T, pred_k).copy_(topv.to(x.dtype).float(), non_blocking=True)
+        ws.host_rs_topv[:T * pred_k].view(T, pred_k).copy_(topv, non_blocking=True)
         return (tres, budget, T, pred_k)
 
     def _rs_finish(self, job, ws: _Workspace) -> None:

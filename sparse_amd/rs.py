@@ -64,6 +64,18 @@ class RoutingScoutResidualMLP(nn.Module):
         return torch.softmax(self.head(self.out_norm(h)), dim=-1)
 
 
+def topk_for_planning(pred: torch.Tensor, pred_k: int, norm_topk_prob: bool, dtype: torch.dtype):
+    """What the prefetch planner is fed from a predictor output ``pred [T,E]`` (fp32): the top
+    ``pred_k`` experts per token, renormalised only for models that renormalise their router,
+    with the probabilities rounded to the activation dtype and widened again
+    (utils/eval_core.py:10985-10996).  Returns ``(topi int64 [T,k], topv float32 [T,k])``."""
+    pred_k = min(int(pred.shape[-1]), int(pred_k))
+    topv, topi = torch.topk(pred.to(torch.float32), k=pred_k, dim=-1)
+    if norm_topk_prob:
+        topv = topv / topv.sum(dim=-1, keepdim=True).clamp_min(1e-12)
+    return topi.to(torch.long), topv.to(dtype).to(torch.float32)
+
+
 def random_init_bank(num_layers: int, hidden: int, num_experts: int, hidden_dim: int = 512, seed: int = 0,
                      device: Optional[torch.device] = None) -> List[Optional[nn.Module]]:
     """One seeded random-init predictor per target layer ``1 .. num_layers-1`` (entry 0 is

@@ -43,7 +43,7 @@ ROOT = Path(__file__).resolve().parents[2]
 if str(ROOT) not in sys.path:
     sys.path.insert(0, str(ROOT))
 
-from tests.helpers import copy_is_late  # noqa: E402  (shared with the tests that replay the fixture)
+from tests.helpers import copy_is_late, seeded_prediction  # noqa: E402  (shared with the tests that replay the fixture)
 
 REF = Path("/root/reference/utils/eval_core.py")
 OUT = Path(__file__).resolve().parent
@@ -73,6 +73,7 @@ METHODS = (
     "_build_prefetch_plan_from_prob_predictions", "_build_target_layer_prob_score_map",
     "_build_prefetch_plan_from_score_map", "_resident_keep_bias", "_pick_victims_by_low_value",
     "_admit_prefetch_plan", "_discard_cache_entry_before_prefetch", "_record_prefetch_event",
+    "_compute_and_schedule_next_layer_rs", "_run_rs_mlp_timed", "_next_layer_rs_feature_mode",
     # environment readers
     "_rank_env_value", "_rank_env_int", "_rank_env_float", "_rs_env_int", "_rs_env_float",
     # lifecycle
@@ -204,7 +205,7 @@ def extract(rec: Recorder, env: Dict[str, str], context: NS):
         _env_int=lambda name, default=0: int(env.get(name, default)),
         _env_float=lambda name, default=0.0: float(env.get(name, default)),
         _hclm_cp_now_ns=lambda: 0, tensor_nbytes=lambda t: 0, _append_prefetch_h2d_event=lambda *a, **k: None,
-        Metrics=object)
+        Metrics=object, time=__import__("time"), nn=torch.nn)
     exec(compile(ast.fix_missing_locations(module), str(REF), "exec"), ns)
     return ns, compute, torch
 
@@ -224,6 +225,7 @@ class StubBlock:
         self.expert_offload, self.experts_kind = "cpu", "modulelist"
         self.planner_mode = cfg["planner_mode"]
         self.placement_mode, self.oracle_mode = "round_robin", "none"
+        self.expert_source = self.exec_routing_mode = "router"
         self.comm_rank = self.rank = 0
         self.metrics = Counters()
         self.norm_topk_prob = False
@@ -479,7 +481,8 @@ def run_case(method: str, kw: Dict[str, Any]) -> Dict[str, Any]:
     if cfg["pred_topk"] is not None:
         env["SPARSE_RS_PREFETCH_PRED_TOPK"] = str(cfg["pred_topk"])
     context = NS(current_phase="none", runtime_call_id=-1, layer_blocks={}, global_expert_cache_enabled=False,
-                 prefill_scp_transient_demoted_for_decode=False)
+                 prefill_scp_transient_demoted_for_decode=False, rs_bank=None, rs_bank_layout="next_layer",
+                 rs_bank_source_layers=[l - 1 for l in range(kw["layers"])], routing_cache={})
     recs, blocks = [], []
     torch_mod = None
     for layer in range(kw["layers"]):
@@ -503,6 +506,15 @@ def run_case(method: str, kw: Dict[str, Any]) -> Dict[str, Any]:
         sizes = {e: policy_expert_bytes(e) for e in range(kw["E"])}
         for l, blk in enumerate(blocks):
             blk._light_policy = mod.LocalPolicy(profile, 0, l, sizes, ())
+    dense = bool(kw.get("dense"))
+    if dense:
+        # the reference's own scheduling function runs, fed by stand-in predictors that return a
+        # dense probability matrix rebuilt from the seed by the tests
+        current = {}
+        context.rs_bank = [None] + [(lambda x, _l=l: current[_l]) for l in range(1, kw["layers"])]
+        context.layer_blocks = {l: blk for l, blk in enumerate(blocks)}
+        for blk in blocks:
+            blk.norm_topk_prob = bool(kw.get("norm_topk_prob", False))
     model = RoutingModel(kw["E"], kw["K"], kw["T"], kw["seed"])
     steps, executors = [], []
     for step in range(kw["steps"]):
@@ -519,7 +531,7 @@ def run_case(method: str, kw: Dict[str, Any]) -> Dict[str, Any]:
                     blk.reset_runtime_state_for_new_request(clear_expert_cache=bool(clear), clear_cache_metadata=True)
         context.current_phase, context.runtime_call_id = phase, step
         routes = [model.route() for _ in range(kw["layers"])]
-        planning = cfg["planner_mode"] == "rs_prefetch" and phase == "decode"
+        planning = cfg["planner_mode"] == "rs_prefetch" and phase == "decode" and not dense
         pred_k = blocks[0]._rs_prefetch_predict_topk() if planning else kw["K"]
         preds = [model.predict(routes[l + 1], pred_k) if planning and l + 1 < kw["layers"] else None
                  for l in range(kw["layers"])]
@@ -528,6 +540,17 @@ def run_case(method: str, kw: Dict[str, Any]) -> Dict[str, Any]:
         for rec in recs:
             rec.step = step
         for l, blk in enumerate(blocks):
+            blk._current_forward_batch_size = kw["T"] if phase == "decode" else 1
+            blk._current_forward_seq_len = 1 if phase == "decode" else kw["T"]
+            if dense:
+                if l + 1 < kw["layers"]:
+                    current[l + 1] = seeded_prediction(kw["seed"], step, l, kw["T"], kw["E"])
+                    tgt = blocks[l + 1]
+                    before = set(tgt._prefetched_ids_this_group)
+                    x = torch_mod.zeros(kw["T"], 4, dtype=torch_mod.bfloat16)
+                    blk._compute_and_schedule_next_layer_rs(x=x, seq_len=1 if phase == "decode" else kw["T"])
+                executors.append(execute(blk, torch_mod, cfg, routes[l]))
+                continue
             if cfg["planner_mode"] == "rs_prefetch" and l + 1 < kw["layers"] and phase == "decode":
                 tgt = blocks[l + 1]
                 key = ("next_layer_rs", phase, step, l, l + 1)
@@ -546,8 +569,6 @@ def run_case(method: str, kw: Dict[str, Any]) -> Dict[str, Any]:
                     if len(plan) > 0:
                         tgt._rec.trace.append(("plan", [[int(e), None if v is None else int(v)] for e, v in plan]))
                         tgt._admit_prefetch_plan(plan, group_end=l + 2)
-            blk._current_forward_batch_size = kw["T"] if phase == "decode" else 1
-            blk._current_forward_seq_len = 1 if phase == "decode" else kw["T"]
             executors.append(execute(blk, torch_mod, cfg, routes[l]))
     expect = []
     for blk, rec in zip(blocks, recs):
@@ -558,7 +579,7 @@ def run_case(method: str, kw: Dict[str, Any]) -> Dict[str, Any]:
             compute=[x[1] for x in t if x[0] == "compute"],
             waits=[x[1] for x in t if x[0] == "wait"],
             side_waits=[[x[0], x[1]] for x in t if x[0].startswith("wait_")],
-            plans=[x[1] for x in t if x[0] == "plan"],
+            plans=None if dense else [x[1] for x in t if x[0] == "plan"],
             residents=[int(e) for e in blk._cache.resident_ids()],
             extra=[int(e) for e in blk._epipe_prefill_extra_cache.resident_ids()]))
     return dict(method=method, kw=kw, steps=steps, executors=executors, expect=expect)
@@ -566,7 +587,8 @@ def run_case(method: str, kw: Dict[str, Any]) -> Dict[str, Any]:
 
 def cases() -> List[Tuple[str, Dict[str, Any]]]:
     base = dict(steps=24, layers=3, E=16, K=2, T=4, capacity=4, top_m=3, seed=0, late_rate=0.0, prefill_steps=0,
-                overrides={}, formal=True, policy_costs=None, resets=[])
+                overrides={}, formal=True, policy_costs=None, resets=[], dense=False,
+                norm_topk_prob=False)
 
     def c(method: str, **kw: Any) -> Tuple[str, Dict[str, Any]]:
         return method, {**base, **kw}
@@ -605,6 +627,11 @@ def cases() -> List[Tuple[str, Dict[str, Any]]]:
         c("epipe", prefill_steps=4, capacity=6, T=8,
           overrides=dict(mt, epipe_prefill_enable=True, epipe_prefill_commit=False,
                          epipe_prefill_extra_cache_slots=2, epipe_prefill_lookahead_min_ready_items=1), seed=20),
+        # the reference's own next-layer scheduling function on dense predictor outputs
+        c("rs", dense=True, seed=31), c("rs", dense=True, formal=False, capacity=6, T=8, top_m=5, seed=32),
+        c("rs-epipe", dense=True, late_rate=0.4, seed=33),
+        c("rs", dense=True, norm_topk_prob=True, overrides=dict(pred_topk=3), seed=34),
+        c("rs-epipe", dense=True, late_rate=0.3, prefill_steps=2, seed=35),
         # requests following one another: metadata reset, and reset with the cache cleared
         c("rs-epipe", late_rate=0.3, resets=[[8, 0], [16, 1]], seed=27),
         c("rs", resets=[[6, 0], [12, 0], [18, 1]], formal=False, seed=28),

@@ -80,3 +80,10 @@ def seeded_moe_layer(shape, T, dtype, seed, shared_gate=True, std=0.25):
         total = total + sum(t.double().abs().sum() for t in triple)
     out["checksum"] = float(total)
     return out
+
+
+def seeded_prediction(seed: int, step: int, layer: int, T: int, E: int) -> "torch.Tensor":
+    """Dense predictor output ``[T, E]`` (rows sum to one) for the prefetch planned at ``step``
+    by ``layer`` for the next one; a pure function of its arguments."""
+    g = torch.Generator().manual_seed(1000003 * seed + 1009 * step + layer)
+    return torch.softmax(torch.randn(T, E, generator=g) * 2.0, dim=-1)
