@@ -36,7 +36,7 @@ Pinned by (tests/test_residency.py and tests/golden/):
                      taken out of the reference source with ``ast`` and run as written
                      against recording stand-ins for streams, events and weights, because
                      they refuse to run without a CUDA device (:11881, :12184, :12530,
-                     :12860).  42 cases cover every method switch, late prefetch copies,
+                     :12860).  55 cases cover every method switch, late prefetch copies,
                      prefill commits / side cache / transient marks, the tiered cache,
                      request resets and the local policy; tests/test_layer_golden.py
                      replays them through this oracle and through the product.  Hand-made

@@ -299,6 +299,7 @@ class StubBlock:
             _prefetch_replace_advantage=cfg["replace_advantage"], _prefetch_replace_margin=cfg["replace_margin"],
             _prefetch_allow_active_replace=cfg["allow_active_replace"], _transition_prefetch_enabled=False,
             _global_expert_cache_enabled=False, prefetch_top_m=cfg["prefetch_top_m"],
+            _cache_ttl_steps=cfg["cache_ttl_steps"],
         ).items():
             setattr(self, name, value)
 
@@ -632,6 +633,23 @@ def cases() -> List[Tuple[str, Dict[str, Any]]]:
         c("rs-epipe", dense=True, late_rate=0.4, seed=33),
         c("rs", dense=True, norm_topk_prob=True, overrides=dict(pred_topk=3), seed=34),
         c("rs-epipe", dense=True, late_rate=0.3, prefill_steps=2, seed=35),
+        # less travelled switches of the prefetch planner and the cache guard
+        c("rs", overrides=dict(cache_ttl_steps=2), seed=36),
+        c("rs-epipe", late_rate=0.3, overrides=dict(cache_ttl_steps=3, recent_protect_steps=3), seed=37),
+        c("rs", overrides=dict(protect_mode="minimal"), seed=38),
+        c("rs-epipe", late_rate=0.5, overrides=dict(wait_before_evict=False), seed=39),
+        c("rs", overrides=dict(allow_active_replace=False), capacity=6, seed=40),
+        c("rs", formal=False, overrides=dict(rs_policy="cache_safe"), seed=41),
+        c("rs", formal=False, top_m=6, capacity=8, overrides=dict(min_candidate_score=0.0, replace_advantage=0.0,
+                                                                  replace_margin=1.0), seed=42),
+        c("rr", overrides=dict(cache_ttl_steps=2), seed=43),
+        c("epipe", overrides=dict(epipe_min_ready_experts=2, epipe_min_ready_items=3, epipe_min_missing_experts=2),
+          T=8, capacity=6, seed=44),
+        c("epipe", overrides=dict(epipe_transient_staging=False), seed=45),
+        c("rs-epipe", late_rate=0.3, overrides=dict(epipe_rs_rolling_gate=False), seed=46),
+        c("rs-epipe", late_rate=0.1, overrides=dict(epipe_rs_gate_window=4, epipe_rs_gate_skip_steps=3,
+                                                    epipe_rs_handle_demand_miss=False), seed=47),
+        c("rs-epipe", late_rate=0.3, overrides=dict(epipe_rs_demand_commit=False), seed=48),
         # requests following one another: metadata reset, and reset with the cache cleared
         c("rs-epipe", late_rate=0.3, resets=[[8, 0], [16, 1]], seed=27),
         c("rs", resets=[[6, 0], [12, 0], [18, 1]], formal=False, seed=28),
