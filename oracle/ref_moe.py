@@ -14,12 +14,14 @@ How each function is pinned (see tests/test_oracle_moe.py):
                             tie rule on hand-made ties.  torch.topk leaves tie order
                             unspecified; the rule here is "higher probability first, then
                             lower expert id".
-  deepseek_router           parity unpinned: the reference delegates to the model's own
-                            ``MoEGate`` (third-party, loaded with trust_remote_code, no
-                            version pin, source not in the reference tree).  Restated from
-                            the published DeepSeek-V2 gate: fp32 logits, fp32 softmax,
-                            top-k, times routed_scaling_factor.  Tests compare per-token
-                            index sets.
+  deepseek_router           the reference delegates to the model's own ``MoEGate`` (third-party,
+                            loaded with trust_remote_code, no version pin, source not in the
+                            reference tree), so no reference code exists to run.  Restated
+                            from the published DeepSeek-V2 gate (fp32 logits, fp32 softmax,
+                            top-k, times routed_scaling_factor) and pinned against the port
+                            of that gate in the installed ``transformers``
+                            (``DeepseekV2TopkRouter``, ``greedy`` method): same experts and
+                            weights in fp32 and bf16.
   experts_world1_exact      fp64 per-token closed form sum_k w_k*down(silu(gate x)*up x)
                             (the expected value of the reference's own
                             tests/test_lightweight_policy.py:122-127), permutation
@@ -71,7 +73,7 @@ def deepseek_router(x: torch.Tensor, gate_w: torch.Tensor, top_k: int, routed_sc
                     router_logits: Optional[torch.Tensor] = None):
     """DeepSeek-family router as seen at the reference's call site :9503-9517.
 
-    The gate itself is third-party (parity unpinned, see the module docstring): fp32
+    The gate itself is third-party (see the module docstring for what pins this restatement): fp32
     logits from fp32-cast x and W, fp32 softmax, greedy top-k, weights scaled and cast to
     x.dtype.  Returns (topv, topi, pseudo_logits) with pseudo_logits built as :9490-9499.
     """

@@ -32,7 +32,10 @@ from .weights import ExpertSlab, HostExpertArena, tile_weight
 
 
 def _is_silu(fn: Any) -> bool:
-    return fn is None or fn is F.silu or isinstance(fn, nn.SiLU) or getattr(fn, "__name__", "") == "silu"
+    if fn is None or fn is F.silu or isinstance(fn, nn.SiLU) or getattr(fn, "__name__", "") == "silu":
+        return True
+    # Hugging Face wraps it in its own module class in some versions
+    return type(fn).__name__.lower() in ("silu", "siluactivation")
 
 
 def _bump(metrics: Any, name: str, value: int) -> None:
@@ -230,7 +233,12 @@ class DistributedSparseMoeBlock(nn.Module):
         self.num_layers = int(num_layers)
         self.top_k = int(top_k)
         self.dtype = dtype
-        self.norm_topk_prob = bool(getattr(mlp_block, "norm_topk_prob", False))
+        # newer Hugging Face layouts keep the routing options on the router module
+        gate_mod = getattr(mlp_block, "gate", None)
+        self.norm_topk_prob = bool(getattr(mlp_block, "norm_topk_prob", getattr(gate_mod, "norm_topk_prob", False)))
+        # None: the reference's rule (tensor only for the DeepSeek family, :9485-9488); a harness
+        # sets it when the decoder layer it swaps into expects the other convention
+        self.return_router_logits: Optional[bool] = None
         # enum validation, same messages as the reference (:4475-4498, :4799-4804)
         self.exec_routing_mode = str(routing_mode)
         if self.exec_routing_mode not in ("router", "rs"):
@@ -326,6 +334,8 @@ class DistributedSparseMoeBlock(nn.Module):
 
     # ------------------------------------------------------------------ helpers
     def _return_tensor_only_mlp(self) -> bool:
+        if self.return_router_logits is not None:
+            return not self.return_router_logits
         return self.moe_family == "deepseek_shared"
 
     def _current_stage(self, seq_len: Optional[int] = None) -> str:

@@ -42,9 +42,10 @@ def decoder_layers(model: Any) -> List[Any]:
 
 
 def _expert_count(mlp: Any, default: int = 0) -> int:
-    for name in ("num_experts", "n_routed_experts"):
-        if int(getattr(mlp, name, 0) or 0) > 0:
-            return int(getattr(mlp, name))
+    for owner in (mlp, getattr(mlp, "gate", None)):
+        for name in ("num_experts", "n_routed_experts"):
+            if int(getattr(owner, name, 0) or 0) > 0:
+                return int(getattr(owner, name))
     experts = mlp.experts
     if hasattr(experts, "gate_up_proj"):
         return int(experts.gate_up_proj.shape[0])
@@ -63,8 +64,8 @@ def install_sparse_blocks(model: Any, *, env: Optional[DistEnv] = None, dtype: t
     """Replace every sparse MLP of ``model``'s decoder layers by a block built from it.
 
     Expert count and top-k are read from the module (``num_experts`` / ``n_routed_experts``,
-    ``top_k`` / ``num_experts_per_tok``) as the reference does (:17943-17955); ``top_k``
-    overrides.  Remaining keywords (``expert_offload``, ``expert_cache``, ``planner_mode``,
+    ``top_k`` / ``num_experts_per_tok``) as the reference does (:17943-17955), or from its router
+    module where newer Hugging Face layouts keep them; ``top_k`` overrides.  Remaining keywords (``expert_offload``, ``expert_cache``, ``planner_mode``,
     ``prefetch_top_m``, ``cache_policy`` ...) go to every block unchanged.  With ``rs_dir``
     the next-layer predictor bank is loaded and registered.  Returns the blocks in layer order.
     """
@@ -76,14 +77,19 @@ def install_sparse_blocks(model: Any, *, env: Optional[DistEnv] = None, dtype: t
         mlp = getattr(layer, "mlp", None)
         if mlp is None or isinstance(mlp, DistributedSparseMoeBlock) or not looks_like_sparse_moe_block(mlp):
             continue
+        router = getattr(mlp, "gate", None)
         k = top_k if top_k is not None else int(
-            getattr(mlp, "top_k", 0) or getattr(mlp, "num_experts_per_tok", 0) or 0)
+            getattr(mlp, "top_k", 0) or getattr(mlp, "num_experts_per_tok", 0) or getattr(router, "top_k", 0) or 0)
         if k <= 0:
             raise RuntimeError(f"Cannot infer top_k at layer {idx}")
         block = DistributedSparseMoeBlock(
             layer_idx=idx, mlp_block=mlp, env=env, num_layers=len(layers), num_experts=_expert_count(mlp),
             top_k=k, dtype=dtype, metrics=metrics, rs_dir=rs_dir, rs_require_complete=rs_require_complete,
             **block_kwargs)
+        if hasattr(router, "top_k") and hasattr(mlp, "shared_expert"):
+            # Hugging Face layouts whose router module does the top-k: their decoder layer
+            # consumes a tensor, not (tensor, router_logits)
+            block.return_router_logits = False
         layer.mlp = block
         blocks.append(block)
     if rs_dir and blocks:

@@ -1,0 +1,111 @@
+"""The block swapped into a real Hugging Face Qwen2-MoE model (random weights, tiny config):
+logits and greedy generation must follow the model's own MoE modules."""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _tiny_model(dtype):
+    transformers = pytest.importorskip("transformers")
+    try:
+        from transformers import Qwen2MoeConfig, Qwen2MoeForCausalLM
+    except ImportError:
+        pytest.skip("this transformers has no Qwen2-MoE")
+    cfg = Qwen2MoeConfig(vocab_size=160, hidden_size=128, intermediate_size=256, moe_intermediate_size=64,
+                         shared_expert_intermediate_size=128, num_hidden_layers=3, num_attention_heads=4,
+                         num_key_value_heads=2, num_experts=8, num_experts_per_tok=2, decoder_sparse_step=1,
+                         norm_topk_prob=False, max_position_embeddings=128, mlp_only_layers=[])
+    torch.manual_seed(0)
+    model = Qwen2MoeForCausalLM(cfg).eval()
+    with torch.no_grad():
+        for p in model.parameters():                 # enough spread for routing to be decisive
+            if p.dim() >= 2:
+                p.mul_(3.0)
+    return model.to(dtype)
+
+
+@pytest.mark.parametrize("offload", ["gpu", "cpu"])
+def test_qwen2_moe_model_with_swapped_blocks(device, offload):
+    from sparse_amd import harness
+    from sparse_amd.block import DistributedSparseMoeBlock
+    from sparse_amd.context import DistEnv, Metrics, SparseContext
+    model = _tiny_model(torch.float32).to(device)
+    ids = torch.tensor([[5, 17, 42, 99, 3, 64], [7, 7, 120, 33, 8, 1]], device=device)
+    mask = torch.ones_like(ids)
+    SparseContext.reset()
+    with torch.no_grad():
+        want_logits = model(input_ids=ids, attention_mask=mask, use_cache=False, return_dict=True).logits.float().cpu()
+        want_ids = harness.greedy_decode(model, ids, mask, 6).cpu()
+
+    SparseContext.reset()
+    metrics = Metrics()
+    kw = dict(expert_offload="gpu") if offload == "gpu" else dict(expert_offload="cpu", expert_cache=3)
+    blocks = harness.install_sparse_blocks(model, env=DistEnv(0, 1, 0, device), dtype=torch.float32, metrics=metrics,
+                                           **kw)
+    assert len(blocks) == 3 and all(isinstance(l.mlp, DistributedSparseMoeBlock) for l in model.model.layers)
+    assert blocks[0].top_k == 2 and blocks[0].num_experts == 8 and blocks[0].experts_kind == "fused"
+    with torch.no_grad():
+        harness.begin_request()
+        SparseContext.current_phase = "prefill"
+        SparseContext.begin_runtime_call(0)
+        got_logits = model(input_ids=ids, attention_mask=mask, use_cache=False, return_dict=True).logits.float().cpu()
+        torch.testing.assert_close(got_logits, want_logits, rtol=2e-4, atol=2e-4)
+        harness.begin_request()
+        got_ids = harness.greedy_decode(model, ids, mask, 6, metrics).cpu()
+    assert torch.equal(got_ids, want_ids)
+    if offload == "cpu":
+        assert metrics.cache_miss_count > 0
+
+
+def _tiny_deepseek(dtype):
+    pytest.importorskip("transformers")
+    try:
+        from transformers import DeepseekV2Config, DeepseekV2ForCausalLM
+    except ImportError:
+        pytest.skip("this transformers has no DeepSeek-V2")
+    cfg = DeepseekV2Config(vocab_size=160, hidden_size=128, intermediate_size=256, moe_intermediate_size=64,
+                           num_hidden_layers=3, num_attention_heads=4, num_key_value_heads=4, n_routed_experts=16,
+                           num_experts_per_tok=6, n_shared_experts=2, first_k_dense_replace=1, topk_method="greedy",
+                           routed_scaling_factor=1.0, norm_topk_prob=False, max_position_embeddings=128,
+                           kv_lora_rank=32, q_lora_rank=None, qk_rope_head_dim=16, qk_nope_head_dim=16, v_head_dim=32,
+                           head_dim=16)
+    torch.manual_seed(1)
+    model = DeepseekV2ForCausalLM(cfg).eval()
+    with torch.no_grad():
+        for p in model.parameters():
+            if p.dim() >= 2:
+                p.mul_(3.0)
+    return model.to(dtype)
+
+
+def test_deepseek_v2_model_with_swapped_blocks(device):
+    """DeepSeek-V2-Lite layout: a dense first layer stays as it is, the sparse layers are
+    swapped; routing follows the model's own gate (greedy top-6 of an fp32 softmax)."""
+    from sparse_amd import harness
+    from sparse_amd.block import DistributedSparseMoeBlock
+    from sparse_amd.context import DistEnv, Metrics, SparseContext
+    model = _tiny_deepseek(torch.float32).to(device)
+    ids = torch.tensor([[5, 17, 42, 99, 3, 64], [7, 7, 120, 33, 8, 1]], device=device)
+    mask = torch.ones_like(ids)
+    SparseContext.reset()
+    with torch.no_grad():
+        want_logits = model(input_ids=ids, attention_mask=mask, use_cache=False, return_dict=True).logits.float().cpu()
+        want_ids = harness.greedy_decode(model, ids, mask, 5).cpu()
+    SparseContext.reset()
+    metrics = Metrics()
+    blocks = harness.install_sparse_blocks(model, env=DistEnv(0, 1, 0, device), dtype=torch.float32, metrics=metrics,
+                                           expert_offload="cpu", expert_cache=6)
+    assert [b.layer_idx for b in blocks] == [1, 2]                       # layer 0 is dense
+    assert not isinstance(model.model.layers[0].mlp, DistributedSparseMoeBlock)
+    assert blocks[0].moe_family == "deepseek_shared" and blocks[0].top_k == 6 and blocks[0].num_experts == 16
+    with torch.no_grad():
+        harness.begin_request()
+        SparseContext.current_phase = "prefill"
+        SparseContext.begin_runtime_call(0)
+        got_logits = model(input_ids=ids, attention_mask=mask, use_cache=False, return_dict=True).logits.float().cpu()
+        torch.testing.assert_close(got_logits, want_logits, rtol=2e-4, atol=2e-4)
+        harness.begin_request()
+        got_ids = harness.greedy_decode(model, ids, mask, 5, metrics).cpu()
+    assert torch.equal(got_ids, want_ids)
+    assert metrics.cache_miss_count > 0

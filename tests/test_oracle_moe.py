@@ -241,3 +241,34 @@ def test_rs_routing_closed_form():
     gate_w = torch.randn(E, H, generator=g)
     out, topv, topi, _ = ref_moe.moe_forward(x, gate_w, experts, 2)
     torch.testing.assert_close(ref_moe.moe_forward_routed(x, topv, topi, experts), out)
+
+
+def test_deepseek_router_against_the_transformers_port_of_the_gate():
+    """The reference delegates DeepSeek routing to the checkpoint's own gate, which is not in
+    its tree.  The installed ``transformers`` carries a port of that gate
+    (``DeepseekV2TopkRouter``); with the ``greedy`` method DeepSeek-V2-Lite uses, the oracle
+    must choose the same experts with the same weights."""
+    transformers = pytest.importorskip("transformers")
+    try:
+        from transformers import DeepseekV2Config
+        from transformers.models.deepseek_v2.modeling_deepseek_v2 import DeepseekV2TopkRouter
+    except ImportError:
+        pytest.skip("this transformers has no DeepSeek-V2")
+    g = torch.Generator().manual_seed(11)
+    for dtype, scale in ((torch.float32, 1.0), (torch.bfloat16, 1.0), (torch.float32, 2.5)):
+        cfg = DeepseekV2Config(hidden_size=64, n_routed_experts=16, num_experts_per_tok=6, topk_method="greedy",
+                               routed_scaling_factor=scale, num_hidden_layers=1, vocab_size=32)
+        gate = DeepseekV2TopkRouter(cfg)
+        gate.weight.data = (torch.randn(16, 64, generator=g) * 0.3)
+        x = torch.randn(40, 64, generator=g).to(dtype)
+        gate = gate.to(dtype)
+        with torch.no_grad():
+            logits, weights, idx = gate(x)
+        topv, topi, pseudo = ref_moe.deepseek_router(x, gate.weight.data, 6, routed_scaling_factor=scale)
+        # the third output is the reference's pseudo logits: log(weight) at the chosen experts
+        assert torch.isinf(pseudo).sum() == 40 * (16 - 6)
+        order_ref, order_hf = torch.sort(topi, 1), torch.sort(idx, 1)
+        assert torch.equal(order_ref.values, order_hf.values)
+        # the reference casts the gate's weights to the activation dtype at its call site (:9514)
+        torch.testing.assert_close(torch.gather(topv.float(), 1, order_ref.indices),
+                                   torch.gather(weights.to(dtype).float(), 1, order_hf.indices), rtol=1e-6, atol=1e-7)
