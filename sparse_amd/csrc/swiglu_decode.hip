@@ -133,20 +133,28 @@ __global__ __launch_bounds__(kDecThreads) void decode_ffn_kernel(const DecodeArg
   const uint16_t* wt1 = kGateUp ? w1 + static_cast<size_t>(row0 >> 4) * group_stride + lane * 8 : nullptr;
   const int ND = Kdim >> 6;
 
-  bf16x8 cb[NT][2], cw[NM][kDecTiles][2];  // fragments being multiplied
-  bf16x8 nb[NT][2], nw[NM][kDecTiles][2];  // fragments in flight for the next slice
+  // Two register stages per wavefront, used in turn: while one slice is multiplied the next
+  // one is already in flight and the one after that is requested as soon as its stage is
+  // free.  The steady-state loop below has no branches, so the wait before each batch of
+  // MFMAs counts exactly the newer stage's loads as still outstanding; a conditional load
+  // inside the loop would make every wait a full drain and leave one slice in flight.
+  bf16x8 b0[NT][2], w0s[NM][kDecTiles][2];
+  bf16x8 b1[NT][2], w1s[NM][kDecTiles][2];
+
+  // token columns past the segment read the block's first activation row (always mapped):
+  // their products land in output columns the epilogue never stores, so they need neither a
+  // branch around the loads nor a mask
+  const uint16_t* bsafe = is_shared ? a.act_s : a.act_r;
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt)
+    if (brow[nt] == nullptr) brow[nt] = bsafe;
 
 #define SP_DEC_LOAD(B, W, d)                                                             \
   do {                                                                                   \
     const int koff_ = (d) << 6;                                                          \
     _Pragma("unroll") for (int nt = 0; nt < NT; ++nt) {                                  \
-      if (brow[nt] != nullptr) {                                                         \
-        B[nt][0] = ld_bf16x8(brow[nt] + koff_ + (q << 4));                               \
-        B[nt][1] = ld_bf16x8(brow[nt] + koff_ + (q << 4) + 8);                           \
-      } else {                                                                           \
-        B[nt][0] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};                                       \
-        B[nt][1] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};                                       \
-      }                                                                                  \
+      B[nt][0] = ld_bf16x8(brow[nt] + koff_ + (q << 4));                                 \
+      B[nt][1] = ld_bf16x8(brow[nt] + koff_ + (q << 4) + 8);                             \
     }                                                                                    \
     _Pragma("unroll") for (int tl = 0; tl < kDecTiles; ++tl) {                           \
       const size_t o_ = tl * group_stride + (static_cast<size_t>(d) << 10);              \
@@ -159,35 +167,45 @@ __global__ __launch_bounds__(kDecThreads) void decode_ffn_kernel(const DecodeArg
     }                                                                                    \
   } while (0)
 
-  int d = wave;
-  if (d < ND) SP_DEC_LOAD(cb, cw, d);
-  for (; d < ND; d += kDecWaves) {
-    const bool more = d + kDecWaves < ND;
-    if (more) SP_DEC_LOAD(nb, nw, d + kDecWaves);
-#pragma unroll
-    for (int tl = 0; tl < kDecTiles; ++tl)
-#pragma unroll
-      for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-        for (int m = 0; m < NM; ++m) {
-          acc[m][tl][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cw[m][tl][0], cb[nt][0], acc[m][tl][nt], 0, 0, 0);
-          acc[m][tl][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cw[m][tl][1], cb[nt][1], acc[m][tl][nt], 0, 0, 0);
-        }
-    if (more) {
-#pragma unroll
-      for (int nt = 0; nt < NT; ++nt) {
-        cb[nt][0] = nb[nt][0];
-        cb[nt][1] = nb[nt][1];
-      }
-#pragma unroll
-      for (int m = 0; m < NM; ++m)
-#pragma unroll
-        for (int tl = 0; tl < kDecTiles; ++tl) {
-          cw[m][tl][0] = nw[m][tl][0];
-          cw[m][tl][1] = nw[m][tl][1];
-        }
-    }
+#define SP_DEC_MFMA(B, W)                                                                                   \
+  do {                                                                                                      \
+    _Pragma("unroll") for (int tl = 0; tl < kDecTiles; ++tl)                                                \
+    _Pragma("unroll") for (int nt = 0; nt < NT; ++nt)                                                       \
+    _Pragma("unroll") for (int m = 0; m < NM; ++m) {                                                        \
+      acc[m][tl][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(W[m][tl][0], B[nt][0], acc[m][tl][nt], 0, 0, 0); \
+      acc[m][tl][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(W[m][tl][1], B[nt][1], acc[m][tl][nt], 0, 0, 0); \
+    }                                                                                                       \
+  } while (0)
+
+  // slice number i of this wavefront is 64-wide slice wave + i * kDecWaves of the reduction
+  const int n = (ND - wave + kDecWaves - 1) / kDecWaves;
+#define SP_DEC_SLICE(i) (wave + (i) * kDecWaves)
+  int i = 0;
+  // the first two loads are unconditional (a wavefront with fewer slices re-reads the last
+  // valid one and never multiplies it): a branch around them would merge two different
+  // outstanding-load states at the loop's entry and turn the loop's waits into full drains
+  SP_DEC_LOAD(b0, w0s, min(SP_DEC_SLICE(0), ND - 1));
+  SP_DEC_LOAD(b1, w1s, min(SP_DEC_SLICE(1), ND - 1));
+  for (; i + 4 <= n; i += 2) {
+    // fences keep the scheduler from sinking a stage's reload below the other stage's MFMAs
+    SP_DEC_MFMA(b0, w0s);
+    __builtin_amdgcn_sched_barrier(0);
+    SP_DEC_LOAD(b0, w0s, SP_DEC_SLICE(i + 2));
+    __builtin_amdgcn_sched_barrier(0);
+    SP_DEC_MFMA(b1, w1s);
+    __builtin_amdgcn_sched_barrier(0);
+    SP_DEC_LOAD(b1, w1s, SP_DEC_SLICE(i + 3));
+    __builtin_amdgcn_sched_barrier(0);
   }
+  // up to three slices left; stage 0 holds slice i, stage 1 slice i + 1
+  if (i < n) {
+    SP_DEC_MFMA(b0, w0s);
+    if (i + 2 < n) SP_DEC_LOAD(b0, w0s, SP_DEC_SLICE(i + 2));
+  }
+  if (i + 1 < n) SP_DEC_MFMA(b1, w1s);
+  if (i + 2 < n) SP_DEC_MFMA(b0, w0s);
+#undef SP_DEC_SLICE
+#undef SP_DEC_MFMA
 #undef SP_DEC_LOAD
 
   // ---- split-K partials meet in LDS ----------------------------------------
