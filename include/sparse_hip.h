@@ -51,6 +51,8 @@ extern "C" {
 #define SPARSE_HIP_MAX_EXPERTS 256
 #define SPARSE_HIP_MAX_TOPK 16
 #define SPARSE_HIP_DECODE_MAX_TOKENS 32
+#define SPARSE_HIP_ROUTE_PACKED_MAX_TOKENS 16
+#define SPARSE_HIP_ROUTE_PACKED_ROWS 64
 
 /* ---- library identity ------------------------------------------------------ */
 
@@ -160,6 +162,23 @@ int sparse_hip_route_decode(const void* x_dev, const void* wg_dev, const void* w
                             void* shared_gate_dev, void* topv_dev, int64_t* topi_dev, int32_t* perm_dev,
                             int32_t* inv_perm_dev, int32_t* seg_offsets_dev, int32_t* active_eids_dev,
                             int32_t* n_active_dev, int32_t* counter_dev, void* stream);
+
+/*
+ * The same routing step (utils/eval_core.py:9519-9520, :9590-9595, and the stable bucketing
+ * of :13224-13243) for bf16 activations and at most SPARSE_HIP_ROUTE_PACKED_MAX_TOKENS tokens,
+ * on a gate matrix packed ahead of time so that one workgroup streams it with contiguous
+ * wave loads and finishes logits, top-k and permutation without waiting for another
+ * workgroup: `gate_packed_dev` is a [SPARSE_HIP_ROUTE_PACKED_ROWS, H] bf16 matrix in the tiled
+ * layout (`sparse_hip_tile_weight` of the row-major matrix whose rows are the E gate rows,
+ * then the shared-expert gate vector if `has_shared_gate`, then zero rows); H % 64 == 0 and
+ * E + has_shared_gate <= SPARSE_HIP_ROUTE_PACKED_ROWS.  Outputs are those of
+ * `sparse_hip_route_decode`; the logits differ from it only in the order of the fp32 sum.
+ */
+int sparse_hip_route_decode_packed(const void* x_dev, const void* gate_packed_dev, int has_shared_gate,
+                                   int logits_dtype, int T, int H, int E, int K, int renorm, void* logits_dev,
+                                   void* shared_gate_dev, void* topv_dev, int64_t* topi_dev, int32_t* perm_dev,
+                                   int32_t* inv_perm_dev, int32_t* seg_offsets_dev, int32_t* active_eids_dev,
+                                   int32_t* n_active_dev, void* stream);
 
 /* ---- A4/A6: grouped SwiGLU expert FFN -------------------------------------- */
 

@@ -64,6 +64,8 @@ SIGNATURES = {
     "sparse_hip_gate_topk": (_i, [_vp, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp]),
     "sparse_hip_route_decode": (
         _i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "sparse_hip_route_decode_packed": (
+        _i, [_vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "sparse_hip_permute_ws_bytes": (_sz, [_i, _i, _i]),
     "sparse_hip_permute_build": (_i, [_vp, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "sparse_hip_grouped_swiglu_decode": (

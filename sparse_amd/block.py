@@ -305,6 +305,9 @@ class DistributedSparseMoeBlock(nn.Module):
         self.shared_gate_weight = (
             sg.weight.detach().to(self.device, self.dtype).reshape(-1).contiguous() if sg is not None else None)
         self.logits_dtype = torch.float32 if self.moe_family == "deepseek_shared" else self.dtype
+        # decode-size batches route on a packed copy of the gate (and shared gate) rows where
+        # the shapes allow it; everything else reads the row-major weights
+        self.gate_packed = ops.pack_router_gate(self.gate_weight, self.shared_gate_weight)
 
         E, H, I = self.num_experts, self.hidden_size, self.inter_size
         self.local_expert_ids = list(range(E))
@@ -358,6 +361,11 @@ class DistributedSparseMoeBlock(nn.Module):
         Returns the logits, a fresh tensor the caller owns."""
         logits = torch.empty((x.shape[0], self.num_experts), device=x.device, dtype=self.logits_dtype)
         shared_gate = ws.shared_gate if self.shared_gate_weight is not None else None
+        if (self.gate_packed is not None and x.shape[0] <= ops.ROUTE_PACKED_MAX_TOKENS
+                and self.routed_scaling_factor == 1.0):
+            ops.route_decode_packed(x, self.gate_packed, self.num_experts, self.shared_gate_weight is not None,
+                                    self.top_k, self.norm_topk_prob, logits, shared_gate, ws.topv, ws.topi, ws.perm)
+            return logits
         if x.shape[0] <= ops.DECODE_MAX_TOKENS and self.routed_scaling_factor == 1.0:
             ops.route_decode(x, self.gate_weight, self.shared_gate_weight, self.top_k, self.norm_topk_prob, logits,
                              shared_gate, ws.topv, ws.topi, ws.perm, ws.route_counter)

@@ -178,13 +178,14 @@ __global__ __launch_bounds__(256) void router_logits_mfma_kernel(
 // l, l+64, l+128, l+192.  Selection runs K rounds of a wave-wide arg-max whose order is
 // (probability descending, expert id ascending): the largest probability first, then
 // the lowest id among the lanes that hold it.  All cross-lane steps are DPP reductions.
+// Lane r < K also returns the r-th selected expert.
 // ---------------------------------------------------------------------------
 constexpr int kTopkWaves = 4;
 constexpr int kTopkNV = SPARSE_HIP_MAX_EXPERTS / 64;
 
 template <typename TL, typename TO>
-__device__ __forceinline__ void topk_token(const TL* __restrict__ row, int E, int K, int renorm,
-                                           TO* __restrict__ topv_row, int64_t* __restrict__ topi_row, int lane) {
+__device__ __forceinline__ int topk_token(const TL* __restrict__ row, int E, int K, int renorm,
+                                          TO* __restrict__ topv_row, int64_t* __restrict__ topi_row, int lane) {
   float p[kTopkNV];
   float m = -INFINITY;
 #pragma unroll
@@ -244,6 +245,7 @@ __device__ __forceinline__ void topk_token(const TL* __restrict__ row, int E, in
     Elem<TO>::store(topv_row + lane, v);
     topi_row[lane] = static_cast<int64_t>(sel_i);
   }
+  return sel_i;  // lane r < K: the r-th selected expert
 }
 
 template <typename TL, typename TO>
@@ -280,6 +282,7 @@ struct RouteArgs {
   int32_t* n_active;
   int32_t* counter;
   int32_t T, H, E, K, renorm;
+  int32_t packed_shared_gate;  // packed gate matrix only: row E is the shared-expert gate vector
 };
 
 constexpr int kRouteThreads = 1024;
@@ -310,31 +313,44 @@ __device__ __forceinline__ void permute_small_block(const int64_t* __restrict__ 
     }
   }
   __syncthreads();
-  if (tid < E) {  // every thread reads the same mask words at a time: LDS broadcasts
-    int32_t off = 0, act = 0;
-    for (int e0 = 0; e0 < E; e0 += 16) {  // words past E are zero
-      uint4 m4[4];
+  // thread e < E owns expert e: segment start = items of lower ids (an exclusive prefix sum
+  // of the popcounts, scanned inside each wavefront and carried across the at most four
+  // wavefronts through LDS), rank among the active experts likewise
+  constexpr int kScanWaves = SPARSE_HIP_MAX_EXPERTS / 64;
+  __shared__ int32_t wave_items[kScanWaves], wave_active[kScanWaves];
+  const int lane = tid & 63, wave = tid >> 6;
+  int32_t mine = 0, upto = 0, act = 0;
+  if (tid < SPARSE_HIP_MAX_EXPERTS) {
+    mine = (tid < E) ? __popc(mask[tid]) : 0;
+    upto = mine;
 #pragma unroll
-      for (int q = 0; q < 4; ++q) m4[q] = *reinterpret_cast<const uint4*>(&mask[e0 + 4 * q]);
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const uint32_t w[4] = {m4[q].x, m4[q].y, m4[q].z, m4[q].w};
-#pragma unroll
-        for (int c = 0; c < 4; ++c) {
-          const int32_t cnt = __popc(w[c]);
-          if (e0 + 4 * q + c < tid) {
-            off += cnt;
-            act += cnt > 0;
-          }
-        }
+    for (int d = 1; d < 64; d <<= 1) {
+      const int32_t below = __shfl_up(upto, d);
+      if (lane >= d) upto += below;
+    }
+    const unsigned long long has = __ballot(mine > 0);
+    act = __popcll(has & ((1ull << lane) - 1ull));
+    if (lane == 63) {
+      wave_items[wave] = upto;
+      wave_active[wave] = __popcll(has);
+    }
+  }
+  if (E > 64) {  // the same for every thread of the block
+    __syncthreads();
+    if (tid < SPARSE_HIP_MAX_EXPERTS) {
+      for (int w = 0; w < wave; ++w) {
+        upto += wave_items[w];
+        act += wave_active[w];
       }
     }
-    const int32_t mine = __popc(mask[tid]);
+  }
+  if (tid < E) {
+    const int32_t off = upto - mine;
     base[tid] = off;
     seg_offsets[tid] = off;
     if (mine > 0) active_eids[act] = tid;
     if (tid == E - 1) {
-      seg_offsets[E] = off + mine;
+      seg_offsets[E] = upto;
       n_active[0] = act + (mine > 0);
     }
   }
@@ -430,6 +446,112 @@ __global__ __launch_bounds__(kRouteThreads) void route_decode_kernel(const Route
     __syncthreads();
   }
   permute_small_block(a.topi, a.T, a.K, E, a.perm, a.inv_perm, a.seg_offsets, a.active_eids, a.n_active);
+}
+
+// ---------------------------------------------------------------------------
+// Decode router for up to 16 bf16 tokens in ONE workgroup, on a gate matrix packed ahead of
+// time: 64 rows (the E <= 64 gate rows, then the shared-expert gate vector when there is
+// one, then zero rows) in the tiled weight layout, so that every load instruction of a
+// wavefront reads 1 KB straight, as the expert kernels do.  No step waits for another
+// workgroup or reads its own results back from memory: the 16 wavefronts take the 64-wide
+// k blocks in turn and multiply the token rows (A operand) with the four 16-row groups (B
+// operand) as 16x16x32 MFMAs, two blocks = 20 loads in flight before the first MFMA; the 16
+// partial tiles are folded to 8 and summed in wavefront order in LDS; wavefront t runs
+// softmax/top-k of token t on the LDS copy of its logits, and the permutation is built from
+// the selections kept in LDS.
+// ---------------------------------------------------------------------------
+constexpr int kRpTok = SPARSE_HIP_ROUTE_PACKED_MAX_TOKENS;
+static_assert(kRpTok == kRouteWaves && SPARSE_HIP_ROUTE_PACKED_ROWS == kRlRows, "one wavefront per token, four 16-row groups");
+
+template <typename TL>
+__global__ __launch_bounds__(kRouteThreads) void route_decode_packed_kernel(const RouteArgs a) {
+  __shared__ float part[kRouteWaves / 2][kRpTok][kRlPad];
+  __shared__ float s_logit[kRpTok][kRlRows];
+  __shared__ int64_t s_topi[kRpTok * SPARSE_HIP_MAX_TOPK];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int r = lane & 15, q = lane >> 4;
+  const int T = a.T, H = a.H, E = a.E;
+  const int R = E + (a.packed_shared_gate ? 1 : 0);
+  const uint16_t* xrow = static_cast<const uint16_t*>(a.x) + static_cast<size_t>(min(r, T - 1)) * H + q * 16;
+  const uint16_t* wt = static_cast<const uint16_t*>(a.wg) + lane * 8;
+  const size_t group_stride = static_cast<size_t>(16) * H;
+  const int nblk = H >> 6;
+  f32x4 acc[4];
+#pragma unroll
+  for (int nt = 0; nt < 4; ++nt) acc[nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  int b = wave;
+  for (; b + kRouteWaves < nblk; b += 2 * kRouteWaves) {
+    bf16x8 av[2][2], bv[2][4][2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int blk = b + j * kRouteWaves;
+      av[j][0] = *reinterpret_cast<const bf16x8*>(xrow + blk * 64);
+      av[j][1] = *reinterpret_cast<const bf16x8*>(xrow + blk * 64 + 8);
+#pragma unroll
+      for (int nt = 0; nt < 4; ++nt) {
+        const uint16_t* p = wt + nt * group_stride + static_cast<size_t>(blk) * 1024;
+        bv[j][nt][0] = *reinterpret_cast<const bf16x8*>(p);
+        bv[j][nt][1] = *reinterpret_cast<const bf16x8*>(p + 512);
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);  // all 20 loads in flight before the first MFMA
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt)
+          acc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[j][h], bv[j][nt][h], acc[nt], 0, 0, 0);
+  }
+  if (b < nblk) {
+    const bf16x8 av0 = *reinterpret_cast<const bf16x8*>(xrow + b * 64);
+    const bf16x8 av1 = *reinterpret_cast<const bf16x8*>(xrow + b * 64 + 8);
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt) {
+      const uint16_t* p = wt + nt * group_stride + static_cast<size_t>(b) * 1024;
+      acc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av0, *reinterpret_cast<const bf16x8*>(p), acc[nt], 0, 0, 0);
+      acc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av1, *reinterpret_cast<const bf16x8*>(p + 512), acc[nt], 0, 0, 0);
+    }
+  }
+  // D: lane holds gate row nt*16 + r for tokens q*4 .. q*4+3.  Wavefronts 8..15 hand their
+  // tiles to wavefronts 0..7, whose sums are then added in wavefront order.
+  if (wave >= kRouteWaves / 2) {
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) part[wave - kRouteWaves / 2][q * 4 + v][nt * 16 + r] = acc[nt][v];
+  }
+  __syncthreads();
+  if (wave < kRouteWaves / 2) {
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) part[wave][q * 4 + v][nt * 16 + r] += acc[nt][v];
+  }
+  __syncthreads();
+  {
+    const int tok = tid >> 6, col = tid & 63;
+    float sum = part[0][tok][col];
+#pragma unroll
+    for (int w = 1; w < kRouteWaves / 2; ++w) sum += part[w][tok][col];
+    if (tok < T && col < R) {
+      if (col < E) {
+        Elem<TL>::store(static_cast<TL*>(a.logits) + static_cast<size_t>(tok) * E + col, sum);
+        s_logit[tok][col] = Elem<TL>::round(sum);
+      } else {
+        static_cast<uint16_t*>(a.shared_gate)[tok] = f32_to_bf16_bits(sum);
+      }
+    }
+  }
+  __syncthreads();
+  if (wave < T) {
+    const int sel = topk_token<float, uint16_t>(s_logit[wave], E, a.K, a.renorm,
+                                                static_cast<uint16_t*>(a.topv) + static_cast<size_t>(wave) * a.K,
+                                                a.topi + static_cast<size_t>(wave) * a.K, lane);
+    if (lane < a.K) s_topi[wave * a.K + lane] = static_cast<int64_t>(sel);
+  }
+  __syncthreads();
+  permute_small_block(s_topi, T, a.K, E, a.perm, a.inv_perm, a.seg_offsets, a.active_eids, a.n_active);
 }
 
 template <typename T, typename TL>
@@ -536,11 +658,44 @@ int sparse_hip_route_decode(const void* x_dev, const void* wg_dev, const void* w
   SP_REQUIRE(wsg_dev == nullptr || shared_gate_dev != nullptr, "route_decode: shared gate output is NULL");
   RouteArgs a = {x_dev,     wg_dev,       wsg_dev,         logits_dev,      shared_gate_dev, topv_dev,   topi_dev,
                  perm_dev,  inv_perm_dev, seg_offsets_dev, active_eids_dev, n_active_dev,    counter_dev,
-                 T,         H,            E,               K,               renorm};
+                 T,         H,            E,               K,               renorm,          0};
   hipStream_t st = as_stream(stream);
   if (dtype == SPARSE_HIP_F32) return launch_route_decode<float, float>(a, st);
   if (logits_dtype == SPARSE_HIP_F32) return launch_route_decode<uint16_t, float>(a, st);
   return launch_route_decode<uint16_t, uint16_t>(a, st);
+}
+
+int sparse_hip_route_decode_packed(const void* x_dev, const void* gate_packed_dev, int has_shared_gate,
+                                   int logits_dtype, int T, int H, int E, int K, int renorm, void* logits_dev,
+                                   void* shared_gate_dev, void* topv_dev, int64_t* topi_dev, int32_t* perm_dev,
+                                   int32_t* inv_perm_dev, int32_t* seg_offsets_dev, int32_t* active_eids_dev,
+                                   int32_t* n_active_dev, void* stream) {
+  SP_REQUIRE(logits_dtype == SPARSE_HIP_BF16 || logits_dtype == SPARSE_HIP_F32,
+             "route_decode_packed: logits_dtype must be bf16 or fp32");
+  SP_REQUIRE(T >= 1 && T <= SPARSE_HIP_ROUTE_PACKED_MAX_TOKENS, "route_decode_packed: T=%d outside [1,%d]", T,
+             SPARSE_HIP_ROUTE_PACKED_MAX_TOKENS);
+  SP_REQUIRE(H > 0 && H % 64 == 0, "route_decode_packed: H=%d must be a positive multiple of 64", H);
+  SP_REQUIRE(E >= 1 && E + (has_shared_gate ? 1 : 0) <= SPARSE_HIP_ROUTE_PACKED_ROWS,
+             "route_decode_packed: E=%d (+ shared gate row) exceeds the %d packed rows", E,
+             SPARSE_HIP_ROUTE_PACKED_ROWS);
+  SP_REQUIRE(K >= 1 && K <= SPARSE_HIP_MAX_TOPK && K <= E, "route_decode_packed: K=%d outside [1,min(%d,E)]", K,
+             SPARSE_HIP_MAX_TOPK);
+  SP_REQUIRE(x_dev && gate_packed_dev && logits_dev && topv_dev && topi_dev && perm_dev && inv_perm_dev &&
+                 seg_offsets_dev && active_eids_dev && n_active_dev,
+             "route_decode_packed: NULL pointer");
+  SP_REQUIRE(!has_shared_gate || shared_gate_dev != nullptr, "route_decode_packed: shared gate output is NULL");
+  RouteArgs a = {x_dev,    gate_packed_dev, nullptr,         logits_dev,      shared_gate_dev, topv_dev, topi_dev,
+                 perm_dev, inv_perm_dev,    seg_offsets_dev, active_eids_dev, n_active_dev,    nullptr,
+                 T,        H,               E,               K,               renorm,          has_shared_gate ? 1 : 0};
+  hipStream_t st = as_stream(stream);
+  ProfScope prof(SPARSE_HIP_K_ROUTE_DECODE, st);
+  if (logits_dtype == SPARSE_HIP_F32) {
+    hipLaunchKernelGGL((route_decode_packed_kernel<float>), dim3(1), dim3(kRouteThreads), 0, st, a);
+  } else {
+    hipLaunchKernelGGL((route_decode_packed_kernel<uint16_t>), dim3(1), dim3(kRouteThreads), 0, st, a);
+  }
+  SP_LAUNCH_CHECK("route_decode_packed_kernel");
+  return SPARSE_HIP_OK;
 }
 
 }  // extern "C"

@@ -143,6 +143,50 @@ def route_decode(x: torch.Tensor, wg: torch.Tensor, wsg: Optional[torch.Tensor],
     _lib.check(rc, "sparse_hip_route_decode")
 
 
+ROUTE_PACKED_MAX_TOKENS = 16
+ROUTE_PACKED_ROWS = 64
+
+
+def pack_router_gate(wg: torch.Tensor, wsg: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
+    """The gate matrix ``route_decode_packed`` reads: 64 bf16 rows (the E gate rows, then the
+    shared-expert gate vector when there is one, then zeros) in the tiled weight layout,
+    flattened.  ``None`` when the shapes do not fit (more than 64 rows, H not a multiple of
+    64, not bf16): the caller then stays on ``route_decode``."""
+    from .weights import tile_weight
+    E, H = wg.shape
+    rows = E + (1 if wsg is not None else 0)
+    if wg.dtype != torch.bfloat16 or H % 64 or rows > ROUTE_PACKED_ROWS:
+        return None
+    full = torch.zeros((ROUTE_PACKED_ROWS, H), dtype=wg.dtype, device=wg.device)
+    full[:E] = wg
+    if wsg is not None:
+        full[E] = wsg.reshape(-1).to(wg.dtype)
+    return tile_weight(full).contiguous()
+
+
+def route_decode_packed(x: torch.Tensor, gate_packed: torch.Tensor, num_experts: int, has_shared_gate: bool, k: int,
+                        renorm: bool, logits: torch.Tensor, shared_gate: Optional[torch.Tensor], topv: torch.Tensor,
+                        topi: torch.Tensor, perm: Permutation) -> None:
+    """Router logits + top-k + permutation of up to 16 bf16 tokens by one workgroup, on the
+    matrix ``pack_router_gate`` made."""
+    lib = _lib.load()
+    T, H = x.shape
+    E = int(num_experts)
+    _need(x, "x", torch.bfloat16)
+    _need(gate_packed, "packed gate", torch.bfloat16, (ROUTE_PACKED_ROWS * H,))
+    _need(logits, "logits", None, (T, E))
+    _need(topv, "topv", x.dtype, (T, k))
+    _need(topi, "topi", torch.int64, (T, k))
+    if has_shared_gate:
+        _need(shared_gate, "shared gate logits", x.dtype, (T,))
+    rc = lib.sparse_hip_route_decode_packed(_ptr(x), _ptr(gate_packed), int(bool(has_shared_gate)),
+                                            dtype_code(logits.dtype), T, H, E, int(k), int(bool(renorm)),
+                                            _ptr(logits), _ptr(shared_gate), _ptr(topv), _ptr(topi),
+                                            _ptr(perm.perm), _ptr(perm.inv_perm), _ptr(perm.seg_offsets),
+                                            _ptr(perm.active_eids), _ptr(perm.n_active), _stream())
+    _lib.check(rc, "sparse_hip_route_decode_packed")
+
+
 # --------------------------------------------------------------------------- experts
 def make_experts(slab: torch.Tensor, expert_slot: torch.Tensor, num_experts: int, hidden: int, inter: int,
                  slot_stride_bytes: Optional[int] = None) -> Experts:

@@ -188,6 +188,62 @@ def test_route_decode_shapes_against_oracle(device, T, E, K):
     assert n == p_active.size and np.array_equal(perm.active_eids.cpu().numpy()[:n], p_active)
 
 
+@pytest.mark.parametrize("ldt", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("T,H,E,K,shared_gate,renorm", [
+    (1, 2048, 60, 4, True, False), (8, 2048, 60, 4, True, False), (3, 2048, 64, 6, False, True),
+    (16, 2048, 63, 8, True, False), (8, 64, 60, 4, True, False), (5, 2560, 8, 8, True, True),
+    (16, 4096, 64, 1, False, False), (7, 192, 15, 3, True, False), (2, 1088, 33, 16, False, False)])
+def test_route_decode_packed_shapes(device, T, H, E, K, shared_gate, renorm, ldt):
+    """One-workgroup decode router on the packed gate matrix (one to sixty-four rows, H from
+    one 64-wide block to several per wavefront, an odd number of blocks): logits and shared
+    gate against fp32 linear algebra, top-k and permutation bit for bit what gate_topk and
+    permute_build return on the logits it wrote, indices against the oracle's rule wherever
+    those logits leave no rounding tie, and the same answer call after call."""
+    ops = _ops()
+    dtype = torch.bfloat16
+    layer = make_layer(H, E, 64, K, Is=64, shared_gate=shared_gate, dtype=dtype, seed=23 + T)
+    wsg = layer["shared_gate_w"].to(device) if shared_gate else None
+    packed = ops.pack_router_gate(layer["gate_w"].to(device), wsg)
+    assert packed is not None and packed.numel() == 64 * H
+    for rep in range(2):
+        x = make_hidden(T, H, dtype, seed=400 + rep)
+        logits = torch.empty(T, E, dtype=ldt, device=device)
+        sg = torch.empty(T, dtype=dtype, device=device) if shared_gate else None
+        topv = torch.empty(T, K, dtype=dtype, device=device)
+        topi = torch.empty(T, K, dtype=torch.int64, device=device)
+        perm = ops.Permutation(T, K, E, device)
+        ops.route_decode_packed(x.to(device), packed, E, shared_gate, K, renorm, logits, sg, topv, topi, perm)
+        torch.cuda.synchronize()
+        ref = torch.nn.functional.linear(x.float(), layer["gate_w"].float())
+        tol = dict(rtol=1e-2, atol=1e-2) if ldt == torch.bfloat16 else dict(rtol=1e-4, atol=1e-4)
+        torch.testing.assert_close(logits.float().cpu(), ref, **tol)
+        if shared_gate:
+            ref_sg = torch.nn.functional.linear(x.float(), layer["shared_gate_w"].float().reshape(1, -1)).reshape(-1)
+            torch.testing.assert_close(sg.float().cpu(), ref_sg, rtol=1e-2, atol=1e-2)
+        topv_a, topi_a = ops.gate_topk(logits, K, renorm=renorm, out_dtype=dtype)
+        perm_a = ops.permute_build(topi_a, E)
+        torch.cuda.synchronize()
+        assert torch.equal(topv_a, topv) and torch.equal(topi_a, topi)
+        n = int(perm_a.n_active.item())
+        assert n == int(perm.n_active.item())
+        for name in ("perm", "inv_perm", "seg_offsets"):
+            assert torch.equal(getattr(perm_a, name), getattr(perm, name)), name
+        assert torch.equal(perm_a.active_eids[:n], perm.active_eids[:n])
+        probs = torch.softmax(logits.cpu(), dim=-1, dtype=torch.float32)
+        ref_i = torch.sort(probs, dim=-1, descending=True, stable=True).indices[:, :K]
+        safe = _boundary_safe(logits.cpu(), K) if K < E else torch.ones(T, dtype=torch.bool)
+        assert torch.equal(topi.cpu()[safe], ref_i[safe])
+
+
+def test_pack_router_gate_declines_what_does_not_fit():
+    from sparse_amd import ops
+    wg = torch.zeros(64, 128, dtype=torch.bfloat16)
+    assert ops.pack_router_gate(wg, None) is not None
+    assert ops.pack_router_gate(wg, torch.zeros(128, dtype=torch.bfloat16)) is None      # 65 rows
+    assert ops.pack_router_gate(wg[:, :96].contiguous(), None) is None                    # H % 64
+    assert ops.pack_router_gate(wg.float(), None) is None
+
+
 # ------------------------------------------------------------------ permute
 @pytest.mark.parametrize("T,E,K", [(1, 60, 4), (8, 60, 4), (32, 60, 4), (255, 64, 6), (256, 64, 6),
                                     (257, 64, 6), (2048, 64, 6), (4096, 64, 6), (1000, 256, 16), (3, 4, 4)])
