@@ -158,6 +158,11 @@ def prefill_workload(shape, tokens, steps, warmup, dtype, device):
     blocks = build_stack(shape, dtype, device)
     inputs = make_inputs(shape, 1, tokens, 2, dtype, device)
     wall = time_steps(blocks, inputs, warmup, steps, use_graph=False)
+    # per-kernel durations are taken with the launches in one stream: beside another kernel a
+    # launch's event-to-event time says nothing about the kernel itself
+    for blk in blocks:
+        blk.overlap_shared = False
+    wall_serial = time_steps(blocks, inputs, 1, steps, use_graph=False)
     stats, _ = instrumented_pass(blocks, inputs, min(steps, 2))
     H, I, Is, K, E = shape["hidden"], shape["inter"], shape["shared_inter"], shape["top_k"], shape["num_experts"]
     flops_layer = 2.0 * tokens * K * 3 * H * I + 2.0 * tokens * 3 * H * Is + 2.0 * tokens * H * E
@@ -170,6 +175,7 @@ def prefill_workload(shape, tokens, steps, warmup, dtype, device):
     ms_per_step = wall / steps * 1e3
     out = dict(
         tokens=tokens, ms_per_step=ms_per_step, tokens_per_s=tokens * steps / wall,
+        ms_per_step_one_stream=wall_serial / steps * 1e3,
         layer_tflops=flops_layer * len(blocks) / (ms_per_step / 1e3) / 1e12,
         mfma_frac=flops_layer * len(blocks) / (ms_per_step / 1e3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
         gateup=dict(kernel=gu_name, launches=gu_n, est_routed_avg_us=gu_routed_s * 1e6,

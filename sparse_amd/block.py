@@ -276,6 +276,9 @@ class DistributedSparseMoeBlock(nn.Module):
         self.rs_prob_to_logit_eps = float(rs_prob_to_logit_eps)
         self.prefetch_top_m = int(prefetch_top_m)
         self.metrics = metrics if metrics is not None else Metrics()
+        # prefill-size batches run the shared expert on a second stream beside the routing
+        self.overlap_shared = str(os.environ.get("SPARSE_HIP_OVERLAP_SHARED", "1")).strip().lower() not in (
+            "", "0", "false", "no", "off")
 
         # ---- weights --------------------------------------------------------
         if not hasattr(mlp_block, "gate") or not hasattr(mlp_block, "experts"):
@@ -355,23 +358,41 @@ class DistributedSparseMoeBlock(nn.Module):
         return _Workspace.get(T, self.top_k, self.num_experts, self.hidden_size, self.inter_size,
                               self.shared_inter_size, self.dtype, self.logits_dtype, self.device)
 
+    _shared_streams: dict = {}
+
+    def _shared_stream(self) -> "torch.cuda.Stream":
+        """The stream (default priority, one per device) the shared expert of prefill-size
+        batches runs on."""
+        key = (self.device.type, self.device.index)
+        st = DistributedSparseMoeBlock._shared_streams.get(key)
+        if st is None:
+            st = torch.cuda.Stream(device=self.device)
+            DistributedSparseMoeBlock._shared_streams[key] = st
+        return st
+
     # ------------------------------------------------------------------ routing
-    def _route(self, x: torch.Tensor, ws: _Workspace) -> torch.Tensor:
+    def _route(self, x: torch.Tensor, ws: _Workspace, after_logits=None) -> torch.Tensor:
         """Router logits (+ shared gate), fused softmax/top-k, permutation (:9519-9595).
-        Returns the logits, a fresh tensor the caller owns."""
+        Returns the logits, a fresh tensor the caller owns.  ``after_logits`` is called once
+        the logits (and the shared gate) are queued: the point from which the shared expert
+        no longer depends on anything the rest of the routing does."""
+        after_logits = after_logits or (lambda: None)
         logits = torch.empty((x.shape[0], self.num_experts), device=x.device, dtype=self.logits_dtype)
         shared_gate = ws.shared_gate if self.shared_gate_weight is not None else None
         if (self.gate_packed is not None and x.shape[0] <= ops.ROUTE_PACKED_MAX_TOKENS
                 and self.routed_scaling_factor == 1.0):
             ops.route_decode_packed(x, self.gate_packed, self.num_experts, self.shared_gate_weight is not None,
                                     self.top_k, self.norm_topk_prob, logits, shared_gate, ws.topv, ws.topi, ws.perm)
+            after_logits()
             return logits
         if x.shape[0] <= ops.DECODE_MAX_TOKENS and self.routed_scaling_factor == 1.0:
             ops.route_decode(x, self.gate_weight, self.shared_gate_weight, self.top_k, self.norm_topk_prob, logits,
                              shared_gate, ws.topv, ws.topi, ws.perm, ws.route_counter)
+            after_logits()
             return logits
         ops.router_logits(x, self.gate_weight, self.shared_gate_weight, self.logits_dtype, out=logits,
                           shared_gate_out=shared_gate)
+        after_logits()
         ops.gate_topk(logits, self.top_k, self.norm_topk_prob, out_dtype=self.dtype, topv=ws.topv, topi=ws.topi)
         if self.routed_scaling_factor != 1.0:
             ws.topv.mul_(self.routed_scaling_factor)
@@ -504,17 +525,32 @@ class DistributedSparseMoeBlock(nn.Module):
                 self.residency.staging = None
             rs_job = self._rs_begin(x, S, ws)
 
-        if self.expert_source == "rs" and self.layer_idx in SparseContext.routing_cache:
-            logits = self._route_from_cache(x, ws)
-        else:
-            # also the first layer and prefill of an RS-routed run (:11128-11136)
-            logits = self._route(x, ws)
         shared_gate = ws.shared_gate if self.shared_gate_weight is not None else None
         fused = (self.residency is None and self.shared_weights is not None and self.dtype == torch.bfloat16
                  and T <= ops.DECODE_MAX_TOKENS)
-        if self.shared_weights is not None and not fused:
+        # Prefill-size batches: the shared expert needs only x and the shared gate, so it runs
+        # on a second stream from the moment the logits kernel is queued, beside top-k,
+        # permutation, tile map and the first routed tiles, and is joined before combine.
+        side = (self._shared_stream() if self.shared_weights is not None and not fused and self.overlap_shared
+                and x.is_cuda and T > ops.DECODE_MAX_TOKENS else None)
+
+        def run_shared() -> None:
+            if self.shared_weights is None or fused:
+                return
             gw, uw, dw = self.shared_weights
-            ops.shared_expert(x, gw, uw, dw, shared_gate, ws.shared_inter, ws.shared_out)
+            if side is None:
+                ops.shared_expert(x, gw, uw, dw, shared_gate, ws.shared_inter, ws.shared_out)
+                return
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                ops.shared_expert(x, gw, uw, dw, shared_gate, ws.shared_inter, ws.shared_out)
+
+        if self.expert_source == "rs" and self.layer_idx in SparseContext.routing_cache:
+            logits = self._route_from_cache(x, ws)
+            run_shared()
+        else:
+            # also the first layer and prefill of an RS-routed run (:11128-11136)
+            logits = self._route(x, ws, after_logits=run_shared)
 
         if fused:
             ops.moe_ffn_decode(self._experts_desc, x, ws.topv, ws.perm, ws.segs_dev, ws.inter, ws.parts,
@@ -543,6 +579,8 @@ class DistributedSparseMoeBlock(nn.Module):
             torch.cuda.current_stream().synchronize()
             self._rs_finish(rs_job, ws)
 
+        if side is not None:
+            torch.cuda.current_stream().wait_stream(side)
         out = torch.empty((T, H), device=x.device, dtype=self.dtype)
         ops.combine(ws.parts, ws.perm, ws.shared_out, T, self.top_k, out)
         out = out.view(B, S, H)

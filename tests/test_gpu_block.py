@@ -104,6 +104,27 @@ def test_deepseek_bf16_prefill_512(device):
     _check(DEEPSEEK, torch.bfloat16, 512, device, seed=2)
 
 
+@pytest.mark.parametrize("shape", [SMALL_Q, SMALL_D], ids=["qwen", "deepseek"])
+def test_shared_expert_on_its_own_stream_changes_nothing(device, shape):
+    """Prefill-size batches run the shared expert on a second stream beside the routing; the
+    kernels and their inputs are the same, so the layer output is bit for bit the one-stream
+    result, call after call, also when calls alternate between the two forms."""
+    from sparse_amd.synthetic import make_hidden
+    _, blk = _build(shape, torch.bfloat16, device, seed=3)
+    assert blk.overlap_shared
+    H = shape["hidden"]
+    outs = {}
+    for rep in range(3):
+        x = make_hidden(256, H, torch.bfloat16, seed=50 + rep).view(1, 256, H).to(device)
+        for overlap in (True, False, True):
+            blk.overlap_shared = overlap
+            ret = blk(x)
+            out = (ret[0] if isinstance(ret, tuple) else ret).clone()
+            torch.cuda.synchronize()
+            outs.setdefault(rep, out)
+            assert torch.equal(out, outs[rep]), (rep, overlap)
+
+
 def test_constructor_rejects_bad_enums(device):
     from sparse_amd.block import DistributedSparseMoeBlock
     from sparse_amd.context import DistEnv
