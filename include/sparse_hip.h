@@ -125,6 +125,19 @@ int sparse_hip_gate_topk(const void* logits_dev, int logits_dtype, int T, int E,
                          int renorm, int out_dtype, void* topv_dev, int64_t* topi_dev,
                          void* stream);
 
+/*
+ * The same with DeepSeek-V2's group-limited selection in front of the top-k: the experts form
+ * `n_group` equal runs of ids, a group scores its largest probability, the `topk_group` best
+ * groups stay (ties to the lower group id) and every other expert's probability is replaced
+ * by 0 before the top-k.  This is the `group_limited_greedy` method of the gate the reference
+ * delegates to (`self.gate(...)`, utils/eval_core.py:9503-9517; the gate module itself is the
+ * model's, e.g. transformers' DeepseekV2TopkRouter).  n_group <= 64, E % n_group == 0;
+ * n_group == 1 or topk_group == n_group is plain top-k.
+ */
+int sparse_hip_gate_topk_grouped(const void* logits_dev, int logits_dtype, int T, int E, int K,
+                                 int renorm, int n_group, int topk_group, int out_dtype,
+                                 void* topv_dev, int64_t* topi_dev, void* stream);
+
 /* ---- A5: token x K expansion + permutation --------------------------------- */
 
 /*

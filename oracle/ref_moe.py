@@ -20,8 +20,9 @@ How each function is pinned (see tests/test_oracle_moe.py):
                             from the published DeepSeek-V2 gate (fp32 logits, fp32 softmax,
                             top-k, times routed_scaling_factor) and pinned against the port
                             of that gate in the installed ``transformers``
-                            (``DeepseekV2TopkRouter``, ``greedy`` method): same experts and
-                            weights in fp32 and bf16.
+                            (``DeepseekV2TopkRouter``, ``greedy`` and
+                            ``group_limited_greedy`` methods): same experts and weights in
+                            fp32 and bf16.
   experts_world1_exact      fp64 per-token closed form sum_k w_k*down(silu(gate x)*up x)
                             (the expected value of the reference's own
                             tests/test_lightweight_policy.py:122-127), permutation
@@ -69,17 +70,32 @@ def routing_router(x: torch.Tensor, gate_w: torch.Tensor, top_k: int, norm_topk_
     return topv.to(dtype=x.dtype), topi.to(torch.long), router_logits
 
 
+def group_limited_scores(probs: torch.Tensor, n_group: int, topk_group: int) -> torch.Tensor:
+    """DeepSeek-V2's ``group_limited_greedy`` mask: experts form ``n_group`` equal runs of ids, a
+    group scores its largest probability, the ``topk_group`` best groups (ties to the lower
+    group id) keep their probabilities, every other entry becomes 0."""
+    T, E = probs.shape
+    group_scores = probs.view(T, n_group, E // n_group).max(dim=-1).values
+    _, keep = topk_lower_id_first(group_scores, topk_group)
+    mask = torch.zeros_like(group_scores, dtype=torch.bool)
+    mask.scatter_(1, keep, True)
+    return torch.where(mask.repeat_interleave(E // n_group, dim=1), probs, torch.zeros_like(probs))
+
+
 def deepseek_router(x: torch.Tensor, gate_w: torch.Tensor, top_k: int, routed_scaling_factor: float = 1.0,
-                    router_logits: Optional[torch.Tensor] = None):
+                    router_logits: Optional[torch.Tensor] = None, n_group: int = 1, topk_group: int = 1):
     """DeepSeek-family router as seen at the reference's call site :9503-9517.
 
     The gate itself is third-party (see the module docstring for what pins this restatement): fp32
-    logits from fp32-cast x and W, fp32 softmax, greedy top-k, weights scaled and cast to
-    x.dtype.  Returns (topv, topi, pseudo_logits) with pseudo_logits built as :9490-9499.
+    logits from fp32-cast x and W, fp32 softmax, greedy top-k (optionally limited to the best
+    groups, the method of the full-size DeepSeek-V2), weights scaled and cast to x.dtype.
+    Returns (topv, topi, pseudo_logits) with pseudo_logits built as :9490-9499.
     """
     if router_logits is None:
         router_logits = F.linear(x.to(torch.float32), gate_w.to(torch.float32))
     probs = torch.softmax(router_logits, dim=-1, dtype=torch.float32)
+    if n_group > 1 and topk_group < n_group:
+        probs = group_limited_scores(probs, n_group, topk_group)
     topv, topi = topk_lower_id_first(probs, top_k)
     topv = (topv * routed_scaling_factor).to(dtype=x.dtype)
     pseudo = torch.full((x.shape[0], gate_w.shape[0]), float("-inf"), dtype=torch.float32)

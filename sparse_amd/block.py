@@ -287,6 +287,17 @@ class DistributedSparseMoeBlock(nn.Module):
         self.routed_scaling_factor = float(getattr(mlp_block.gate, "routed_scaling_factor",
                                                    getattr(mlp_block, "routed_scaling_factor", 1.0)) or 1.0)
         self.gate_weight = mlp_block.gate.weight.detach().to(self.device, self.dtype).contiguous()
+        # selection method of a DeepSeek-family gate module (the reference runs whatever gate the
+        # model brings, :9503-9517): plain greedy top-k, or limited to the best expert groups
+        method = str(getattr(gate_mod, "topk_method", "greedy") or "greedy")
+        if method not in ("greedy", "group_limited_greedy"):
+            raise NotImplementedError(f"gate topk_method={method} is not built (greedy | group_limited_greedy)")
+        self.n_group = self.topk_group = 1
+        if method == "group_limited_greedy":
+            self.n_group = int(getattr(gate_mod, "num_group", None) or getattr(gate_mod, "n_group", None) or 1)
+            self.topk_group = int(getattr(gate_mod, "topk_group", None) or self.n_group)
+            if self.topk_group >= self.n_group:
+                self.n_group = self.topk_group = 1          # every group kept: plain top-k
         self.experts_kind, expert_weights = extract_experts(mlp_block.experts)
         self.num_experts = int(num_experts) if num_experts is not None else len(expert_weights)
         if self.num_experts != len(expert_weights) or self.gate_weight.shape[0] != self.num_experts:
@@ -379,13 +390,13 @@ class DistributedSparseMoeBlock(nn.Module):
         after_logits = after_logits or (lambda: None)
         logits = torch.empty((x.shape[0], self.num_experts), device=x.device, dtype=self.logits_dtype)
         shared_gate = ws.shared_gate if self.shared_gate_weight is not None else None
-        if (self.gate_packed is not None and x.shape[0] <= ops.ROUTE_PACKED_MAX_TOKENS
-                and self.routed_scaling_factor == 1.0):
+        one_launch = self.routed_scaling_factor == 1.0 and self.n_group == 1
+        if self.gate_packed is not None and x.shape[0] <= ops.ROUTE_PACKED_MAX_TOKENS and one_launch:
             ops.route_decode_packed(x, self.gate_packed, self.num_experts, self.shared_gate_weight is not None,
                                     self.top_k, self.norm_topk_prob, logits, shared_gate, ws.topv, ws.topi, ws.perm)
             after_logits()
             return logits
-        if x.shape[0] <= ops.DECODE_MAX_TOKENS and self.routed_scaling_factor == 1.0:
+        if x.shape[0] <= ops.DECODE_MAX_TOKENS and one_launch:
             ops.route_decode(x, self.gate_weight, self.shared_gate_weight, self.top_k, self.norm_topk_prob, logits,
                              shared_gate, ws.topv, ws.topi, ws.perm, ws.route_counter)
             after_logits()
@@ -393,7 +404,8 @@ class DistributedSparseMoeBlock(nn.Module):
         ops.router_logits(x, self.gate_weight, self.shared_gate_weight, self.logits_dtype, out=logits,
                           shared_gate_out=shared_gate)
         after_logits()
-        ops.gate_topk(logits, self.top_k, self.norm_topk_prob, out_dtype=self.dtype, topv=ws.topv, topi=ws.topi)
+        ops.gate_topk(logits, self.top_k, self.norm_topk_prob, out_dtype=self.dtype, topv=ws.topv, topi=ws.topi,
+                      n_group=self.n_group, topk_group=self.topk_group)
         if self.routed_scaling_factor != 1.0:
             ws.topv.mul_(self.routed_scaling_factor)
         ops.permute_build(ws.topi, self.num_experts, out=ws.perm)

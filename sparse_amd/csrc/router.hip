@@ -185,7 +185,8 @@ constexpr int kTopkNV = SPARSE_HIP_MAX_EXPERTS / 64;
 
 template <typename TL, typename TO>
 __device__ __forceinline__ int topk_token(const TL* __restrict__ row, int E, int K, int renorm,
-                                          TO* __restrict__ topv_row, int64_t* __restrict__ topi_row, int lane) {
+                                          TO* __restrict__ topv_row, int64_t* __restrict__ topi_row, int lane,
+                                          int n_group = 0, int topk_group = 0) {
   float p[kTopkNV];
   float m = -INFINITY;
 #pragma unroll
@@ -210,6 +211,36 @@ __device__ __forceinline__ int topk_token(const TL* __restrict__ row, int E, int
   for (int j = 0; j < kTopkNV; ++j) {
     const int e = lane + 64 * j;
     p[j] = (e < E) ? p[j] / s : -1.f;  // -1 marks "not a candidate"
+  }
+
+  if (n_group > 1) {
+    // group-limited selection: the experts form n_group equal runs of ids; a group's score is
+    // its largest probability, the topk_group best groups (score descending, then lower group
+    // id) stay, every other expert's probability becomes 0 and still takes part in the top-k
+    const int gsz = E / n_group;
+    float gscore = -2.f;  // lane g < n_group: score of group g
+    for (int g = 0; g < n_group; ++g) {
+      float m = -1.f;
+#pragma unroll
+      for (int j = 0; j < kTopkNV; ++j) {
+        const int e = lane + 64 * j;
+        if (e < E && e / gsz == g) m = fmaxf(m, p[j]);
+      }
+      m = wave_max(m);
+      if (lane == g) gscore = m;
+    }
+    unsigned long long keep = 0ull;
+    for (int r = 0; r < topk_group; ++r) {
+      const float wv = wave_max(gscore);
+      const int wi = wave_min_int(gscore == wv ? lane : 0x7fffffff);
+      keep |= 1ull << wi;
+      if (lane == wi) gscore = -2.f;
+    }
+#pragma unroll
+    for (int j = 0; j < kTopkNV; ++j) {
+      const int e = lane + 64 * j;
+      if (e < E && !((keep >> (e / gsz)) & 1ull)) p[j] = 0.f;
+    }
   }
 
   float sel_v = 0.f;  // lane r keeps the r-th selection
@@ -251,11 +282,11 @@ __device__ __forceinline__ int topk_token(const TL* __restrict__ row, int E, int
 template <typename TL, typename TO>
 __global__ __launch_bounds__(kTopkWaves * 64) void gate_topk_kernel(
     const TL* __restrict__ logits, int Ttok, int E, int K, int renorm, TO* __restrict__ topv,
-    int64_t* __restrict__ topi) {
+    int64_t* __restrict__ topi, int n_group, int topk_group) {
   const int t = blockIdx.x * kTopkWaves + (threadIdx.x >> 6);
   if (t >= Ttok) return;
   topk_token<TL, TO>(logits + static_cast<size_t>(t) * E, E, K, renorm, topv + static_cast<size_t>(t) * K,
-                     topi + static_cast<size_t>(t) * K, threadIdx.x & 63);
+                     topi + static_cast<size_t>(t) * K, threadIdx.x & 63, n_group, topk_group);
 }
 
 // ---------------------------------------------------------------------------
@@ -579,11 +610,12 @@ static int launch_router_logits(const void* x, const void* wg, const void* wsg, 
 
 template <typename TL, typename TO>
 static int launch_gate_topk(const void* logits, int Ttok, int E, int K, int renorm, void* topv,
-                            int64_t* topi, hipStream_t st) {
+                            int64_t* topi, hipStream_t st, int n_group = 0, int topk_group = 0) {
   dim3 grid((Ttok + kTopkWaves - 1) / kTopkWaves);
   ProfScope prof(SPARSE_HIP_K_GATE_TOPK, st);
   hipLaunchKernelGGL((gate_topk_kernel<TL, TO>), grid, dim3(kTopkWaves * 64), 0, st,
-                     static_cast<const TL*>(logits), Ttok, E, K, renorm, static_cast<TO*>(topv), topi);
+                     static_cast<const TL*>(logits), Ttok, E, K, renorm, static_cast<TO*>(topv), topi, n_group,
+                     topk_group);
   SP_LAUNCH_CHECK("gate_topk_kernel");
   return SPARSE_HIP_OK;
 }
@@ -623,7 +655,18 @@ int sparse_hip_router_logits(const void* x_dev, const void* wg_dev, const void* 
 
 int sparse_hip_gate_topk(const void* logits_dev, int logits_dtype, int T, int E, int K, int renorm,
                          int out_dtype, void* topv_dev, int64_t* topi_dev, void* stream) {
+  return sparse_hip_gate_topk_grouped(logits_dev, logits_dtype, T, E, K, renorm, 1, 1, out_dtype, topv_dev, topi_dev,
+                                      stream);
+}
+
+int sparse_hip_gate_topk_grouped(const void* logits_dev, int logits_dtype, int T, int E, int K, int renorm,
+                                 int n_group, int topk_group, int out_dtype, void* topv_dev, int64_t* topi_dev,
+                                 void* stream) {
   SP_REQUIRE(valid_dtype(logits_dtype) && valid_dtype(out_dtype), "gate_topk: unknown dtype");
+  SP_REQUIRE(n_group >= 1 && n_group <= 64 && E % n_group == 0, "gate_topk: n_group=%d must divide E=%d and be <= 64",
+             n_group, E);
+  SP_REQUIRE(topk_group >= 1 && topk_group <= n_group, "gate_topk: topk_group=%d outside [1,n_group=%d]", topk_group,
+             n_group);
   SP_REQUIRE(T >= 0, "gate_topk: T=%d", T);
   SP_REQUIRE(E >= 1 && E <= SPARSE_HIP_MAX_EXPERTS, "gate_topk: E=%d outside [1,%d]", E, SPARSE_HIP_MAX_EXPERTS);
   SP_REQUIRE(K >= 1 && K <= SPARSE_HIP_MAX_TOPK && K <= E, "gate_topk: K=%d outside [1,min(%d,E)]", K,
@@ -632,10 +675,12 @@ int sparse_hip_gate_topk(const void* logits_dev, int logits_dtype, int T, int E,
   if (T == 0) return SPARSE_HIP_OK;
   hipStream_t st = as_stream(stream);
   const bool lb = logits_dtype == SPARSE_HIP_BF16, ob = out_dtype == SPARSE_HIP_BF16;
-  if (lb && ob) return launch_gate_topk<uint16_t, uint16_t>(logits_dev, T, E, K, renorm, topv_dev, topi_dev, st);
-  if (lb) return launch_gate_topk<uint16_t, float>(logits_dev, T, E, K, renorm, topv_dev, topi_dev, st);
-  if (ob) return launch_gate_topk<float, uint16_t>(logits_dev, T, E, K, renorm, topv_dev, topi_dev, st);
-  return launch_gate_topk<float, float>(logits_dev, T, E, K, renorm, topv_dev, topi_dev, st);
+  const int ng = (n_group > 1 && topk_group < n_group) ? n_group : 0;  // every group kept = plain top-k
+  if (lb && ob)
+    return launch_gate_topk<uint16_t, uint16_t>(logits_dev, T, E, K, renorm, topv_dev, topi_dev, st, ng, topk_group);
+  if (lb) return launch_gate_topk<uint16_t, float>(logits_dev, T, E, K, renorm, topv_dev, topi_dev, st, ng, topk_group);
+  if (ob) return launch_gate_topk<float, uint16_t>(logits_dev, T, E, K, renorm, topv_dev, topi_dev, st, ng, topk_group);
+  return launch_gate_topk<float, float>(logits_dev, T, E, K, renorm, topv_dev, topi_dev, st, ng, topk_group);
 }
 
 int sparse_hip_route_decode(const void* x_dev, const void* wg_dev, const void* wsg_dev, int dtype,

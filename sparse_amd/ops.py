@@ -71,8 +71,11 @@ def router_logits(x: torch.Tensor, wg: torch.Tensor, wsg: Optional[torch.Tensor]
 
 
 def gate_topk(logits: torch.Tensor, k: int, renorm: bool = False, out_dtype: Optional[torch.dtype] = None,
-              topv: Optional[torch.Tensor] = None, topi: Optional[torch.Tensor] = None):
-    """Fused softmax(fp32) + top-k: returns ``(topv [T,k] out_dtype, topi [T,k] int64)``."""
+              topv: Optional[torch.Tensor] = None, topi: Optional[torch.Tensor] = None,
+              n_group: int = 1, topk_group: int = 1):
+    """Fused softmax(fp32) + top-k: returns ``(topv [T,k] out_dtype, topi [T,k] int64)``.
+    With ``n_group > 1`` only experts of the ``topk_group`` best groups keep their probability
+    (DeepSeek-V2's group-limited selection); the others enter the top-k with 0."""
     lib = _lib.load()
     _need(logits, "logits")
     T, E = logits.shape
@@ -83,9 +86,10 @@ def gate_topk(logits: torch.Tensor, k: int, renorm: bool = False, out_dtype: Opt
         topi = torch.empty((T, k), device=logits.device, dtype=torch.int64)
     _need(topv, "topv", odt, (T, k))
     _need(topi, "topi", torch.int64, (T, k))
-    rc = lib.sparse_hip_gate_topk(_ptr(logits), dtype_code(logits.dtype), T, E, int(k), int(bool(renorm)),
-                                  dtype_code(odt), _ptr(topv), _ptr(topi), _stream())
-    _lib.check(rc, "sparse_hip_gate_topk")
+    rc = lib.sparse_hip_gate_topk_grouped(_ptr(logits), dtype_code(logits.dtype), T, E, int(k), int(bool(renorm)),
+                                          int(n_group), int(topk_group), dtype_code(odt), _ptr(topv), _ptr(topi),
+                                          _stream())
+    _lib.check(rc, "sparse_hip_gate_topk_grouped")
     return topv, topi
 
 

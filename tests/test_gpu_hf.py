@@ -58,7 +58,7 @@ def test_qwen2_moe_model_with_swapped_blocks(device, offload):
         assert metrics.cache_miss_count > 0
 
 
-def _tiny_deepseek(dtype):
+def _tiny_deepseek(dtype, **routing):
     pytest.importorskip("transformers")
     try:
         from transformers import DeepseekV2Config, DeepseekV2ForCausalLM
@@ -66,8 +66,9 @@ def _tiny_deepseek(dtype):
         pytest.skip("this transformers has no DeepSeek-V2")
     cfg = DeepseekV2Config(vocab_size=160, hidden_size=128, intermediate_size=256, moe_intermediate_size=64,
                            num_hidden_layers=3, num_attention_heads=4, num_key_value_heads=4, n_routed_experts=16,
-                           num_experts_per_tok=6, n_shared_experts=2, first_k_dense_replace=1, topk_method="greedy",
-                           routed_scaling_factor=1.0, norm_topk_prob=False, max_position_embeddings=128,
+                           num_experts_per_tok=6, n_shared_experts=2, first_k_dense_replace=1,
+                           **{**dict(topk_method="greedy", routed_scaling_factor=1.0), **routing},
+                           norm_topk_prob=False, max_position_embeddings=128,
                            kv_lora_rank=32, q_lora_rank=None, qk_rope_head_dim=16, qk_nope_head_dim=16, v_head_dim=32,
                            head_dim=16)
     torch.manual_seed(1)
@@ -109,3 +110,34 @@ def test_deepseek_v2_model_with_swapped_blocks(device):
         got_ids = harness.greedy_decode(model, ids, mask, 5, metrics).cpu()
     assert torch.equal(got_ids, want_ids)
     assert metrics.cache_miss_count > 0
+
+
+def test_deepseek_v2_group_limited_gate_and_scaling_factor(device):
+    """The gate of the full-size DeepSeek-V2: experts in four groups of which two compete, and a
+    routed scaling factor.  The swapped blocks read both from the model's gate module and
+    reproduce the model's own logits and greedy continuation."""
+    from sparse_amd import harness
+    from sparse_amd.context import DistEnv, Metrics, SparseContext
+    model = _tiny_deepseek(torch.float32, topk_method="group_limited_greedy", n_group=4, topk_group=2,
+                           routed_scaling_factor=2.0).to(device)
+    ids = torch.tensor([[5, 17, 42, 99, 3, 64], [7, 7, 120, 33, 8, 1]], device=device)
+    mask = torch.ones_like(ids)
+    SparseContext.reset()
+    with torch.no_grad():
+        want_logits = model(input_ids=ids, attention_mask=mask, use_cache=False, return_dict=True).logits.float().cpu()
+        want_ids = harness.greedy_decode(model, ids, mask, 5).cpu()
+    SparseContext.reset()
+    blocks = harness.install_sparse_blocks(model, env=DistEnv(0, 1, 0, device), dtype=torch.float32, metrics=Metrics())
+    assert (blocks[0].n_group, blocks[0].topk_group, blocks[0].routed_scaling_factor) == (4, 2, 2.0)
+    with torch.no_grad():
+        harness.begin_request()
+        SparseContext.current_phase = "prefill"
+        SparseContext.begin_runtime_call(0)
+        got_logits = model(input_ids=ids, attention_mask=mask, use_cache=False, return_dict=True).logits.float().cpu()
+        torch.testing.assert_close(got_logits, want_logits, rtol=2e-4, atol=2e-4)
+        ws = blocks[0]._workspace(ids.numel())
+        groups = torch.div(ws.topi.cpu(), 4, rounding_mode="floor")
+        assert max(len(set(row.tolist())) for row in groups) <= 2          # chosen experts come from two groups
+        harness.begin_request()
+        got_ids = harness.greedy_decode(model, ids, mask, 5).cpu()
+    assert torch.equal(got_ids, want_ids)

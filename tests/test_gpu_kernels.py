@@ -58,6 +58,41 @@ def test_gate_topk_matches_oracle(device, E, K, ldt):
     torch.testing.assert_close(topv.float()[safe], ref_v.to(ldt).float()[safe], rtol=1e-2, atol=1e-6)
 
 
+@pytest.mark.parametrize("E,n_group,topk_group,K", [(16, 4, 2, 6), (160, 8, 3, 6), (256, 64, 5, 16), (64, 2, 1, 8),
+                                                      (60, 6, 6, 4), (12, 4, 1, 5)])
+@pytest.mark.parametrize("ldt", [torch.float32, torch.bfloat16])
+def test_gate_topk_group_limited(device, E, n_group, topk_group, K, ldt):
+    """Group-limited selection against the oracle: indices exact wherever neither the group
+    choice nor the top-k boundary is a rounding tie; K larger than the experts left picks
+    zero-probability experts in id order, as the oracle's rule says."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(E + n_group)
+    logits = (torch.randn(300, E, generator=g) * 2.0).to(ldt)
+    topv, topi = ops.gate_topk(logits.to(device), K, out_dtype=torch.float32, n_group=n_group, topk_group=topk_group)
+    probs = torch.softmax(logits, dim=-1, dtype=torch.float32)
+    masked = ref_moe.group_limited_scores(probs, n_group, topk_group) if topk_group < n_group else probs
+    ref_v, ref_i = ref_moe.topk_lower_id_first(masked, K)
+    # rows whose group ranking or top-k boundary could flip on an ulp of exp/sum are left out
+    gs = probs.view(300, n_group, E // n_group).max(-1).values.sort(-1, descending=True).values
+    safe = torch.ones(300, dtype=torch.bool)
+    if topk_group < n_group:
+        a, b = gs[:, topk_group - 1], gs[:, topk_group]
+        safe &= (a == b) | ((a - b) / a > 1e-5)
+    srt = masked.sort(dim=-1, descending=True, stable=True).values
+    if K < E:
+        a, b = srt[:, K - 1], srt[:, K]
+        safe &= (a == b) | ((a - b) / a.clamp_min(1e-30) > 1e-5)
+    pairs = srt[:, :K]
+    safe &= ((pairs[:, :-1] == pairs[:, 1:]) | ((pairs[:, :-1] - pairs[:, 1:]) / pairs[:, :-1].clamp_min(1e-30) > 1e-5)).all(1)
+    assert safe.float().mean() > 0.8
+    assert torch.equal(topi.cpu()[safe], ref_i[safe])
+    torch.testing.assert_close(topv.cpu()[safe], ref_v[safe], rtol=1e-5, atol=1e-7)
+    if topk_group < n_group:
+        grp = torch.div(topi.cpu(), E // n_group, rounding_mode="floor")
+        live = (masked > 0).sum(1) >= K                     # enough experts left in the kept groups
+        assert max((len(set(r.tolist())) for r in grp[live]), default=0) <= topk_group
+
+
 def test_gate_topk_ties_go_to_lower_id(device):
     ops = _ops()
     logits = torch.zeros(5, 60)

@@ -272,3 +272,50 @@ def test_deepseek_router_against_the_transformers_port_of_the_gate():
         # the reference casts the gate's weights to the activation dtype at its call site (:9514)
         torch.testing.assert_close(torch.gather(topv.float(), 1, order_ref.indices),
                                    torch.gather(weights.to(dtype).float(), 1, order_hf.indices), rtol=1e-6, atol=1e-7)
+
+
+def test_deepseek_group_limited_router_against_the_transformers_port():
+    """The ``group_limited_greedy`` method of the full-size DeepSeek-V2 gate (experts in equal
+    groups, only the best groups compete): same experts and weights as the transformers port,
+    a hand-made case where the limit changes the answer, and the degenerate settings that
+    must reduce to plain top-k."""
+    pytest.importorskip("transformers")
+    try:
+        from transformers import DeepseekV2Config
+        from transformers.models.deepseek_v2.modeling_deepseek_v2 import DeepseekV2TopkRouter
+    except ImportError:
+        pytest.skip("this transformers has no DeepSeek-V2")
+    g = torch.Generator().manual_seed(12)
+    for dtype, scale, E, ng, kg, K in ((torch.float32, 1.0, 16, 4, 2, 6), (torch.bfloat16, 16.0, 32, 8, 3, 6),
+                                       (torch.float32, 1.0, 160, 8, 3, 6)):
+        cfg = DeepseekV2Config(hidden_size=64, n_routed_experts=E, num_experts_per_tok=K,
+                               topk_method="group_limited_greedy", n_group=ng, topk_group=kg,
+                               routed_scaling_factor=scale, num_hidden_layers=1, vocab_size=32)
+        gate = DeepseekV2TopkRouter(cfg)
+        gate.weight.data = (torch.randn(E, 64, generator=g) * 0.3)
+        x = torch.randn(50, 64, generator=g).to(dtype)
+        gate = gate.to(dtype)
+        with torch.no_grad():
+            _, weights, idx = gate(x)
+        topv, topi, _ = ref_moe.deepseek_router(x, gate.weight.data, K, routed_scaling_factor=scale,
+                                                n_group=ng, topk_group=kg)
+        order_ref, order_hf = torch.sort(topi, 1), torch.sort(idx, 1)
+        assert torch.equal(order_ref.values, order_hf.values)
+        torch.testing.assert_close(torch.gather(topv.float(), 1, order_ref.indices),
+                                   torch.gather(weights.to(dtype).float(), 1, order_hf.indices), rtol=1e-6, atol=1e-7)
+        # every chosen expert sits in one of kg groups
+        assert (torch.div(topi, E // ng, rounding_mode="floor").sort(1).values.diff(dim=1) != 0).sum(1).max() < kg
+        plain = ref_moe.deepseek_router(x, gate.weight.data, K, routed_scaling_factor=scale)
+        assert not torch.equal(torch.sort(plain[1], 1).values, order_ref.values)      # the limit matters here
+        for ng2, kg2 in ((1, 1), (ng, ng)):
+            same = ref_moe.deepseek_router(x, gate.weight.data, K, routed_scaling_factor=scale, n_group=ng2,
+                                           topk_group=kg2)
+            assert torch.equal(same[1], plain[1]) and torch.equal(same[0], plain[0])
+    # by hand: 2 groups of 3, one group allowed, K=2: the runner-up overall (id 3) is outside the best group
+    probs = torch.tensor([[0.30, 0.05, 0.10, 0.28, 0.02, 0.25]])
+    masked = ref_moe.group_limited_scores(probs, 2, 1)
+    assert torch.equal(masked, torch.tensor([[0.30, 0.05, 0.10, 0.0, 0.0, 0.0]]))
+    assert ref_moe.topk_lower_id_first(masked, 2)[1].tolist() == [[0, 2]]
+    # equal group scores: the lower group wins
+    tie = torch.tensor([[0.25, 0.0, 0.25, 0.0]])
+    assert ref_moe.group_limited_scores(tie, 2, 1).tolist() == [[0.25, 0.0, 0.0, 0.0]]
