@@ -365,8 +365,9 @@ class DistributedSparseMoeBlock(nn.Module):
             return "decode" if seq == 1 else "prefill"
         return "decode"
 
-    def _workspace(self, T: int) -> _Workspace:
-        return _Workspace.get(T, self.top_k, self.num_experts, self.hidden_size, self.inter_size,
+    def _workspace(self, T: int, K: Optional[int] = None) -> _Workspace:
+        return _Workspace.get(T, self.top_k if K is None else int(K), self.num_experts, self.hidden_size,
+                              self.inter_size,
                               self.shared_inter_size, self.dtype, self.logits_dtype, self.device)
 
     _shared_streams: dict = {}
@@ -417,9 +418,8 @@ class DistributedSparseMoeBlock(nn.Module):
         logits: log of the replayed weight at the chosen experts, -1e9 elsewhere."""
         w, idx = SparseContext.routing_cache[self.layer_idx]
         T = int(x.shape[0])
-        if tuple(idx.shape) != (T, self.top_k) or tuple(w.shape) != (T, self.top_k):
-            raise NotImplementedError(
-                f"RS routing replay with {tuple(idx.shape)} predictions for top_k={self.top_k} is not built")
+        if tuple(idx.shape) != tuple(ws.topi.shape) or tuple(w.shape) != tuple(ws.topv.shape):
+            raise RuntimeError(f"cached routing of shape {tuple(idx.shape)} does not fit {T} tokens")
         ws.topv.copy_(w.to(self.dtype))
         ws.topi.copy_(idx)
         ops.permute_build(ws.topi, self.num_experts, out=ws.perm)
@@ -523,7 +523,11 @@ class DistributedSparseMoeBlock(nn.Module):
         if T == 0:
             logits = torch.empty((0, self.num_experts), device=x.device, dtype=self.logits_dtype)
             return hidden_states if self._return_tensor_only_mlp() else (hidden_states, logits)
-        ws = self._workspace(T)
+        # a layer that replays its predecessor's prediction executes as many experts per token as
+        # that prediction holds (SPARSE_RS_EXEC_TOPK, :10979-10987), not necessarily its own top-k
+        from_cache = self.expert_source == "rs" and self.layer_idx in SparseContext.routing_cache
+        k_exec = int(SparseContext.routing_cache[self.layer_idx][1].shape[-1]) if from_cache else self.top_k
+        ws = self._workspace(T, k_exec)
         staging = SparseContext.staging
         staged = (staging is not None and self.residency is not None and staging.handles(self, S))
         if staged:
@@ -557,7 +561,7 @@ class DistributedSparseMoeBlock(nn.Module):
             with torch.cuda.stream(side):
                 ops.shared_expert(x, gw, uw, dw, shared_gate, ws.shared_inter, ws.shared_out)
 
-        if self.expert_source == "rs" and self.layer_idx in SparseContext.routing_cache:
+        if from_cache:
             logits = self._route_from_cache(x, ws)
             run_shared()
         else:
@@ -594,7 +598,7 @@ class DistributedSparseMoeBlock(nn.Module):
         if side is not None:
             torch.cuda.current_stream().wait_stream(side)
         out = torch.empty((T, H), device=x.device, dtype=self.dtype)
-        ops.combine(ws.parts, ws.perm, ws.shared_out, T, self.top_k, out)
+        ops.combine(ws.parts, ws.perm, ws.shared_out, T, k_exec, out)
         out = out.view(B, S, H)
         if self._return_tensor_only_mlp():
             return out

@@ -258,3 +258,62 @@ def test_expert_source_rs_executes_the_predicted_routing(device, dtype, offload)
             torch.testing.assert_close(out.view(T, -1).cpu().float(), want.float(), **tol)
             prev_in = xin
             hid = out
+
+
+@pytest.mark.parametrize("exec_topk", [2, 7])
+@pytest.mark.parametrize("offload", ["gpu", "cpu"])
+def test_rs_routing_with_its_own_number_of_experts_per_token(device, monkeypatch, exec_topk, offload):
+    """``SPARSE_RS_EXEC_TOPK`` (reference :10979-10987): the replayed routing holds that many
+    experts per token, fewer or more than the layer's own top-k, and the layer executes
+    exactly them; router-routed calls keep the layer's top-k."""
+    from sparse_amd.block import DistributedSparseMoeBlock
+    from sparse_amd.context import DistEnv, SparseContext
+    from sparse_amd.rs import random_init_bank
+    from sparse_amd.synthetic import make_hidden, make_mlp_block
+    monkeypatch.setenv("SPARSE_RS_EXEC_TOPK", str(exec_topk))
+    shape, T, L, dtype = SMALL_Q, 5, 3, torch.bfloat16
+    SparseContext.reset()
+    mlps = [make_mlp_block(shape, dtype=dtype, seed=40 + l) for l in range(L)]
+    kw = dict(expert_offload="cpu", expert_cache=5, planner_mode="rs_prefetch", prefetch_top_m=3) \
+        if offload == "cpu" else dict(expert_offload="gpu", routing_mode="rs")
+    blocks = [DistributedSparseMoeBlock(l, mlps[l], None, DistEnv(0, 1, 0, device), num_layers=L,
+                                        num_experts=shape["num_experts"], top_k=shape["top_k"], dtype=dtype,
+                                        expert_source="rs", **kw) for l in range(L)]
+    SparseContext.set_rs_bank(random_init_bank(L, shape["hidden"], shape["num_experts"], hidden_dim=32, seed=2,
+                                               device=device))
+    for call, phase in enumerate(["prefill", "decode", "decode"]):
+        SparseContext.current_phase = phase
+        SparseContext.begin_runtime_call(call)
+        x = make_hidden(T, shape["hidden"], dtype, seed=500 + call)
+        hid = (x.view(1, T, -1) if phase == "prefill" else x.view(T, 1, -1)).to(device)
+        for l, blk in enumerate(blocks):
+            replay = phase == "decode" and l > 0
+            if replay:
+                w_dev, i_dev = (t.cpu() for t in SparseContext.routing_cache[l])
+                assert tuple(i_dev.shape) == (T, exec_topk)
+            out, logits = blk(hid)
+            torch.cuda.synchronize()
+            lay = oracle_layer(mlps[l])
+            xin = hid.view(T, -1).cpu()
+            if replay:
+                ws = blk._workspace(T, exec_topk)
+                assert torch.equal(ws.topi.cpu(), i_dev) and torch.equal(ws.topv.cpu(), w_dev)
+                assert int((logits.cpu() > -1e8).sum()) == T * exec_topk
+                want = ref_moe.moe_forward_routed(xin, w_dev, i_dev, lay["experts"], lay["shared"],
+                                                  lay["shared_gate_w"])
+            else:
+                want, _, ref_topi, _ = ref_moe.moe_forward(
+                    xin, lay["gate_w"], lay["experts"], shape["top_k"], lay["shared"], lay["shared_gate_w"],
+                    router_logits=logits.cpu())
+                # compare the choice where it does not hang on the last bit of exp(): the two
+                # probabilities around the top-k boundary are equal or clearly apart
+                srt = logits.cpu().float().sort(dim=-1, descending=True, stable=True)
+                p = torch.softmax(logits.cpu().float(), -1).gather(1, srt.indices)
+                k = shape["top_k"]
+                clear = (srt.values[:, k - 1] == srt.values[:, k]) | ((p[:, k - 1] - p[:, k]) / p[:, k - 1] > 1e-4)
+                got_topi = blk._workspace(T).topi.cpu()
+                assert torch.equal(got_topi[clear], ref_topi[clear])
+                want = ref_moe.moe_forward_routed(xin, blk._workspace(T).topv.cpu(), got_topi, lay["experts"],
+                                                  lay["shared"], lay["shared_gate_w"])
+            torch.testing.assert_close(out.view(T, -1).cpu().float(), want.float(), **BF16_TOL)
+            hid = out
