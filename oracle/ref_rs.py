@@ -10,6 +10,10 @@ as identity, Linear, Softmax) in numpy float32.  Pinned by closed form against
 ``select_candidates`` restates utils/rs_staging.py:97-118, the staging adapter's scoring
 (the same formula as utils/eval_core.py:10104-10106).  Pinned by the reference's own
 known-answer tests, tests/test_rs_staging.py:147-150 and :308-312.
+
+``router_topk_feature`` restates utils/eval_core.py:10903-10908, the extra predictor input of
+``feature_mode="hidden_router_topk"``.  Pinned by vectors recorded from the reference's own
+method (tests/golden/make_rs_golden.py, tests/test_rs_golden.py) and by hand-made rows.
 """
 from __future__ import annotations
 
@@ -66,3 +70,20 @@ def plan_inputs(pred, pred_k: int, norm_topk_prob: bool, dtype):
     if norm_topk_prob:
         vals = vals / vals.sum(dim=-1, keepdim=True).clamp_min(1e-12)
     return ids.reshape(-1).tolist(), vals.to(dtype).to(torch.float32).reshape(-1).tolist()
+
+
+def router_topk_feature(idx, w, num_experts: int) -> np.ndarray:
+    """``[T, E]`` float32: token t's routing weights, divided by their sum (at least 1e-12),
+    added at its chosen experts; zero elsewhere (utils/eval_core.py:10903-10908).  The sum
+    and the division run in float32 as in the reference."""
+    idx = np.asarray(idx, dtype=np.int64)
+    ww = np.asarray(w, dtype=np.float32)
+    total = np.zeros(ww.shape[0], dtype=np.float32)
+    for k in range(ww.shape[1]):                     # left to right, as a float32 row sum
+        total = (total + ww[:, k]).astype(np.float32)
+    ww = (ww / np.maximum(total, np.float32(1e-12))[:, None]).astype(np.float32)
+    feat = np.zeros((idx.shape[0], int(num_experts)), dtype=np.float32)
+    for t in range(idx.shape[0]):
+        for k in range(idx.shape[1]):
+            feat[t, idx[t, k]] = np.float32(feat[t, idx[t, k]] + ww[t, k])
+    return feat

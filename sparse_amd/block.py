@@ -27,7 +27,7 @@ from torch import nn
 from . import ops
 from .context import DistEnv, Metrics, SparseContext
 from .residency import Backend, LayerResidency, ResidencyConfig
-from .rs import topk_for_planning
+from .rs import router_topk_feature, topk_for_planning
 from .weights import ExpertSlab, HostExpertArena, tile_weight
 
 
@@ -441,9 +441,17 @@ class DistributedSparseMoeBlock(nn.Module):
         return ws.topv, ws.topi, logits
 
     # ------------------------------------------------------------------ RS prefetch
-    def _rs_begin(self, x: torch.Tensor, seq_len: int, ws: _Workspace):
+    def _next_layer_rs_feature_mode(self) -> str:
+        """What the predictor of the next layer reads (:10910-10914)."""
+        target = self.layer_idx + 1
+        if SparseContext.rs_bank is None or target >= len(SparseContext.rs_bank):
+            return "hidden"
+        return str(getattr(SparseContext.rs_bank[target], "rs_feature_mode", "hidden"))
+
+    def _rs_begin(self, x: torch.Tensor, seq_len: int, ws: _Workspace, source=None):
         """Device half of ``_compute_and_schedule_next_layer_rs`` (:10916-11010): budget on
-        the host, predictor + top-k on the device, async copy of the top-k to the host."""
+        the host, predictor + top-k on the device, async copy of the top-k to the host.
+        ``source`` = this layer's own (ids, weights) for predictors that read them."""
         for_routing = self.expert_source == "rs" or self.exec_routing_mode == "rs"
         if (self.planner_mode != "rs_prefetch" and not for_routing) or SparseContext.rs_bank is None:
             return None
@@ -475,7 +483,15 @@ class DistributedSparseMoeBlock(nn.Module):
             policy = tres.light_policy
             here = policy.profile.cost(self.rank, self.layer_idx)
             policy.window_ms = here.compute(self.top_k, int(x.shape[0]) * self.top_k) + policy.cost.attention
-        pred = SparseContext.rs_bank[target](x.float()).to(torch.float32)
+        rs_in = x.float()
+        mode = self._next_layer_rs_feature_mode()
+        if mode == "hidden_router_topk":
+            if source is None:
+                return None
+            rs_in = torch.cat([rs_in, router_topk_feature(source[0], source[1], self.num_experts)], dim=-1)
+        elif mode != "hidden":
+            raise RuntimeError(f"Unsupported next-layer RS feature_mode={mode}")
+        pred = SparseContext.rs_bank[target](rs_in).to(torch.float32)
         self.metrics.rs_next_layer_pred_calls += 1
         self.metrics.rs_mlp_calls += 1
         if for_routing:
@@ -539,7 +555,8 @@ class DistributedSparseMoeBlock(nn.Module):
         else:
             if self.residency is not None:
                 self.residency.staging = None
-            rs_job = self._rs_begin(x, S, ws)
+            # a predictor that also reads this layer's routing runs after it (:16466-16506)
+            rs_job = self._rs_begin(x, S, ws) if self._next_layer_rs_feature_mode() == "hidden" else None
 
         shared_gate = ws.shared_gate if self.shared_gate_weight is not None else None
         fused = (self.residency is None and self.shared_weights is not None and self.dtype == torch.bfloat16
@@ -567,6 +584,8 @@ class DistributedSparseMoeBlock(nn.Module):
         else:
             # also the first layer and prefill of an RS-routed run (:11128-11136)
             logits = self._route(x, ws, after_logits=run_shared)
+        if not staged and self._next_layer_rs_feature_mode() == "hidden_router_topk":
+            rs_job = self._rs_begin(x, S, ws, source=(ws.topi, ws.topv))
 
         if fused:
             ops.moe_ffn_decode(self._experts_desc, x, ws.topv, ws.perm, ws.segs_dev, ws.inter, ws.parts,

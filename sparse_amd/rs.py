@@ -158,14 +158,14 @@ def _state_dict_of(payload: Any) -> Dict[str, torch.Tensor]:
 def module_from_payload(payload: Any, fallback_input_dim: int, fallback_num_experts: int) -> nn.Module:
     """Build the predictor a checkpoint payload describes (utils/eval_core.py:3490-3550):
     ``model_type`` picks the class, a bare state dict is a 1024-wide ``RoutingScoutMLP``.
-    Only predictors of routing probabilities read from the layer's hidden state are built;
-    cache-value checkpoints and the ``hidden_router_topk`` feature raise."""
+    Only predictors of routing probabilities are built; cache-value checkpoints raise.  The
+    checkpoint's ``feature_mode`` is left on the module as ``rs_feature_mode`` (``hidden``: the
+    layer's hidden state; ``hidden_router_topk``: that plus ``router_topk_feature`` of the
+    source layer's own routing), as the reference does (:3522, :3539)."""
     meta = payload if isinstance(payload, dict) else {}
     if meta.get("task", "") == "cache_value_rs":
         raise NotImplementedError("cache_value_rs checkpoints are not supported")
     feature = str(meta.get("feature_mode", "hidden"))
-    if feature != "hidden":
-        raise NotImplementedError(f"RS feature_mode {feature!r} is not supported")
     kind = meta.get("model_type", "")
     input_dim = int(meta.get("input_dim", fallback_input_dim))
     num_experts = int(meta.get("num_experts", fallback_num_experts))
@@ -178,7 +178,19 @@ def module_from_payload(payload: Any, fallback_input_dim: int, fallback_num_expe
     else:
         module = RoutingScoutMLP(fallback_input_dim, fallback_num_experts, hidden_dim=1024)
     module.load_state_dict(_state_dict_of(payload), strict=True)
+    if kind in ("next_layer_residual_logits_rs", "independent_light_logits_rs"):
+        module.rs_feature_mode = feature
     return module
+
+
+def router_topk_feature(idx: torch.Tensor, w: torch.Tensor, num_experts: int) -> torch.Tensor:
+    """Dense ``[T, E]`` fp32 rows holding each token's routing weights, renormalised to sum 1,
+    at its chosen experts (utils/eval_core.py:10903-10908)."""
+    feat = torch.zeros((idx.shape[0], int(num_experts)), device=idx.device, dtype=torch.float32)
+    ww = w.float()
+    ww = ww / ww.sum(dim=-1, keepdim=True).clamp_min(1e-12)
+    feat.scatter_add_(1, idx.to(torch.long), ww)
+    return feat
 
 
 def load_rs_bank(rs_dir: str, num_layers: int, hidden_dim: int, num_experts: int,

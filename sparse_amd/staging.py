@@ -270,6 +270,9 @@ class BoundedRS:
                 continue
             target = self.blocks[layer + 1].residency
             kk = int(k) if k is not None else min(block.num_experts, target.predict_topk())
+            # the captured prediction reads the hidden state only (utils/rs_overlap.py:124)
+            if str(getattr(rs_bank[layer + 1], "rs_feature_mode", "hidden")) != "hidden":
+                raise ValueError("the bounded staging engine needs predictors with feature_mode='hidden'")
             graph = GraphPrediction(rs_bank[layer + 1], batch, block.hidden_size, kk, dtype,
                                     block.norm_topk_prob, block.device)
             for seed in range(3):

@@ -10,7 +10,8 @@ top-level definitions of ``utils/eval_core.py``; they are taken out of the sourc
 and run on the CPU.  Recorded: state dicts of small predictors, their eval-mode outputs on a
 fixed input, and what the loader returns for directories with complete, incomplete and
 differently named checkpoint sets (layout, source layers, missing list, module classes,
-outputs of the loaded bank).
+outputs of the loaded bank), the block method that builds the ``hidden_router_topk`` input
+feature, and a checkpoint that asks for it.
 """
 from __future__ import annotations
 
@@ -42,6 +43,17 @@ def extract():
                               Optional=Optional, Tuple=Tuple, Sequence=Sequence)
     exec(compile(ast.fix_missing_locations(ast.Module(body=[future, *nodes], type_ignores=[])), str(REF), "exec"), ns)
     return ns
+
+
+def block_method(name: str):
+    """A method of the reference's ``DistributedSparseMoeBlock`` as a plain function."""
+    tree = ast.parse(REF.read_text())
+    cls = next(n for n in tree.body if isinstance(n, ast.ClassDef) and n.name == "DistributedSparseMoeBlock")
+    fn = next(n for n in cls.body if isinstance(n, ast.FunctionDef) and n.name == name)
+    future = ast.ImportFrom(module="__future__", names=[ast.alias(name="annotations")], level=0)
+    ns: Dict[str, Any] = dict(torch=torch)
+    exec(compile(ast.fix_missing_locations(ast.Module(body=[future, fn], type_ignores=[])), str(REF), "exec"), ns)
+    return ns[name]
 
 
 def lists(state: Dict[str, torch.Tensor]) -> Dict[str, Any]:
@@ -115,6 +127,36 @@ def main() -> None:
             except RuntimeError as err:
                 rec.update(error=str(err).splitlines()[0])
             out["directories"].append(rec)
+    # the extra predictor input of ``feature_mode="hidden_router_topk"``: the source layer's own
+    # routing as a dense [T, E] row of renormalised weights
+    from types import SimpleNamespace
+    build = block_method("_build_router_topk_feature")
+    g = torch.Generator().manual_seed(21)
+    out["router_topk_feature"] = []
+    for dtype, T, E2, K in ((torch.float32, 4, 5, 2), (torch.bfloat16, 3, 7, 3), (torch.float32, 2, 4, 4)):
+        w = torch.rand(T, K, generator=g).to(dtype)
+        idx = torch.stack([torch.randperm(E2, generator=g)[:K] for _ in range(T)])
+        feat = build(SimpleNamespace(num_experts=E2), idx, w)
+        out["router_topk_feature"].append(dict(dtype=str(dtype).replace("torch.", ""), num_experts=E2,
+                                               idx=idx.tolist(), w=w.float().tolist(), feat=feat.tolist()))
+    # a checkpoint that asks for that input: what the loader leaves on the module
+    mod = ns["RoutingScoutMLP"](D + E, E, hidden_dim=W).eval()
+    randomize(mod, 31)
+    meta = dict(model_type="independent_light_logits_rs", input_dim=D + E, num_experts=E, hidden_dim=W,
+                feature_mode="hidden_router_topk")
+    with tempfile.TemporaryDirectory() as tmp:
+        d = Path(tmp)
+        torch.save({**meta, "state_dict": mod.state_dict()}, d / "rs_l1_inL0.pth")
+        bank, task, layout, sources, missing = ns["_load_runtime_rs_bank"](
+            rs_path=d, num_layers=2, hidden_dim=D, num_experts=E, device=torch.device("cpu"), require_complete=True)
+        w = torch.rand(6, 2, generator=g)
+        idx = torch.stack([torch.randperm(E, generator=g)[:2] for _ in range(6)])
+        full = torch.cat([x, build(SimpleNamespace(num_experts=E), idx, w)], dim=-1)
+        with torch.no_grad():
+            out["feature_checkpoint"] = dict(
+                meta=meta, state=lists(mod.state_dict()), layout=layout, task=task,
+                feature_modes=[str(getattr(m, "rs_feature_mode", "hidden")) for m in bank],
+                idx=idx.tolist(), w=w.tolist(), output=bank[1](full).tolist())
     (OUT / "rs_bank.json").write_text(json.dumps(out, separators=(",", ":")))
     print("wrote", OUT / "rs_bank.json")
 

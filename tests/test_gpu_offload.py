@@ -300,3 +300,70 @@ def test_cost_aware_local_policy_on_the_device(device, tmp_path):
     _stack(device, "rr", capacity, top_m, "cpu")
     with pytest.raises(ValueError):
         install_lightweight_policies(CostProfile(path, 1))
+
+
+def test_predictor_reading_the_source_layers_routing(device):
+    """Checkpoints with ``feature_mode="hidden_router_topk"`` (reference :10964-10968): the
+    predictor of layer l+1 reads layer l's hidden state and layer l's own routing, so it runs
+    after that routing.  The ids and probabilities the planner receives must be the oracle's
+    top-k of the prediction recomputed on the CPU from the device's routing; outputs stay
+    those of the all-resident block."""
+    from oracle import ref_rs
+    from sparse_amd.context import SparseContext
+    from sparse_amd.rs import RoutingScoutMLP
+    from sparse_amd.synthetic import make_hidden
+    H, E, L, T = SHAPE["hidden"], SHAPE["num_experts"], SHAPE["num_layers"], 4
+    blocks, _ = _stack(device, "rs", 5, 3, "cpu")
+    bank = []
+    for l in range(L):
+        torch.manual_seed(70 + l)
+        m = RoutingScoutMLP(H + E, E, hidden_dim=32).eval()
+        m.rs_feature_mode = "hidden_router_topk"
+        bank.append(m.to(device))
+    SparseContext.set_rs_bank(bank)
+    seen, checked = [], 0
+    for blk in blocks:
+        blk._rs_plan_hook = lambda layer, ids, probs, budget, plan: seen.append((layer, list(ids), list(probs)))
+    for step in range(3):
+        SparseContext.current_phase = "decode"
+        SparseContext.begin_runtime_call(step)
+        hid = make_hidden(T, H, torch.bfloat16, seed=900 + step).view(T, 1, -1).to(device)
+        for l, blk in enumerate(blocks):
+            before = len(seen)
+            out, _ = blk(hid)
+            torch.cuda.synchronize()
+            if l + 1 < L and len(seen) > before:        # no plan when the target has no budget left
+                assert len(seen) == before + 1 and seen[-1][0] == l
+                checked += 1
+                ws = blk._workspace(T)
+                feat = ref_rs.router_topk_feature(ws.topi.cpu().numpy(), ws.topv.float().cpu().numpy(), E)
+                full = torch.cat([hid.view(T, H).float().cpu(), torch.from_numpy(feat)], dim=-1)
+                with torch.no_grad():
+                    pred = bank[l + 1].cpu()(full)
+                    bank[l + 1].to(device)
+                pred_k = len(seen[-1][1]) // T
+                ids, probs = ref_rs.plan_inputs(pred, pred_k, blk.norm_topk_prob, torch.bfloat16)
+                got_ids, got_probs = seen[-1][1], seen[-1][2]
+                # the device's fp32 prediction differs from the CPU's in the last bits: compare ids
+                # where the ranking is clear, probabilities to bf16 resolution
+                srt = pred.sort(dim=-1, descending=True).values
+                kk = min(pred_k, E - 1)
+                clear = ((srt[:, :kk] - srt[:, 1:kk + 1]) / srt[:, :kk] > 1e-3).all(1)
+                for t in range(T):
+                    if bool(clear[t]):
+                        assert got_ids[t * pred_k:(t + 1) * pred_k] == ids[t * pred_k:(t + 1) * pred_k]
+                        assert got_probs[t * pred_k:(t + 1) * pred_k] == pytest.approx(
+                            probs[t * pred_k:(t + 1) * pred_k], rel=2e-2)
+                assert bool(clear.any())
+            elif l + 1 == L:
+                assert len(seen) == before
+            hid = out
+    assert checked >= 3
+    # a feature mode nobody defines: the reference's forward calls the predictor for neither of
+    # the two modes it knows (:16467, :16505), so nothing is predicted and nothing is planned
+    bank[1].rs_feature_mode = "something_else"
+    SparseContext.begin_runtime_call(3)
+    before = len(seen)
+    blocks[0](make_hidden(T, H, torch.bfloat16, seed=1).view(T, 1, -1).to(device))
+    torch.cuda.synchronize()
+    assert len(seen) == before

@@ -56,3 +56,37 @@ def test_directory_loading_matches_the_reference(rec, tmp_path):
         if want is not None:
             with torch.no_grad():
                 torch.testing.assert_close(module(X), torch.tensor(want), rtol=1e-6, atol=1e-7)
+
+
+@pytest.mark.parametrize("rec", DATA["router_topk_feature"], ids=lambda r: f"{r['dtype']}-E{r['num_experts']}")
+def test_router_topk_feature_matches_the_reference(rec):
+    """The extra predictor input of ``feature_mode="hidden_router_topk"`` against the rows the
+    reference's own method returned: bit for bit from the host code (same PyTorch ops on the
+    same CPU), to float32 rounding from the numpy oracle."""
+    from sparse_amd.rs import router_topk_feature
+    idx = torch.tensor(rec["idx"])
+    w = torch.tensor(rec["w"], dtype=torch.float32).to(getattr(torch, rec["dtype"]))
+    want = torch.tensor(rec["feat"], dtype=torch.float32)
+    got = router_topk_feature(idx, w, rec["num_experts"])
+    assert got.dtype == torch.float32 and torch.equal(got, want)
+    np.testing.assert_allclose(ref_rs.router_topk_feature(rec["idx"], w.float().numpy(), rec["num_experts"]),
+                               want.numpy(), rtol=2e-7, atol=0)
+    assert torch.allclose(got.sum(1), torch.ones(len(idx)))
+
+
+def test_router_topk_feature_by_hand():
+    feat = ref_rs.router_topk_feature([[2, 0], [1, 3]], [[1.0, 3.0], [0.0, 0.0]], 4)
+    assert feat.tolist() == [[0.75, 0.0, 0.25, 0.0], [0.0, 0.0, 0.0, 0.0]]      # an all-zero row stays zero
+
+
+def test_checkpoint_asking_for_the_router_topk_feature(tmp_path):
+    """What the loader leaves on the modules, and the prediction from hidden state + feature."""
+    from sparse_amd.rs import router_topk_feature
+    rec = DATA["feature_checkpoint"]
+    torch.save({**rec["meta"], "state_dict": state_dict(rec["state"])}, tmp_path / "rs_l1_inL0.pth")
+    bank, sources, missing = load_rs_bank(str(tmp_path), 2, D, E, require_complete=True)
+    assert [str(getattr(m, "rs_feature_mode", "hidden")) for m in bank] == rec["feature_modes"]
+    feat = router_topk_feature(torch.tensor(rec["idx"]), torch.tensor(rec["w"]), E)
+    with torch.no_grad():
+        got = bank[1](torch.cat([X, feat], dim=-1))
+    torch.testing.assert_close(got, torch.tensor(rec["output"]), rtol=1e-6, atol=1e-7)
