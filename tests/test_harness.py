@@ -135,9 +135,10 @@ def test_payload_variants():
     assert isinstance(module_from_payload({"model_state_dict": plain.state_dict()}, 8, 5), RoutingScoutMLP)
     with pytest.raises(NotImplementedError):
         module_from_payload({"task": "cache_value_rs", "state_dict": {}}, 8, 5)
-    with pytest.raises(NotImplementedError):
-        module_from_payload({"model_type": "independent_light_logits_rs", "feature_mode": "hidden_router_topk",
-                             "state_dict": plain.state_dict()}, 8, 5)
+    wide = RoutingScoutMLP(8 + 5, 5, hidden_dim=1024)
+    mod = module_from_payload({"model_type": "independent_light_logits_rs", "feature_mode": "hidden_router_topk",
+                               "input_dim": 13, "state_dict": wide.state_dict()}, 8, 5)
+    assert mod.rs_feature_mode == "hidden_router_topk"
     with pytest.raises(RuntimeError):
         module_from_payload([1, 2, 3], 8, 5)
 
