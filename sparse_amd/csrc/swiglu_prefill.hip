@@ -301,10 +301,16 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_ffn_kernel(const Prefil
     cur = (cur == kPfStages - 1) ? 0 : cur + 1;
     nxt2 = (nxt2 == kPfStages - 1) ? 0 : nxt2 + 1;
   };
-  for (int kt = 0; kt < nk; kt += 2) {
+  // Slabs go in pairs with no branch inside the loop: a conditional second slab would give the
+  // loop head two different pictures of the outstanding fragment loads, and the waits the
+  // compiler puts before each MFMA would then assume the shorter one (eight loads behind
+  // instead of sixteen), i.e. drain the loads issued for the slab after next.
+  int kt = 0;
+  for (; kt + 2 <= nk; kt += 2) {
     slab(std::integral_constant<int, 0>{}, kt);
-    if (kt + 1 < nk) slab(std::integral_constant<int, 1>{}, kt + 1);
+    slab(std::integral_constant<int, 1>{}, kt + 1);
   }
+  if (kt < nk) slab(std::integral_constant<int, 0>{}, kt);
   __builtin_amdgcn_s_waitcnt(kWaitVm0);  // no copy may land in LDS after the epilogue starts to reuse it
   __syncthreads();
 
