@@ -57,6 +57,11 @@ struct DecodeArgs {
 __device__ __forceinline__ bf16x8 ld_bf16x8(const uint16_t* p) {
   return *reinterpret_cast<const bf16x8*>(p);
 }
+// Weights are read once per launch: a non-temporal load keeps them from displacing the
+// activations and partial results in the caches on their way through.
+__device__ __forceinline__ bf16x8 ld_stream_bf16x8(const uint16_t* p) {
+  return __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(p));
+}
 
 template <bool kGateUp, int NT>
 __global__ __launch_bounds__(kDecThreads) void decode_ffn_kernel(const DecodeArgs a) {
@@ -158,11 +163,11 @@ __global__ __launch_bounds__(kDecThreads) void decode_ffn_kernel(const DecodeArg
     }                                                                                    \
     _Pragma("unroll") for (int tl = 0; tl < kDecTiles; ++tl) {                           \
       const size_t o_ = tl * group_stride + (static_cast<size_t>(d) << 10);              \
-      W[0][tl][0] = ld_bf16x8(wt0 + o_);                                                 \
-      W[0][tl][1] = ld_bf16x8(wt0 + o_ + 512);                                           \
+      W[0][tl][0] = ld_stream_bf16x8(wt0 + o_);                                                 \
+      W[0][tl][1] = ld_stream_bf16x8(wt0 + o_ + 512);                                           \
       if (kGateUp) {                                                                     \
-        W[NM - 1][tl][0] = ld_bf16x8(wt1 + o_);                                          \
-        W[NM - 1][tl][1] = ld_bf16x8(wt1 + o_ + 512);                                    \
+        W[NM - 1][tl][0] = ld_stream_bf16x8(wt1 + o_);                                          \
+        W[NM - 1][tl][1] = ld_stream_bf16x8(wt1 + o_ + 512);                                    \
       }                                                                                  \
     }                                                                                    \
   } while (0)
