@@ -429,6 +429,7 @@ def test_tile_weight_kernel_matches_host_packing(device, dtype):
 
 # ------------------------------------------------------------------ shared expert + combine
 @pytest.mark.parametrize("dtype,T", [(torch.bfloat16, 8), (torch.bfloat16, 32), (torch.bfloat16, 200),
+                                     (torch.bfloat16, 2048), (torch.bfloat16, 2500),   # XCDs own bands of M-tiles
                                      (torch.float32, 8), (torch.float32, 100)])
 @pytest.mark.parametrize("gated", [True, False])
 def test_shared_expert(device, dtype, T, gated):
