@@ -313,6 +313,7 @@ def cached_decode_workload(dtype, device, steps, batch=8, capacity=15, top_m=8):
                                   ("rs_informed", "rs", "informed"), ("rs-epipe_informed", "rs-epipe", "informed"),
                                   ("rs-epipe_light_informed", "rs-epipe", "informed"),
                                   ("rs-epipe_staged_informed", "rs-epipe", "informed")):
+        print(f"[bench] cached decode: {name}, {steps} steps", file=sys.stderr, flush=True)
         staged = "staged" in name
         kw = dict(staging_pool_slots=4) if staged else {}
         blocks, metrics, _ = build_offload_stack(shape, dtype, device, method, capacity, top_m, rs_kind=rs_kind,
@@ -370,6 +371,7 @@ def epipe_prefill_workload(dtype, device, tokens=4096, chunk=2048, capacity=19, 
     del blocks
     release_stack()
     for method in ("rr", "rs-epipe", "sparse"):
+        print(f"[bench] chunked prefill: {method}", file=sys.stderr, flush=True)
         blocks, metrics, _ = build_offload_stack(shape, dtype, device, method, capacity, top_m, rs_kind="informed",
                                                  epipe_prefill_enable=True)
         wall = run_phase_steps(blocks, inputs, "prefill")   # cold cache
