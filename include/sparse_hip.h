@@ -245,16 +245,27 @@ int sparse_hip_shared_expert(const void* x_dev, const void* gate_w_dev, const vo
  * Decode fast path: sparse_hip_grouped_swiglu_decode and sparse_hip_shared_expert of one
  * call in a single launch pair (gate/up of every routed segment and of the shared
  * expert, then all down projections), so the chip sees one fat stream of weights
- * instead of four thinner launches.  Results are identical to the two separate calls.
- * bf16 only, T <= SPARSE_HIP_DECODE_MAX_TOKENS.  Arguments as in those two functions;
- * `sh_*` are the shared expert's (utils/eval_core.py:16520-16526).
+ * instead of four thinner launches.  bf16 only, T <= SPARSE_HIP_DECODE_MAX_TOKENS.
+ * Arguments as in those two functions; `sh_*` are the shared expert's
+ * (utils/eval_core.py:16520-16526).
+ * `split_ws_dev` is NULL or a workspace of sparse_hip_decode_split_ws_bytes(T, H) bytes.  With
+ * NULL the results are identical to the two separate calls.  With a workspace, and when
+ * sparse_hip_decode_split_parts(Is) > 1, the shared expert's down projection, whose reduction
+ * is Is long against the routed experts' I, is cut into that many workgroups per tile so that
+ * it no longer trails the launch: `shared_dev` is then NOT written, the workspace receives the
+ * fp32 partial sums [parts][T][H], and sparse_hip_combine_split finishes them (adds them in
+ * their order, rounds, applies the shared gate) while it combines -- the same rounding steps
+ * as the one-workgroup form, with the fp32 sum grouped differently.
  */
+size_t sparse_hip_decode_split_ws_bytes(int T, int H);
+int sparse_hip_decode_split_parts(int Is);
 int sparse_hip_moe_ffn_decode(const sparse_hip_experts* experts, const void* x_dev, const void* topv_dev,
                               const int32_t* perm_dev, const int32_t* seg_offsets_dev,
                               const sparse_hip_seglist* segs, int T, int K, void* inter_ws_dev,
                               void* parts_dev, const void* sh_gate_w_dev, const void* sh_up_w_dev,
                               const void* sh_down_w_dev, const void* shared_gate_dev, int Is,
-                              void* sh_inter_ws_dev, void* shared_dev, void* stream);
+                              void* sh_inter_ws_dev, void* shared_dev, void* split_ws_dev,
+                              void* stream);
 
 /* ---- A7: combine ----------------------------------------------------------- */
 
@@ -269,6 +280,17 @@ int sparse_hip_moe_ffn_decode(const sparse_hip_experts* experts, const void* x_d
 int sparse_hip_combine(const void* parts_dev, const int32_t* inv_perm_dev,
                        const void* shared_dev, int dtype, int T, int K, int H, void* out_dev,
                        void* stream);
+
+/*
+ * The same for a decode call whose shared expert was left as partial sums by
+ * sparse_hip_moe_ffn_decode(split_ws_dev): shared[t] = bf16(bf16(sum of the `nparts` fp32
+ * parts) * bf16(sigmoid(shared_gate[t]))) (no factor when `shared_gate_dev` is NULL) -- the
+ * tail of `_shared_expert_forward` (utils/eval_core.py:9455-9463) -- added after the routed
+ * parts as above.  bf16 only.
+ */
+int sparse_hip_combine_split(const void* parts_dev, const int32_t* inv_perm_dev, const void* split_ws_dev,
+                             int nparts, const void* shared_gate_dev, int T, int K, int H,
+                             void* out_dev, void* stream);
 
 /* ---- A11/A12/A13: expert residency ----------------------------------------- */
 

@@ -89,6 +89,12 @@ class _Workspace:
         self.shared_out = torch.empty((T, H), device=device, dtype=dtype) if Is else None
         self.segs_dev = ops.seglist_device(self.perm, min(E, T * K))
         self.route_counter = torch.zeros((1,), device=device, dtype=torch.int32)
+        # small decode calls cut the shared down projection's long reduction into parts (fp32
+        # sums here) that the combine step finishes; from 17 tokens on the routed experts are
+        # enough work beside it and the extra reads of the combine step cost more than they save
+        self.split_parts = (ops.decode_split_parts(Is) if Is and T <= 16
+                            and dtype == torch.bfloat16 and torch.device(device).type == "cuda" else 1)
+        self.split_ws = ops.decode_split_workspace(T, H, device) if self.split_parts > 1 else None
         # host mirrors for the offloaded path (pinned, written by async D2H copies)
         self.host_offsets = torch.empty((E + 1,), dtype=torch.int32, pin_memory=True)
         self.host_rs_topi = torch.empty((T * E,), dtype=torch.int64, pin_memory=True)
@@ -589,7 +595,7 @@ class DistributedSparseMoeBlock(nn.Module):
 
         if fused:
             ops.moe_ffn_decode(self._experts_desc, x, ws.topv, ws.perm, ws.segs_dev, ws.inter, ws.parts,
-                               self.shared_weights, shared_gate, ws.shared_inter, ws.shared_out)
+                               self.shared_weights, shared_gate, ws.shared_inter, ws.shared_out, ws.split_ws)
         elif self.residency is None:
             ops.grouped_swiglu(self._experts_desc, x, ws.topv, ws.perm, ws.segs_dev, ws.inter, ws.parts)
         else:
@@ -617,7 +623,10 @@ class DistributedSparseMoeBlock(nn.Module):
         if side is not None:
             torch.cuda.current_stream().wait_stream(side)
         out = torch.empty((T, H), device=x.device, dtype=self.dtype)
-        ops.combine(ws.parts, ws.perm, ws.shared_out, T, k_exec, out)
+        if fused and ws.split_ws is not None:
+            ops.combine_split(ws.parts, ws.perm, ws.split_ws, ws.split_parts, shared_gate, T, k_exec, out)
+        else:
+            ops.combine(ws.parts, ws.perm, ws.shared_out, T, k_exec, out)
         out = out.view(B, S, H)
         if self._return_tensor_only_mlp():
             return out

@@ -11,7 +11,9 @@ int decode_shared_bf16(const void*, const void*, const void*, const void*, const
                        void*, hipStream_t);
 int decode_fused_bf16(const sparse_hip_experts*, const void*, const void*, const int32_t*, const int32_t*,
                       const sparse_hip_seglist*, int, int, void*, void*, const void*, const void*, const void*,
-                      const void*, int, void*, void*, hipStream_t);
+                      const void*, int, void*, void*, void*, hipStream_t);
+size_t decode_split_ws_bytes(int, int);
+int decode_split_parts(int);
 int prefill_routed_bf16(const sparse_hip_experts*, const void*, const void*, const int32_t*, const int32_t*,
                         const sparse_hip_seglist*, int, int, void*, void*, void*, hipStream_t);
 size_t prefill_ws_bytes(int, int, int, int, int);
@@ -115,7 +117,7 @@ int sparse_hip_moe_ffn_decode(const sparse_hip_experts* experts, const void* x_d
                               const sparse_hip_seglist* segs, int T, int K, void* inter_ws_dev, void* parts_dev,
                               const void* sh_gate_w_dev, const void* sh_up_w_dev, const void* sh_down_w_dev,
                               const void* shared_gate_dev, int Is, void* sh_inter_ws_dev, void* shared_dev,
-                              void* stream) {
+                              void* split_ws_dev, void* stream) {
   int rc = check_routed("moe_ffn_decode", experts, x_dev, topv_dev, perm_dev, seg_offsets_dev, segs, T, K,
                         inter_ws_dev, parts_dev);
   if (rc != SPARSE_HIP_OK) return rc;
@@ -127,13 +129,20 @@ int sparse_hip_moe_ffn_decode(const sparse_hip_experts* experts, const void* x_d
              "moe_ffn_decode: NULL shared-expert pointer");
   SP_REQUIRE(((reinterpret_cast<uintptr_t>(sh_gate_w_dev) | reinterpret_cast<uintptr_t>(sh_up_w_dev) |
                reinterpret_cast<uintptr_t>(sh_down_w_dev) | reinterpret_cast<uintptr_t>(sh_inter_ws_dev) |
-               reinterpret_cast<uintptr_t>(shared_dev)) &
+               reinterpret_cast<uintptr_t>(shared_dev) | reinterpret_cast<uintptr_t>(split_ws_dev)) &
               15) == 0,
              "moe_ffn_decode: shared-expert pointers must be 16-byte aligned");
   return decode_fused_bf16(experts, x_dev, topv_dev, perm_dev, seg_offsets_dev, segs, T, K, inter_ws_dev,
                            parts_dev, sh_gate_w_dev, sh_up_w_dev, sh_down_w_dev, shared_gate_dev, Is,
-                           sh_inter_ws_dev, shared_dev, as_stream(stream));
+                           sh_inter_ws_dev, shared_dev, split_ws_dev, as_stream(stream));
 }
+
+size_t sparse_hip_decode_split_ws_bytes(int T, int H) {
+  if (T < 1 || H < 1) return 0;
+  return decode_split_ws_bytes(T, H);
+}
+
+int sparse_hip_decode_split_parts(int Is) { return Is > 0 && Is % 64 == 0 ? decode_split_parts(Is) : 1; }
 
 int sparse_hip_shared_expert(const void* x_dev, const void* gate_w_dev, const void* up_w_dev,
                              const void* down_w_dev, const void* shared_gate_dev, int dtype, int T, int H,

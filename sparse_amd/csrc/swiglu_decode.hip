@@ -24,6 +24,7 @@ constexpr int kDecThreads = 256;
 constexpr int kDecWaves = 4;
 constexpr int kDecTiles = 2;                    // 16-row tiles per workgroup
 constexpr int kDecRows = kDecTiles * 16;        // output rows per workgroup
+constexpr int kDecSplit = 4;                    // parts of the shared down projection's reduction
 
 struct DecodeArgs {
   // routed experts
@@ -51,6 +52,10 @@ struct DecodeArgs {
   int32_t Ndim_s;
   int32_t tiles_s;
   int32_t T;
+  // shared down projection with its reduction cut into `split_s` parts, one workgroup each
+  // (1 = not cut): fp32 partial sums [split_s][T][Ndim_s], finished by the combine step
+  int32_t split_s;
+  float* split_sums;
   sparse_hip_seglist segs;
 };
 
@@ -70,18 +75,24 @@ __global__ __launch_bounds__(kDecThreads) void decode_ffn_kernel(const DecodeArg
   const int r = lane & 15, q = lane >> 4;
 
   // ---- which tile of which matrix ------------------------------------------
-  const bool is_shared = static_cast<int>(blockIdx.x) < a.tiles_s;
+  const int split = kGateUp ? 1 : a.split_s;
+  const bool is_shared = static_cast<int>(blockIdx.x) < a.tiles_s * split;
   const uint16_t *w0, *w1 = nullptr;
   int Kdim, Ndim, row0, M, r0 = 0;
+  int tile_s = 0, part = 0, kbeg = 0, klen = 0;  // which part of the shared reduction (whole: part 0 of 1)
   if (is_shared) {
     Kdim = a.Kdim_s;
     Ndim = a.Ndim_s;
-    row0 = blockIdx.x * kDecRows;
+    tile_s = blockIdx.x / split;
+    part = blockIdx.x - tile_s * split;
+    row0 = tile_s * kDecRows;
     M = a.T;
     w0 = a.w_s;
     w1 = a.w2_s;
+    klen = Kdim / split;
+    kbeg = part * klen;
   } else {
-    const int b = blockIdx.x - a.tiles_s;
+    const int b = blockIdx.x - a.tiles_s * split;
     const int si = b / a.tiles_r;
     int eid, slot_id;
     if (a.segs.eids_dev != nullptr) {
@@ -96,6 +107,7 @@ __global__ __launch_bounds__(kDecThreads) void decode_ffn_kernel(const DecodeArg
     }
     Kdim = a.Kdim;
     Ndim = a.Ndim;
+    klen = Kdim;
     row0 = (b - si * a.tiles_r) * kDecRows;
     r0 = a.seg_offsets[eid];
     M = a.seg_offsets[eid + 1] - r0;
@@ -113,7 +125,7 @@ __global__ __launch_bounds__(kDecThreads) void decode_ffn_kernel(const DecodeArg
     brow[nt] = nullptr;
     if (n < M) {
       if (is_shared) {
-        brow[nt] = a.act_s + static_cast<size_t>(n) * Kdim;
+        brow[nt] = a.act_s + static_cast<size_t>(n) * Kdim + kbeg;
       } else if (kGateUp) {
         brow[nt] = a.act_r + static_cast<size_t>(a.perm[r0 + n] / a.topk) * Kdim;
       } else {
@@ -134,9 +146,10 @@ __global__ __launch_bounds__(kDecThreads) void decode_ffn_kernel(const DecodeArg
   // of 64 k; the first KB of a block is the first MFMA's A operand in lane order, the
   // second KB the second MFMA's, so every load instruction of a wave reads 1 KB straight.
   const size_t group_stride = static_cast<size_t>(16) * Kdim;
-  const uint16_t* wt0 = w0 + static_cast<size_t>(row0 >> 4) * group_stride + lane * 8;
+  const size_t kskip = static_cast<size_t>(kbeg >> 6) << 10;  // 64-wide blocks before this part, 1 K elements each
+  const uint16_t* wt0 = w0 + static_cast<size_t>(row0 >> 4) * group_stride + kskip + lane * 8;
   const uint16_t* wt1 = kGateUp ? w1 + static_cast<size_t>(row0 >> 4) * group_stride + lane * 8 : nullptr;
-  const int ND = Kdim >> 6;
+  const int ND = klen >> 6;
 
   // Two register stages per wavefront, used in turn: while one slice is multiplied the next
   // one is already in flight and the one after that is requested as soon as its stage is
@@ -149,7 +162,7 @@ __global__ __launch_bounds__(kDecThreads) void decode_ffn_kernel(const DecodeArg
   // token columns past the segment read the block's first activation row (always mapped):
   // their products land in output columns the epilogue never stores, so they need neither a
   // branch around the loads nor a mask
-  const uint16_t* bsafe = is_shared ? a.act_s : a.act_r;
+  const uint16_t* bsafe = is_shared ? a.act_s + kbeg : a.act_r;
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt)
     if (brow[nt] == nullptr) brow[nt] = bsafe;
@@ -224,17 +237,8 @@ __global__ __launch_bounds__(kDecThreads) void decode_ffn_kernel(const DecodeArg
       for (int m = 0; m < NM; ++m) red[wave][(tl * NT + nt) * NM + m][lane] = acc[m][tl][nt];
   __syncthreads();
 
-  for (int f = wave; f < NFRAG; f += kDecWaves) {
-    const int tl = f / NT, nt = f - tl * NT;
-    const int n = r + 16 * nt;
-    if (n >= M) continue;
-    f32x4 s0 = red[0][f * NM][lane];
-    f32x4 s1 = kGateUp ? red[0][f * NM + 1][lane] : f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int w = 1; w < kDecWaves; ++w) {
-      s0 += red[w][f * NM][lane];
-      if (kGateUp) s1 += red[w][f * NM + 1][lane];
-    }
+  // one fragment of the tile: rows row0 + 16 tl + 4 q .. + 3 of token column n, as fp32 sums
+  auto emit = [&](int tl, int n, const f32x4& s0, const f32x4& s1) {
     const int orow = row0 + tl * 16 + q * 4;
     float scale = 1.f;
     bool has_scale = false;
@@ -269,12 +273,43 @@ __global__ __launch_bounds__(kDecThreads) void decode_ffn_kernel(const DecodeArg
     pk.x = static_cast<uint32_t>(o[0]) | (static_cast<uint32_t>(o[1]) << 16);
     pk.y = static_cast<uint32_t>(o[2]) | (static_cast<uint32_t>(o[3]) << 16);
     *reinterpret_cast<uint2*>(dst) = pk;
+  };
+
+  if (!kGateUp && is_shared && split > 1) {
+    // A part of a shared tile: its fp32 sums go to memory as they are; the combine step adds
+    // the parts in their order, rounds, applies the shared gate and adds the result in.
+    const size_t part_stride = static_cast<size_t>(a.T) * Ndim;
+    for (int f = wave; f < NFRAG; f += kDecWaves) {
+      const int tl = f / NT, nt = f - tl * NT;
+      const int n = r + 16 * nt;
+      if (n >= M) continue;
+      f32x4 s0 = red[0][f][lane];
+#pragma unroll
+      for (int w = 1; w < kDecWaves; ++w) s0 += red[w][f][lane];
+      *reinterpret_cast<f32x4*>(a.split_sums + part * part_stride + static_cast<size_t>(n) * Ndim + row0 + tl * 16 +
+                                q * 4) = s0;
+    }
+    return;
+  }
+
+  for (int f = wave; f < NFRAG; f += kDecWaves) {
+    const int tl = f / NT, nt = f - tl * NT;
+    const int n = r + 16 * nt;
+    if (n >= M) continue;
+    f32x4 s0 = red[0][f * NM][lane];
+    f32x4 s1 = kGateUp ? red[0][f * NM + 1][lane] : f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int w = 1; w < kDecWaves; ++w) {
+      s0 += red[w][f * NM][lane];
+      if (kGateUp) s1 += red[w][f * NM + 1][lane];
+    }
+    emit(tl, n, s0, s1);
   }
 }
 
 template <bool kGateUp>
 static int launch_decode(const DecodeArgs& a, int n_seg, hipStream_t st) {
-  const int grid = a.tiles_s + n_seg * a.tiles_r;
+  const int grid = a.tiles_s * (kGateUp ? 1 : a.split_s) + n_seg * a.tiles_r;
   if (grid == 0) return SPARSE_HIP_OK;
   ProfScope prof(kGateUp ? SPARSE_HIP_K_DECODE_GATEUP : SPARSE_HIP_K_DECODE_DOWN, st);
   if (a.T <= 16) {
@@ -292,6 +327,7 @@ int decode_routed_bf16(const sparse_hip_experts* ex, const void* x, const void* 
                        void* inter_ws, void* parts, hipStream_t st) {
   const uint64_t H = ex->hidden, I = ex->inter;
   DecodeArgs a = {};
+  a.split_s = 1;
   a.slab = static_cast<const uint16_t*>(ex->slab_dev);
   a.slot_stride = ex->slot_stride / 2;
   a.expert_slot = ex->expert_slot_dev;
@@ -327,9 +363,11 @@ int decode_routed_bf16(const sparse_hip_experts* ex, const void* x, const void* 
 int decode_fused_bf16(const sparse_hip_experts* ex, const void* x, const void* topv, const int32_t* perm,
                       const int32_t* seg_offsets, const sparse_hip_seglist* segs, int T, int K, void* inter_ws,
                       void* parts, const void* sh_gate_w, const void* sh_up_w, const void* sh_down_w,
-                      const void* shared_gate, int Is, void* sh_inter_ws, void* shared_out, hipStream_t st) {
+                      const void* shared_gate, int Is, void* sh_inter_ws, void* shared_out, void* split_ws,
+                      hipStream_t st) {
   const uint64_t H = ex->hidden, I = ex->inter;
   DecodeArgs a = {};
+  a.split_s = 1;
   a.slab = static_cast<const uint16_t*>(ex->slab_dev);
   a.slot_stride = ex->slot_stride / 2;
   a.expert_slot = ex->expert_slot_dev;
@@ -372,14 +410,25 @@ int decode_fused_bf16(const sparse_hip_experts* ex, const void* x, const void* t
   a.Kdim_s = Is;
   a.Ndim_s = static_cast<int32_t>(H);
   a.tiles_s = a.Ndim_s / kDecRows;
+  // The shared down projection reduces over Is, several times the routed experts' I: as one
+  // workgroup per tile it would still be streaming when everything else has finished.  With a
+  // workspace it is cut into kDecSplit parts whose fp32 sums the combine step adds up.
+  if (split_ws != nullptr && (Is / 64) % kDecSplit == 0) {
+    a.split_s = kDecSplit;
+    a.split_sums = static_cast<float*>(split_ws);
+  }
   return launch_decode<false>(a, segs->n, st);
 }
+
+size_t decode_split_ws_bytes(int T, int H) { return static_cast<size_t>(kDecSplit) * T * H * sizeof(float); }
+int decode_split_parts(int Is) { return (Is / 64) % kDecSplit == 0 ? kDecSplit : 1; }
 
 // Shared expert, bf16, T <= 32.
 int decode_shared_bf16(const void* x, const void* gate_w, const void* up_w, const void* down_w,
                        const void* shared_gate, int T, int H, int Is, void* inter_ws, void* shared_out,
                        hipStream_t st) {
   DecodeArgs a = {};
+  a.split_s = 1;
   a.T = T;
   a.topk = 1;
   a.tiles_r = 1;

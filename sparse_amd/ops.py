@@ -303,6 +303,24 @@ def combine(parts: torch.Tensor, perm: Permutation, shared: Optional[torch.Tenso
     _lib.check(rc, "sparse_hip_combine")
 
 
+def combine_split(parts: torch.Tensor, perm: Permutation, split_ws: torch.Tensor, nparts: int,
+                  shared_gate: Optional[torch.Tensor], T: int, K: int, out: torch.Tensor) -> None:
+    """``combine`` for a decode call whose shared down projection was left as ``nparts`` fp32
+    partial sums in ``split_ws`` (``moe_ffn_decode(split_ws=...)``)."""
+    lib = _lib.load()
+    H = parts.shape[1]
+    _need(parts, "parts", torch.bfloat16, (T * K, H))
+    _need(out, "out", parts.dtype, (T, H))
+    _need(split_ws, "split workspace", torch.float32)
+    if split_ws.numel() < int(nparts) * T * H:
+        raise ValueError("split workspace is too small for this T and H")
+    if shared_gate is not None:
+        _need(shared_gate, "shared gate logits", parts.dtype, (T,))
+    rc = lib.sparse_hip_combine_split(_ptr(parts), _ptr(perm.inv_perm), _ptr(split_ws), int(nparts), _ptr(shared_gate),
+                                      T, K, H, _ptr(out), _stream())
+    _lib.check(rc, "sparse_hip_combine_split")
+
+
 # --------------------------------------------------------------------------- residency
 class Event:
     """A HIP event owned through the C ABI (no timing unless asked)."""
@@ -411,8 +429,11 @@ def profile_read() -> dict:
 
 def moe_ffn_decode(experts: Experts, x: torch.Tensor, topv: torch.Tensor, perm: Permutation, segs: SegList,
                    inter_ws: torch.Tensor, parts: torch.Tensor, shared_w, shared_gate: Optional[torch.Tensor],
-                   shared_inter_ws: torch.Tensor, shared_out: torch.Tensor) -> None:
-    """Routed experts + shared expert of a decode call in one launch pair (bf16, T <= 32)."""
+                   shared_inter_ws: torch.Tensor, shared_out: torch.Tensor,
+                   split_ws: Optional[torch.Tensor] = None) -> None:
+    """Routed experts + shared expert of a decode call in one launch pair (bf16, T <= 32).
+    ``split_ws`` (from ``decode_split_workspace``) lets the shared down projection spread its
+    long reduction over four workgroups per tile."""
     lib = _lib.load()
     T, H = x.shape
     K = topv.shape[1]
@@ -427,8 +448,26 @@ def moe_ffn_decode(experts: Experts, x: torch.Tensor, topv: torch.Tensor, perm: 
     _need(dw, "shared down_proj", x.dtype, (H, Is))
     _need(shared_inter_ws, "shared inter_ws", x.dtype, (T, Is))
     _need(shared_out, "shared out", x.dtype, (T, H))
+    if split_ws is not None:
+        _need(split_ws, "split workspace", torch.float32)
+        if split_ws.numel() * 4 < int(lib.sparse_hip_decode_split_ws_bytes(T, H)):
+            raise ValueError("split workspace is too small for this T and H")
     rc = lib.sparse_hip_moe_ffn_decode(C.byref(experts), _ptr(x), _ptr(topv), _ptr(perm.perm),
                                        _ptr(perm.seg_offsets), C.byref(segs), T, K, _ptr(inter_ws), _ptr(parts),
                                        _ptr(gw), _ptr(uw), _ptr(dw), _ptr(shared_gate), Is, _ptr(shared_inter_ws),
-                                       _ptr(shared_out), _stream())
+                                       _ptr(shared_out), _ptr(split_ws), _stream())
     _lib.check(rc, "sparse_hip_moe_ffn_decode")
+
+
+def decode_split_workspace(T: int, H: int, device) -> torch.Tensor:
+    """fp32 workspace for ``moe_ffn_decode(split_ws=...)``: the partial sums of the shared down
+    projection, ``[parts, T, H]``."""
+    lib = _lib.load()
+    n = int(lib.sparse_hip_decode_split_ws_bytes(int(T), int(H)))
+    return torch.empty(n // 4, dtype=torch.float32, device=device)
+
+
+def decode_split_parts(shared_inter: int) -> int:
+    """Parts the fused decode call cuts the shared down projection into when it is given a
+    workspace (1: it is not cut and ``shared_out`` is written as usual)."""
+    return int(_lib.load().sparse_hip_decode_split_parts(int(shared_inter)))

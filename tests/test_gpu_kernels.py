@@ -449,6 +449,66 @@ def test_shared_expert(device, dtype, T, gated):
     torch.testing.assert_close(out.cpu().float(), ref.float(), **tol(dtype))
 
 
+@pytest.mark.parametrize("T", [1, 8, 17, 32])
+@pytest.mark.parametrize("gated", [True, False])
+def test_fused_decode_with_the_shared_reduction_split(device, T, gated):
+    """The fused decode launch pair with the workspace that spreads the shared expert's long
+    down-projection reduction over four workgroups per tile, finished by combine_split: routed
+    parts bit for bit those of the one-workgroup form, the layer output within one bf16
+    rounding of combine() on that form (the fp32 sum is grouped differently) and within
+    tolerance of the oracle, the same bits call after call, also when the two forms alternate."""
+    ops = _ops()
+    from sparse_amd.weights import ExpertSlab, tile_weight
+    H, E, I, K, Is = 512, 8, 128, 2, 1024
+    dtype = torch.bfloat16
+    layer = make_layer(H, E, I, K, Is=Is, shared_gate=gated, dtype=dtype, seed=81, std=0.05)
+    xc = make_hidden(T, H, dtype, seed=82)
+    x = xc.to(device)
+    slab = ExpertSlab.resident(layer["experts"], H, I, dtype, device)
+    experts = ops.make_experts(slab.data, slab.expert_slot, E, H, I)
+    logits, sg = ops.router_logits(x, layer["gate_w"].to(device), layer["shared_gate_w"].to(device) if gated else None)
+    topv, topi = ops.gate_topk(logits, K, out_dtype=dtype)
+    perm = ops.permute_build(topi, E)
+    segs = ops.seglist_device(perm, min(E, T * K))
+    sw = tuple(tile_weight(t).reshape(t.shape).contiguous().to(device) for t in layer["shared"])
+    nparts = ops.decode_split_parts(Is)
+    assert nparts == 4 and ops.decode_split_parts(64 * 7) == 1
+    ws = ops.decode_split_workspace(T, H, device)
+
+    def run(split):
+        inter = torch.empty((T * K, I), device=device, dtype=dtype)
+        parts = torch.empty((T * K, H), device=device, dtype=dtype)
+        sh_inter = torch.empty((T, Is), device=device, dtype=dtype)
+        sh_out = torch.full((T, H), float("nan"), device=device, dtype=dtype)
+        out = torch.empty((T, H), device=device, dtype=dtype)
+        ws.fill_(float("nan"))
+        ops.moe_ffn_decode(experts, x, topv, perm, segs, inter, parts, sw, sg if gated else None, sh_inter, sh_out,
+                           ws if split else None)
+        if split:
+            assert torch.isnan(sh_out.float()).all()            # left to combine_split
+            ops.combine_split(parts, perm, ws, nparts, sg if gated else None, T, K, out)
+        else:
+            ops.combine(parts, perm, sh_out, T, K, out)
+        torch.cuda.synchronize()
+        return parts, out
+
+    parts0, out0 = run(False)
+    ref, _, _, _ = ref_moe.moe_forward(xc, layer["gate_w"], layer["experts"], K, layer["shared"], layer["shared_gate_w"],
+                                       router_logits=logits.cpu())
+    first = None
+    for split in (True, False, True, True):
+        parts1, out1 = run(split)
+        assert torch.equal(parts1, parts0)
+        if not split:
+            assert torch.equal(out1, out0)
+            continue
+        first = out1 if first is None else first
+        assert torch.equal(out1, first) and not torch.isnan(out1.float()).any()
+        torch.testing.assert_close(out1.float(), out0.float(), rtol=1.6e-2, atol=1e-6)   # two bf16 roundings apart at most
+        torch.testing.assert_close(out1.cpu().float(), ref.float(), **tol(dtype))
+    assert (first == out0).float().mean() > 0.9                      # most sums round the same way
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 def test_combine_is_ordered_sum(device, dtype):
     ops = _ops()
