@@ -34,13 +34,17 @@ int hip_fail(hipError_t err, const char* what);
     if (_e != hipSuccess) return sparse::hip_fail(_e, name);      \
   } while (0)
 
-// Brackets one kernel launch with an event pair while profiling is enabled.
+// Times one kernel launch while profiling is enabled.  Either the scope records an event
+// before and after the launch (the interval then contains the dispatch latency of the launch,
+// 2-3 us), or the launch site asks for the pair with `dispatch_events` and hands it to
+// hipExtLaunchKernelGGL, which stamps the events with the dispatch's own begin and end.
 struct ProfScope {
-  ProfScope(int kernel, hipStream_t stream);
+  ProfScope(int kernel, hipStream_t stream, bool dispatch_events = false);
   ~ProfScope();
+  bool active() const { return start_ != nullptr && stop_ != nullptr; }
   int kernel_;
   hipStream_t stream_;
-  hipEvent_t start_;
+  hipEvent_t start_, stop_;  // stop_ is set only for dispatch events
 };
 
 inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }

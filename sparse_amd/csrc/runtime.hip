@@ -44,16 +44,30 @@ static hipEvent_t prof_take_event() {
   return e;
 }
 
-ProfScope::ProfScope(int kernel, hipStream_t stream) : kernel_(kernel), stream_(stream), start_(nullptr) {
+ProfScope::ProfScope(int kernel, hipStream_t stream, bool dispatch_events)
+    : kernel_(kernel), stream_(stream), start_(nullptr), stop_(nullptr) {
   if (!g_prof_on) return;
   std::lock_guard<std::mutex> lk(g_prof_mu);
   start_ = prof_take_event();
-  if (start_ != nullptr) (void)hipEventRecord(start_, stream_);
+  if (start_ == nullptr) return;
+  if (dispatch_events) {
+    stop_ = prof_take_event();
+    if (stop_ == nullptr) {
+      g_prof_free.push_back(start_);
+      start_ = nullptr;
+    }
+    return;
+  }
+  (void)hipEventRecord(start_, stream_);
 }
 
 ProfScope::~ProfScope() {
   if (start_ == nullptr) return;
   std::lock_guard<std::mutex> lk(g_prof_mu);
+  if (stop_ != nullptr) {  // stamped by the launch itself
+    g_prof_recs[kernel_].push_back(ProfRec{start_, stop_});
+    return;
+  }
   hipEvent_t stop = prof_take_event();
   if (stop == nullptr) {
     g_prof_free.push_back(start_);

@@ -17,6 +17,7 @@
 // A and B use the same k mapping, so any permutation of k inside a 64-wide slice
 // applied to both leaves the product unchanged; the 32-byte-per-lane load relies on it.
 #include "common.h"
+#include <hip/hip_ext.h>
 
 namespace sparse {
 
@@ -311,8 +312,16 @@ template <bool kGateUp>
 static int launch_decode(const DecodeArgs& a, int n_seg, hipStream_t st) {
   const int grid = a.tiles_s * (kGateUp ? 1 : a.split_s) + n_seg * a.tiles_r;
   if (grid == 0) return SPARSE_HIP_OK;
-  ProfScope prof(kGateUp ? SPARSE_HIP_K_DECODE_GATEUP : SPARSE_HIP_K_DECODE_DOWN, st);
-  if (a.T <= 16) {
+  ProfScope prof(kGateUp ? SPARSE_HIP_K_DECODE_GATEUP : SPARSE_HIP_K_DECODE_DOWN, st, /*dispatch_events=*/true);
+  if (prof.active()) {  // profiling: the launch stamps the event pair with the dispatch's begin and end
+    if (a.T <= 16) {
+      hipExtLaunchKernelGGL((decode_ffn_kernel<kGateUp, 1>), dim3(grid), dim3(kDecThreads), 0, st, prof.start_,
+                            prof.stop_, 0, a);
+    } else {
+      hipExtLaunchKernelGGL((decode_ffn_kernel<kGateUp, 2>), dim3(grid), dim3(kDecThreads), 0, st, prof.start_,
+                            prof.stop_, 0, a);
+    }
+  } else if (a.T <= 16) {
     hipLaunchKernelGGL((decode_ffn_kernel<kGateUp, 1>), dim3(grid), dim3(kDecThreads), 0, st, a);
   } else {
     hipLaunchKernelGGL((decode_ffn_kernel<kGateUp, 2>), dim3(grid), dim3(kDecThreads), 0, st, a);
