@@ -317,3 +317,49 @@ def test_rs_routing_with_its_own_number_of_experts_per_token(device, monkeypatch
                                                   lay["shared"], lay["shared_gate_w"])
             torch.testing.assert_close(out.view(T, -1).cpu().float(), want.float(), **BF16_TOL)
             hid = out
+
+
+@pytest.mark.parametrize("T", [1, 8, 32])
+def test_decode_stack_in_a_hip_graph_replays_like_eager(device, T):
+    """The decode path of a small stack captured into a HIP graph (one-launch router, fused FFN
+    launch pair, combine): every replay, on new inputs and with eager calls and
+    synchronisations of the same blocks in between, gives bit for bit what the eager call
+    gives on those inputs.  None of the kernels' self-resetting counters or workspaces may
+    depend on having been run eagerly last."""
+    from sparse_amd.block import DistributedSparseMoeBlock
+    from sparse_amd.context import DistEnv, SparseContext
+    from sparse_amd.synthetic import make_hidden, make_mlp_block
+    shape = dict(family="qwen_shared", hidden=512, num_experts=12, inter=256, top_k=4, shared_inter=1024)
+    dtype = torch.bfloat16
+    SparseContext.reset()
+    SparseContext.current_phase = "decode"
+    blocks = [DistributedSparseMoeBlock(l, make_mlp_block(shape, dtype=dtype, seed=60 + l), None, DistEnv(0, 1, 0, device),
+                                        num_layers=2, num_experts=12, top_k=4, dtype=dtype, expert_offload="gpu")
+              for l in range(2)]
+
+    def step(h):
+        outs = []
+        for blk in blocks:
+            h, logits = blk(h)
+            outs += [h, logits]
+        return outs
+
+    inputs = [make_hidden(T, 512, dtype, seed=700 + i).view(T, 1, -1).to(device) for i in range(5)]
+    static_in = inputs[0].clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step(static_in)                                   # workspaces exist before capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = step(static_in)
+    for i in (1, 2, 3, 4, 1):
+        want = [t.clone() for t in step(inputs[i])]       # eager, between the replays
+        torch.cuda.synchronize()
+        static_in.copy_(inputs[i])
+        graph.replay()
+        torch.cuda.synchronize()
+        for got, ref in zip(captured, want):
+            assert torch.equal(got, ref), (T, i)
