@@ -319,10 +319,11 @@ def test_rs_routing_with_its_own_number_of_experts_per_token(device, monkeypatch
             hid = out
 
 
-@pytest.mark.parametrize("T", [1, 8, 32])
+@pytest.mark.parametrize("T", [1, 8, 32, 96])
 def test_decode_stack_in_a_hip_graph_replays_like_eager(device, T):
     """The decode path of a small stack captured into a HIP graph (one-launch router, fused FFN
-    launch pair, combine): every replay, on new inputs and with eager calls and
+    launch pair, combine; at 96 tokens the prefill-size kernels with the shared expert forked
+    onto its second stream inside the capture): every replay, on new inputs and with eager calls and
     synchronisations of the same blocks in between, gives bit for bit what the eager call
     gives on those inputs.  None of the kernels' self-resetting counters or workspaces may
     depend on having been run eagerly last."""
