@@ -53,6 +53,7 @@ extern "C" {
 #define SPARSE_HIP_DECODE_MAX_TOKENS 32
 #define SPARSE_HIP_ROUTE_PACKED_MAX_TOKENS 16
 #define SPARSE_HIP_ROUTE_PACKED_ROWS 64
+#define SPARSE_HIP_PERMUTE_STATIC_MAX_TOKENS 65536
 
 /* ---- library identity ------------------------------------------------------ */
 
@@ -157,6 +158,22 @@ int sparse_hip_permute_build(const int64_t* topi_dev, int T, int K, int E, int32
                              int32_t* inv_perm_dev, int32_t* seg_offsets_dev,
                              int32_t* active_eids_dev, int32_t* n_active_dev, void* ws_dev,
                              void* stream);
+
+/*
+ * sparse_hip_permute_build for callers that cannot allocate device memory (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc): same inputs, same
+ * outputs, no workspace argument.  It has no counterpart in the reference.  The per-block
+ * histograms live in a 256 KB array built into the library (one copy per GPU, held until
+ * the process ends), which bounds T at SPARSE_HIP_PERMUTE_STATIC_MAX_TOKENS; a larger T is
+ * rejected with SPARSE_HIP_EINVAL.  The call allocates nothing; the first call on a device
+ * looks up the array's address (make that call outside a graph capture).  All calls on one
+ * GPU share the array: calls that overlap there, on different streams or from different
+ * threads, race.  Nothing has to be cleared between calls -- every entry that is read was
+ * written by the same call.
+ */
+int sparse_hip_permute_build_static(const int64_t* topi_dev, int T, int K, int E, int32_t* perm_dev,
+                                    int32_t* inv_perm_dev, int32_t* seg_offsets_dev,
+                                    int32_t* active_eids_dev, int32_t* n_active_dev, void* stream);
 
 /*
  * Decode fast path: sparse_hip_router_logits + sparse_hip_gate_topk +

@@ -17,6 +17,7 @@ MAX_TOPK = 16
 DECODE_MAX_TOKENS = 32
 ENOTREADY = 1
 ABI_VERSION = 1
+PERMUTE_STATIC_MAX_TOKENS = 65536
 
 
 class SparseHipMissing(RuntimeError):
@@ -69,6 +70,7 @@ SIGNATURES = {
         _i, [_vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "sparse_hip_permute_ws_bytes": (_sz, [_i, _i, _i]),
     "sparse_hip_permute_build": (_i, [_vp, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "sparse_hip_permute_build_static": (_i, [_vp, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp]),
     "sparse_hip_grouped_swiglu_decode": (
         _i, [C.POINTER(Experts), _vp, _vp, _vp, _vp, C.POINTER(SegList), _i, _i, _vp, _vp, _vp]),
     "sparse_hip_prefill_ws_bytes": (_sz, [_i, _i, _i, _i, _i]),

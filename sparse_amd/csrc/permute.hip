@@ -8,7 +8,37 @@
 // order of a stable sort, with no atomics on positions, so it is deterministic.
 #include "permute_device.h"
 
+#include <mutex>
+
 namespace sparse {
+
+// Per-block histograms of the entry point that allocates nothing: one copy of this array
+// per GPU, held until the process ends.  Host code never passes the array's name to a
+// kernel (on the host it is a stand-in, not a device address); it asks the runtime for
+// the address on the current device once and keeps it.
+constexpr int kPermStaticBlocks = SPARSE_HIP_PERMUTE_STATIC_MAX_TOKENS / kPermThreads;
+static __device__ __align__(256) int32_t scratch[kPermStaticBlocks * SPARSE_HIP_MAX_EXPERTS];
+
+constexpr int kPermMaxDevices = 64;
+static std::mutex g_scratch_mu;
+static int32_t* g_scratch_ptr[kPermMaxDevices] = {nullptr};
+
+// Device address of `scratch` on the current device (looked up on the first call there).
+static int static_scratch(int32_t** out) {
+  int dev = -1;
+  SP_HIP(hipGetDevice(&dev));
+  SP_REQUIRE(dev >= 0 && dev < kPermMaxDevices, "permute_build_static: device ordinal %d outside [0,%d)", dev,
+             kPermMaxDevices);
+  std::lock_guard<std::mutex> lk(g_scratch_mu);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    SP_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    SP_REQUIRE(p != nullptr, "permute_build_static: hipGetSymbolAddress returned NULL");
+    g_scratch_ptr[dev] = static_cast<int32_t*>(p);
+  }
+  *out = g_scratch_ptr[dev];
+  return SPARSE_HIP_OK;
+}
 
 __global__ __launch_bounds__(kPermThreads) void permute_count_kernel(const int64_t* __restrict__ topi, int T,
                                                                      int K, int E,
@@ -50,9 +80,11 @@ size_t sparse_hip_permute_ws_bytes(int T, int K, int E) {
   return nb * static_cast<size_t>(E) * sizeof(int32_t);
 }
 
-int sparse_hip_permute_build(const int64_t* topi_dev, int T, int K, int E, int32_t* perm_dev,
-                             int32_t* inv_perm_dev, int32_t* seg_offsets_dev, int32_t* active_eids_dev,
-                             int32_t* n_active_dev, void* ws_dev, void* stream) {
+}  // extern "C"
+
+static int permute_build_impl(const int64_t* topi_dev, int T, int K, int E, int32_t* perm_dev,
+                              int32_t* inv_perm_dev, int32_t* seg_offsets_dev, int32_t* active_eids_dev,
+                              int32_t* n_active_dev, void* ws_dev, void* stream) {
   SP_REQUIRE(T >= 1, "permute_build: T=%d must be >= 1", T);
   SP_REQUIRE(E >= 1 && E <= SPARSE_HIP_MAX_EXPERTS, "permute_build: E=%d outside [1,%d]", E,
              SPARSE_HIP_MAX_EXPERTS);
@@ -79,6 +111,31 @@ int sparse_hip_permute_build(const int64_t* topi_dev, int T, int K, int E, int32
                      counts, perm_dev, inv_perm_dev, seg_offsets_dev, active_eids_dev, n_active_dev);
   SP_LAUNCH_CHECK("permute_scatter_kernel");
   return SPARSE_HIP_OK;
+}
+
+extern "C" {
+
+int sparse_hip_permute_build(const int64_t* topi_dev, int T, int K, int E, int32_t* perm_dev,
+                             int32_t* inv_perm_dev, int32_t* seg_offsets_dev, int32_t* active_eids_dev,
+                             int32_t* n_active_dev, void* ws_dev, void* stream) {
+  return permute_build_impl(topi_dev, T, K, E, perm_dev, inv_perm_dev, seg_offsets_dev, active_eids_dev,
+                            n_active_dev, ws_dev, stream);
+}
+
+int sparse_hip_permute_build_static(const int64_t* topi_dev, int T, int K, int E, int32_t* perm_dev,
+                                    int32_t* inv_perm_dev, int32_t* seg_offsets_dev, int32_t* active_eids_dev,
+                                    int32_t* n_active_dev, void* stream) {
+  SP_REQUIRE(T <= SPARSE_HIP_PERMUTE_STATIC_MAX_TOKENS,
+             "permute_build_static: T=%d exceeds the built-in scratch (at most %d tokens); use "
+             "sparse_hip_permute_build with a workspace",
+             T, SPARSE_HIP_PERMUTE_STATIC_MAX_TOKENS);
+  int32_t* counts = nullptr;
+  const int rc = static_scratch(&counts);
+  if (rc != SPARSE_HIP_OK) return rc;
+  // The counting pass writes every histogram entry the scatter pass reads (blocks < ceil(T/256),
+  // experts < E), so nothing of an earlier call's contents is ever read and nothing needs clearing.
+  return permute_build_impl(topi_dev, T, K, E, perm_dev, inv_perm_dev, seg_offsets_dev, active_eids_dev,
+                            n_active_dev, counts, stream);
 }
 
 }  // extern "C"
