@@ -120,6 +120,9 @@ int sparse_hip_router_logits(const void* x_dev, const void* wg_dev, const void* 
  * probs = softmax(logits, fp32); (topv, topi) = top-K of probs, descending, ties to
  * the lower expert id; optional renormalisation topv /= max(sum topv, 1e-12); topv is
  * rounded to `out_dtype`, topi is int64 -- utils/eval_core.py:9520, :9590-9595.
+ * The ranking is done on the logits (descending, then lower id), which is the order of the
+ * probabilities wherever two of them differ and does not depend on the rounding of exp: the
+ * indices are a function of the logits alone.
  * logits [T,E] in `logits_dtype`; topv [T,K]; topi [T,K].  E <= 256, K <= 16, K <= E.
  */
 int sparse_hip_gate_topk(const void* logits_dev, int logits_dtype, int T, int E, int K,
@@ -138,6 +141,17 @@ int sparse_hip_gate_topk(const void* logits_dev, int logits_dtype, int T, int E,
 int sparse_hip_gate_topk_grouped(const void* logits_dev, int logits_dtype, int T, int E, int K,
                                  int renorm, int n_group, int topk_group, int out_dtype,
                                  void* topv_dev, int64_t* topi_dev, void* stream);
+
+/*
+ * Top-K of each row of given probabilities, no softmax: values descending, ties to the lower
+ * index; optional renormalisation as above; topv rounded to `out_dtype`.  This is the
+ * `torch.topk` the reference applies to the next-layer predictor's output before planning
+ * prefetches and before replaying a predicted routing (utils/eval_core.py:10985-10996,
+ * :10971-10983), with the tie order torch leaves open fixed.  values [T,E] fp32; E <= 256,
+ * K <= 16, K <= E.
+ */
+int sparse_hip_topk(const void* values_dev, int T, int E, int K, int renorm, int out_dtype,
+                    void* topv_dev, int64_t* topi_dev, void* stream);
 
 /* ---- A5: token x K expansion + permutation --------------------------------- */
 

@@ -12,8 +12,12 @@ How each function is pinned (see tests/test_oracle_moe.py):
   routing_router            closed form (fp64 softmax + brute-force top-k on small E),
                             invariants (distinct ids, descending, sum <= 1), the chosen
                             tie rule on hand-made ties.  torch.topk leaves tie order
-                            unspecified; the rule here is "higher probability first, then
-                            lower expert id".
+                            unspecified; the rule here is "higher LOGIT first, then lower
+                            expert id" (``topk_by_logit``).  Softmax is monotone, so this is
+                            the probability order wherever two probabilities differ; where
+                            two distinct logits round to one probability the reference's
+                            own order is whatever torch.topk happens to do, and the rule
+                            here picks the mathematically larger one.
   deepseek_router           the reference delegates to the model's own ``MoEGate`` (third-party,
                             loaded with trust_remote_code, no version pin, source not in the
                             reference tree), so no reference code exists to run.  Restated
@@ -52,6 +56,14 @@ def topk_lower_id_first(probs: torch.Tensor, k: int) -> Tuple[torch.Tensor, torc
     return order.values[..., :k].contiguous(), order.indices[..., :k].contiguous()
 
 
+def topk_by_logit(logits: torch.Tensor, probs: torch.Tensor, k: int) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Top-k of ``probs = softmax(logits)`` ranked on the logits: logit descending, ties to the
+    lower index; the values are the probabilities of the winners.  ``logits`` may carry -inf
+    for entries whose probability was forced to 0."""
+    order = torch.sort(logits.to(torch.float32), dim=-1, descending=True, stable=True).indices[..., :k].contiguous()
+    return torch.gather(probs, -1, order), order
+
+
 def routing_router(x: torch.Tensor, gate_w: torch.Tensor, top_k: int, norm_topk_prob: bool = False,
                    router_logits: Optional[torch.Tensor] = None):
     """Qwen-family router, :9519-9520 and :9590-9595.
@@ -64,22 +76,29 @@ def routing_router(x: torch.Tensor, gate_w: torch.Tensor, top_k: int, norm_topk_
     if router_logits is None:
         router_logits = F.linear(x, gate_w)
     probs = torch.softmax(router_logits, dim=-1, dtype=torch.float32)
-    topv, topi = topk_lower_id_first(probs, top_k)
+    topv, topi = topk_by_logit(router_logits, probs, top_k)
     if norm_topk_prob:
         topv = topv / topv.sum(dim=-1, keepdim=True).clamp_min(1e-12)
     return topv.to(dtype=x.dtype), topi.to(torch.long), router_logits
 
 
-def group_limited_scores(probs: torch.Tensor, n_group: int, topk_group: int) -> torch.Tensor:
+def group_limited_scores(probs: torch.Tensor, n_group: int, topk_group: int, logits: Optional[torch.Tensor] = None):
     """DeepSeek-V2's ``group_limited_greedy`` mask: experts form ``n_group`` equal runs of ids, a
     group scores its largest probability, the ``topk_group`` best groups (ties to the lower
-    group id) keep their probabilities, every other entry becomes 0."""
+    group id) keep their probabilities, every other entry becomes 0.  With ``logits`` the
+    groups are ranked on their largest logit (the same order, see ``topk_by_logit``) and the
+    masked logits (-inf where the probability became 0) are returned as well."""
     T, E = probs.shape
-    group_scores = probs.view(T, n_group, E // n_group).max(dim=-1).values
+    ranked = probs if logits is None else logits.to(torch.float32)
+    group_scores = ranked.view(T, n_group, E // n_group).max(dim=-1).values
     _, keep = topk_lower_id_first(group_scores, topk_group)
     mask = torch.zeros_like(group_scores, dtype=torch.bool)
     mask.scatter_(1, keep, True)
-    return torch.where(mask.repeat_interleave(E // n_group, dim=1), probs, torch.zeros_like(probs))
+    full = mask.repeat_interleave(E // n_group, dim=1)
+    masked = torch.where(full, probs, torch.zeros_like(probs))
+    if logits is None:
+        return masked
+    return masked, torch.where(full, ranked, torch.full_like(ranked, float("-inf")))
 
 
 def deepseek_router(x: torch.Tensor, gate_w: torch.Tensor, top_k: int, routed_scaling_factor: float = 1.0,
@@ -94,9 +113,10 @@ def deepseek_router(x: torch.Tensor, gate_w: torch.Tensor, top_k: int, routed_sc
     if router_logits is None:
         router_logits = F.linear(x.to(torch.float32), gate_w.to(torch.float32))
     probs = torch.softmax(router_logits, dim=-1, dtype=torch.float32)
+    keys = router_logits.to(torch.float32)
     if n_group > 1 and topk_group < n_group:
-        probs = group_limited_scores(probs, n_group, topk_group)
-    topv, topi = topk_lower_id_first(probs, top_k)
+        probs, keys = group_limited_scores(probs, n_group, topk_group, logits=keys)
+    topv, topi = topk_by_logit(keys, probs, top_k)
     topv = (topv * routed_scaling_factor).to(dtype=x.dtype)
     pseudo = torch.full((x.shape[0], gate_w.shape[0]), float("-inf"), dtype=torch.float32)
     pseudo.scatter_(1, topi, topv.to(torch.float32).clamp_min(1e-12).log())

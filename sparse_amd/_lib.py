@@ -64,6 +64,7 @@ SIGNATURES = {
     "sparse_hip_router_logits": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _vp, _vp]),
     "sparse_hip_gate_topk": (_i, [_vp, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp]),
     "sparse_hip_gate_topk_grouped": (_i, [_vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp]),
+    "sparse_hip_topk": (_i, [_vp, _i, _i, _i, _i, _i, _vp, _vp, _vp]),
     "sparse_hip_route_decode": (
         _i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "sparse_hip_route_decode_packed": (

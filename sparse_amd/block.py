@@ -27,7 +27,7 @@ from torch import nn
 from . import ops
 from .context import DistEnv, Metrics, SparseContext
 from .residency import Backend, LayerResidency, ResidencyConfig
-from .rs import router_topk_feature, topk_for_planning
+from .rs import router_topk_feature, stable_topk, topk_for_planning
 from .weights import ExpertSlab, HostExpertArena, tile_weight
 
 
@@ -107,6 +107,10 @@ class _Workspace:
             ws = cls(*key)
             cls._cache[key] = ws
         return ws
+
+
+def _NO_SEGMENTS():
+    return ops.seglist_host([], [])
 
 
 class _EventRing:
@@ -504,7 +508,7 @@ class DistributedSparseMoeBlock(nn.Module):
             # the next layer may execute with this prediction instead of its router (:10971-10983)
             raw = os.environ.get("SPARSE_RS_EXEC_TOPK", "").strip()
             exec_topk = max(1, min(int(raw) if raw else self.top_k, int(pred.shape[-1])))
-            route_v, route_i = torch.topk(pred, k=exec_topk, dim=-1)
+            route_v, route_i = stable_topk(pred, exec_topk)
             if self.norm_topk_prob:
                 route_v = route_v / route_v.sum(dim=-1, keepdim=True).clamp_min(1e-12)
             SparseContext.routing_cache[target] = (route_v.to(x.dtype), route_i.to(torch.long))
@@ -573,10 +577,21 @@ class DistributedSparseMoeBlock(nn.Module):
         side = (self._shared_stream() if self.shared_weights is not None and not fused and self.overlap_shared
                 and x.is_cuda and T > ops.DECODE_MAX_TOKENS else None)
 
+        # Whether the shared expert's down projection is left as partial sums for the combine
+        # step depends on the call's size and dtype only, never on where the routed experts
+        # live: an offloaded layer must give the bits of the all-resident one.
+        split_shared = self.shared_weights is not None and ws.split_ws is not None
+
         def run_shared() -> None:
             if self.shared_weights is None or fused:
                 return
             gw, uw, dw = self.shared_weights
+            if split_shared:
+                # the fused decode entry point with no routed segment: the shared expert alone,
+                # in the same split form the all-resident call uses
+                ops.moe_ffn_decode(self._experts_desc, x, ws.topv, ws.perm, _NO_SEGMENTS(), ws.inter, ws.parts,
+                                   self.shared_weights, shared_gate, ws.shared_inter, ws.shared_out, ws.split_ws)
+                return
             if side is None:
                 ops.shared_expert(x, gw, uw, dw, shared_gate, ws.shared_inter, ws.shared_out)
                 return
@@ -623,7 +638,7 @@ class DistributedSparseMoeBlock(nn.Module):
         if side is not None:
             torch.cuda.current_stream().wait_stream(side)
         out = torch.empty((T, H), device=x.device, dtype=self.dtype)
-        if fused and ws.split_ws is not None:
+        if split_shared:
             ops.combine_split(ws.parts, ws.perm, ws.split_ws, ws.split_parts, shared_gate, T, k_exec, out)
         else:
             ops.combine(ws.parts, ws.perm, ws.shared_out, T, k_exec, out)

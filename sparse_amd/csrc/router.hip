@@ -175,10 +175,14 @@ __global__ __launch_bounds__(256) void router_logits_mfma_kernel(
 
 // ---------------------------------------------------------------------------
 // Fused softmax(fp32) + top-k of one token by one wavefront; lane l holds experts
-// l, l+64, l+128, l+192.  Selection runs K rounds of a wave-wide arg-max whose order is
-// (probability descending, expert id ascending): the largest probability first, then
-// the lowest id among the lanes that hold it.  All cross-lane steps are DPP reductions.
-// Lane r < K also returns the r-th selected expert.
+// l, l+64, l+128, l+192.  Selection runs K rounds of a wave-wide arg-max on the LOGITS
+// themselves, in the order (logit descending, expert id ascending): softmax is monotone, so
+// this is the order of the probabilities wherever those differ, and it does not depend on
+// how exp and the division round when two logits one ulp apart collapse to one probability.
+// A probability is computed only for the K winners (and nothing else of the row needs one:
+// a group's best probability belongs to its best logit).  With `softmax` off the row is
+// ranked and returned as it is (top-k of given probabilities).  All cross-lane steps are
+// DPP reductions.  Lane r < K also returns the r-th selected expert.
 // ---------------------------------------------------------------------------
 constexpr int kTopkWaves = 4;
 constexpr int kTopkNV = SPARSE_HIP_MAX_EXPERTS / 64;
@@ -186,60 +190,60 @@ constexpr int kTopkNV = SPARSE_HIP_MAX_EXPERTS / 64;
 template <typename TL, typename TO>
 __device__ __forceinline__ int topk_token(const TL* __restrict__ row, int E, int K, int renorm,
                                           TO* __restrict__ topv_row, int64_t* __restrict__ topi_row, int lane,
-                                          int n_group = 0, int topk_group = 0) {
-  float p[kTopkNV];
+                                          int n_group = 0, int topk_group = 0, bool softmax = true) {
+  float key[kTopkNV];  // what is ranked: the logit (-inf once masked by the group limit)
+  unsigned alive = 0u;  // bit j: expert lane + 64*j exists and has not been selected yet
   float m = -INFINITY;
 #pragma unroll
   for (int j = 0; j < kTopkNV; ++j) {
     const int e = lane + 64 * j;
-    p[j] = -INFINITY;
+    key[j] = -INFINITY;
     if (64 * j < E) {  // uniform: whole groups of 64 experts that do not exist cost nothing
-      p[j] = (e < E) ? Elem<TL>::load(row + e) : -INFINITY;
-      m = fmaxf(m, p[j]);
+      if (e < E) {
+        key[j] = Elem<TL>::load(row + e);
+        alive |= 1u << j;
+      }
+      m = fmaxf(m, key[j]);
     }
   }
-  m = wave_max(m);
-  float s = 0.f;
+  float s = 1.f;
+  if (softmax) {
+    m = wave_max(m);
+    s = 0.f;
 #pragma unroll
-  for (int j = 0; j < kTopkNV; ++j) {
-    const int e = lane + 64 * j;
-    p[j] = (e < E) ? expf(p[j] - m) : 0.f;
-    s += p[j];
-  }
-  s = wave_sum(s);
-#pragma unroll
-  for (int j = 0; j < kTopkNV; ++j) {
-    const int e = lane + 64 * j;
-    p[j] = (e < E) ? p[j] / s : -1.f;  // -1 marks "not a candidate"
+    for (int j = 0; j < kTopkNV; ++j) s += ((alive >> j) & 1u) ? expf(key[j] - m) : 0.f;
+    s = wave_sum(s);
   }
 
   if (n_group > 1) {
     // group-limited selection: the experts form n_group equal runs of ids; a group's score is
-    // its largest probability, the topk_group best groups (score descending, then lower group
-    // id) stay, every other expert's probability becomes 0 and still takes part in the top-k
+    // its largest probability, i.e. that of its largest logit; the topk_group best groups
+    // (score descending, then lower group id) stay; every other expert's probability becomes
+    // 0 and still takes part in the top-k -- here: its key becomes -inf, whose probability is 0
     const int gsz = E / n_group;
-    float gscore = -2.f;  // lane g < n_group: score of group g
+    float gscore = -INFINITY;  // lane g < n_group: score of group g
     for (int g = 0; g < n_group; ++g) {
-      float m = -1.f;
+      float gm = -INFINITY;
 #pragma unroll
       for (int j = 0; j < kTopkNV; ++j) {
         const int e = lane + 64 * j;
-        if (e < E && e / gsz == g) m = fmaxf(m, p[j]);
+        if (e < E && e / gsz == g) gm = fmaxf(gm, key[j]);
       }
-      m = wave_max(m);
-      if (lane == g) gscore = m;
+      gm = wave_max(gm);
+      if (lane == g) gscore = gm;
     }
-    unsigned long long keep = 0ull;
+    unsigned long long keep = 0ull, taken = 0ull;
     for (int r = 0; r < topk_group; ++r) {
-      const float wv = wave_max(gscore);
-      const int wi = wave_min_int(gscore == wv ? lane : 0x7fffffff);
+      const bool cand = lane < n_group && !((taken >> lane) & 1ull);
+      const float wv = wave_max(cand ? gscore : -INFINITY);
+      const int wi = wave_min_int((cand && gscore == wv) ? lane : 0x7fffffff);
       keep |= 1ull << wi;
-      if (lane == wi) gscore = -2.f;
+      taken |= 1ull << wi;
     }
 #pragma unroll
     for (int j = 0; j < kTopkNV; ++j) {
       const int e = lane + 64 * j;
-      if (e < E && !((keep >> (e / gsz)) & 1ull)) p[j] = 0.f;
+      if (e < E && !((keep >> (e / gsz)) & 1ull)) key[j] = -INFINITY;
     }
   }
 
@@ -247,28 +251,26 @@ __device__ __forceinline__ int topk_token(const TL* __restrict__ row, int E, int
   int sel_i = 0;
   float sum_sel = 0.f;
   for (int r = 0; r < K; ++r) {
-    float bv = -1.f;
-    int bi = 0x7fffffff;
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;  // a lane without a candidate never wins the id comparison
 #pragma unroll
     for (int j = 0; j < kTopkNV; ++j) {
-      if (64 * j < E && p[j] > bv) {  // ascending j == ascending id, so strict > keeps the lower id
-        bv = p[j];
+      // ascending j == ascending id, so strict > keeps the lower id among equal keys
+      if (((alive >> j) & 1u) && (bi == 0x7fffffff || key[j] > bv)) {
+        bv = key[j];
         bi = lane + 64 * j;
       }
     }
     const float wv = wave_max(bv);
     const int wi = wave_min_int(bv == wv ? bi : 0x7fffffff);
     // every lane now holds the winner; its owner retires it
-    if ((wi & 63) == lane) {
-#pragma unroll
-      for (int j = 0; j < kTopkNV; ++j)
-        if ((wi >> 6) == j) p[j] = -1.f;
-    }
+    if ((wi & 63) == lane) alive &= ~(1u << (wi >> 6));
+    const float pv = softmax ? expf(wv - m) / s : wv;
     if (lane == r) {
-      sel_v = wv;
+      sel_v = pv;
       sel_i = wi;
     }
-    sum_sel += wv;
+    sum_sel += pv;
   }
   if (lane < K) {
     float v = sel_v;
@@ -282,11 +284,11 @@ __device__ __forceinline__ int topk_token(const TL* __restrict__ row, int E, int
 template <typename TL, typename TO>
 __global__ __launch_bounds__(kTopkWaves * 64) void gate_topk_kernel(
     const TL* __restrict__ logits, int Ttok, int E, int K, int renorm, TO* __restrict__ topv,
-    int64_t* __restrict__ topi, int n_group, int topk_group) {
+    int64_t* __restrict__ topi, int n_group, int topk_group, int softmax) {
   const int t = blockIdx.x * kTopkWaves + (threadIdx.x >> 6);
   if (t >= Ttok) return;
   topk_token<TL, TO>(logits + static_cast<size_t>(t) * E, E, K, renorm, topv + static_cast<size_t>(t) * K,
-                     topi + static_cast<size_t>(t) * K, threadIdx.x & 63, n_group, topk_group);
+                     topi + static_cast<size_t>(t) * K, threadIdx.x & 63, n_group, topk_group, softmax != 0);
 }
 
 // ---------------------------------------------------------------------------
@@ -610,12 +612,12 @@ static int launch_router_logits(const void* x, const void* wg, const void* wsg, 
 
 template <typename TL, typename TO>
 static int launch_gate_topk(const void* logits, int Ttok, int E, int K, int renorm, void* topv,
-                            int64_t* topi, hipStream_t st, int n_group = 0, int topk_group = 0) {
+                            int64_t* topi, hipStream_t st, int n_group = 0, int topk_group = 0, int softmax = 1) {
   dim3 grid((Ttok + kTopkWaves - 1) / kTopkWaves);
   ProfScope prof(SPARSE_HIP_K_GATE_TOPK, st);
   hipLaunchKernelGGL((gate_topk_kernel<TL, TO>), grid, dim3(kTopkWaves * 64), 0, st,
                      static_cast<const TL*>(logits), Ttok, E, K, renorm, static_cast<TO*>(topv), topi, n_group,
-                     topk_group);
+                     topk_group, softmax);
   SP_LAUNCH_CHECK("gate_topk_kernel");
   return SPARSE_HIP_OK;
 }
@@ -681,6 +683,20 @@ int sparse_hip_gate_topk_grouped(const void* logits_dev, int logits_dtype, int T
   if (lb) return launch_gate_topk<uint16_t, float>(logits_dev, T, E, K, renorm, topv_dev, topi_dev, st, ng, topk_group);
   if (ob) return launch_gate_topk<float, uint16_t>(logits_dev, T, E, K, renorm, topv_dev, topi_dev, st, ng, topk_group);
   return launch_gate_topk<float, float>(logits_dev, T, E, K, renorm, topv_dev, topi_dev, st, ng, topk_group);
+}
+
+int sparse_hip_topk(const void* values_dev, int T, int E, int K, int renorm, int out_dtype, void* topv_dev,
+                    int64_t* topi_dev, void* stream) {
+  SP_REQUIRE(valid_dtype(out_dtype), "topk: unknown dtype");
+  SP_REQUIRE(T >= 0, "topk: T=%d", T);
+  SP_REQUIRE(E >= 1 && E <= SPARSE_HIP_MAX_EXPERTS, "topk: E=%d outside [1,%d]", E, SPARSE_HIP_MAX_EXPERTS);
+  SP_REQUIRE(K >= 1 && K <= SPARSE_HIP_MAX_TOPK && K <= E, "topk: K=%d outside [1,min(%d,E)]", K, SPARSE_HIP_MAX_TOPK);
+  SP_REQUIRE(values_dev && topv_dev && topi_dev, "topk: NULL pointer");
+  if (T == 0) return SPARSE_HIP_OK;
+  hipStream_t st = as_stream(stream);
+  if (out_dtype == SPARSE_HIP_BF16)
+    return launch_gate_topk<float, uint16_t>(values_dev, T, E, K, renorm, topv_dev, topi_dev, st, 0, 0, 0);
+  return launch_gate_topk<float, float>(values_dev, T, E, K, renorm, topv_dev, topi_dev, st, 0, 0, 0);
 }
 
 int sparse_hip_route_decode(const void* x_dev, const void* wg_dev, const void* wsg_dev, int dtype,

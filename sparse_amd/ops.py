@@ -93,6 +93,26 @@ def gate_topk(logits: torch.Tensor, k: int, renorm: bool = False, out_dtype: Opt
     return topv, topi
 
 
+def topk_values(values: torch.Tensor, k: int, renorm: bool = False, out_dtype: Optional[torch.dtype] = None,
+                topv: Optional[torch.Tensor] = None, topi: Optional[torch.Tensor] = None):
+    """Top-k of given fp32 probabilities (no softmax), descending, ties to the lower index:
+    returns ``(topv [T,k] out_dtype, topi [T,k] int64)``."""
+    lib = _lib.load()
+    _need(values, "values", torch.float32)
+    T, E = values.shape
+    odt = out_dtype or torch.float32
+    if topv is None:
+        topv = torch.empty((T, k), device=values.device, dtype=odt)
+    if topi is None:
+        topi = torch.empty((T, k), device=values.device, dtype=torch.int64)
+    _need(topv, "topv", odt, (T, k))
+    _need(topi, "topi", torch.int64, (T, k))
+    rc = lib.sparse_hip_topk(_ptr(values), T, E, int(k), int(bool(renorm)), dtype_code(odt), _ptr(topv), _ptr(topi),
+                             _stream())
+    _lib.check(rc, "sparse_hip_topk")
+    return topv, topi
+
+
 # --------------------------------------------------------------------------- permute
 class Permutation:
     """Outputs of ``permute_build`` (all int32 device tensors)."""

@@ -15,6 +15,8 @@ from typing import Any, Dict, List, Optional, Tuple
 import torch
 from torch import nn
 
+from . import _lib
+
 
 class RoutingScoutMLP(nn.Module):
     def __init__(self, input_dim: int, num_experts: int, hidden_dim: int = 1024) -> None:
@@ -70,10 +72,23 @@ def topk_for_planning(pred: torch.Tensor, pred_k: int, norm_topk_prob: bool, dty
     with the probabilities rounded to the activation dtype and widened again
     (utils/eval_core.py:10985-10996).  Returns ``(topi int64 [T,k], topv float32 [T,k])``."""
     pred_k = min(int(pred.shape[-1]), int(pred_k))
-    topv, topi = torch.topk(pred.to(torch.float32), k=pred_k, dim=-1)
+    topv, topi = stable_topk(pred.to(torch.float32), pred_k)
     if norm_topk_prob:
         topv = topv / topv.sum(dim=-1, keepdim=True).clamp_min(1e-12)
     return topi.to(torch.long), topv.to(dtype).to(torch.float32)
+
+
+def stable_topk(values: torch.Tensor, k: int):
+    """Top-k of fp32 rows, descending, equal values in ascending index order (``torch.topk``
+    leaves that order open, and the planner's candidate order depends on it).  Device rows go
+    through the HIP top-k kernel; rows wider than the kernel takes, more than its 16
+    selections, or host tensors (planner logic exercised without a device) are ranked by a
+    stable sort."""
+    if values.is_cuda and k <= _lib.MAX_TOPK and values.shape[-1] <= _lib.MAX_EXPERTS and values.dim() == 2:
+        from . import ops
+        return ops.topk_values(values.contiguous(), k)
+    order = torch.sort(values, dim=-1, descending=True, stable=True)
+    return order.values[..., :k].contiguous(), order.indices[..., :k].contiguous()
 
 
 def random_init_bank(num_layers: int, hidden: int, num_experts: int, hidden_dim: int = 512, seed: int = 0,

@@ -25,19 +25,6 @@ def _ops():
     return ops
 
 
-def _boundary_safe(logits: torch.Tensor, k: int, eps: float = 1e-6) -> torch.Tensor:
-    """Tokens whose top-k cannot flip under ulp-level differences in exp/sum: every
-    adjacent pair among the k+1 largest is either an exact logit tie (equal inputs give
-    equal probabilities everywhere, the id rule decides) or clearly separated."""
-    srt = torch.sort(logits.float(), dim=-1, descending=True, stable=True)
-    top_l = srt.values[:, : k + 1]
-    probs = torch.softmax(logits, dim=-1, dtype=torch.float32)
-    top_p = torch.gather(probs, 1, srt.indices[:, : k + 1])
-    gap = (top_p[:, :-1] - top_p[:, 1:]) / top_p[:, :-1].clamp_min(1e-30)
-    ok = (top_l[:, :-1] == top_l[:, 1:]) | (gap > eps)
-    return ok.all(dim=1)
-
-
 # ------------------------------------------------------------------ gate_topk
 @pytest.mark.parametrize("E,K", [(60, 4), (64, 6), (16, 2), (200, 8)])
 @pytest.mark.parametrize("ldt", [torch.float32, torch.bfloat16])
@@ -45,48 +32,39 @@ def test_gate_topk_matches_oracle(device, E, K, ldt):
     ops = _ops()
     g = torch.Generator().manual_seed(E * 100 + K)
     logits = (torch.randn(257, E, generator=g) * 2.0).to(ldt)
+    # a third of the rows get logits one ulp apart around the K-th place: the indices are a
+    # function of the logits alone, so they must agree there too
+    srt = torch.sort(logits.float(), dim=-1, descending=True)
+    for t in range(0, 257, 3):
+        a, b = int(srt.indices[t, K - 1]), int(srt.indices[t, K])
+        logits[t, b] = torch.nextafter(logits[t, a].float(), torch.tensor(-1e30)).to(ldt) if ldt == torch.float32 \
+            else logits[t, a]
     probs = torch.softmax(logits, dim=-1, dtype=torch.float32)
-    ref_v, ref_i = ref_moe.topk_lower_id_first(probs, K)
+    ref_v, ref_i = ref_moe.topk_by_logit(logits, probs, K)
     topv, topi = ops.gate_topk(logits.to(device), K, out_dtype=ldt)
     topv, topi = topv.cpu(), topi.cpu()
-    safe = _boundary_safe(logits, K)
-    assert safe.float().mean() > 0.9
-    assert torch.equal(topi[safe], ref_i[safe])
-    # tokens with a near-tie still pick a valid top-k set
-    both = torch.sort(topi, dim=1).values
-    assert (both[:, 1:] != both[:, :-1]).all()
-    torch.testing.assert_close(topv.float()[safe], ref_v.to(ldt).float()[safe], rtol=1e-2, atol=1e-6)
+    assert torch.equal(topi, ref_i)
+    torch.testing.assert_close(topv.float(), ref_v.to(ldt).float(), rtol=1e-2 if ldt == torch.bfloat16 else 1e-5,
+                               atol=1e-6)
 
 
 @pytest.mark.parametrize("E,n_group,topk_group,K", [(16, 4, 2, 6), (160, 8, 3, 6), (256, 64, 5, 16), (64, 2, 1, 8),
                                                       (60, 6, 6, 4), (12, 4, 1, 5)])
 @pytest.mark.parametrize("ldt", [torch.float32, torch.bfloat16])
 def test_gate_topk_group_limited(device, E, n_group, topk_group, K, ldt):
-    """Group-limited selection against the oracle: indices exact wherever neither the group
-    choice nor the top-k boundary is a rounding tie; K larger than the experts left picks
-    zero-probability experts in id order, as the oracle's rule says."""
+    """Group-limited selection against the oracle, indices exact on every row; K larger than
+    the experts left picks zero-probability experts in id order, as the oracle's rule says."""
     ops = _ops()
     g = torch.Generator().manual_seed(E + n_group)
     logits = (torch.randn(300, E, generator=g) * 2.0).to(ldt)
     topv, topi = ops.gate_topk(logits.to(device), K, out_dtype=torch.float32, n_group=n_group, topk_group=topk_group)
     probs = torch.softmax(logits, dim=-1, dtype=torch.float32)
-    masked = ref_moe.group_limited_scores(probs, n_group, topk_group) if topk_group < n_group else probs
-    ref_v, ref_i = ref_moe.topk_lower_id_first(masked, K)
-    # rows whose group ranking or top-k boundary could flip on an ulp of exp/sum are left out
-    gs = probs.view(300, n_group, E // n_group).max(-1).values.sort(-1, descending=True).values
-    safe = torch.ones(300, dtype=torch.bool)
+    masked, keys = probs, logits.float()
     if topk_group < n_group:
-        a, b = gs[:, topk_group - 1], gs[:, topk_group]
-        safe &= (a == b) | ((a - b) / a > 1e-5)
-    srt = masked.sort(dim=-1, descending=True, stable=True).values
-    if K < E:
-        a, b = srt[:, K - 1], srt[:, K]
-        safe &= (a == b) | ((a - b) / a.clamp_min(1e-30) > 1e-5)
-    pairs = srt[:, :K]
-    safe &= ((pairs[:, :-1] == pairs[:, 1:]) | ((pairs[:, :-1] - pairs[:, 1:]) / pairs[:, :-1].clamp_min(1e-30) > 1e-5)).all(1)
-    assert safe.float().mean() > 0.8
-    assert torch.equal(topi.cpu()[safe], ref_i[safe])
-    torch.testing.assert_close(topv.cpu()[safe], ref_v[safe], rtol=1e-5, atol=1e-7)
+        masked, keys = ref_moe.group_limited_scores(probs, n_group, topk_group, logits=logits)
+    ref_v, ref_i = ref_moe.topk_by_logit(keys, masked, K)
+    assert torch.equal(topi.cpu(), ref_i)
+    torch.testing.assert_close(topv.cpu(), ref_v, rtol=1e-5, atol=1e-7)
     if topk_group < n_group:
         grp = torch.div(topi.cpu(), E // n_group, rounding_mode="floor")
         live = (masked > 0).sum(1) >= K                     # enough experts left in the kept groups
@@ -102,7 +80,7 @@ def test_gate_topk_ties_go_to_lower_id(device):
     logits[4] = torch.arange(60, dtype=torch.float32).flip(0) * 0.0  # all equal
     for ldt in (torch.float32, torch.bfloat16):
         probs = torch.softmax(logits.to(ldt), dim=-1, dtype=torch.float32)
-        ref_v, ref_i = ref_moe.topk_lower_id_first(probs, 4)
+        ref_v, ref_i = ref_moe.topk_by_logit(logits.to(ldt), probs, 4)
         topv, topi = ops.gate_topk(logits.to(ldt).to(device), 4)
         assert torch.equal(topi.cpu(), ref_i)
         assert topi.cpu()[0].tolist() == [0, 1, 2, 3]
@@ -119,9 +97,8 @@ def test_gate_topk_renorm(device):
     torch.testing.assert_close(topv.cpu().sum(dim=1), torch.ones(33), rtol=1e-5, atol=1e-5)
     x = torch.zeros(33, 8)
     ref_v, ref_i, _ = ref_moe.routing_router(x, torch.zeros(60, 8), 4, True, router_logits=logits)
-    safe = _boundary_safe(logits, 4)
-    assert torch.equal(topi.cpu()[safe], ref_i[safe])
-    torch.testing.assert_close(topv.cpu()[safe], ref_v[safe], rtol=1e-5, atol=1e-6)
+    assert torch.equal(topi.cpu(), ref_i)
+    torch.testing.assert_close(topv.cpu(), ref_v, rtol=1e-5, atol=1e-6)
 
 
 def test_gate_topk_rejects_bad_arguments(device):
@@ -131,6 +108,24 @@ def test_gate_topk_rejects_bad_arguments(device):
         ops.gate_topk(logits, 4)
     with pytest.raises(ValueError):
         ops.gate_topk(torch.zeros(4, 8, device=device), 9)
+
+
+def test_topk_of_given_probabilities(device):
+    """``sparse_hip_topk``: rows ranked as they are (no softmax), equal values in id order."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(9)
+    pred = torch.softmax(torch.randn(50, 60, generator=g) * 3.0, dim=-1)
+    pred[3, [40, 5, 17]] = pred[3].max() + 0.1          # three-way tie at the top
+    pred[4] = 1.0 / 60                                   # all equal
+    for K in (1, 8, 16):
+        order = torch.sort(pred, dim=-1, descending=True, stable=True)
+        topv, topi = ops.topk_values(pred.to(device), K)
+        assert torch.equal(topi.cpu(), order.indices[:, :K])
+        assert torch.equal(topv.cpu(), order.values[:, :K])
+    topv, _ = ops.topk_values(pred.to(device), 8, out_dtype=torch.bfloat16)
+    assert torch.equal(topv.cpu(), torch.sort(pred, dim=-1, descending=True).values[:, :8].to(torch.bfloat16))
+    with pytest.raises(ValueError):
+        ops.topk_values(pred.to(device), 17)
 
 
 # ------------------------------------------------------------------ router logits
@@ -196,7 +191,7 @@ def test_route_decode_equals_the_three_separate_calls(device, dtype, ldt, T):
 @pytest.mark.parametrize("T,E,K", [(1, 4, 4), (32, 256, 16), (7, 64, 6), (32, 60, 1)])
 def test_route_decode_shapes_against_oracle(device, T, E, K):
     """Corner shapes of the decode router (K == E, the largest E and K, K == 1) against the
-    CPU oracle: indices exact wherever the top-k boundary is not a rounding tie."""
+    CPU oracle: logits within fp32 summation error, indices exact given the logits the kernel wrote."""
     ops = _ops()
     H = 512
     dtype = torch.float32
@@ -210,11 +205,11 @@ def test_route_decode_shapes_against_oracle(device, T, E, K):
     counter = torch.zeros(1, dtype=torch.int32, device=device)
     ops.route_decode(x, wg, None, K, False, logits, None, topv, topi, perm, counter)
     torch.cuda.synchronize()
-    ref_v, ref_i, ref_logits = ref_moe.routing_router(x.cpu(), layer["gate_w"], K, False)
+    _, _, ref_logits = ref_moe.routing_router(x.cpu(), layer["gate_w"], K, False)
     torch.testing.assert_close(logits.cpu(), ref_logits, rtol=1e-5, atol=1e-5)
-    safe = _boundary_safe(ref_logits, K)
-    assert torch.equal(topi.cpu()[safe], ref_i[safe])
-    torch.testing.assert_close(topv.cpu()[safe], ref_v[safe], rtol=1e-5, atol=1e-6)
+    ref_v, ref_i, _ = ref_moe.routing_router(x.cpu(), layer["gate_w"], K, False, router_logits=logits.cpu())
+    assert torch.equal(topi.cpu(), ref_i)
+    torch.testing.assert_close(topv.cpu(), ref_v, rtol=1e-5, atol=1e-6)
     p_perm, p_inv, p_off, p_active = ref_permute.permute_build(topi.cpu().numpy(), E)
     assert np.array_equal(perm.perm.cpu().numpy(), p_perm)
     assert np.array_equal(perm.inv_perm.cpu().numpy(), p_inv)
@@ -232,8 +227,8 @@ def test_route_decode_packed_shapes(device, T, H, E, K, shared_gate, renorm, ldt
     """One-workgroup decode router on the packed gate matrix (one to sixty-four rows, H from
     one 64-wide block to several per wavefront, an odd number of blocks): logits and shared
     gate against fp32 linear algebra, top-k and permutation bit for bit what gate_topk and
-    permute_build return on the logits it wrote, indices against the oracle's rule wherever
-    those logits leave no rounding tie, and the same answer call after call."""
+    permute_build return on the logits it wrote, indices equal to the oracle's on those logits,
+    and the same answer call after call."""
     ops = _ops()
     dtype = torch.bfloat16
     layer = make_layer(H, E, 64, K, Is=64, shared_gate=shared_gate, dtype=dtype, seed=23 + T)
@@ -265,9 +260,8 @@ def test_route_decode_packed_shapes(device, T, H, E, K, shared_gate, renorm, ldt
             assert torch.equal(getattr(perm_a, name), getattr(perm, name)), name
         assert torch.equal(perm_a.active_eids[:n], perm.active_eids[:n])
         probs = torch.softmax(logits.cpu(), dim=-1, dtype=torch.float32)
-        ref_i = torch.sort(probs, dim=-1, descending=True, stable=True).indices[:, :K]
-        safe = _boundary_safe(logits.cpu(), K) if K < E else torch.ones(T, dtype=torch.bool)
-        assert torch.equal(topi.cpu()[safe], ref_i[safe])
+        _, ref_i = ref_moe.topk_by_logit(logits.cpu(), probs, K)
+        assert torch.equal(topi.cpu(), ref_i)
 
 
 def test_pack_router_gate_declines_what_does_not_fit():

@@ -15,32 +15,44 @@ pytestmark = pytest.mark.gpu
 SHAPE = dict(family="qwen_shared", hidden=512, num_experts=12, inter=256, top_k=4, shared_inter=384, num_layers=3)
 
 
-def _stack(device, method, capacity, top_m, offload, seed0=0, **overrides):
+def _stack(device, method, capacity, top_m, offload, seed0=0, shape=None, structured=False, **overrides):
+    """``shape``: the toy stack unless given.  ``structured``: skewed, co-activating routing
+    (Zipf popularity + clusters of 4) written into the gates; the blocks then carry the
+    structure the inputs must be drawn with as ``blocks[0].test_structure``."""
     from sparse_amd.block import DistributedSparseMoeBlock
     from sparse_amd.context import DistEnv, Metrics, SparseContext
     from sparse_amd.methods import method_settings, residency_config
     from sparse_amd.rs import random_init_bank
-    from sparse_amd.synthetic import make_mlp_block
+    from sparse_amd.synthetic import add_routing_structure, make_mlp_block
+    shape = shape or SHAPE
     SparseContext.reset()
     metrics = Metrics()
     metrics.events = []
     kw = method_settings(method)["kwargs"]
     blocks = []
-    for layer in range(SHAPE["num_layers"]):
-        mlp = make_mlp_block(SHAPE, dtype=torch.bfloat16, seed=seed0 + layer)
+    structure = None
+    for layer in range(shape["num_layers"]):
+        mlp = make_mlp_block(shape, dtype=torch.bfloat16, seed=seed0 + layer, fused=shape is not SHAPE,
+                             device=device if shape is not SHAPE else "cpu")
+        if structured:
+            structure = add_routing_structure(mlp, shape["num_experts"], seed=layer)
         cfg = residency_config(method, capacity, top_m, **overrides) if offload == "cpu" else None
         blocks.append(DistributedSparseMoeBlock(
-            layer, mlp, None, DistEnv(0, 1, 0, device), num_layers=SHAPE["num_layers"],
-            num_experts=SHAPE["num_experts"], top_k=SHAPE["top_k"], dtype=torch.bfloat16, expert_offload=offload,
+            layer, mlp, None, DistEnv(0, 1, 0, device), num_layers=shape["num_layers"],
+            num_experts=shape["num_experts"], top_k=shape["top_k"], dtype=torch.bfloat16, expert_offload=offload,
             expert_cache=capacity, planner_mode=kw["planner_mode"] if offload == "cpu" else "none",
             prefetch_top_m=top_m, placement_mode=kw["placement_mode"], metrics=metrics, residency_config=cfg))
+        del mlp
+    blocks[0].test_structure = structure
     if offload == "cpu" and kw["planner_mode"] == "rs_prefetch":
-        SparseContext.set_rs_bank(random_init_bank(SHAPE["num_layers"], SHAPE["hidden"], SHAPE["num_experts"],
+        SparseContext.set_rs_bank(random_init_bank(shape["num_layers"], shape["hidden"], shape["num_experts"],
                                                    hidden_dim=64, seed=5, device=device))
     return blocks, metrics
 
 
-def _run(blocks, device, steps, T, record=None, sync_prefetch=False, prefill_first=False):
+def _run(blocks, device, steps, T, record=None, sync_prefetch=False, prefill_first=False, calls=None):
+    """``calls``: explicit list of ``(phase, hidden [B,S,H] on the device)`` instead of the toy
+    schedule of ``steps`` decode steps of ``T`` tokens."""
     from sparse_amd.block import _SideStreams
     from sparse_amd.context import SparseContext
     from sparse_amd.synthetic import make_hidden
@@ -62,24 +74,31 @@ def _run(blocks, device, steps, T, record=None, sync_prefetch=False, prefill_fir
                 if sync_prefetch:
                     _SideStreams.get().prefetch.synchronize()
             blk._rs_plan_hook = hook
-    for step in range(steps):
-        prefill = prefill_first and step == 0
-        SparseContext.current_phase = "prefill" if prefill else "decode"
+    if calls is None:
+        calls = []
+        for step in range(steps):
+            prefill = prefill_first and step == 0
+            n = 40 if prefill else T
+            x = make_hidden(n, SHAPE["hidden"], torch.bfloat16, seed=1000 + step).to(device)
+            calls.append(("prefill" if prefill else "decode", x.view(1, n, -1) if prefill else x.view(n, 1, -1)))
+    for step, (phase, hid) in enumerate(calls):
+        SparseContext.current_phase = phase
         SparseContext.begin_runtime_call(step)
-        n = 40 if prefill else T
-        x = make_hidden(n, SHAPE["hidden"], torch.bfloat16, seed=1000 + step).to(device)
-        hid = x.view(1, n, -1) if prefill else x.view(n, 1, -1)
         for blk in blocks:
-            out, _logits = blk(hid)
+            ret = blk(hid)
+            out = ret[0] if isinstance(ret, tuple) else ret
             outs.append(out.clone())
     torch.cuda.synchronize()
     return outs
 
 
-def _replay_oracle(record, cfg, capacity):
+def _replay_oracle(record, cfg, capacity, shape=None, expert_bytes=0):
+    shape = shape or SHAPE
     names = [n for n in vars(RefConfig()) if hasattr(cfg, n)]
     rc = {n: getattr(cfg, n) for n in names}
-    lays = [RefLayer(l, SHAPE["num_experts"], SHAPE["top_k"], RefConfig(**rc)) for l in range(SHAPE["num_layers"])]
+    lays = [RefLayer(l, shape["num_experts"], shape["top_k"], RefConfig(**rc)) for l in range(shape["num_layers"])]
+    for lay in lays:
+        lay.expert_bytes = expert_bytes
     plans, executors = [], []
     pending_rs = None
     for item in record:
@@ -149,6 +168,105 @@ def test_offloaded_methods_match_resident_values_and_oracle_events(device, metho
         assert any(k == "prefetch_hit" for k, _l, _e in metrics.events) or method == "rs"
     if method in ("epipe", "rs-epipe", "sparse"):
         assert any(n.startswith("epipe") for n in executors)
+
+
+# ---- the offload configurations at their real layer shapes ---------------------------------
+def _structured_calls(blocks, shape, device, phase, n_calls, tokens, seed0):
+    from sparse_amd.synthetic import make_structured_hidden
+    st = blocks[0].test_structure
+    calls = []
+    for i in range(n_calls):
+        x = make_structured_hidden(tokens, shape["hidden"], shape["num_experts"] // 4, st["cluster_prob"],
+                                   torch.bfloat16, seed=seed0 + i).to(device)
+        calls.append((phase, x.view(1, tokens, -1) if phase == "prefill" else x.view(tokens, 1, -1)))
+    return calls
+
+
+def _check_against_oracle(blocks, metrics, record, cfg, capacity, shape):
+    lays, plans, executors = _replay_oracle(record, cfg, capacity, shape, blocks[0].arena.expert_bytes)
+    assert executors == [r[2] for r in record if r[0] == "executor"]
+    for l, lay in enumerate(lays):
+        want_events = [t for t in lay.trace if t[0] in ("hit", "prefetch_hit", "miss")]
+        got_events = [(k, e) for k, ll, e in metrics.events if ll == l]
+        assert got_events == want_events, f"layer {l}: cache events differ from the oracle"
+        assert blocks[l].residency.cache.resident_ids() == lay.cache.resident_ids()
+        assert blocks[l].residency.extra_cache.resident_ids() == lay.extra.resident_ids()
+    misses = sum(1 for k, _l, _e in metrics.events if k == "miss")
+    assert metrics.cache_miss_count == misses and misses > 0
+    assert metrics.demand_h2d_bytes == misses * blocks[0].arena.expert_bytes
+    return lays, plans, executors
+
+
+@pytest.mark.parametrize("method,overrides", [
+    ("rr", {}), ("rs-epipe", {}), ("sparse", {}),
+    # the prefill side cache: staged experts that are not committed to the LRU are parked there,
+    # ten slots, of which the default 128 MB byte bound lets seven 17.3 MB experts in
+    ("rs-epipe", dict(epipe_prefill_extra_cache_slots=10, epipe_prefill_commit=False)),
+    ("epipe", dict(epipe_prefill_extra_cache_slots=4, epipe_prefill_extra_cache_max_mb=0.0)),
+])
+def test_chunked_epipe_prefill_at_the_deepseek_shape(device, method, overrides):
+    """Readiness-aware chunked prefill as the benchmark configuration states it, on two layers:
+    DeepSeek-V2-Lite layer shape, a 4096-token prefill as two 2048-token prefill-phase calls,
+    HBM cache of 19 of 64 experts (30 %), Zipf / co-activation routing, the EPIPE prefill
+    stage on (reference utils/eval_core.py:11867-12167; side cache :5637-5720).  Outputs equal
+    the all-resident stack bit for bit; cache events, executor per call, the final LRU order
+    and the side cache equal the oracle's."""
+    from sparse_amd.methods import residency_config
+    from sparse_amd.synthetic import DEEPSEEK
+    shape = dict(DEEPSEEK, num_layers=2)
+    capacity, top_m = 19, 8
+    overrides = dict(overrides, epipe_prefill_enable=True)
+    # the first chunk finds a cold cache (nothing ready: plain order), the second stages; the side
+    # cache cases take a third chunk, which reads what the second one parked
+    n_calls = 3 if overrides.get("epipe_prefill_extra_cache_slots") else 2
+    ref_blocks, _ = _stack(device, "rr", capacity, top_m, "gpu", shape=shape, structured=True)
+    calls = _structured_calls(ref_blocks, shape, device, "prefill", n_calls, 2048, 7100)
+    want = _run(ref_blocks, device, 0, 0, calls=calls)
+    del ref_blocks
+    blocks, metrics = _stack(device, method, capacity, top_m, "cpu", shape=shape, structured=True, **overrides)
+    record = []
+    got = _run(blocks, device, 0, 0, record=record, sync_prefetch=True, calls=calls)
+    assert len(got) == len(want) == 2 * n_calls
+    for i, (a, b) in enumerate(zip(got, want)):
+        assert torch.equal(a, b), f"output {i} differs from the all-resident stack"
+    cfg = residency_config(method, capacity, top_m, **overrides)
+    lays, _plans, executors = _check_against_oracle(blocks, metrics, record, cfg, capacity, shape)
+    # a 2048-token chunk touches (nearly) every expert, so most of each call misses
+    assert metrics.cache_miss_count >= n_calls * 2 * (shape["num_experts"] - capacity) * 0.8
+    if method != "rr":
+        assert any(n.startswith("epipe") for n in executors)
+    if overrides.get("epipe_prefill_extra_cache_slots"):
+        kept = [len(lay.extra.resident_ids()) for lay in lays]
+        assert sum(kept) > 0, "nothing was ever parked in the prefill side cache"
+        hits = metrics.counters.get("epipe_prefill_extra_cache_hit_count", 0)
+        assert hits == sum(lay.counters.get("epipe_prefill_extra_cache_hit_count", 0) for lay in lays) > 0
+        assert max(kept) <= (128 * 1024 * 1024) // blocks[0].arena.expert_bytes
+
+
+@pytest.mark.parametrize("method", ["rr", "rs", "rs-epipe"])
+def test_cached_decode_at_the_qwen_shape(device, method):
+    """Cached-expert decode as the benchmark configuration states it, on two layers: Qwen layer
+    shape, 15 of 60 experts in HBM, the rest in pinned host memory (17.3 MB per upload), batch
+    8, Zipf / co-activation routing, next-layer predictor with top-8 prefetch.  Outputs equal
+    the all-resident stack bit for bit; events, plans and final LRU order equal the oracle's."""
+    from sparse_amd.methods import residency_config
+    from sparse_amd.synthetic import QWEN
+    shape = dict(QWEN, num_layers=2)
+    capacity, top_m, steps, batch = 15, 8, 10, 8
+    ref_blocks, _ = _stack(device, "rr", capacity, top_m, "gpu", shape=shape, structured=True)
+    calls = _structured_calls(ref_blocks, shape, device, "decode", steps, batch, 5000)
+    want = _run(ref_blocks, device, 0, 0, calls=calls)
+    del ref_blocks
+    blocks, metrics = _stack(device, method, capacity, top_m, "cpu", shape=shape, structured=True)
+    assert blocks[0].arena.expert_bytes == 17301504
+    record = []
+    got = _run(blocks, device, 0, 0, record=record, sync_prefetch=True, calls=calls)
+    for i, (a, b) in enumerate(zip(got, want)):
+        assert torch.equal(a, b), f"output {i} differs from the all-resident stack"
+    cfg = residency_config(method, capacity, top_m)
+    _check_against_oracle(blocks, metrics, record, cfg, capacity, shape)
+    if method != "rr":
+        assert metrics.prefetch_admitted_count > 0 and metrics.prefetch_h2d_bytes > 0
 
 
 def test_values_do_not_depend_on_copy_timing(device):

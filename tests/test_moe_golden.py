@@ -142,17 +142,21 @@ def test_hip_block_against_the_reference_vectors(device, case):
     if logits is not None:
         torch.testing.assert_close(logits.cpu().float(), c.want["logits"].float(),
                                    **(dict(rtol=2e-2, atol=2e-2) if dtype == torch.bfloat16 else tol))
-    # on the device's own logits the choice is exact; against the reference's logits it is the
-    # same set wherever the k-th and (k+1)-th probabilities are not within rounding of each other
-    probs = torch.softmax(c.want["logits"].float(), -1)
-    srt = torch.sort(probs, -1, descending=True).values
-    clear = (srt[:, K - 1] - srt[:, K]) > (2e-2 if dtype == torch.bfloat16 else 1e-5) if K < E else torch.ones(T, dtype=torch.bool)
+    # indices: exact, on every row, given the logits the device itself wrote
+    if logits is not None:
+        _, own_i, _ = ref_moe.routing_router(c.x, c.gate_w, K, c.renorm, router_logits=logits.cpu())
+        assert torch.equal(ws.topi.cpu(), own_i)
+    # against the reference's recorded run: its logits differ from the device's in the order of
+    # the sum, so a token whose K-th and (K+1)-th logits nearly tie may route elsewhere; rows
+    # that chose the reference's experts (nearly all) are held to the recorded layer output
+    got = out.view(T, H).cpu().float()
     got_i = torch.sort(ws.topi.cpu(), 1).values
-    want_i = torch.sort(c.want["topi"], 1).values
-    assert torch.equal(got_i[clear], want_i[clear])
-    if bool(clear.all()):
-        # these layers have weights of std 0.25, so outputs are O(10): the absolute part of the
-        # tolerance is taken relative to the output's scale
-        want = c.want["layer_out"].float()
-        scale = max(1.0, float(want.abs().max()))
-        torch.testing.assert_close(out.view(T, H).cpu().float(), want, rtol=tol["rtol"], atol=tol["atol"] * scale)
+    same = (got_i == torch.sort(c.want["topi"], 1).values).all(dim=1)
+    assert float(same.float().mean()) >= 0.9, "too few rows route like the reference for the comparison to mean much"
+    torch.testing.assert_close(got[same], c.want["layer_out"].float()[same], **tol)
+    # the other rows: the oracle on the device's own routing
+    if not bool(same.all()):
+        want = ref_moe.moe_forward_routed(c.x, ws.topv.cpu(), ws.topi.cpu(), c.experts, c.shared, c.shared_gate_w)
+        torch.testing.assert_close(got[~same], want.float()[~same], **tol)
+    # the output scale is that of the full-size layers, so atol 1e-2 bites
+    assert 0.05 < float(c.want["layer_out"].float().abs().mean()) < 2.0

@@ -50,6 +50,41 @@ def test_router_tie_rule():
     assert topi.tolist() == [[0, 1, 2], [2, 6, 0], [7, 0, 1]]
 
 
+def test_ranking_on_logits_is_the_probability_ranking_wherever_probabilities_differ():
+    """``topk_by_logit`` against the plain top-k of the probabilities (what the reference
+    computes): identical indices and values on every row whose k+1 largest probabilities are
+    distinct or come from equal logits -- softmax is monotone."""
+    g = torch.Generator().manual_seed(3)
+    for dtype in (torch.float32, torch.bfloat16):
+        logits = (torch.randn(2000, 60, generator=g) * 2.0).to(dtype)
+        probs = torch.softmax(logits, dim=-1, dtype=torch.float32)
+        v1, i1 = ref_moe.topk_by_logit(logits, probs, 4)
+        v2, i2 = ref_moe.topk_lower_id_first(probs, 4)
+        top5 = torch.sort(probs, dim=-1, descending=True).values[:, :5]
+        lt5 = torch.sort(logits.float(), dim=-1, descending=True).values[:, :5]
+        clear = ((top5[:, :-1] != top5[:, 1:]) | (lt5[:, :-1] == lt5[:, 1:])).all(dim=1)
+        assert clear.float().mean() > 0.99
+        assert torch.equal(i1[clear], i2[clear]) and torch.equal(v1[clear], v2[clear])
+        tv, ti = torch.topk(probs, 4, dim=-1)                 # the reference's call
+        assert torch.equal(v1, tv)                            # values never depend on the tie order
+        distinct = (top5[:, :-1] != top5[:, 1:]).all(dim=1)   # torch.topk leaves equal values in any order
+        assert torch.equal(i1[distinct], ti[distinct])
+
+
+def test_ranking_on_logits_when_two_logits_collapse_to_one_probability():
+    """Two logits one ulp apart close to the maximum round to the same probability; the rule
+    still prefers the larger logit, whichever id it has, and the selected set is a valid top-k
+    of the probabilities either way."""
+    lo = torch.tensor(-0.1)
+    logits = torch.stack([torch.tensor(0.0), torch.nextafter(lo, torch.tensor(-100.0)), lo]).view(1, 3)
+    probs = torch.softmax(logits, dim=-1)
+    assert probs[0, 1] == probs[0, 2]                         # collapsed
+    v, i = ref_moe.topk_by_logit(logits, probs, 2)
+    assert i.tolist() == [[0, 2]]
+    assert ref_moe.topk_lower_id_first(probs, 2)[1].tolist() == [[0, 1]]
+    assert torch.equal(v, torch.topk(probs, 2).values)
+
+
 def test_deepseek_router_is_fp32_and_builds_pseudo_logits():
     g = torch.Generator().manual_seed(1)
     x = (torch.randn(10, 16, generator=g)).to(torch.bfloat16)
