@@ -298,6 +298,28 @@ int sparse_hip_moe_ffn_decode(const sparse_hip_experts* experts, const void* x_d
                               void* sh_inter_ws_dev, void* shared_dev, void* split_ws_dev,
                               void* stream);
 
+/*
+ * sparse_hip_moe_ffn_decode followed by sparse_hip_combine_split, without the second launch:
+ * in the down projection, the workgroup that finishes a 32-column tile last (counted per
+ * tile) sums that tile's columns of every token -- the K routed rows in ascending expert id,
+ * then the shared expert from its partial sums, with the rounding steps of
+ * sparse_hip_combine_split, bit for bit -- and writes `out_dev` [T,H]
+ * (utils/eval_core.py:16520-16526, :14690-14721, :523-538, :9455-9463).  Needs
+ * sparse_hip_decode_split_parts(Is) > 1.  `split_ws_dev` holds
+ * sparse_hip_decode_split_ws_bytes(T, H) bytes: the partial sums, then, from
+ * sparse_hip_decode_split_counter_offset(T, H) on, one int32 counter per tile, which must be
+ * zero before the first call; every call leaves them zero.  Calls that share a workspace must
+ * not overlap.  `parts_dev` is written as by sparse_hip_moe_ffn_decode.
+ */
+size_t sparse_hip_decode_split_counter_offset(int T, int H);
+int sparse_hip_moe_ffn_decode_combine(const sparse_hip_experts* experts, const void* x_dev, const void* topv_dev,
+                                      const int32_t* perm_dev, const int32_t* inv_perm_dev,
+                                      const int32_t* seg_offsets_dev, const sparse_hip_seglist* segs, int T,
+                                      int K, void* inter_ws_dev, void* parts_dev, const void* sh_gate_w_dev,
+                                      const void* sh_up_w_dev, const void* sh_down_w_dev,
+                                      const void* shared_gate_dev, int Is, void* sh_inter_ws_dev,
+                                      void* split_ws_dev, void* out_dev, void* stream);
+
 /* ---- A7: combine ----------------------------------------------------------- */
 
 /*

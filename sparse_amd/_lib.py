@@ -80,6 +80,10 @@ SIGNATURES = {
     "sparse_hip_moe_ffn_decode": (
         _i, [C.POINTER(Experts), _vp, _vp, _vp, _vp, C.POINTER(SegList), _i, _i, _vp, _vp,
              _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _vp]),
+    "sparse_hip_moe_ffn_decode_combine": (
+        _i, [C.POINTER(Experts), _vp, _vp, _vp, _vp, _vp, C.POINTER(SegList), _i, _i, _vp, _vp,
+             _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _vp]),
+    "sparse_hip_decode_split_counter_offset": (_sz, [_i, _i]),
     "sparse_hip_decode_split_ws_bytes": (_sz, [_i, _i]),
     "sparse_hip_decode_split_parts": (_i, [_i]),
     "sparse_hip_combine_split": (_i, [_vp, _vp, _vp, _i, _vp, _i, _i, _i, _vp, _vp]),

@@ -286,6 +286,10 @@ class DistributedSparseMoeBlock(nn.Module):
         self.rs_prob_to_logit_eps = float(rs_prob_to_logit_eps)
         self.prefetch_top_m = int(prefetch_top_m)
         self.metrics = metrics if metrics is not None else Metrics()
+        # all-resident decode calls of up to 16 tokens: combine inside the down projection's launch
+        # (SPARSE_HIP_FOLD_COMBINE=0 keeps the separate combine launch; same bits either way)
+        self.fold_combine = str(os.environ.get("SPARSE_HIP_FOLD_COMBINE", "1")).strip().lower() not in (
+            "", "0", "false", "no", "off")
         # prefill-size batches run the shared expert on a second stream beside the routing
         self.overlap_shared = str(os.environ.get("SPARSE_HIP_OVERLAP_SHARED", "1")).strip().lower() not in (
             "", "0", "false", "no", "off")
@@ -608,7 +612,14 @@ class DistributedSparseMoeBlock(nn.Module):
         if not staged and self._next_layer_rs_feature_mode() == "hidden_router_topk":
             rs_job = self._rs_begin(x, S, ws, source=(ws.topi, ws.topv))
 
-        if fused:
+        out = torch.empty((T, H), device=x.device, dtype=self.dtype)
+        combined = False
+        if fused and split_shared and self.fold_combine:
+            # small decode call, everything resident: the down projection's launch also combines
+            ops.moe_ffn_decode_combine(self._experts_desc, x, ws.topv, ws.perm, ws.segs_dev, ws.inter, ws.parts,
+                                       self.shared_weights, shared_gate, ws.shared_inter, ws.split_ws, out)
+            combined = True
+        elif fused:
             ops.moe_ffn_decode(self._experts_desc, x, ws.topv, ws.perm, ws.segs_dev, ws.inter, ws.parts,
                                self.shared_weights, shared_gate, ws.shared_inter, ws.shared_out, ws.split_ws)
         elif self.residency is None:
@@ -637,8 +648,9 @@ class DistributedSparseMoeBlock(nn.Module):
 
         if side is not None:
             torch.cuda.current_stream().wait_stream(side)
-        out = torch.empty((T, H), device=x.device, dtype=self.dtype)
-        if split_shared:
+        if combined:
+            pass
+        elif split_shared:
             ops.combine_split(ws.parts, ws.perm, ws.split_ws, ws.split_parts, shared_gate, T, k_exec, out)
         else:
             ops.combine(ws.parts, ws.perm, ws.shared_out, T, k_exec, out)

@@ -11,8 +11,9 @@ int decode_shared_bf16(const void*, const void*, const void*, const void*, const
                        void*, hipStream_t);
 int decode_fused_bf16(const sparse_hip_experts*, const void*, const void*, const int32_t*, const int32_t*,
                       const sparse_hip_seglist*, int, int, void*, void*, const void*, const void*, const void*,
-                      const void*, int, void*, void*, void*, hipStream_t);
+                      const void*, int, void*, void*, void*, const int32_t*, void*, hipStream_t);
 size_t decode_split_ws_bytes(int, int);
+size_t decode_split_counter_offset(int, int);
 int decode_split_parts(int);
 int prefill_routed_bf16(const sparse_hip_experts*, const void*, const void*, const int32_t*, const int32_t*,
                         const sparse_hip_seglist*, int, int, void*, void*, void*, hipStream_t);
@@ -134,7 +135,40 @@ int sparse_hip_moe_ffn_decode(const sparse_hip_experts* experts, const void* x_d
              "moe_ffn_decode: shared-expert pointers must be 16-byte aligned");
   return decode_fused_bf16(experts, x_dev, topv_dev, perm_dev, seg_offsets_dev, segs, T, K, inter_ws_dev,
                            parts_dev, sh_gate_w_dev, sh_up_w_dev, sh_down_w_dev, shared_gate_dev, Is,
-                           sh_inter_ws_dev, shared_dev, split_ws_dev, as_stream(stream));
+                           sh_inter_ws_dev, shared_dev, split_ws_dev, nullptr, nullptr, as_stream(stream));
+}
+
+int sparse_hip_moe_ffn_decode_combine(const sparse_hip_experts* experts, const void* x_dev, const void* topv_dev,
+                                      const int32_t* perm_dev, const int32_t* inv_perm_dev,
+                                      const int32_t* seg_offsets_dev, const sparse_hip_seglist* segs, int T, int K,
+                                      void* inter_ws_dev, void* parts_dev, const void* sh_gate_w_dev,
+                                      const void* sh_up_w_dev, const void* sh_down_w_dev, const void* shared_gate_dev,
+                                      int Is, void* sh_inter_ws_dev, void* split_ws_dev, void* out_dev, void* stream) {
+  int rc = check_routed("moe_ffn_decode_combine", experts, x_dev, topv_dev, perm_dev, seg_offsets_dev, segs, T, K,
+                        inter_ws_dev, parts_dev);
+  if (rc != SPARSE_HIP_OK) return rc;
+  SP_REQUIRE(experts->dtype == SPARSE_HIP_BF16, "moe_ffn_decode_combine: bf16 only");
+  SP_REQUIRE(T <= SPARSE_HIP_DECODE_MAX_TOKENS, "moe_ffn_decode_combine: T=%d exceeds %d", T,
+             SPARSE_HIP_DECODE_MAX_TOKENS);
+  SP_REQUIRE(Is > 0 && Is % 64 == 0, "moe_ffn_decode_combine: Is=%d must be a positive multiple of 64", Is);
+  SP_REQUIRE(decode_split_parts(Is) > 1,
+             "moe_ffn_decode_combine: Is=%d cannot be cut into parts; use sparse_hip_moe_ffn_decode + sparse_hip_combine", Is);
+  SP_REQUIRE(sh_gate_w_dev && sh_up_w_dev && sh_down_w_dev && sh_inter_ws_dev && split_ws_dev && inv_perm_dev && out_dev,
+             "moe_ffn_decode_combine: NULL pointer");
+  SP_REQUIRE(((reinterpret_cast<uintptr_t>(sh_gate_w_dev) | reinterpret_cast<uintptr_t>(sh_up_w_dev) |
+               reinterpret_cast<uintptr_t>(sh_down_w_dev) | reinterpret_cast<uintptr_t>(sh_inter_ws_dev) |
+               reinterpret_cast<uintptr_t>(out_dev) | reinterpret_cast<uintptr_t>(split_ws_dev)) &
+              15) == 0,
+             "moe_ffn_decode_combine: pointers must be 16-byte aligned");
+  return decode_fused_bf16(experts, x_dev, topv_dev, perm_dev, seg_offsets_dev, segs, T, K, inter_ws_dev,
+                           parts_dev, sh_gate_w_dev, sh_up_w_dev, sh_down_w_dev, shared_gate_dev, Is,
+                           sh_inter_ws_dev, /*shared_out=*/out_dev, split_ws_dev, inv_perm_dev, out_dev,
+                           as_stream(stream));
+}
+
+size_t sparse_hip_decode_split_counter_offset(int T, int H) {
+  if (T < 1 || H < 1) return 0;
+  return decode_split_counter_offset(T, H);
 }
 
 size_t sparse_hip_decode_split_ws_bytes(int T, int H) {

@@ -57,8 +57,26 @@ struct DecodeArgs {
   // (1 = not cut): fp32 partial sums [split_s][T][Ndim_s], finished by the combine step
   int32_t split_s;
   float* split_sums;
+  // combine folded into the down projection (needs split_s > 1): the workgroup that finishes a
+  // 32-column tile last, counted per tile in `tile_counters`, sums that tile's columns of
+  // every token over its K routed rows and the shared expert and writes `final_out`
+  int32_t* tile_counters;       // [Ndim / kDecRows], zero between launches; NULL: no combine here
+  const int32_t* inv_perm;      // [T*K]
+  uint16_t* final_out;          // [T, Ndim]
   sparse_hip_seglist segs;
 };
+
+// Results that another workgroup of the same launch reads travel as device-scope relaxed
+// atomics: such a store is written through to memory instead of staying in the writer's
+// L2 (each XCD has its own), such a load is served from memory instead of a stale line of the
+// reader's L2.  No cache-wide write-back or invalidate is involved, which is what a
+// release / acquire fence at device scope costs.
+__device__ __forceinline__ void st_device_u64(void* p, uint64_t v) {
+  __hip_atomic_store(reinterpret_cast<uint64_t*>(p), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ uint64_t ld_device_u64(const void* p) {
+  return __hip_atomic_load(reinterpret_cast<const uint64_t*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 
 __device__ __forceinline__ bf16x8 ld_bf16x8(const uint16_t* p) {
   return *reinterpret_cast<const bf16x8*>(p);
@@ -112,7 +130,7 @@ __global__ __launch_bounds__(kDecThreads) void decode_ffn_kernel(const DecodeArg
     row0 = (b - si * a.tiles_r) * kDecRows;
     r0 = a.seg_offsets[eid];
     M = a.seg_offsets[eid + 1] - r0;
-    if (M <= 0) return;
+    if (M <= 0 && (kGateUp || a.tile_counters == nullptr)) return;  // (an empty segment still counts as arrived)
     const uint16_t* slot = a.slab + static_cast<uint64_t>(slot_id) * a.slot_stride;
     w0 = slot + a.mat_offset;
     w1 = slot + a.mat2_offset;
@@ -273,8 +291,13 @@ __global__ __launch_bounds__(kDecThreads) void decode_ffn_kernel(const DecodeArg
     uint2 pk;
     pk.x = static_cast<uint32_t>(o[0]) | (static_cast<uint32_t>(o[1]) << 16);
     pk.y = static_cast<uint32_t>(o[2]) | (static_cast<uint32_t>(o[3]) << 16);
-    *reinterpret_cast<uint2*>(dst) = pk;
+    if (!kGateUp && a.tile_counters != nullptr) {
+      st_device_u64(dst, static_cast<uint64_t>(pk.x) | (static_cast<uint64_t>(pk.y) << 32));
+    } else {
+      *reinterpret_cast<uint2*>(dst) = pk;
+    }
   };
+  const bool fuse = !kGateUp && a.tile_counters != nullptr;
 
   if (!kGateUp && is_shared && split > 1) {
     // A part of a shared tile: its fp32 sums go to memory as they are; the combine step adds
@@ -287,24 +310,107 @@ __global__ __launch_bounds__(kDecThreads) void decode_ffn_kernel(const DecodeArg
       f32x4 s0 = red[0][f][lane];
 #pragma unroll
       for (int w = 1; w < kDecWaves; ++w) s0 += red[w][f][lane];
-      *reinterpret_cast<f32x4*>(a.split_sums + part * part_stride + static_cast<size_t>(n) * Ndim + row0 + tl * 16 +
-                                q * 4) = s0;
+      float* dst = a.split_sums + part * part_stride + static_cast<size_t>(n) * Ndim + row0 + tl * 16 + q * 4;
+      if (fuse) {
+        st_device_u64(dst, static_cast<uint64_t>(__float_as_uint(s0[0])) | (static_cast<uint64_t>(__float_as_uint(s0[1])) << 32));
+        st_device_u64(dst + 2, static_cast<uint64_t>(__float_as_uint(s0[2])) | (static_cast<uint64_t>(__float_as_uint(s0[3])) << 32));
+      } else {
+        *reinterpret_cast<f32x4*>(dst) = s0;
+      }
     }
-    return;
+    if (!fuse) return;
+  } else {
+    for (int f = wave; f < NFRAG; f += kDecWaves) {
+      const int tl = f / NT, nt = f - tl * NT;
+      const int n = r + 16 * nt;
+      if (n >= M) continue;
+      f32x4 s0 = red[0][f * NM][lane];
+      f32x4 s1 = kGateUp ? red[0][f * NM + 1][lane] : f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int w = 1; w < kDecWaves; ++w) {
+        s0 += red[w][f * NM][lane];
+        if (kGateUp) s1 += red[w][f * NM + 1][lane];
+      }
+      emit(tl, n, s0, s1);
+    }
   }
 
-  for (int f = wave; f < NFRAG; f += kDecWaves) {
-    const int tl = f / NT, nt = f - tl * NT;
-    const int n = r + 16 * nt;
-    if (n >= M) continue;
-    f32x4 s0 = red[0][f * NM][lane];
-    f32x4 s1 = kGateUp ? red[0][f * NM + 1][lane] : f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int w = 1; w < kDecWaves; ++w) {
-      s0 += red[w][f * NM][lane];
-      if (kGateUp) s1 += red[w][f * NM + 1][lane];
+  if constexpr (!kGateUp) {
+    if (!fuse) return;
+    // ---- combine, by the workgroup that finishes this 32-column tile last ----------------
+    // Every workgroup of the tile (one per active routed segment, `split` for the shared
+    // expert) has written its rows through to memory; once its own writes are acknowledged it
+    // counts itself in.  The last one finds everybody's rows in memory.
+    __shared__ int s_last;
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wavefront's stores have been acknowledged
+    __syncthreads();
+    const int tile = row0 / kDecRows;
+    if (threadIdx.x == 0) {
+      const int nseg = (a.segs.eids_dev != nullptr) ? min(a.segs.count_dev[0], a.segs.n) : a.segs.n;
+      const int prev = __hip_atomic_fetch_add(a.tile_counters + tile, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      s_last = (prev == nseg + split - 1);
+      if (s_last) __hip_atomic_store(a.tile_counters + tile, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
-    emit(tl, n, s0, s1);
+    __syncthreads();
+    if (!s_last) return;
+    // thread -> (token, four columns); the arithmetic is that of the stand-alone combine step:
+    // K ordered adds rounded to bf16, then the shared expert finished from its parts
+    const int Ttok = a.T, K = a.topk, H = a.Ndim_s;
+    const int t = threadIdx.x >> 3, c4 = (threadIdx.x & 7) * 4;
+    if (t >= Ttok) return;
+    int32_t pos[SPARSE_HIP_MAX_TOPK];
+#pragma unroll
+    for (int k = 0; k < SPARSE_HIP_MAX_TOPK; ++k) pos[k] = (k < K) ? a.inv_perm[t * K + k] : 0x7fffffff;
+#pragma unroll
+    for (int i = 1; i < SPARSE_HIP_MAX_TOPK; ++i) {
+#pragma unroll
+      for (int j = i; j > 0; --j) {
+        const int32_t lo = min(pos[j - 1], pos[j]), hi = max(pos[j - 1], pos[j]);
+        pos[j - 1] = lo;
+        pos[j] = hi;
+      }
+    }
+    const int h = row0 + c4;
+    float accv[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int k = 0; k < SPARSE_HIP_MAX_TOPK; ++k) {
+      if (k < K) {
+        const uint64_t v = ld_device_u64(a.out_r + static_cast<size_t>(pos[k]) * H + h);
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          accv[j] = round_bf16(accv[j] + bf16_bits_to_f32(static_cast<uint16_t>(v >> (16 * j))));
+      }
+    }
+    const size_t part_stride = static_cast<size_t>(Ttok) * H;
+    const float* src = a.split_sums + static_cast<size_t>(t) * H + h;
+    float sh[4];
+    {
+      const uint64_t lo = ld_device_u64(src), hi = ld_device_u64(src + 2);
+      sh[0] = __uint_as_float(static_cast<uint32_t>(lo));
+      sh[1] = __uint_as_float(static_cast<uint32_t>(lo >> 32));
+      sh[2] = __uint_as_float(static_cast<uint32_t>(hi));
+      sh[3] = __uint_as_float(static_cast<uint32_t>(hi >> 32));
+    }
+    for (int p = 1; p < split; ++p) {
+      const uint64_t lo = ld_device_u64(src + p * part_stride), hi = ld_device_u64(src + p * part_stride + 2);
+      sh[0] += __uint_as_float(static_cast<uint32_t>(lo));
+      sh[1] += __uint_as_float(static_cast<uint32_t>(lo >> 32));
+      sh[2] += __uint_as_float(static_cast<uint32_t>(hi));
+      sh[3] += __uint_as_float(static_cast<uint32_t>(hi >> 32));
+    }
+    const bool gated = a.gate_s != nullptr;
+    const float scale = gated ? round_bf16(sigmoid_f32(bf16_bits_to_f32(a.gate_s[t]))) : 1.f;
+    uint16_t o[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      float v = round_bf16(sh[j]);
+      if (gated) v = v * scale;
+      o[j] = f32_to_bf16_bits(accv[j] + round_bf16(v));
+    }
+    uint2 pk;
+    pk.x = static_cast<uint32_t>(o[0]) | (static_cast<uint32_t>(o[1]) << 16);
+    pk.y = static_cast<uint32_t>(o[2]) | (static_cast<uint32_t>(o[3]) << 16);
+    *reinterpret_cast<uint2*>(a.final_out + static_cast<size_t>(t) * H + h) = pk;
   }
 }
 
@@ -373,7 +479,7 @@ int decode_fused_bf16(const sparse_hip_experts* ex, const void* x, const void* t
                       const int32_t* seg_offsets, const sparse_hip_seglist* segs, int T, int K, void* inter_ws,
                       void* parts, const void* sh_gate_w, const void* sh_up_w, const void* sh_down_w,
                       const void* shared_gate, int Is, void* sh_inter_ws, void* shared_out, void* split_ws,
-                      hipStream_t st) {
+                      const int32_t* inv_perm, void* final_out, hipStream_t st) {
   const uint64_t H = ex->hidden, I = ex->inter;
   DecodeArgs a = {};
   a.split_s = 1;
@@ -425,11 +531,20 @@ int decode_fused_bf16(const sparse_hip_experts* ex, const void* x, const void* t
   if (split_ws != nullptr && (Is / 64) % kDecSplit == 0) {
     a.split_s = kDecSplit;
     a.split_sums = static_cast<float*>(split_ws);
+    if (final_out != nullptr) {  // the per-tile arrival counters follow the partial sums in the workspace
+      a.tile_counters = reinterpret_cast<int32_t*>(static_cast<float*>(split_ws) + static_cast<size_t>(kDecSplit) * T * H);
+      a.inv_perm = inv_perm;
+      a.final_out = static_cast<uint16_t*>(final_out);
+    }
   }
   return launch_decode<false>(a, segs->n, st);
 }
 
-size_t decode_split_ws_bytes(int T, int H) { return static_cast<size_t>(kDecSplit) * T * H * sizeof(float); }
+// fp32 partial sums [kDecSplit][T][H], then one int32 arrival counter per 32-column tile
+size_t decode_split_ws_bytes(int T, int H) {
+  return static_cast<size_t>(kDecSplit) * T * H * sizeof(float) + static_cast<size_t>((H + kDecRows - 1) / kDecRows) * sizeof(int32_t);
+}
+size_t decode_split_counter_offset(int T, int H) { return static_cast<size_t>(kDecSplit) * T * H * sizeof(float); }
 int decode_split_parts(int Is) { return (Is / 64) % kDecSplit == 0 ? kDecSplit : 1; }
 
 // Shared expert, bf16, T <= 32.

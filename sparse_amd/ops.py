@@ -481,10 +481,40 @@ def moe_ffn_decode(experts: Experts, x: torch.Tensor, topv: torch.Tensor, perm: 
 
 def decode_split_workspace(T: int, H: int, device) -> torch.Tensor:
     """fp32 workspace for ``moe_ffn_decode(split_ws=...)``: the partial sums of the shared down
-    projection, ``[parts, T, H]``."""
+    projection, ``[parts, T, H]``, followed by the per-tile arrival counters of
+    ``moe_ffn_decode_combine``, which start out (and are always left) at zero."""
     lib = _lib.load()
     n = int(lib.sparse_hip_decode_split_ws_bytes(int(T), int(H)))
-    return torch.empty(n // 4, dtype=torch.float32, device=device)
+    return torch.zeros((n + 3) // 4, dtype=torch.float32, device=device)
+
+
+def moe_ffn_decode_combine(experts: Experts, x: torch.Tensor, topv: torch.Tensor, perm: Permutation, segs: SegList,
+                           inter_ws: torch.Tensor, parts: torch.Tensor, shared_w, shared_gate: Optional[torch.Tensor],
+                           shared_inter_ws: torch.Tensor, split_ws: torch.Tensor, out: torch.Tensor) -> None:
+    """``moe_ffn_decode`` with the combine step folded into the down projection's launch:
+    writes the layer's expert output ``out [T,H]`` (routed sum + shared expert)."""
+    lib = _lib.load()
+    T, H = x.shape
+    K = topv.shape[1]
+    gw, uw, dw = shared_w
+    Is = gw.shape[0]
+    _need(x, "x", torch.bfloat16)
+    _need(topv, "topv", x.dtype, (T, K))
+    _need(inter_ws, "inter_ws", x.dtype, (T * K, experts.inter))
+    _need(parts, "parts", x.dtype, (T * K, H))
+    _need(gw, "shared gate_proj", x.dtype, (Is, H))
+    _need(uw, "shared up_proj", x.dtype, (Is, H))
+    _need(dw, "shared down_proj", x.dtype, (H, Is))
+    _need(shared_inter_ws, "shared inter_ws", x.dtype, (T, Is))
+    _need(out, "out", x.dtype, (T, H))
+    _need(split_ws, "split workspace", torch.float32)
+    if split_ws.numel() * 4 < int(lib.sparse_hip_decode_split_ws_bytes(T, H)):
+        raise ValueError("split workspace is too small for this T and H")
+    rc = lib.sparse_hip_moe_ffn_decode_combine(
+        C.byref(experts), _ptr(x), _ptr(topv), _ptr(perm.perm), _ptr(perm.inv_perm), _ptr(perm.seg_offsets),
+        C.byref(segs), T, K, _ptr(inter_ws), _ptr(parts), _ptr(gw), _ptr(uw), _ptr(dw), _ptr(shared_gate), Is,
+        _ptr(shared_inter_ws), _ptr(split_ws), _ptr(out), _stream())
+    _lib.check(rc, "sparse_hip_moe_ffn_decode_combine")
 
 
 def decode_split_parts(shared_inter: int) -> int:

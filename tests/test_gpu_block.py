@@ -319,6 +319,35 @@ def test_rs_routing_with_its_own_number_of_experts_per_token(device, monkeypatch
             hid = out
 
 
+@pytest.mark.parametrize("shape_name,T", [("qwen", 1), ("qwen", 8), ("qwen", 16), ("small", 3), ("small", 16)])
+def test_combine_folded_into_the_down_projection_gives_the_same_bits(device, shape_name, T):
+    """Small all-resident decode calls combine inside the down projection's launch (the
+    workgroup that finishes a 32-column tile last sums it): bit for bit the output of the
+    separate combine launch, call after call on new inputs (the arrival counters go back to
+    zero), and every routed row is still written."""
+    from sparse_amd.synthetic import QWEN, make_hidden
+    shape = QWEN if shape_name == "qwen" else dict(family="qwen_shared", hidden=512, num_experts=12, inter=256,
+                                                     top_k=4, shared_inter=1024)
+    _mlp, blk = _build(shape, torch.bfloat16, device, seed=3)
+    H = shape["hidden"]
+    assert blk._workspace(T).split_ws is not None
+    for i in range(6):
+        x = make_hidden(T, H, torch.bfloat16, seed=4000 + i).view(T, 1, H).to(device)
+        blk.fold_combine = True
+        got, _ = blk(x)
+        parts_a = blk._workspace(T).parts.clone()
+        blk.fold_combine = False
+        want, _ = blk(x)
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), f"call {i}"
+        assert torch.equal(parts_a, blk._workspace(T).parts)
+    # the counters are back at zero
+    from sparse_amd import _lib
+    ws = blk._workspace(T)
+    off = int(_lib.load().sparse_hip_decode_split_counter_offset(T, H)) // 4
+    assert int(ws.split_ws[off:].view(torch.int32).abs().sum().item()) == 0
+
+
 @pytest.mark.parametrize("T", [1, 8, 32, 96])
 def test_decode_stack_in_a_hip_graph_replays_like_eager(device, T):
     """The decode path of a small stack captured into a HIP graph (one-launch router, fused FFN
