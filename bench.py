@@ -281,7 +281,7 @@ def offload_report(metrics, blocks, wall, n_steps, tokens_per_step, resident_ms)
     )
 
 
-def cached_decode_workload(dtype, device, steps, batch=8, capacity=15, top_m=8):
+def cached_decode_workload(dtype, device, steps, batch=8, capacity=15, top_m=8, short_steps=None, variants=None):
     """BASELINE configs[3]: Qwen shape, HBM cache of 25 % of each layer's experts, the rest in
     pinned host memory, skewed co-activating routing, rr vs rs (random-init predictor, as the
     config says, and a predictor that reproduces the next layer's router)."""
@@ -289,7 +289,13 @@ def cached_decode_workload(dtype, device, steps, batch=8, capacity=15, top_m=8):
     from sparse_amd.synthetic import QWEN, make_structured_hidden
     shape = QWEN
     n_clusters = shape["num_experts"] // 4
-    out = {"steps": steps, "batch": batch, "capacity": capacity, "experts": shape["num_experts"], "top_m": top_m}
+    # The configuration states 512 decode steps and names two methods, rr and rs with a
+    # random-init predictor: those run `steps` steps.  The other variants (predictors that
+    # reproduce the next router, EPIPE, the cost-aware policy, the staging engine) are this
+    # build's additions and run `short_steps` steps; every entry says how many it ran.
+    short_steps = steps if short_steps is None else min(steps, short_steps)
+    out = {"steps": steps, "config_steps": 512, "batch": batch, "capacity": capacity, "experts": shape["num_experts"],
+           "top_m": top_m}
 
     def inputs_for(structure):
         return [make_structured_hidden(batch, shape["hidden"], n_clusters, structure["cluster_prob"], dtype,
@@ -298,8 +304,8 @@ def cached_decode_workload(dtype, device, steps, batch=8, capacity=15, top_m=8):
     blocks, _m, structure = build_offload_stack(shape, dtype, device, "rr", capacity, top_m, offload="gpu")
     inputs = inputs_for(structure)
     run_phase_steps(blocks, inputs[:8], "decode")
-    wall = run_phase_steps(blocks, inputs, "decode")
-    resident_ms = wall / steps * 1e3
+    wall = run_phase_steps(blocks, inputs[:short_steps], "decode")
+    resident_ms = wall / short_steps * 1e3
     out["resident_eager_ms_per_step"] = resident_ms
     # cost table for the cost-aware local policy, measured on this GPU with the resident layer 0
     from sparse_amd.local_policy import CostProfile, install_lightweight_policies, measure_costs, write_profile
@@ -309,11 +315,15 @@ def cached_decode_workload(dtype, device, steps, batch=8, capacity=15, top_m=8):
     write_profile(profile_path, costs, calibrated=True, provenance="bench.py measure_costs on the running GPU")
     del blocks
     release_stack()
-    for name, method, rs_kind in (("rr", "rr", "random"), ("rs_random_init", "rs", "random"),
-                                  ("rs_informed", "rs", "informed"), ("rs-epipe_informed", "rs-epipe", "informed"),
-                                  ("rs-epipe_light_informed", "rs-epipe", "informed"),
-                                  ("rs-epipe_staged_informed", "rs-epipe", "informed")):
-        print(f"[bench] cached decode: {name}, {steps} steps", file=sys.stderr, flush=True)
+    all_variants = (("rr", "rr", "random"), ("rs_random_init", "rs", "random"),
+                    ("rs_informed", "rs", "informed"), ("rs-epipe_informed", "rs-epipe", "informed"),
+                    ("rs-epipe_light_informed", "rs-epipe", "informed"),
+                    ("rs-epipe_staged_informed", "rs-epipe", "informed"))
+    for name, method, rs_kind in all_variants:
+        if variants is not None and name not in variants:
+            continue
+        n_steps = steps if name in ("rr", "rs_random_init") else short_steps
+        print(f"[bench] cached decode: {name}, {n_steps} steps", file=sys.stderr, flush=True)
         staged = "staged" in name
         kw = dict(staging_pool_slots=4) if staged else {}
         blocks, metrics, _ = build_offload_stack(shape, dtype, device, method, capacity, top_m, rs_kind=rs_kind,
@@ -330,8 +340,10 @@ def cached_decode_workload(dtype, device, steps, batch=8, capacity=15, top_m=8):
             engine.enabled = True
             SparseContext.staging = engine
             engine.begin(name)
-        wall = run_phase_steps(blocks, inputs, "decode")   # cold cache, all steps timed
-        out[name] = offload_report(metrics, blocks, wall, steps, batch, resident_ms)
+        wall = run_phase_steps(blocks, inputs[:n_steps], "decode")   # cold cache, all steps timed
+        out[name] = offload_report(metrics, blocks, wall, n_steps, batch, resident_ms)
+        out[name]["steps"] = n_steps
+        out[name]["shortened"] = n_steps < 512
         if policies:
             out[name]["policy"] = {k: sum(p.stats[k] for p in policies)
                                    for k in ("prefetch_calls", "candidate_scores", "feedback_updates",
@@ -370,14 +382,19 @@ def epipe_prefill_workload(dtype, device, tokens=4096, chunk=2048, capacity=19, 
     out["resident_ms_per_request"] = resident_ms
     del blocks
     release_stack()
-    for method in ("rr", "rs-epipe", "sparse"):
-        print(f"[bench] chunked prefill: {method}", file=sys.stderr, flush=True)
+    # rr / rs-epipe / sparse as the configuration names them (the reference stages one missing
+    # expert per call beside the resident work), then the same with every missing expert
+    # streamed on the EPIPE lane (this build's stream-all ordering)
+    for name, method, extra_kw in (("rr", "rr", {}), ("rs-epipe", "rs-epipe", {}), ("sparse", "sparse", {}),
+                                   ("rs-epipe_stream_all", "rs-epipe", dict(epipe_stream_all=True))):
+        print(f"[bench] chunked prefill: {name}", file=sys.stderr, flush=True)
+        # rr is the plain baseline: demand copies on the compute lane, no EPIPE stage in prefill
         blocks, metrics, _ = build_offload_stack(shape, dtype, device, method, capacity, top_m, rs_kind="informed",
-                                                 epipe_prefill_enable=True)
+                                                 epipe_prefill_enable=method != "rr", **extra_kw)
         wall = run_phase_steps(blocks, inputs, "prefill")   # cold cache
         rep = offload_report(metrics, blocks, wall, 1, tokens, resident_ms)
         rep["ms_per_request"] = rep.pop("ms_per_step")
-        out[method] = rep
+        out[name] = rep
         del blocks, metrics
         release_stack()
     return out
@@ -398,11 +415,36 @@ def measured_traffic_ratio(kernel="decode_gateup"):
     return None
 
 
+def usable_cores():
+    """Host cores this process may use: the scheduler affinity, cut down by the cgroup's CPU
+    quota and by the thread share the machine's operator exports (OMP_NUM_THREADS) where
+    those are set.  Returns (count, how it was derived)."""
+    total = os.cpu_count() or 1
+    try:
+        n = len(os.sched_getaffinity(0))
+    except (AttributeError, OSError):
+        n = total
+    note = [f"os.cpu_count()={total}", f"affinity={n}"]
+    try:
+        quota, period = open("/sys/fs/cgroup/cpu.max").read().split()[:2]
+        if quota != "max":
+            q = max(1, int(int(quota) / int(period)))
+            note.append(f"cgroup quota={q}")
+            n = min(n, q)
+    except (OSError, ValueError):
+        pass
+    env = os.environ.get("OMP_NUM_THREADS", "").strip()
+    if env.isdigit() and int(env) > 0:
+        note.append(f"OMP_NUM_THREADS={env}")
+        n = min(n, int(env))
+    return max(1, n), ", ".join(note)
+
+
 def cpu_baseline(shape, batch, dtype, device, budget_s=12.0):
     """The CPU oracle of one layer of the same workload on this box's host cores."""
     from oracle import ref_moe
     from sparse_amd.synthetic import make_hidden, make_mlp_block
-    cores = min(16, os.cpu_count() or 1)
+    cores, core_note = usable_cores()
     torch.set_num_threads(cores)
     mlp = make_mlp_block(shape, dtype=dtype, seed=0, device=device, fused=True)
     gu, dn = mlp.experts.gate_up_proj.cpu(), mlp.experts.down_proj.cpu()
@@ -430,7 +472,7 @@ def cpu_baseline(shape, batch, dtype, device, budget_s=12.0):
     torch.set_num_threads(cores)
     layers = shape["num_layers"]
     return dict(value=batch / (dt / n * layers), unit="tokens/s", cores=cores, kind="port",
-                value_1_thread=batch / (dt1 / n1 * layers),
+                value_1_thread=batch / (dt1 / n1 * layers), host_cpu_count=os.cpu_count(), cores_note=core_note,
                 sample=f"{n} decode layer-calls (batch {batch}, 1 of {layers} layers, bf16) of the CPU oracle in "
                        f"{dt:.1f} s on {cores} threads, and {n1} in {dt1:.1f} s on 1 thread, each scaled linearly "
                        f"to {layers} layers")
@@ -496,9 +538,10 @@ def main():
         extra["prefill_4k_deepseek"] = prefill_workload(DEEPSEEK, 4096, max(2, min(10, args.steps // 10)), 1, dtype,
                                                         device)
     if not args.no_extra:
-        # the offloaded configurations, shortened (64 decode steps from a cold cache); a failure
+        # the offloaded configurations: rr and rs as the configuration states them (512 decode steps
+        # from a cold cache), this build's other variants at 64 steps and labelled so; a failure
         # here (e.g. no pinned memory to be had) must not cost the main line
-        for name, leg in (("cached_decode_qwen", lambda: cached_decode_workload(dtype, device, 64)),
+        for name, leg in (("cached_decode_qwen", lambda: cached_decode_workload(dtype, device, 512, short_steps=64)),
                           ("epipe_prefill_deepseek", lambda: epipe_prefill_workload(dtype, device))):
             try:
                 extra[name] = leg()
@@ -532,9 +575,13 @@ def main():
         "roofline": {
             "bound": "hbm", "achieved": gu["gbps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
             "frac": gu["gbps"] / HBM_PEAK_GBPS,
-            # counter-measured HBM bytes per launch: the ratio recorded in profiles/ (FETCH_SIZE +
-            # WRITE_SIZE runs scaled by a plain copy) applied to this run's algorithmic bytes
+            # HBM bytes per launch: NOT measured in this run (counters need the profiler); the ratio
+            # recorded in profiles/ (FETCH_SIZE + WRITE_SIZE runs scaled by a plain copy) applied to
+            # this run's algorithmic bytes
             "traffic": (gu["bytes_per_launch"] * ratio) if ratio else None,
+            "traffic_source": ("recorded: profiles/decode_b8_qwen_hbm_traffic.txt (rocprofv3 --pmc FETCH_SIZE / "
+                               "WRITE_SIZE, scaled by a plain copy kernel) x this run's algorithmic bytes"
+                               if ratio else None),
             "traffic_over_algorithmic": ratio, "kernel": gu["kernel"],
             "bytes_per_launch": gu["bytes_per_launch"], "avg_launch_us": gu["avg_us"], "launches": gu["launches"],
             "mean_distinct_experts": main_res["mean_distinct_experts"],

@@ -114,6 +114,7 @@ class RefConfig:
         self.epipe_prefill_lookahead_min_ready_items = 256
         self.epipe_decode_rs_commit = True
         self.epipe_decode_no_rs_commit = True
+        self.epipe_stream_all = False                 # this build's addition, see RefLayer.execute
         for k, v in kw.items():
             if not hasattr(self, k):
                 raise ValueError(f"unknown option {k}")
@@ -134,6 +135,7 @@ class RefLayer:
         self.extra = RefEpipePrefillExtraCache(cfg.epipe_prefill_extra_cache_slots)
         self.expert_bytes = 0                    # size of one expert for the side cache's byte guard
         self.copy_done = copy_done or (lambda eid: True)
+        self.miss_lane = "compute"
         self.prefetched: Set[int] = set()        # _prefetched_ids_this_group
         self.used: Set[int] = set()              # _prefetch_used_ids_this_group
         self.events: Dict[int, int] = {}         # _prefetch_events: eid -> token
@@ -217,9 +219,11 @@ class RefLayer:
         if self.extra_get(eid):
             return
         self.trace.append(("miss", eid))
-        self.trace.append(("h2d", "compute", eid))
+        self.trace.append(("h2d", self.miss_lane, eid))
         self.on_demand_access(eid)
         self.cache_put_guarded(eid)
+        if self.miss_lane != "compute":     # stream-all EPIPE (not in the reference): the compute lane waits this copy
+            self.trace.append(("wait", eid))
 
     # ---- prefill side cache (:5637-5720) -----------------------------------------------
     def extra_enabled(self) -> bool:
@@ -278,8 +282,19 @@ class RefLayer:
         if not segments:
             return "empty"
         c = self.cfg
+        epipe = self.epipe_stage_enabled() and c.epipe_mode != "off"
+        # stream-all EPIPE, an addition of this build: every miss inside an EPIPE call is copied
+        # on the EPIPE lane and awaited by the compute lane; events and cache state are unchanged
+        self.miss_lane = "epipe" if (epipe and getattr(c, "epipe_stream_all", False)) else "compute"
+        try:
+            return self._execute(segments, epipe)
+        finally:
+            self.miss_lane = "compute"
+
+    def _execute(self, segments: Sequence[Segment], epipe: bool) -> str:
+        c = self.cfg
         result = None
-        if self.epipe_stage_enabled() and c.epipe_mode != "off":
+        if epipe:
             rs_active = c.planner_mode == "rs_prefetch"
             if self.stage == "decode" and rs_active and c.epipe_decode_rs_mode == "off":
                 result = None

@@ -93,6 +93,12 @@ class ResidencyConfig:
     epipe_no_evict: bool = True
     epipe_transient_staging: bool = True
     epipe_max_staged_experts: int = 1
+    # Not in the reference, which copies exactly one missing expert per call beside the resident
+    # work and the others on the compute lane: with this on, every expert an EPIPE executor finds
+    # missing is copied on the EPIPE lane, back to back, and its segment runs behind its own
+    # event, after the resident segments.  Cache events, eviction order and final contents are
+    # those of the one-staged-expert executors; only lanes and waits change.
+    epipe_stream_all: bool = False
     epipe_min_ready_experts: int = 1
     epipe_min_ready_items: int = 1
     epipe_min_missing_experts: int = 1
@@ -161,6 +167,7 @@ class ResidencyConfig:
         c.epipe_no_evict = _env_flag("SPARSE_EPIPE_NO_EVICT", "1")
         c.epipe_transient_staging = _env_flag("SPARSE_EPIPE_TRANSIENT_STAGING", "1")
         c.epipe_max_staged_experts = _env_int("SPARSE_EPIPE_MAX_STAGED_EXPERTS", 1)
+        c.epipe_stream_all = _env_flag("SPARSE_HIP_EPIPE_STREAM_ALL", "0")
         c.epipe_sort_ready_by_work = _env_flag("SPARSE_EPIPE_SORT_READY_BY_WORK", "0")
         # the prefill policy sets the defaults of commit and transient mark (reference :5007-5016)
         policy = str(os.environ.get("SPARSE_EPIPE_PREFILL_POLICY", "deferred_lru_commit")
@@ -273,6 +280,8 @@ class LayerResidency:
         self._slot_fence: Dict[int, Any] = {}    # compute-lane event after the last read
         self._slot_upload: Dict[int, Tuple[Any, str]] = {}  # last upload (event, lane)
         self._slot_of: Dict[int, int] = {}       # resident expert -> slot (mirrors the cache)
+        self._miss_lane = "compute"              # where a demand miss is copied ("epipe": stream-all EPIPE)
+        self._slot_ready: Dict[int, Any] = {}    # slot -> event of a side-lane demand copy nobody has waited yet
         # prefetch cycle state (reference :5056-5083)
         self.prefetched_ids: Set[int] = set()
         self.prefetch_used_ids: Set[int] = set()
@@ -331,6 +340,12 @@ class LayerResidency:
         return ev
 
     def _enqueue(self, eid: int, slot: int) -> None:
+        ready = self._slot_ready.pop(int(slot), None)
+        if ready is not None:
+            # weights still travelling on a side lane: what is queued goes first, then the
+            # compute lane waits this copy and this segment opens the next batch
+            self.flush()
+            self.backend.wait_event(ready, "compute")
         self._pending.append((int(eid), int(slot)))
         self._pending_slots.add(int(slot))
 
@@ -449,7 +464,13 @@ class LayerResidency:
             return extra
         self._event("miss", eid)
         slot = self._acquire_slot()
-        self._upload(eid, slot, "compute")
+        if self._miss_lane == "compute":
+            self._upload(eid, slot, "compute")
+        else:
+            # stream-all EPIPE: the copy travels on the side lane; the segment is launched behind
+            # its event (see _enqueue), whatever was queued before it runs meanwhile
+            self._slot_ready[slot] = self._upload(eid, slot, self._miss_lane)
+            self.metrics.bump("epipe_stream_all_copies")
         self.metrics.demand_h2d_bytes += self.expert_bytes
         self._on_demand_access(eid)
         self._cache_put(eid, slot)
@@ -510,7 +531,17 @@ class LayerResidency:
         if not segments:
             return "empty"
         name = None
-        if self._epipe_stage_enabled() and self.cfg.epipe_mode != "off" and not self.cfg.world1_exact:
+        epipe = self._epipe_stage_enabled() and self.cfg.epipe_mode != "off" and not self.cfg.world1_exact
+        self._miss_lane = "epipe" if (epipe and self.cfg.epipe_stream_all) else "compute"
+        try:
+            name = self._execute(segments, epipe)
+        finally:
+            self._miss_lane = "compute"
+        return name
+
+    def _execute(self, segments: Sequence[Segment], epipe: bool) -> str:
+        name = None
+        if epipe:
             rs_active = self.cfg.planner_mode == "rs_prefetch"
             mode = self.cfg.epipe_decode_rs_mode
             if self.stage == "decode" and rs_active and mode == "off":

@@ -139,6 +139,10 @@ def _replay_oracle(record, cfg, capacity, shape=None, expert_bytes=0):
     ("epipe", dict(epipe_mode="miss_triggered", epipe_lookahead_min_ready_items=1), False),
     ("epipe", dict(epipe_mode="miss_triggered", epipe_prefill_enable=True, epipe_lookahead_min_ready_items=1,
                    epipe_prefill_lookahead_min_ready_items=1), True),
+    # stream-all EPIPE: every missing expert of an EPIPE call travels on the EPIPE lane
+    ("epipe", dict(epipe_stream_all=True), False),
+    ("rs-epipe", dict(epipe_stream_all=True), False),
+    ("epipe", dict(epipe_stream_all=True, epipe_prefill_enable=True), True),
 ])
 def test_offloaded_methods_match_resident_values_and_oracle_events(device, method, overrides, prefill_first):
     from sparse_amd.methods import residency_config
@@ -203,6 +207,8 @@ def _check_against_oracle(blocks, metrics, record, cfg, capacity, shape):
     # ten slots, of which the default 128 MB byte bound lets seven 17.3 MB experts in
     ("rs-epipe", dict(epipe_prefill_extra_cache_slots=10, epipe_prefill_commit=False)),
     ("epipe", dict(epipe_prefill_extra_cache_slots=4, epipe_prefill_extra_cache_max_mb=0.0)),
+    # resident experts run while ALL the missing ones stream in on the EPIPE lane
+    ("rs-epipe", dict(epipe_stream_all=True)),
 ])
 def test_chunked_epipe_prefill_at_the_deepseek_shape(device, method, overrides):
     """Readiness-aware chunked prefill as the benchmark configuration states it, on two layers:
@@ -235,6 +241,9 @@ def test_chunked_epipe_prefill_at_the_deepseek_shape(device, method, overrides):
     assert metrics.cache_miss_count >= n_calls * 2 * (shape["num_experts"] - capacity) * 0.8
     if method != "rr":
         assert any(n.startswith("epipe") for n in executors)
+    if overrides.get("epipe_stream_all"):
+        # every miss of the calls that found resident experts went over the EPIPE lane
+        assert metrics.counters.get("epipe_stream_all_copies", 0) >= (shape["num_experts"] - capacity) * 2 * 0.8
     if overrides.get("epipe_prefill_extra_cache_slots"):
         kept = [len(lay.extra.resident_ids()) for lay in lays]
         assert sum(kept) > 0, "nothing was ever parked in the prefill side cache"

@@ -372,6 +372,13 @@ METHOD_CASES = [
                    overrides=dict(epipe_mode="miss_triggered", epipe_prefill_enable=True, epipe_prefill_commit=False,
                                   epipe_prefill_extra_cache_slots=2, epipe_prefill_lookahead_min_ready_items=1,
                                   epipe_lookahead_min_ready_items=1))),
+    # stream-all EPIPE (this build's addition): every miss of an EPIPE call on the EPIPE lane
+    ("epipe", dict(overrides=dict(epipe_stream_all=True))),
+    ("rs-epipe", dict(late_rate=0.3, overrides=dict(epipe_stream_all=True))),
+    ("sparse", dict(capacity=15, E=60, K=4, T=8, top_m=8, overrides=dict(epipe_stream_all=True))),
+    ("epipe", dict(prefill_steps=4, capacity=6, T=8, overrides=dict(epipe_stream_all=True, epipe_prefill_enable=True))),
+    ("epipe", dict(capacity=6, T=8, overrides=dict(epipe_stream_all=True, epipe_mode="miss_triggered",
+                                                   epipe_lookahead_min_ready_items=1))),
 ]
 
 
@@ -389,6 +396,56 @@ def test_product_reproduces_the_oracle_event_for_event(method, kw):
             assert g["residents"] == w["residents"], f"layer {l}: final LRU order differs"
     if method in ("epipe", "rs-epipe", "sparse"):
         assert any(e.startswith("epipe") for e in ex_o), "EPIPE never triggered in this trace"
+
+
+@pytest.mark.parametrize("method,kw", [
+    ("epipe", {}), ("rs-epipe", dict(late_rate=0.3)), ("sparse", dict(capacity=15, E=60, K=4, T=8, top_m=8)),
+    ("epipe", dict(prefill_steps=4, capacity=6, T=8, overrides=dict(epipe_prefill_enable=True))),
+])
+def test_stream_all_changes_lanes_and_waits_only(method, kw):
+    """Stream-all EPIPE against the reference's one-staged-expert executors on the same trace:
+    the same cache events in the same order, the same execution order, the same final LRU
+    order and executor per call; every copy that was a demand copy on the compute lane inside
+    an EPIPE call now travels on the EPIPE lane and is awaited exactly once; nothing else moves."""
+    kw = dict(kw)
+    over = dict(kw.pop("overrides", {}))
+    for which in ("oracle", "product"):
+        base, ex_b = run_trace(method, which, seed=5, overrides=over, **kw)
+        strm, ex_s = run_trace(method, which, seed=5, overrides=dict(over, epipe_stream_all=True), **kw)
+        assert ex_b == ex_s
+        moved = 0
+        for b, s_ in zip(base, strm):
+            assert s_["events"] == b["events"] and s_["compute"] == b["compute"] and s_["residents"] == b["residents"]
+            assert [(e) for _h, _lane, e in s_["h2d"]] == [(e) for _h, _lane, e in b["h2d"]]     # same copies, same order
+            for (_h, lane_b, e), (_h2, lane_s, _e) in zip(b["h2d"], s_["h2d"]):
+                assert lane_s == lane_b or (lane_b == "compute" and lane_s == "epipe")
+                moved += lane_s != lane_b
+            assert len(s_["waits"]) == len(b["waits"]) + sum(
+                1 for (_h, lb, _e), (_h2, ls, _e2) in zip(b["h2d"], s_["h2d"]) if lb != ls)
+        assert moved > 0, "no copy ever moved to the EPIPE lane"
+
+
+def test_stream_all_runs_resident_segments_before_it_waits(which="product"):
+    """In the product's device trace of a stream-all call the resident segments are launched
+    before the compute lane waits for the first streamed copy, and every streamed segment is
+    launched after its own wait."""
+    cfg = residency_config("epipe", 4, 2, epipe_stream_all=True)
+    lay, be, m = product_layer(cfg)
+    lay.phase, lay.call_id, lay.stage = "decode", 0, "decode"
+    lay.execute([(1, 2), (3, 1)])                        # cold: plain path, still streamed? (no EPIPE trigger)
+    be.trace.clear()
+    lay.call_id = 1
+    name = lay.execute([(1, 1), (2, 2), (3, 1), (5, 1), (7, 3)])
+    assert name == "epipe_upfront"
+    t = be.trace
+    first_wait = min(i for i, x in enumerate(t) if x[0] == "wait")
+    for eid in (1, 3):
+        assert t.index(("compute", eid)) < first_wait
+    for eid in (2, 5, 7):
+        assert ("h2d", "epipe", eid) in t
+        assert t.index(("h2d", "epipe", eid)) < t.index(("wait", eid)) < t.index(("compute", eid))
+    # all three copies are enqueued before the second streamed segment runs (they are back to back on their lane)
+    assert t.index(("h2d", "epipe", 5)) < t.index(("compute", 5))
 
 
 def test_transient_mark_of_prefill_commits_changes_later_evictions():
