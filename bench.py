@@ -337,8 +337,7 @@ def cached_decode_workload(dtype, device, steps, batch=8, capacity=15, top_m=8, 
             from sparse_amd.staging import BoundedRS
             engine = BoundedRS(slots=4)
             engine.prepare({b.layer_idx: b for b in blocks}, SparseContext.rs_bank, batch=batch, dtype=dtype)
-            engine.enabled = True
-            SparseContext.staging = engine
+            engine.install()
             engine.begin(name)
         wall = run_phase_steps(blocks, inputs[:n_steps], "decode")   # cold cache, all steps timed
         out[name] = offload_report(metrics, blocks, wall, n_steps, batch, resident_ms)
@@ -350,6 +349,7 @@ def cached_decode_workload(dtype, device, steps, batch=8, capacity=15, top_m=8, 
                                              "residual_calls")}
         if engine is not None:
             st = engine.finish()
+            engine.restore()
             engine.shutdown()
             out[name]["staging"] = {k: st[k] for k in ("predictions", "issued", "used", "wasted", "retained",
                                                         "skipped_slots", "closed_before_publish")}

@@ -561,10 +561,10 @@ class DistributedSparseMoeBlock(nn.Module):
         staging = SparseContext.staging
         staged = (staging is not None and self.residency is not None and staging.handles(self, S))
         if staged:
-            # bounded staging engine: the prediction for layer l+1 leaves on a side stream and
-            # is never joined; this layer's own staged copies are exposed at the executor
+            # forecast staging: the prediction for layer l+1 leaves on a side stream and is never
+            # joined; this layer's own ring window is sealed at the executor
             self.residency.staging = staging
-            staging.predict(self, x, int(SparseContext.runtime_call_id))
+            staging.forecast_next(self, x, int(SparseContext.runtime_call_id))
             rs_job = None
         else:
             if self.residency is not None:
@@ -636,12 +636,12 @@ class DistributedSparseMoeBlock(nn.Module):
             res.stage = self._current_stage(S)
             self._backend.bind(x, ws)
             if staged:
-                staging.activate_at_demand(self, int(SparseContext.runtime_call_id))
+                staging.seal(self, int(SparseContext.runtime_call_id))
             try:
                 self.last_executor = res.execute(segments)
             finally:
                 if staged:
-                    staging.release(self)
+                    staging.settle(self)
         if self.residency is None and rs_job is not None:
             torch.cuda.current_stream().synchronize()
             self._rs_finish(rs_job, ws)

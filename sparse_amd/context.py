@@ -80,7 +80,7 @@ class SparseContext:
     rs_bank_source_layers: List[int] = []
     routing_cache: Dict[int, Tuple[torch.Tensor, torch.Tensor]] = {}
     prefill_scp_transient_demoted_for_decode: bool = False
-    staging: Optional[Any] = None          # bounded RS staging engine (sparse_amd.staging.BoundedRS)
+    staging: Optional[Any] = None          # forecast staging engine (sparse_amd.staging.BoundedRS) while installed
 
     @classmethod
     def register_layer_block(cls, layer_idx: int, block: Any) -> None:

@@ -22,6 +22,7 @@ from typing import Any, Callable, Dict, List, Optional, Sequence, Set, Tuple
 
 from .cache import TieredExpertWeightCache, tiered_capacity_split, EpipePrefillExtraCache, ExpertWeightCache
 from .context import Metrics
+from .ring import StagingRing
 
 Segment = Tuple[int, int]  # (expert id, routed rows)
 
@@ -209,6 +210,19 @@ class ResidencyConfig:
         return c
 
 
+@dataclass
+class StagedExpert:
+    """An expert readable from a slot of the staging ring during one layer call."""
+
+    pos: int                  # ring position that lent the slot
+    slot: int
+    event: Any                # recorded behind the copy
+    touched: bool = False     # a lookup used it
+    kept: bool = False        # the LRU took it, and its slot, at the call's end
+    recycled: bool = False    # ... and the ring got the slot of the resident it pushed out
+    ring_slot: Optional[int] = None   # what the ring position holds afterwards, when kept
+
+
 class Backend:
     """Device services the policy needs.  Lanes: ``compute`` (the stream the layer's
     kernels run on), ``prefetch`` and ``epipe`` (side streams for uploads)."""
@@ -268,11 +282,16 @@ class LayerResidency:
         self.extra_cache = EpipePrefillExtraCache(int(config.epipe_prefill_extra_cache_slots))
         self.num_slots = max(0, total_capacity) + max(1, int(config.staging_slots)) + \
             max(0, int(config.epipe_prefill_extra_cache_slots))
-        # slots of the bounded RS staging pool sit after the ordinary ones and never enter the free list
-        self._pool_slots: List[int] = list(range(self.num_slots, self.num_slots + max(0, int(config.staging_pool_slots))))
         self._free_slots: List[int] = list(range(self.num_slots - 1, -1, -1))
-        self.num_slots += len(self._pool_slots)
-        self.staging: Any = None   # the BoundedRS engine while a request runs with it enabled
+        # the staging ring's slots sit after the ordinary ones and never enter the free list
+        ring_slots = max(0, int(config.staging_pool_slots))
+        self.ring: Optional[StagingRing] = \
+            StagingRing(range(self.num_slots, self.num_slots + ring_slots)) if ring_slots else None
+        self.num_slots += ring_slots
+        self.staged: Dict[int, StagedExpert] = {}   # experts readable from ring slots during this call
+        self.staged_touched: List[int] = []         # those a lookup really used, in first-use order
+        self.staged_unconfirmed = 0                 # unused copies whose completion nobody has counted yet
+        self.staging: Any = None   # the forecast engine (sparse_amd.staging) while it serves this layer's calls
         self.light_policy: Optional[Any] = None     # sparse_amd.local_policy.LocalPolicy, when installed
         self._retired: List[int] = []           # evicted, still read by the pending batch
         self._pending: List[Tuple[int, int]] = []  # (eid, slot) not launched yet
@@ -308,7 +327,7 @@ class LayerResidency:
         else:
             m.cache_miss_count += 1
             if self.staging is not None and self.stage == "decode":
-                self.staging.note_demand_miss(self)
+                self.staging.demand_miss(self.layer_idx)
         if m.events is not None:
             m.events.append((kind, self.layer_idx, int(eid)))
 
@@ -455,7 +474,7 @@ class LayerResidency:
 
     def _demand(self, eid: int) -> int:
         """``_get_local_module_weights`` (reference :11388-11435): returns the slot."""
-        slot = self.cache.get(eid)
+        slot = self.find(eid)
         if slot is not None:
             self._record_cached_use(eid, wait_prefetch=True)
             return slot
@@ -550,7 +569,7 @@ class LayerResidency:
                 if self.staging is not None:
                     # staged experts are classified like cached ones by the upfront scan
                     # (utils/rs_overlap.py:474-479)
-                    self.staging.stats["unified_epipe_calls"] += 1
+                    self.staging.count("unified_epipe_calls")
                     name = self._epipe_upfront_scan(segments)
                 else:
                     name = self._epipe_rs_residual_scan(segments)
@@ -581,7 +600,7 @@ class LayerResidency:
 
     def _contains_no_touch(self, eid: int) -> bool:
         """Reference :5815-5851."""
-        return (self._extra_readable() and self.extra_cache.has(eid)) or self.cache.has(eid)
+        return (self._extra_readable() and self.extra_cache.has(eid)) or self.holds(eid)
 
     def _headroom_ok(self) -> bool:
         """A transient needs a slot that no cache entry owns."""
@@ -1044,14 +1063,104 @@ class LayerResidency:
         return "epipe_miss_triggered"
 
     # ------------------------------------------------------------------ RS prefetch
-    # ---- bounded RS staging (utils/rs_overlap.py) -------------------------------------
-    def claim_staging_pool(self, n: int) -> List[int]:
-        """Slot ids reserved for the staging engine (``staging_pool_slots`` of the config)."""
-        if n > len(self._pool_slots):
+    # ---- staged experts: a third state of the slot table ---------------------------------
+    # Besides *resident* (the LRU owns the slot) and *transient* (the slot lives for one batch)
+    # an expert can be *staged*: a forecast copied it into a slot of the layer's ring, this
+    # call's lookups may read it there, and the LRU learns of it only at the call's end and
+    # only if a lookup really used it.  A wrong forecast therefore never evicts and never
+    # moves recency (the ownership rule of utils/rs_staging.py:52-94).
+    @property
+    def _pool_slots(self) -> List[int]:
+        return self.ring.slots if self.ring is not None else []
+
+    def staging_ring(self, positions: int) -> StagingRing:
+        """The layer's ring, which must have at least ``positions`` slots."""
+        have = len(self.ring) if self.ring is not None else 0
+        if positions > have:
             raise ValueError(
-                f"layer {self.layer_idx}: {n} staging pool slots asked, {len(self._pool_slots)} reserved "
+                f"layer {self.layer_idx}: {positions} staging slots asked, {have} reserved "
                 "(set ResidencyConfig.staging_pool_slots before the block is built)")
-        return list(self._pool_slots[:n])
+        return self.ring
+
+    def find(self, eid: int, touch: bool = True) -> Optional[int]:
+        """Slot that holds ``eid`` for this call, or None.  A resident copy wins over a staged
+        one; ``touch`` moves the LRU's recency for the former and records first use of the
+        latter."""
+        slot = self.cache.get(eid) if touch else self.cache.peek(eid)
+        if slot is not None:
+            return slot
+        rec = self.staged.get(int(eid))
+        if rec is None:
+            return None
+        if touch and not rec.touched:
+            rec.touched = True
+            self.staged_touched.append(int(eid))
+        return rec.slot
+
+    def holds(self, eid: int) -> bool:
+        return bool(self.cache.has(eid)) or int(eid) in self.staged
+
+    def expose_staged(self, filled: Sequence[Tuple[int, int, Any]]) -> None:
+        """Make the copies of a sealed ring window readable: ``(expert, ring position, copy
+        event)``.  They count as issued prefetches; the compute lane waits a copy's event on
+        first use like that of any prefetch (utils/rs_overlap.py:326-340)."""
+        assert not self.staged and not self.staged_touched, "the last call's staged experts were not settled"
+        for eid, pos, event in filled:
+            self.staged[int(eid)] = StagedExpert(pos, self.ring.slots[pos], event)
+            self.prefetched_ids.add(int(eid))
+            self.prefetch_events[int(eid)] = event
+            self.metrics.prefetch_h2d_bytes += self.expert_bytes
+            self.metrics.prefetch_issued_count += 1
+            self.metrics.prefetch_admitted_count += 1
+
+    def _keep_staged(self, eid: int, rec: StagedExpert) -> None:
+        """Admit a staged expert that was used to the LRU where its bytes are: its slot becomes
+        the cache's; the ring gets the slot of the resident it pushed out, or a free one while
+        the cache is not full (utils/rs_overlap.py:352-381 exchanges payload objects)."""
+        if self.cache.capacity <= 0:
+            return
+        self._on_demand_access(eid)
+        self.cache.put(int(eid), rec.slot, pinned=False, protect_ids=self._protect_with_fallback(eid))
+        if not self.cache.has(eid):
+            return
+        self._slot_of[int(eid)] = rec.slot
+        self._slot_upload[rec.slot] = (rec.event, "staging")
+        pushed_out = [e for e in self._slot_of if not self.cache.has(e)]
+        assert len(pushed_out) <= 1, "staging needs the plain per-layer LRU"
+        if pushed_out:
+            self.prefetch_events.pop(pushed_out[0], None)
+            rec.ring_slot, rec.recycled = self._slot_of.pop(pushed_out[0]), True
+        else:
+            rec.ring_slot = self._acquire_slot()
+        rec.kept = True
+
+    def settle_staged(self) -> List[Tuple[int, StagedExpert]]:
+        """End of the layer call: keep what was used (first-use order), give every ring position
+        back -- a used one behind a fence on the compute lane, an unused one behind its own
+        copy -- and forget the staged state (utils/rs_overlap.py:383-408).  Returns the settled
+        records, used ones first."""
+        if not self.staged:
+            return []
+        fence = self.backend.fence() if self.staged_touched else None   # after every reader of this call
+        for eid in self.staged_touched:
+            self._keep_staged(eid, self.staged[eid])
+        order = self.staged_touched + [e for e in self.staged if not self.staged[e].touched]
+        settled = [(e, self.staged[e]) for e in order]
+        for eid, rec in settled:
+            self.ring.give_back(rec.pos, fence if rec.touched else rec.event, rec.ring_slot if rec.kept else None)
+            if not rec.touched:
+                self.metrics.prefetch_wasted_count += 1
+                self.staged_unconfirmed += 1
+            self.prefetch_events.pop(eid, None)
+            self.prefetched_ids.discard(eid)
+            self.prefetch_used_ids.discard(eid)
+        self.staged, self.staged_touched = {}, []
+        return settled
+
+    def confirm_staged_copies(self) -> None:
+        """After the copy lane has drained: the unused copies have completed too."""
+        self.metrics.prefetch_completed_count += self.staged_unconfirmed
+        self.staged_unconfirmed = 0
 
     def min_candidate_score(self) -> float:
         """``_prefetch_min_candidate_score`` with the cache-safe floor (reference :4954-4972)."""
@@ -1059,32 +1168,6 @@ class LayerResidency:
         if self.cfg.rs_policy in ("cache_safe", "cache-safe", "benefit_gate", "benefit-gate"):
             score = max(score, float(self.cfg.cache_safe_min_score))
         return score
-
-    def adopt_staged(self, eid: int, slot: int, event: Any) -> Tuple[Optional[int], bool]:
-        """Admit a staged expert that this call really used into the LRU, keeping its bytes
-        where they are: ``slot`` becomes the cache's, and the slot handed back -- the evicted
-        resident's (``recycled``) or a free one -- becomes the pool's
-        (``_retain_used``, utils/rs_overlap.py:352-381).  ``(None, False)`` if the cache did
-        not take the expert."""
-        resident = getattr(self.cache, "resident", self.cache)
-        if resident.capacity <= 0:
-            return None, False
-        self._on_demand_access(eid)
-        protect = self._protect_with_fallback(eid)
-        resident.put(int(eid), int(slot), pinned=False, protect_ids=protect)
-        if not resident.has(eid):
-            return None, False
-        self._slot_of[int(eid)] = int(slot)
-        self._slot_upload[int(slot)] = (event, "staging")
-        evicted = [e for e in self._slot_of if not resident.has(e)]
-        assert len(evicted) <= 1, "Only a layer-local plain LRU is supported"
-        if evicted:
-            self.prefetch_events.pop(evicted[0], None)
-            replacement, recycled = self._slot_of.pop(evicted[0]), True
-        else:
-            replacement, recycled = self._acquire_slot(), False
-        self._pool_slots[self._pool_slots.index(int(slot))] = replacement
-        return replacement, recycled
 
     def effective_top_m(self) -> int:
         return max(0, int(self.cfg.prefetch_top_m))
@@ -1312,6 +1395,6 @@ class LayerResidency:
         self.cache.clear()
         self.extra_cache.clear()
         self._slot_of.clear()
-        pool = set(self._pool_slots)
-        self._free_slots = [s for s in range(self.num_slots - 1, -1, -1) if s not in pool]
+        ring = set(self._pool_slots)
+        self._free_slots = [s for s in range(self.num_slots - 1, -1, -1) if s not in ring]
         self._retired = []

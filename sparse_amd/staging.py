@@ -1,522 +1,423 @@
-"""Bounded next-layer RS staging: the opt-in alternative to the in-line prefetch planner.
+"""Forecast staging for decode: while layer l computes, a predictor names the experts layer
+l+1 will probably route to, and their weights are copied into l+1's staging ring before l+1
+asks for them -- without ever touching l+1's resident cache on a guess.
 
-Mirrors the reference's ownership rules (utils/rs_staging.py:12-118) and pipeline
-(utils/rs_overlap.py:58-497) on this build's slot model:
+This is the build's counterpart of the reference's bounded staging adapter
+(utils/rs_overlap.py:58-433, ownership rules utils/rs_staging.py:12-118); the harness-facing
+surface keeps its names (``BoundedRS``: ``configure``, ``prepare``, ``begin``, ``finish``,
+``install``, ``restore``, ``enabled``; ``select_candidates``), the machinery is this build's:
 
-  * speculation never writes the resident LRU; a staged expert sits in a slot of the
-    target layer's *staging pool* and is visible to demand lookups through
-    ``DemandCacheView`` only;
-  * the predictor's top-k is captured in a graph on a side stream, read back
-    asynchronously into pinned memory, and scored by one worker thread, which publishes
-    copies under the target's lock; the target closes publication when its executor starts
-    (``activate_at_demand``) -- a prediction is never joined;
-  * at the target layer's exit (``release``) the experts that were actually used are
-    admitted to the LRU in first-use order by exchanging slot ownership, not bytes: the
-    evicted resident's slot becomes the pool's next scratch slot.
+  * a staged expert is a state of the target layer's slot table
+    (``LayerResidency.staged`` / ``find`` / ``holds``), not a cache wrapper: the layer's
+    lookups read ring slots directly, and ``settle_staged`` hands a used expert to the LRU
+    by exchanging slot indices with the ring;
+  * publication goes through ``StagingRing`` (sparse_amd/ring.py): ``open`` at the source
+    layer, ``publish`` from the scoring thread, ``seal`` at the target's executor, all under
+    the ring's lock, so a forecast is never joined -- late copies are simply declined;
+  * candidates are scored by ``LayerResidency.score_map``, the in-line planner's own
+    aggregate, after the entries that need no copy are filtered out;
+  * the forecast itself -- predictor, top-k, renormalisation, rounding -- is
+    ``rs.topk_for_planning`` captured once per source layer in a HIP graph, so both planners
+    see the same candidates for the same hidden state.
 
-Where the reference's pool is four free-standing payloads shared by all layers, a payload
-here is a slot index of the target layer's own HBM slab (a kernel addresses weights as
-slab base + slot * stride), so every offloaded layer carries ``pool_slots`` extra slots
-(``ResidencyConfig.staging_pool_slots``).  The engine is wired into the block through
-``SparseContext.staging`` instead of patching methods at run time
-(utils/rs_overlap.py:434-486 lists the seven patch points; the hooks sit at the same
-places).
+One engine serves a whole stack.  Timeline of a decode step at layer l:
+``forecast_next`` (graph launch on the forecast stream, asynchronous read-back into pinned
+memory, scoring task queued; nothing waits) -> router, permutation -> ``seal`` (l's own ring
+window ends, its copies become readable) -> executor -> ``settle`` (admission, ring slots
+returned behind fences).
 """
 from __future__ import annotations
 
 import threading
-import time
 from concurrent.futures import ThreadPoolExecutor
-from dataclasses import dataclass
-from typing import Any, Callable, Dict, Iterable, List, Optional
+from contextlib import contextmanager
+from time import perf_counter
+from typing import Any, Dict, Iterable, List, Optional
 
+import torch
 
-# --------------------------------------------------------------------------- ownership rules
-@dataclass
-class Transfer:
-    """One issued copy (utils/rs_staging.py:12-20)."""
-
-    expert: int
-    payload: Any
-    event: Any
-    slot: Any
-    nbytes: int
-    used: bool = False
-    retained: bool = False
-
-
-class TargetJob:
-    """Copies predicted for one (epoch, step, target layer) (utils/rs_staging.py:23-49)."""
-
-    def __init__(self, ticket, slots) -> None:
-        self.ticket = ticket
-        self.slots = slots
-        self.transfers: Dict[int, Transfer] = {}
-        self.closed = False
-        self.lock = threading.Lock()
-        self.future = None
-        self.plan_count: Optional[int] = None
-
-    def publish(self, expert: int, submit: Callable[[], Transfer]) -> bool:
-        """Submit and publish one transfer atomically, or decline once the target has closed.
-        ``submit`` may only enqueue on preallocated storage."""
-        with self.lock:
-            if self.closed:
-                return False
-            transfer = submit()
-            assert transfer.expert == expert and expert not in self.transfers
-            self.transfers[expert] = transfer
-            return True
-
-    def close(self) -> Dict[int, Transfer]:
-        with self.lock:
-            self.closed = True
-            return dict(self.transfers)
-
-
-class DemandCacheView:
-    """The resident cache plus the copies issued for this layer call; only the resident part
-    has capacity, recency and eviction (utils/rs_staging.py:52-94)."""
-
-    def __init__(self, resident) -> None:
-        self.resident = resident
-        self.staged: Dict[int, Transfer] = {}
-        self.used_in_order: List[Transfer] = []
-
-    def __getattr__(self, name):
-        return getattr(self.resident, name)
-
-    def __len__(self) -> int:
-        return len(self.resident)
-
-    def has(self, expert) -> bool:
-        return self.resident.has(expert) or int(expert) in self.staged
-
-    def get(self, expert):
-        payload = self.resident.get(expert)
-        if payload is not None:
-            return payload
-        transfer = self.staged.get(int(expert))
-        if transfer is None:
-            return None
-        if not transfer.used:
-            transfer.used = True
-            self.used_in_order.append(transfer)
-        return transfer.payload
-
-    def peek(self, expert):
-        payload = self.resident.peek(expert)
-        if payload is not None:
-            return payload
-        transfer = self.staged.get(int(expert))
-        return None if transfer is None else transfer.payload
-
-    def resident_ids(self):
-        return self.resident.resident_ids()
+from .residency import LayerResidency
+from .ring import StagingRing
 
 
 def select_candidates(ids: Iterable[int], weights: Iterable[float], *, allowed, resident, minimum: float,
                       budget: int, diagnostics: Optional[dict] = None) -> List[int]:
-    """Aggregate probability / reuse score without victim selection
-    (utils/rs_staging.py:97-118; the formula of utils/eval_core.py:10104-10106)."""
-    total: Dict[int, float] = {}
-    hits: Dict[int, int] = {}
-    peak: Dict[int, float] = {}
-    skipped_owner = skipped_resident = 0
-    for eid, weight in zip(ids, weights):
-        eid, weight = int(eid), float(weight)
+    """Which forecast experts are worth a copy: drop entries this rank does not own or already
+    holds, score the rest with the planner's aggregate, keep those at or above ``minimum``, best
+    first, at most ``budget`` (utils/rs_staging.py:97-118).  No victim is chosen: a staged
+    copy displaces nothing."""
+    foreign = held = 0
+    keep_ids: List[int] = []
+    keep_w: List[float] = []
+    for eid, w in zip(ids, weights):
+        eid = int(eid)
         if eid not in allowed:
-            skipped_owner += 1
+            foreign += 1
         elif eid in resident:
-            skipped_resident += 1
+            held += 1
         else:
-            total[eid] = total.get(eid, 0.0) + weight
-            hits[eid] = hits.get(eid, 0) + 1
-            peak[eid] = max(peak.get(eid, 0.0), weight)
-    score = {eid: s * (1 + .15 * (hits[eid] - 1)) + .05 * peak[eid] for eid, s in total.items()}
+            keep_ids.append(eid)
+            keep_w.append(float(w))
+    score = LayerResidency.score_map(keep_ids, keep_w)
+    good = [eid for eid in score if score[eid] >= minimum]
     if diagnostics is not None:
-        diagnostics.update(nonlocal_entries=skipped_owner, resident_entries=skipped_resident, scored=len(score),
-                           below_threshold=sum(v < minimum for v in score.values()))
-    ranked = sorted(score, key=score.get, reverse=True)
-    return [eid for eid in ranked if score[eid] >= minimum][:budget]
+        diagnostics.update(nonlocal_entries=foreign, resident_entries=held, scored=len(score),
+                           below_threshold=len(score) - len(good))
+    good.sort(key=score.get, reverse=True)     # stable: equal scores stay in first-seen order
+    return good[:budget]
 
 
-# --------------------------------------------------------------------------- predictor
-class GraphPrediction:
-    """Predictor + top-k of one source layer, captured once and replayed
-    (utils/rs_overlap.py:21-55)."""
+class ForecastPause:
+    """Empty-forecast cool-down (utils/rs_overlap.py:87-109).  A forecast that named nothing
+    worth copying is not repeated for ``steps`` decode steps of that layer, unless a demand
+    miss there or a change of the cache's membership says the situation moved; a change of
+    recency alone does not."""
 
-    def __init__(self, model, batch: int, width: int, k: int, dtype, normalize: bool, device) -> None:
-        import torch
-        self.torch, self.model = torch, model
-        self.k, self.dtype, self.normalize = int(k), dtype, bool(normalize)
-        self.input = torch.zeros((batch, width), device=device, dtype=torch.float32)
-        stream = torch.cuda.Stream(device=device)
-        stream.wait_stream(torch.cuda.current_stream(device))
-        with torch.cuda.stream(stream), torch.inference_mode():
-            for _ in range(3):
-                self.compute(self.input)
-        stream.synchronize()
+    def __init__(self, steps: int = 0) -> None:
+        self.steps = int(steps)
+        self.until: Dict[int, int] = {}            # layer -> first step that forecasts again
+        self.members: Dict[int, frozenset] = {}    # layer -> cache membership when the pause began
+
+    def arm(self, layer: int, step: int, members: Iterable[int]) -> None:
+        self.until[layer] = int(step) + self.steps + 1
+        self.members[layer] = frozenset(members)
+
+    def wake(self, layer: int) -> bool:
+        self.members.pop(layer, None)
+        return self.until.pop(layer, None) is not None
+
+    def verdict(self, layer: int, step: int, members: Iterable[int]) -> str:
+        """``"run"`` (no pause, or it ran out), ``"moved"`` (membership changed: pause dropped)
+        or ``"hold"``."""
+        if step >= self.until.get(layer, 0):
+            self.wake(layer)
+            return "run"
+        if frozenset(members) != self.members[layer]:
+            self.wake(layer)
+            return "moved"
+        return "hold"
+
+    def clear(self) -> None:
+        self.until.clear()
+        self.members.clear()
+
+
+class CapturedForecast:
+    """Predictor and planner top-k of one source layer as a replayable HIP graph
+    (utils/rs_overlap.py:21-55), with the pinned read-back buffers that belong to it."""
+
+    def __init__(self, predictor, rows: int, width: int, k: int, dtype, renorm: bool, device) -> None:
+        from .rs import topk_for_planning
+        self.k = int(k)
+        self._plan = lambda x: topk_for_planning(predictor(x), self.k, bool(renorm), dtype)
+        self.x = torch.zeros((rows, width), dtype=torch.float32, device=device)
         self.graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(self.graph, stream=stream), torch.inference_mode():
-            self.ids, self.values = self.compute(self.input)
-        torch.cuda.current_stream(device).wait_stream(stream)
-        self.validations = 0
+        with torch.inference_mode():
+            for _ in range(3):                      # lazy initialisation happens outside the capture
+                self._plan(self.x)
+            torch.cuda.synchronize(device)
+            with torch.cuda.graph(self.graph):      # captures on a stream of its own and rejoins
+                self.ids, self.probs = self._plan(self.x)
+        self.host_ids = torch.empty((rows, self.k), dtype=torch.long, pin_memory=True)
+        self.host_probs = torch.empty((rows, self.k), dtype=torch.float32, pin_memory=True)
+        self.landed = torch.cuda.Event(blocking=False)
+        self.task = None          # scoring task that reads the host buffers, until it is done
+        self.checked = 0
 
-    def compute(self, x):
-        t = self.torch
-        values, ids = t.topk(self.model(x).to(t.float32), k=self.k, dim=-1)
-        if self.normalize:
-            values = values / values.sum(-1, keepdim=True).clamp_min(1e-12)
-        return ids.to(t.long), values.to(self.dtype)
+    def launch(self, x, stream) -> None:
+        """Replay for hidden state ``x`` on ``stream`` and start the read-back behind it."""
+        with torch.inference_mode(), torch.cuda.stream(stream):
+            self.x.copy_(x)
+            self.graph.replay()
+            for host, dev in ((self.host_ids, self.ids), (self.host_probs, self.probs)):
+                host.copy_(dev, non_blocking=True)
+            self.landed.record(stream)
 
-    def __call__(self, x):
-        self.input.copy_(x)
-        self.graph.replay()
-        return self.ids, self.values
-
-    def verify(self, x) -> None:
-        want_ids, want_values = self.compute(x.float())
-        ids, values = self(x.float())
-        assert self.torch.equal(ids, want_ids) and self.torch.equal(values, want_values)
-        self.validations += 1
+    def check_against_eager(self, x) -> None:
+        """A replay must give the eager result bit for bit."""
+        with torch.inference_mode():
+            want_ids, want_probs = self._plan(x.float())
+            self.x.copy_(x)
+            self.graph.replay()
+        assert torch.equal(self.ids, want_ids) and torch.equal(self.probs, want_probs)
+        self.checked += 1
 
 
-_STAT_KEYS = ("predictions", "plans", "issued", "used", "wasted", "closed_before_publish", "skipped_slots",
-              "skipped_cooldown", "unified_epipe_calls", "demand_deadline_activations", "empty_plan_closes",
-              "unplanned_closes", "planned_no_publish_closes", "observed_decode_misses",
-              "cooldown_miss_invalidations", "cooldown_cache_invalidations", "candidate_nonlocal_entries",
-              "candidate_resident_entries", "candidate_scored", "candidate_below_threshold", "retained",
-              "recycled_payloads", "allocated_replacements")
+_COUNTERS = ("predictions", "plans", "issued", "used", "wasted", "closed_before_publish", "skipped_slots",
+             "skipped_cooldown", "unified_epipe_calls", "demand_deadline_activations", "empty_plan_closes",
+             "unplanned_closes", "planned_no_publish_closes", "observed_decode_misses",
+             "cooldown_miss_invalidations", "cooldown_cache_invalidations", "candidate_nonlocal_entries",
+             "candidate_resident_entries", "candidate_scored", "candidate_below_threshold", "retained",
+             "recycled_payloads", "allocated_replacements")
+_TIMERS = ("worker_ms", "readback_wait_ms", "main_submission_ms", "target_close_ms", "request_drain_ms")
 
 
 class BoundedRS:
-    """The staging controller (utils/rs_overlap.py:58-433).  One instance serves the whole
-    layer stack; ``SparseContext.staging`` points at it while it is installed."""
+    """The staging engine of a layer stack.  ``slots`` ring positions per layer, of which one
+    window uses at most half, so the copies of step s+1 never wait for the readers of step s."""
 
     def __init__(self, *, slots: int = 4, empty_steps: int = 0) -> None:
+        if int(slots) < 2:
+            raise ValueError("the staging ring needs at least two slots per layer")
         self.enabled = False
-        self.slot_count, self.empty_steps = int(slots), int(empty_steps)
-        assert self.slot_count >= 2 and self.empty_steps >= 0
-        self.pool = ThreadPoolExecutor(max_workers=1, thread_name_prefix="rs-staging")
-        self.graphs: Dict[Any, GraphPrediction] = {}
-        self.buffers: Dict[Any, Any] = {}
-        self.jobs: Dict[int, TargetJob] = {}
-        self.retired: List[Any] = []
-        self.slots: Dict[int, List[dict]] = {}      # layer -> pool slot records
-        self.views: Dict[int, DemandCacheView] = {}
-        self.next_probe: Dict[int, int] = {}
-        self.allowed: Dict[int, frozenset] = {}
-        self.cooldown_residents: Dict[int, frozenset] = {}
-        self.pending_completion_metrics: List[Any] = []
+        self.positions = int(slots)
+        self.pause = ForecastPause(empty_steps)
+        if self.pause.steps < 0:
+            raise ValueError("empty_steps must be a nonnegative integer")
+        self.scorer = ThreadPoolExecutor(max_workers=1, thread_name_prefix="forecast-scorer")
+        self.layers: Dict[int, Any] = {}                    # layer -> block
+        self.forecasts: Dict[int, CapturedForecast] = {}    # source layer -> its captured predictor
+        self.copy_events: Dict[int, List[Any]] = {}         # layer -> one event per ring position
+        self.owned: Dict[int, frozenset] = {}               # layer -> experts this rank holds in host memory
+        self.forecast_stream = None
+        self.copy_lane = None
         self.epoch = 0
-        self.stream = None
-        self.copy_stream = None
-        self.owner = threading.get_ident()
         self.case = None
         self.stats: Dict[str, Any] = {}
-        self.blocks: Dict[int, Any] = {}
+        self.home_thread = threading.get_ident()
 
-    # ---- configuration ------------------------------------------------------------
+    # ---- harness surface --------------------------------------------------------------
+    @property
+    def empty_steps(self) -> int:
+        return self.pause.steps
+
+    def _quiet(self) -> bool:
+        return all(b.residency.ring.all_idle() and not b.residency.staged for b in self.layers.values()) \
+            and all(f.task is None for f in self.forecasts.values())
+
     def configure(self, *, empty_steps) -> None:
-        """Set the empty-forecast cool-down, only between drained requests
-        (utils/rs_overlap.py:78-85)."""
+        """Change the cool-down length; only between drained requests (utils/rs_overlap.py:76-83)."""
         if type(empty_steps) is not int or empty_steps < 0:
             raise ValueError("empty_steps must be a nonnegative integer")
-        assert not self.jobs and not self.retired and not self.views
-        self.empty_steps = empty_steps
-        self.next_probe.clear()
-        self.cooldown_residents.clear()
+        assert self._quiet(), "configure() between requests only"
+        self.pause.steps = empty_steps
+        self.pause.clear()
 
-    def note_demand_miss(self, block) -> None:
-        """A new miss invalidates the target's stale empty forecast (utils/rs_overlap.py:87-93)."""
-        layer = int(block.layer_idx)
-        self.stats["observed_decode_misses"] += 1
-        if self.next_probe.pop(layer, None) is not None:
-            self.cooldown_residents.pop(layer, None)
-            self.stats["cooldown_miss_invalidations"] += 1
-
-    def _skip_cooldown(self, layer: int, step: int) -> bool:
-        """utils/rs_overlap.py:95-109."""
-        deadline = self.next_probe.get(layer, 0)
-        if step >= deadline:
-            self.next_probe.pop(layer, None)
-            self.cooldown_residents.pop(layer, None)
-            return False
-        resident = frozenset(self.views[layer].resident_ids())
-        if resident != self.cooldown_residents[layer]:
-            self.next_probe.pop(layer, None)
-            self.cooldown_residents.pop(layer, None)
-            self.stats["cooldown_cache_invalidations"] += 1
-            return False
-        self.stats["skipped_cooldown"] += 1
-        return True
-
-    # ---- set-up ---------------------------------------------------------------------
     def prepare(self, blocks: Dict[int, Any], rs_bank, *, batch: int, dtype, k: Optional[int] = None) -> None:
-        """Capture the predictors and claim every layer's pool slots
-        (``prepare_graphs``, utils/rs_overlap.py:116-166).  Call once, before ``begin``."""
-        import torch
+        """Bind the stack: check every layer's ring, create the copy events, capture one
+        forecast graph per layer that has a successor (``prepare_graphs``,
+        utils/rs_overlap.py:113-157).  Once, before the first ``begin``."""
         from . import ops
-        assert not self.jobs and not self.retired
-        self.blocks = dict(blocks)
-        for layer, block in sorted(self.blocks.items()):
-            res = block.residency
-            assert res is not None and block.expert_offload == "cpu" and block.cache_policy == "lru"
-            pool = res.claim_staging_pool(self.slot_count)
-            self.slots[layer] = [dict(payload=s, event=ops.Event(), retire=None, busy=False,
-                                      nbytes=int(res.expert_bytes), layer=layer) for s in pool]
-            if layer + 1 >= block.num_layers or layer + 1 not in self.blocks:
+        assert not self.layers, "prepare() once per engine"
+        self.layers = dict(sorted(blocks.items()))
+        for layer, block in self.layers.items():
+            if block.residency is None or block.expert_offload != "cpu" or block.cache_policy != "lru":
+                raise ValueError("forecast staging needs offloaded layers with the plain LRU cache")
+            ring = block.residency.staging_ring(self.positions)
+            self.copy_events[layer] = [ops.Event() for _ in range(len(ring))]
+            self.owned[layer] = frozenset(block._local_eid_set)
+        for layer, block in self.layers.items():
+            nxt = self.layers.get(layer + 1)
+            if nxt is None:
                 continue
-            target = self.blocks[layer + 1].residency
-            kk = int(k) if k is not None else min(block.num_experts, target.predict_topk())
-            # the captured prediction reads the hidden state only (utils/rs_overlap.py:124)
+            # a captured forecast can only read what exists before the layer's router has run
             if str(getattr(rs_bank[layer + 1], "rs_feature_mode", "hidden")) != "hidden":
                 raise ValueError("the bounded staging engine needs predictors with feature_mode='hidden'")
-            graph = GraphPrediction(rs_bank[layer + 1], batch, block.hidden_size, kk, dtype,
-                                    block.norm_topk_prob, block.device)
-            for seed in range(3):
-                x = torch.arange(batch * block.hidden_size, device=block.device,
-                                 dtype=torch.float32).reshape(batch, -1)
-                graph.verify(((x % (97 + seed)) - 48) / 30)
-            self.graphs[layer, kk] = graph
-            self.buffers[layer, kk] = (torch.empty((batch, kk), dtype=torch.long, pin_memory=True),
-                                       torch.empty((batch, kk), dtype=dtype, pin_memory=True),
-                                       torch.cuda.Event(blocking=False))
-        device = next(iter(self.blocks.values())).device
-        self.stream = torch.cuda.Stream(device=device, priority=0)
-        self.copy_stream = ops.SideStream()
+            kk = int(k) if k is not None else min(block.num_experts, nxt.residency.predict_topk())
+            fc = CapturedForecast(rs_bank[layer + 1], batch, block.hidden_size, kk, dtype, block.norm_topk_prob,
+                                  block.device)
+            ramp = torch.arange(batch * block.hidden_size, device=block.device, dtype=torch.float32)
+            for modulus in (97, 98, 99):
+                fc.check_against_eager(((ramp % modulus) - 48).reshape(batch, -1) / 30)
+            self.forecasts[layer] = fc
+        device = next(iter(self.layers.values())).device
+        self.forecast_stream = torch.cuda.Stream(device=device)     # default priority
+        self.copy_lane = ops.SideStream()
         torch.cuda.synchronize()
 
     def begin(self, case=None) -> None:
-        """Start a request (utils/rs_overlap.py:168-205)."""
-        assert not self.jobs and not self.retired and not self.views
+        """Start a request (utils/rs_overlap.py:159-195)."""
+        assert self._quiet(), "the previous request was not finished"
         self.epoch += 1
-        self.case, self.next_probe, self.cooldown_residents = case, {}, {}
-        assert not self.pending_completion_metrics
-        self.stats = {key: 0 for key in _STAT_KEYS}
-        self.stats.update(worker_ms=0.0, readback_wait_ms=0.0, main_submission_ms=0.0, target_close_ms=0.0,
-                          request_drain_ms=0.0, effective_empty_steps=self.empty_steps,
-                          staging_bytes=sum(s["nbytes"] for pool in self.slots.values() for s in pool))
-        if not self.enabled:
-            return
-        for layer, block in self.blocks.items():
-            assert block.expert_source == "router" and block.exec_routing_mode == "router"
-            res = block.residency
-            view = DemandCacheView(res.cache)
-            self.views[layer] = view
-            res.cache = view
-            block._cache = view
-            self.allowed[layer] = frozenset(block._local_eid_set)   # one GPU owns every expert
+        self.case = case
+        self.pause.clear()
+        self.stats = {key: 0 for key in _COUNTERS}
+        self.stats.update({key: 0.0 for key in _TIMERS})
+        self.stats.update(effective_empty_steps=self.pause.steps,
+                          staging_bytes=sum(len(b.residency.ring) * int(b.residency.expert_bytes)
+                                            for b in self.layers.values()))
+        if self.enabled:
+            for block in self.layers.values():
+                assert block.expert_source == "router" and block.exec_routing_mode == "router"
 
-    # ---- slot pool ---------------------------------------------------------------------
-    def _retire(self, slot: dict, event) -> None:
-        assert slot["busy"]
-        slot["busy"], slot["retire"] = False, event
+    def install(self) -> None:
+        """Route the blocks' hooks to this engine (the reference patches seven methods of its
+        block class at this point, utils/rs_overlap.py:436-489)."""
+        from .context import SparseContext
+        SparseContext.staging = self
+        self.enabled = True
 
-    def _collect(self) -> None:
-        keep = []
-        for job, transferred in self.retired:
-            if not job.future.done():
-                keep.append((job, transferred))
-                continue
-            row = job.future.result()   # already complete: never a layer join
-            self.stats["worker_ms"] += row["worker_ms"]
-            self.stats["readback_wait_ms"] += row["readback_wait_ms"]
-            for key, value in row.get("candidate_counts", {}).items():
-                self.stats["candidate_" + key] += value
-            used = {id(x.slot) for x in transferred.values()}
-            for slot in job.slots:
-                if id(slot) not in used:
-                    self._retire(slot, None)
-        self.retired = keep
+    def restore(self) -> None:
+        from .context import SparseContext
+        if SparseContext.staging is self:
+            SparseContext.staging = None
+        self.enabled = False
 
-    def _reserve(self, layer: int, budget: int) -> List[dict]:
-        self._collect()
-        free = [s for s in self.slots[layer] if not s["busy"] and (s["retire"] is None or s["retire"].query())]
-        chosen = free[:budget]
-        for slot in chosen:
-            slot["busy"], slot["retire"] = True, None
-        return chosen
+    def count(self, key: str, n: int = 1) -> None:
+        self.stats[key] += n
 
-    # ---- worker thread --------------------------------------------------------------
-    def _work(self, job: TargetJob, target, ids, weights, readback, resident, minimum: float) -> dict:
-        """Wait for the read-back, score, publish copies (utils/rs_overlap.py:230-263).
-        Works on snapshots only; the single mutation is ``job.publish`` under its lock."""
-        from . import ops
-        started = time.perf_counter()
-        counts: Dict[str, int] = {}
-        stamp = time.perf_counter()
-        readback.synchronize()
-        waited = (time.perf_counter() - stamp) * 1000
-        if not job.closed:
-            chosen = select_candidates(ids.reshape(-1).tolist(), weights.float().reshape(-1).tolist(),
-                                       allowed=self.allowed[target.layer_idx], resident=resident, minimum=minimum,
-                                       budget=len(job.slots), diagnostics=counts)
-            job.plan_count = len(chosen)
-            for eid, slot in zip(chosen, job.slots):
-                def submit(eid=eid, slot=slot):
-                    ops.expert_upload_async(target.slab.slot_ptr(slot["payload"]), target.arena.host_ptr(eid),
-                                            target.arena.expert_bytes, self.copy_stream.handle, slot["event"])
-                    return Transfer(eid, slot["payload"], slot["event"], slot, slot["nbytes"])
-                if not job.publish(eid, submit):
-                    break
-        return dict(worker_ms=(time.perf_counter() - started) * 1000, readback_wait_ms=waited,
-                    candidate_counts=counts)
+    @contextmanager
+    def _timed(self, key: str):
+        """Add the host time of the enclosed block to ``stats[key]``, in ms."""
+        t0 = perf_counter()
+        try:
+            yield
+        finally:
+            self.stats[key] += (perf_counter() - t0) * 1e3
 
-    # ---- source layer: predict ---------------------------------------------------------
+    # ---- hooks called by the blocks ---------------------------------------------------------
     def handles(self, block, seq_len: int) -> bool:
+        """Decode calls of layers whose planner is the RS prefetch."""
         return bool(self.enabled and int(seq_len) == 1 and block.planner_mode == "rs_prefetch")
 
-    def predict(self, block, x, step: int) -> None:
-        """Launch the prediction for layer l+1 and hand it to the worker
-        (utils/rs_overlap.py:255-303).  Never waits for anything."""
-        import torch
-        target_layer = int(block.layer_idx) + 1
-        if target_layer >= block.num_layers or target_layer not in self.blocks:
+    def demand_miss(self, layer: int) -> None:
+        """A decode miss at ``layer``: whatever paused its forecasts is out of date."""
+        self.count("observed_decode_misses")
+        if self.pause.wake(int(layer)):
+            self.count("cooldown_miss_invalidations")
+
+    def _paused(self, layer: int, step: int) -> bool:
+        verdict = self.pause.verdict(layer, step, self.layers[layer].residency.cache.resident_ids())
+        if verdict == "moved":
+            self.count("cooldown_cache_invalidations")
+        elif verdict == "hold":
+            self.count("skipped_cooldown")
+        return verdict == "hold"
+
+    def _absorb(self, fc: CapturedForecast) -> None:
+        """Fold a finished scoring task's timings and counts into the request's statistics."""
+        if fc.task is None or not fc.task.done():
             return
-        assert threading.get_ident() == self.owner
-        target = self.blocks[target_layer]
-        if self.empty_steps and self._skip_cooldown(target_layer, step):
+        row, fc.task = fc.task.result(), None       # done: this does not wait
+        self.stats["worker_ms"] += row["ms"]
+        self.stats["readback_wait_ms"] += row["waited_ms"]
+        for key, value in row["seen"].items():
+            self.stats["candidate_" + key] += value
+
+    def forecast_next(self, block, x, step: int) -> None:
+        """At source layer l: open l+1's ring window, launch the forecast, queue the scoring
+        task (utils/rs_overlap.py:255-301).  Waits for nothing."""
+        src = int(block.layer_idx)
+        fc = self.forecasts.get(src)
+        if fc is None:
             return
-        self._collect()   # graph and host buffers must not be reused while an old worker may read them
-        if target_layer in self.jobs or any(j.ticket[2] == target_layer for j, _ in self.retired):
-            self.stats["skipped_slots"] += 1
+        assert threading.get_ident() == self.home_thread, "hooks run on the thread that built the engine"
+        dst, step = src + 1, int(step)
+        target = self.layers[dst]
+        res: LayerResidency = target.residency
+        if self.pause.steps and self._paused(dst, step):
             return
-        tres = target.residency
-        budget = min(int(tres.effective_top_m()), self.slot_count // 2)
-        if budget <= 0:
+        self._absorb(fc)
+        want = min(int(res.effective_top_m()), self.positions // 2)
+        if want <= 0:
             return
-        slots = self._reserve(target_layer, budget)
-        if not slots:
-            self.stats["skipped_slots"] += 1
-            return
-        stamp = time.perf_counter()
-        k = min(block.num_experts, tres.predict_topk())
-        graph = self.graphs[block.layer_idx, k]
-        host_ids, host_weights, event = self.buffers[block.layer_idx, k]
-        assert tuple(x.shape) == tuple(graph.input.shape)
-        self.stream.wait_stream(torch.cuda.current_stream(block.device))
-        x.record_stream(self.stream)
-        with torch.cuda.stream(self.stream), torch.inference_mode():
-            ids, weights = graph(x)
-            host_ids.copy_(ids, non_blocking=True)
-            host_weights.copy_(weights, non_blocking=True)
-            event.record(self.stream)
-        job = TargetJob((self.epoch, int(step), target_layer), slots)
-        self.jobs[target_layer] = job
-        resident = frozenset(self.views[target_layer].resident_ids())
-        job.future = self.pool.submit(self._work, job, target, host_ids, host_weights, event, resident,
-                                      float(tres.min_candidate_score()))
+        # the graph's buffers belong to the last task until it is done, a layer has one window at
+        # a time, and a window needs at least one ring position whose last readers have finished
+        ticket = (self.epoch, step, dst)
+        with self._timed("main_submission_ms"):
+            room = 0 if (fc.task is not None or res.ring.is_open()) else \
+                res.ring.open(ticket, want, res.backend.event_done)
+            if room == 0:
+                self.count("skipped_slots")
+                return
+            assert x.shape == fc.x.shape, "forecast graphs are captured for one batch size"
+            self.forecast_stream.wait_stream(torch.cuda.current_stream(block.device))
+            x.record_stream(self.forecast_stream)
+            fc.launch(x, self.forecast_stream)
+            snapshot = dict(ticket=ticket, room=room, members=frozenset(res.cache.resident_ids()),
+                            minimum=float(res.min_candidate_score()))
+            fc.task = res.ring.worker = self.scorer.submit(self._score_and_publish, fc, target, **snapshot)
         block.metrics.rs_next_layer_pred_calls += 1
-        self.stats["predictions"] += 1
-        self.stats["main_submission_ms"] += (time.perf_counter() - stamp) * 1000
+        self.count("predictions")
 
-    # ---- target layer: close, use, release ----------------------------------------------
-    def activate(self, block, step: int) -> None:
-        """Close publication for this layer and expose what was issued
-        (utils/rs_overlap.py:305-340)."""
-        layer = int(block.layer_idx)
-        view = self.views[layer]
-        assert not view.staged and not view.used_in_order
-        job = self.jobs.pop(layer, None)
-        if job is None:
+    def _score_and_publish(self, fc: CapturedForecast, target, *, ticket, room: int, members: frozenset,
+                           minimum: float) -> dict:
+        """Scoring thread: wait for the read-back, choose, publish copies until the ring declines
+        (utils/rs_overlap.py:227-253).  Reads snapshots only; the ring's lock is the single
+        point of contact with the layer's thread."""
+        from . import ops
+        t0 = perf_counter()
+        fc.landed.synchronize()
+        t1 = perf_counter()
+        ring: StagingRing = target.residency.ring
+        layer = int(target.layer_idx)
+        events, lane, arena = self.copy_events[layer], self.copy_lane.handle, target.arena
+        seen: Dict[str, int] = {}
+
+        def copy_of(eid: int):
+            def enqueue(slot: int, pos: int):
+                ops.expert_upload_async(target.slab.slot_ptr(slot), arena.host_ptr(eid), arena.expert_bytes, lane,
+                                        events[pos])
+                return events[pos]
+            return enqueue
+
+        if ring.ticket == ticket:       # a stale read only costs a scoring pass; publish() decides
+            chosen = select_candidates(fc.host_ids.flatten().tolist(), fc.host_probs.flatten().tolist(),
+                                       allowed=self.owned[layer], resident=members, minimum=minimum, budget=room,
+                                       diagnostics=seen)
+            ring.note_chosen(ticket, len(chosen))
+            for eid in chosen:
+                if not ring.publish(ticket, eid, copy_of(eid)):
+                    break           # sealed, or full: nothing later can get in either
+        return dict(ms=(perf_counter() - t0) * 1e3, waited_ms=(t1 - t0) * 1e3, seen=seen)
+
+    def seal(self, block, step: int) -> None:
+        """At the target's executor, after router and permutation: end the window and make its
+        copies readable (utils/rs_overlap.py:303-346).  A scoring task that has not published
+        yet has lost its chance for this step; it is not waited for."""
+        layer, res = int(block.layer_idx), block.residency
+        self.count("demand_deadline_activations")
+        with self._timed("target_close_ms"):
+            ticket, filled, chosen = res.ring.seal()
+        if ticket is None:
             return
-        stamp = time.perf_counter()
-        transfers = job.close()
-        self.stats["target_close_ms"] += (time.perf_counter() - stamp) * 1000
-        ticket = (self.epoch, int(step), layer)
-        assert job.ticket == ticket, "Stale prediction crossed a request/step boundary"
-        self.retired.append((job, transfers))
-        if job.plan_count == 0 and self.empty_steps:
-            self.next_probe[layer] = ticket[1] + self.empty_steps + 1
-            self.cooldown_residents[layer] = frozenset(view.resident_ids())
-        if not transfers:
-            self.stats["closed_before_publish"] += 1
-            if job.plan_count is None:
-                self.stats["unplanned_closes"] += 1
-            elif job.plan_count == 0:
-                self.stats["empty_plan_closes"] += 1
-            else:
-                self.stats["planned_no_publish_closes"] += 1
-        view.staged = transfers
-        res = block.residency
-        self.stats["plans"] += bool(transfers)
-        for eid, transfer in transfers.items():
-            res.prefetched_ids.add(eid)
-            res.prefetch_events[eid] = transfer.event
-            res.metrics.prefetch_h2d_bytes += transfer.nbytes
-            res.metrics.prefetch_issued_count += 1
-            res.metrics.prefetch_admitted_count += 1
-            self.stats["issued"] += 1
+        assert ticket == (self.epoch, int(step), layer), "a forecast crossed a request or step boundary"
+        if chosen == 0 and self.pause.steps:
+            self.pause.arm(layer, int(step), res.cache.resident_ids())
+        if filled:
+            res.expose_staged(filled)
+            self.count("plans")
+            self.count("issued", len(filled))
+        else:
+            self.count("closed_before_publish")
+            self.count("unplanned_closes" if chosen is None else
+                       "empty_plan_closes" if chosen == 0 else "planned_no_publish_closes")
 
-    def activate_at_demand(self, block, step: int) -> None:
-        """Publication stays open through router and permutation; it closes here, at the
-        executor's entry (utils/rs_overlap.py:342-350)."""
-        self.activate(block, step)
-        self.stats["demand_deadline_activations"] += 1
+    def settle(self, block) -> list:
+        """Layer exit: the residency admits what was used and returns the ring's positions; the
+        engine only keeps count.  Returns the settled ``(expert, record)`` pairs."""
+        settled = block.residency.settle_staged()
+        for _eid, rec in settled:
+            self.count("used" if rec.touched else "wasted")
+            if rec.kept:
+                self.count("retained")
+                self.count("recycled_payloads" if rec.recycled else "allocated_replacements")
+        return settled
 
-    def _retain_used(self, block, transfer: Transfer) -> None:
-        """Admit an expert that was really used, after the layer: exchange slot ownership
-        with the evicted resident instead of moving bytes (utils/rs_overlap.py:352-381)."""
-        assert transfer.used and not transfer.retained
-        replacement, recycled = block.residency.adopt_staged(transfer.expert, transfer.payload, transfer.event)
-        if replacement is None:
-            return
-        self.stats["recycled_payloads" if recycled else "allocated_replacements"] += 1
-        transfer.slot["payload"] = replacement
-        transfer.retained = True
-        self.stats["retained"] += 1
-
-    def release(self, block) -> None:
-        """Layer exit (utils/rs_overlap.py:383-408)."""
-        view = self.views[int(block.layer_idx)]
-        res = block.residency
-        used = [x for x in view.staged.values() if x.used]
-        done = res.backend.fence() if used else None   # after every consumer on the compute lane
-        for transfer in view.used_in_order:
-            self._retain_used(block, transfer)
-        for eid, transfer in view.staged.items():
-            self._retire(transfer.slot, done if transfer.used else transfer.event)
-            self.stats["used" if transfer.used else "wasted"] += 1
-            if not transfer.used:
-                res.metrics.prefetch_wasted_count += 1
-                self.pending_completion_metrics.append(res)
-            res.prefetch_events.pop(eid, None)
-            res.prefetched_ids.discard(eid)
-            res.prefetch_used_ids.discard(eid)
-        view.staged = {}
-        view.used_in_order = []
-
+    # ---- end of request ------------------------------------------------------------------------
     def finish(self) -> dict:
-        """Drain the request (utils/rs_overlap.py:410-432)."""
-        stamp = time.perf_counter()
-        for layer, job in list(self.jobs.items()):
-            transfers = job.close()
-            self.retired.append((job, transfers))
-            for transfer in transfers.values():
-                self._retire(transfer.slot, transfer.event)
-        self.jobs.clear()
-        for job, _ in self.retired:
-            job.future.result(timeout=30)
-        self._collect()
-        if self.stream is not None:
-            self.stream.synchronize()
-            self.copy_stream.synchronize()
-        for layer, view in self.views.items():
-            block = self.blocks[layer]
-            if view.staged:
-                self.release(block)
-            assert block.residency.cache is view
-            block.residency.cache = view.resident
-            block._cache = view.resident
-        self.views = {}
-        for res in self.pending_completion_metrics:
-            res.metrics.prefetch_completed_count += 1
-        self.pending_completion_metrics = []
-        self.stats["request_drain_ms"] = (time.perf_counter() - stamp) * 1000
-        return dict(case=self.case, **self.stats)
+        """Drain: seal what is still open, let the scoring tasks and both streams run out, settle
+        (utils/rs_overlap.py:406-432).  Returns the request's statistics."""
+        t0 = perf_counter()
+        for block in self.layers.values():
+            ring = block.residency.ring
+            _ticket, filled, _chosen = ring.seal()
+            for _eid, pos, event in filled:         # copied for a step that never came
+                ring.give_back(pos, event)
+        for fc in self.forecasts.values():
+            if fc.task is not None:
+                fc.task.result(timeout=30)
+                self._absorb(fc)
+        if self.copy_lane is not None:      # None: the engine was never bound to a device
+            self.forecast_stream.synchronize()
+            self.copy_lane.synchronize()
+        for block in self.layers.values():
+            self.settle(block)
+            block.residency.confirm_staged_copies()
+            block.residency.ring.worker = None
+        self.stats["request_drain_ms"] = (perf_counter() - t0) * 1e3
+        return {"case": self.case, **self.stats}
 
     def shutdown(self) -> None:
-        assert not self.jobs and not self.retired and not self.views
-        self.pool.shutdown(wait=True)
+        assert self._quiet(), "finish() the request first"
+        self.scorer.shutdown(wait=True)

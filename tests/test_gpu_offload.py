@@ -357,8 +357,9 @@ def test_bounded_staging_engine_decode(device):
     blocks, metrics, bank = _staged_stack(device, capacity, top_m, pool_slots=4)
     engine = BoundedRS(slots=4)
     engine.prepare(blocks, bank, batch=T, dtype=torch.bfloat16)
-    engine.enabled = True
-    SparseContext.staging = engine
+    engine.install()
+    assert SparseContext.staging is engine and engine.enabled
+    assert all(fc.checked == 3 for fc in engine.forecasts.values()) and len(engine.forecasts) == len(blocks) - 1
     engine.begin("test")
     got = _run(list(blocks.values()), device, steps, T)
     stats = engine.finish()
@@ -374,19 +375,19 @@ def test_bounded_staging_engine_decode(device):
     assert metrics.prefetch_h2d_bytes == stats["issued"] * blocks[0].arena.expert_bytes
     for layer, blk in blocks.items():
         res = blk.residency
-        assert res.cache is blk._cache and not hasattr(res.cache, "staged")      # views are gone
+        assert res.cache is blk._cache and not res.staged and not res.staged_touched   # nothing left staged
         slots = [res._slot_of[e] for e in res.cache.resident_ids()]
-        pool = [s["payload"] for s in engine.slots[layer]]
-        assert len(set(slots)) == len(slots) and not set(slots) & set(pool)       # no slot has two owners
-        assert sorted(pool) == sorted(res._pool_slots) and not set(pool) & set(res._free_slots)
-        assert all(not s["busy"] for s in engine.slots[layer])
+        ring = res.ring.slots
+        assert len(set(slots)) == len(slots) and not set(slots) & set(ring)       # no slot has two owners
+        assert len(set(ring)) == len(ring) == 4 and not set(ring) & set(res._free_slots)
+        assert res.ring.all_idle() and res.staged_unconfirmed == 0
     # a second request on the same engine, then the ordinary planner again
     engine.begin("again")
     got2 = _run(list(blocks.values()), device, 6, T)
     stats2 = engine.finish()
     assert stats2["predictions"] > 0 and stats2["case"] == "again"
-    engine.enabled = False
-    SparseContext.staging = None
+    engine.restore()
+    assert SparseContext.staging is None and not engine.enabled
     for a, b in zip(got2, want[: len(got2)]):
         assert torch.equal(a, b)
     got3 = _run(list(blocks.values()), device, 6, T)

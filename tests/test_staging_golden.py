@@ -1,9 +1,10 @@
-"""Host logic of the bounded staging adapter against vectors recorded from the reference's
+"""Host logic of forecast staging against vectors recorded from the reference's
 own modules (``tests/golden/staging_ops.json``, written by
 ``tests/golden/make_staging_golden.py`` from utils/rs_staging.py and utils/rs_overlap.py run
 as they are): candidate selection, what a demand lookup sees while copies are staged, the
 empty-forecast cool-down, and the admission of used experts at layer exit with its exchange
-of storage."""
+of storage.  The reference's operations are mapped onto this build's slot table: a payload
+is a slot index, a staged transfer a ``StagedExpert`` in a lent ring position."""
 import json
 from pathlib import Path
 from types import SimpleNamespace as NS
@@ -11,8 +12,9 @@ from types import SimpleNamespace as NS
 import pytest
 
 from oracle import ref_rs, ref_staging
-from sparse_amd.residency import ResidencyConfig
-from sparse_amd.staging import BoundedRS, DemandCacheView, Transfer, select_candidates
+from sparse_amd.residency import ResidencyConfig, StagedExpert
+from sparse_amd.ring import LENT
+from sparse_amd.staging import BoundedRS, select_candidates
 from tests.test_residency import FakeEvent, product_layer
 
 DATA = json.loads((Path(__file__).resolve().parent / "golden" / "staging_ops.json").read_text())
@@ -43,34 +45,31 @@ def _product_session(case):
 
     for e in case["seed_ids"]:
         load(e)
-    view = DemandCacheView(res.cache)
-    owner = BoundedRS.__new__(BoundedRS)
-    owner.jobs, owner.retired, owner.views = {}, [], {0: view}
-    owner.next_probe, owner.cooldown_residents = {}, {}
-    owner.empty_steps = case["empty_steps"]
-    owner.stats = {k: 0 for k in STATS}
-    block = NS(layer_idx=0, residency=res)
-    in_use = set()
+    ring = res.ring
+    engine = BoundedRS(slots=2, empty_steps=case["empty_steps"])
+    engine.layers = {0: NS(layer_idx=0, residency=res)}
+    engine.begin()
+    block = engine.layers[0]
     for (op, *args), want in zip(case["ops"], case["results"]):
         r = None
         if op == "stage":
-            slot = next(s for s in res._pool_slots if s not in in_use)
-            in_use.add(slot)
+            pos = ring.state.index("idle")
+            slot, ring.state[pos] = ring.slots[pos], LENT
             tags[slot] = f"staged{args[0]}"
-            res.backend.slot_content[slot] = args[0]
-            view.staged[args[0]] = Transfer(args[0], slot, FakeEvent("copy", args[0]), {"payload": slot}, 12)
+            backend.slot_content[slot] = args[0]
+            res.staged[args[0]] = StagedExpert(pos, slot, FakeEvent("copy", args[0]))
         elif op in ("get", "peek"):
-            got = getattr(view, op)(args[0])
+            got = res.find(args[0], touch=op == "get")
             r = None if got is None else tags[got]
         elif op == "has":
-            r = bool(view.has(args[0]))
+            r = res.holds(args[0])
         elif op == "miss":
-            owner.note_demand_miss(block)
+            engine.demand_miss(0)
         elif op == "arm":
-            owner.next_probe[0] = args[0]
-            owner.cooldown_residents[0] = frozenset(view.resident_ids())
+            engine.pause.until[0] = args[0]
+            engine.pause.members[0] = frozenset(res.cache.resident_ids())
         elif op == "skip":
-            r = bool(owner._skip_cooldown(0, args[0]))
+            r = engine._paused(0, args[0])
         elif op == "put":
             if res.cache.has(args[0]):
                 # the reference replaces the payload object of a resident entry; here the bytes
@@ -81,18 +80,16 @@ def _product_session(case):
                 load(args[0])
                 res.flush()
         else:
+            free_before = set(res._free_slots)
             r = []
-            for transfer in view.used_in_order:
-                free_before = set(res._free_slots)
-                owner._retain_used(block, transfer)
-                new = transfer.slot["payload"]
-                r.append([transfer.expert, bool(transfer.retained),
-                          "fresh" if (transfer.retained and new in free_before) else tags[new]])
-            in_use.clear()
-            view.staged, view.used_in_order = {}, []
+            for eid, rec in engine.settle(block):
+                if rec.touched:
+                    now = ring.slots[rec.pos]       # what the ring holds in the staged expert's place
+                    r.append([eid, rec.kept, "fresh" if (rec.kept and now in free_before) else tags[now]])
+            assert ring.all_idle() and not res.staged
         freq = sorted(res.access_freq.items()) if op == "exit" else None
-        got = [r, res.cache.resident_ids(), [t.expert for t in view.used_in_order], sorted(view.staged),
-               owner.next_probe.get(0), [owner.stats[k] for k in STATS], freq]
+        got = [r, res.cache.resident_ids(), list(res.staged_touched), sorted(res.staged),
+               engine.pause.until.get(0), [engine.stats[k] for k in STATS], freq]
         yield op, args, got, want
 
 
