@@ -415,6 +415,13 @@ int sparse_hip_calib_copy(const void* src_dev, void* dst_dev, size_t bytes, void
 int sparse_hip_profile_enable(int on);
 int sparse_hip_profile_reset(void);
 int sparse_hip_profile_read(int kernel, double* total_ms_out, int64_t* launches_out);
+/* Checking aid with no counterpart in the reference: while on, the prefill-size expert FFN
+ * (sparse_hip_moe_ffn_prefill, sparse_hip_shared_ffn at prefill sizes) runs the variant of its
+ * kernel whose k loop drains every outstanding vector-memory operation where the normal one
+ * waits for a counted number of them.  Same arithmetic, same bits, slower; a difference
+ * between the two means the counted waits no longer match the code the compiler produced.
+ * Process-wide; returns the previous setting. */
+int sparse_hip_prefill_drain_waits(int on);
 /* Name of the __global__ function behind a kernel id (as rocprofv3 prints it, without
  * template arguments). */
 const char* sparse_hip_kernel_name(int kernel);

@@ -25,6 +25,7 @@ import torch.nn.functional as F
 from torch import nn
 
 from . import ops
+from ._lru import LruTable
 from .context import DistEnv, Metrics, SparseContext
 from .residency import Backend, LayerResidency, ResidencyConfig
 from .rs import router_topk_feature, stable_topk, topk_for_planning
@@ -73,9 +74,10 @@ def extract_experts(experts: Any) -> Tuple[str, List[Tuple[torch.Tensor, torch.T
 
 
 class _Workspace:
-    """Activation buffers for one (T, layer shape); shared by all layers of that shape."""
+    """Activation buffers for one (T, layer shape); shared by all layers of that shape.  The
+    most recently used ``SPARSE_HIP_WORKSPACE_CACHE`` (default 8) shapes are kept."""
 
-    _cache: Dict[Tuple, "_Workspace"] = {}
+    _cache = LruTable.from_env("SPARSE_HIP_WORKSPACE_CACHE", 8)
 
     def __init__(self, T: int, K: int, E: int, H: int, I: int, Is: int, dtype, logits_dtype, device) -> None:
         self.logits_dtype = logits_dtype
@@ -102,11 +104,7 @@ class _Workspace:
 
     @classmethod
     def get(cls, *key) -> "_Workspace":
-        ws = cls._cache.get(key)
-        if ws is None:
-            ws = cls(*key)
-            cls._cache[key] = ws
-        return ws
+        return cls._cache.get_or_make(key, lambda: cls(*key))
 
 
 def _NO_SEGMENTS():

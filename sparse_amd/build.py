@@ -7,6 +7,7 @@ anywhere the ROCm toolchain is installed; the resulting ``.so`` is loaded by
 from __future__ import annotations
 
 import os
+import re
 import shutil
 import subprocess
 import sys
@@ -43,6 +44,39 @@ HIP_FLAGS = [
 ]
 
 
+# Kernels whose pipelines wait for a *counted* number of vector-memory operations.  A register
+# spill adds scratch loads and stores to that count, so a build in which one of these kernels
+# uses scratch memory is refused.
+NO_SCRATCH = {"swiglu_prefill.hip": ("prefill_ffn_kernel",)}
+RESOURCE_REMARKS = "-Rpass-analysis=kernel-resource-usage"
+
+
+def scratch_by_kernel(remarks: str) -> dict[str, int]:
+    """``{mangled kernel name: scratch bytes per lane}`` from hipcc's resource-usage remarks."""
+    out: dict[str, int] = {}
+    name = None
+    for line in remarks.splitlines():
+        if "remark: Function Name:" in line:
+            name = line.split("Function Name:", 1)[1].split("[", 1)[0].strip()
+        elif "ScratchSize [bytes/lane]:" in line and name is not None:
+            out[name] = int(line.split("ScratchSize [bytes/lane]:", 1)[1].split("[", 1)[0])
+    return out
+
+
+def check_no_scratch(source: str, remarks: str) -> None:
+    wanted = NO_SCRATCH.get(source, ())
+    if not wanted:
+        return
+    table = scratch_by_kernel(remarks)
+    for kernel in wanted:
+        hits = {n: b for n, b in table.items() if kernel in n}
+        if not hits:
+            raise RuntimeError(f"{source}: no resource remarks for {kernel}; cannot check its scratch use")
+        bad = {n: b for n, b in hits.items() if b != 0}
+        if bad:
+            raise RuntimeError(f"{source}: {kernel} uses scratch memory {bad}; its counted waits assume none")
+
+
 def lib_path() -> Path:
     return CSRC / LIB_NAME
 
@@ -54,15 +88,20 @@ def _hipcc() -> str:
     return exe
 
 
-def _run(cmd: list[str]) -> None:
+def _run(cmd: list[str]) -> str:
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if proc.returncode != 0:
         raise RuntimeError("command failed: %s\n%s\n%s" % (" ".join(cmd), proc.stdout, proc.stderr))
-    # the host pass prints one "not a recognized feature" line per flag; drop those
+    # the host pass prints one "not a recognized feature" line per flag; drop those, and the
+    # resource remarks (with the source excerpts clang prints under each of them)
+    quiet = RESOURCE_REMARKS in cmd
     for line in proc.stderr.splitlines():
         if "packed-fp32-ops" in line or not line.strip():
             continue
+        if quiet and ("remark:" in line or re.match(r"\s*\d*\s*\|", line)):
+            continue
         print(line, file=sys.stderr)
+    return proc.stderr
 
 
 def build(verbose: bool = True, jobs: int | None = None) -> Path:
@@ -74,9 +113,11 @@ def build(verbose: bool = True, jobs: int | None = None) -> Path:
     def compile_one(name: str) -> str:
         obj = obj_dir / (name + ".o")
         cmd = [hipcc, *HIP_FLAGS, f"-I{INCLUDE}", f"-I{CSRC}", "-c", str(CSRC / name), "-o", str(obj)]
+        if name in NO_SCRATCH:
+            cmd.insert(1, RESOURCE_REMARKS)
         if verbose:
             print("[sparse_amd.build] hipcc -c", name, flush=True)
-        _run(cmd)
+        check_no_scratch(name, _run(cmd))
         return str(obj)
 
     with ThreadPoolExecutor(max_workers=jobs) as pool:

@@ -18,6 +18,7 @@ int decode_split_parts(int);
 int prefill_routed_bf16(const sparse_hip_experts*, const void*, const void*, const int32_t*, const int32_t*,
                         const sparse_hip_seglist*, int, int, void*, void*, void*, hipStream_t);
 size_t prefill_ws_bytes(int, int, int, int, int);
+int prefill_set_drain_waits(int);
 int prefill_shared_bf16(const void*, const void*, const void*, const void*, const void*, int, int, int, void*,
                         void*, hipStream_t);
 template <typename T>
@@ -70,6 +71,8 @@ static int check_routed(const char* fn, const sparse_hip_experts* ex, const void
 using namespace sparse;
 
 extern "C" {
+
+int sparse_hip_prefill_drain_waits(int on) { return prefill_set_drain_waits(on); }
 
 size_t sparse_hip_prefill_ws_bytes(int T, int K, int num_segments, int H, int I) {
   if (T <= 0 || K <= 0 || num_segments < 0 || H <= 0 || I <= 0) return 0;

@@ -27,6 +27,7 @@
 //   D: column c, rows 8*i + 4*g + j for register 4*i + j
 // The weights are passed as A and the activations as B, so D is the transposed output
 // tile: a lane owns one activation row and runs of four consecutive output columns.
+#include <atomic>
 #include <type_traits>
 
 #include "common.h"
@@ -133,7 +134,10 @@ __global__ __launch_bounds__(256) void prefill_tile_map_kernel(const PfMapArgs a
   }
 }
 
-template <bool kGateUp>
+// kDrainWaits replaces the counted vector-memory waits of the k loop by full drains: slower,
+// and correct whatever else the compiler has in flight.  It exists to check the counted
+// waits: both variants must give the same bits.
+template <bool kGateUp, bool kDrainWaits>
 __global__ __launch_bounds__(kPfThreads, 2) void prefill_ffn_kernel(const PrefillArgs a) {
   __shared__ __attribute__((aligned(1024))) uint8_t lds[kPfStages][kPfLdsA];
   __shared__ float s_scale[kPfBM];
@@ -252,7 +256,8 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_ffn_kernel(const Prefil
   // of slab kt+2 and the 8 fragment loads of slab kt's steps -- vmcnt(20) -- and the
   // scheduling fences keep exactly that order.  Slabs past the end refetch the last one
   // instead of branching.
-  constexpr int kWaitVm20 = 0x4F74, kWaitVm0 = 0x0F70;  // s_waitcnt vmcnt(n), other counters untouched
+  // s_waitcnt vmcnt(n), other counters untouched
+  constexpr int kWaitVm0 = 0x0F70, kWaitVm20 = kDrainWaits ? kWaitVm0 : 0x4F74;
   const int nk = Kdim / kPfBK;
   bf16x8 bfrag[2][2][4];
   stage_slab(0, 0);
@@ -364,6 +369,10 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_ffn_kernel(const Prefil
   }
 }
 
+static std::atomic<int> g_prefill_drain_waits{0};
+
+int prefill_set_drain_waits(int on) { return g_prefill_drain_waits.exchange(on ? 1 : 0); }
+
 template <bool kGateUp>
 static int launch_prefill(PrefillArgs& a, int max_mtiles, hipStream_t st) {
   int64_t grid = static_cast<int64_t>(a.ntiles_n) * max_mtiles;
@@ -371,8 +380,12 @@ static int launch_prefill(PrefillArgs& a, int max_mtiles, hipStream_t st) {
   if (grid == 0) return SPARSE_HIP_OK;
   SP_REQUIRE(grid < (1ll << 31), "prefill_ffn: grid too large");
   ProfScope prof(kGateUp ? SPARSE_HIP_K_PREFILL_GATEUP : SPARSE_HIP_K_PREFILL_DOWN, st);
-  hipLaunchKernelGGL((prefill_ffn_kernel<kGateUp>), dim3(static_cast<unsigned>(grid)), dim3(kPfThreads), 0, st,
-                     a);
+  if (g_prefill_drain_waits.load(std::memory_order_relaxed))
+    hipLaunchKernelGGL((prefill_ffn_kernel<kGateUp, true>), dim3(static_cast<unsigned>(grid)), dim3(kPfThreads), 0,
+                       st, a);
+  else
+    hipLaunchKernelGGL((prefill_ffn_kernel<kGateUp, false>), dim3(static_cast<unsigned>(grid)), dim3(kPfThreads), 0,
+                       st, a);
   SP_LAUNCH_CHECK("prefill_ffn_kernel");
   return SPARSE_HIP_OK;
 }

@@ -13,6 +13,7 @@ from typing import Optional, Sequence, Tuple
 import torch
 
 from . import _lib
+from ._lru import LruTable
 from ._lib import BF16, F32, DECODE_MAX_TOKENS, Experts, SegList
 
 
@@ -275,19 +276,17 @@ def grouped_swiglu(experts: Experts, x: torch.Tensor, topv: torch.Tensor, perm: 
     _lib.check(rc, "sparse_hip_grouped_swiglu_prefill")
 
 
-_TILE_WS = {}
+_TILE_WS = LruTable.from_env("SPARSE_HIP_WORKSPACE_CACHE", 8)
 
 
 def prefill_tile_ws(T: int, K: int, num_segments: int, hidden: int, inter: int, device) -> torch.Tensor:
     """Tile-map workspace of the prefill kernels, cached per shape (launches on one stream
     reuse it in order)."""
-    key = (T, K, num_segments, hidden, inter, str(device))
-    ws = _TILE_WS.get(key)
-    if ws is None:
+    def make() -> torch.Tensor:
         nbytes = _lib.load().sparse_hip_prefill_ws_bytes(T, K, num_segments, hidden, inter)
-        ws = torch.empty((max(16, nbytes),), device=device, dtype=torch.uint8)
-        _TILE_WS[key] = ws
-    return ws
+        return torch.empty((max(16, nbytes),), device=device, dtype=torch.uint8)
+
+    return _TILE_WS.get_or_make((T, K, num_segments, hidden, inter, str(device)), make)
 
 
 def shared_expert(x: torch.Tensor, gate_w: torch.Tensor, up_w: torch.Tensor, down_w: torch.Tensor,

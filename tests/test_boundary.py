@@ -172,3 +172,19 @@ def test_boundary_hook_counts_and_clears_the_side_cache_only_on_request():
         assert m.counters["epipe_prefill_extra_cache_resident_at_decode_end"] == 1
     finally:
         SparseContext.reset()
+
+
+def test_workspace_tables_are_bounded():
+    """Per-shape workspaces are kept for the most recently used shapes only."""
+    from sparse_amd._lru import LruTable
+    made = []
+    table = LruTable(3)
+    for key in (1, 2, 3, 1, 4):          # 1 is refreshed before 4 arrives, so 2 is the one dropped
+        table.get_or_make(key, lambda key=key: made.append(key) or object())
+    assert table.keys() == [3, 1, 4] and made == [1, 2, 3, 4] and 2 not in table
+    assert table.get_or_make(1, lambda: pytest.fail("still held")) is not None
+    with pytest.raises(ValueError):
+        LruTable(0)
+    from sparse_amd import ops
+    from sparse_amd.block import _Workspace
+    assert isinstance(_Workspace._cache, LruTable) and isinstance(ops._TILE_WS, LruTable)

@@ -370,6 +370,50 @@ def test_prefill_and_decode_kernels_agree(device):
     torch.testing.assert_close(a.float(), b.float(), **BF16_TOL)
 
 
+@pytest.mark.parametrize("H,E,I,K,T", [(512, 12, 256, 4, 300), (2048, 60, 1408, 4, 1531), (7168, 8, 2048, 2, 777)])
+def test_prefill_counted_waits_equal_full_drains(device, H, E, I, K, T):
+    """The prefill kernel's k loop waits for a counted number of vector-memory operations.
+    The same kernel built with full drains in their place must give the same bits, over
+    ragged segments (routing of random rows: segment sizes from empty to several row tiles,
+    odd and even numbers of k slabs across the three shapes), for the routed rows, the
+    combined output and the shared expert."""
+    from sparse_amd import _lib
+    ops = _ops()
+    lib = _lib.load()
+    layer = make_layer(H, E, I, K, Is=I, shared_gate=True, dtype=torch.bfloat16, seed=61)
+    x = make_hidden(T, H, torch.bfloat16, seed=62)
+    g = torch.Generator().manual_seed(63)
+    popularity = 1.0 / torch.arange(1, E + 1, dtype=torch.float32) ** 1.2    # a few busy experts, a long tail
+    popularity[E - 1] = 0.0                                                   # and one nobody routes to
+    topi = torch.multinomial(popularity.expand(T, E), K, replacement=False, generator=g)
+    topv = torch.rand(T, K, generator=g).to(torch.bfloat16)
+    counts = torch.bincount(topi.reshape(-1), minlength=E)
+    assert int(counts.max()) > 256 and int(counts[counts > 0].min()) < 128 and int(counts.min()) == 0
+    sh = [w.to(device) for w in layer["shared"]]
+    xd = x.to(device)
+    sg = torch.nn.functional.linear(x.float(), layer["shared_gate_w"].float().reshape(1, -1)).reshape(-1)
+    sg = sg.to(torch.bfloat16).to(device)
+
+    def run():
+        out, parts, _ = _run_routed(ops, layer, x, topv, topi, device, decode=False)
+        inter = torch.zeros((T, I), device=device, dtype=torch.bfloat16)
+        shared = torch.zeros((T, H), device=device, dtype=torch.bfloat16)
+        ops.shared_expert(xd, sh[0], sh[1], sh[2], sg, inter, shared)
+        torch.cuda.synchronize()
+        return out, parts, shared.cpu()
+
+    assert lib.sparse_hip_prefill_drain_waits(0) == 0
+    fast = run()
+    assert lib.sparse_hip_prefill_drain_waits(1) == 0
+    try:
+        safe = run()
+    finally:
+        assert lib.sparse_hip_prefill_drain_waits(0) == 1
+    for a, b, what in zip(fast, safe, ("combined output", "routed rows", "shared expert")):
+        assert torch.equal(a, b), f"{what}: counted waits and full drains differ"
+    assert float(fast[0].float().abs().max()) > 0
+
+
 @pytest.mark.parametrize("T,decode", [(8, True), (128, False)])
 def test_ffn_fp32_matches_oracle(device, T, decode):
     ops = _ops()
