@@ -239,133 +239,145 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_ffn_kernel(const Prefil
     bptr[ni] = base + static_cast<size_t>(n >> 4) * 16 * Kdim + kh * 512 + r16 * 8;
   }
 
-  f32x16 acc[4][2];
-#pragma unroll
-  for (int mi = 0; mi < 4; ++mi)
-#pragma unroll
-    for (int ni = 0; ni < 2; ++ni)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) acc[mi][ni][v] = 0.f;
-
-  // Pipeline: while slab kt is multiplied, the activation rows of slab kt+2 travel to the
-  // third LDS buffer and the weight fragments of slab kt+2 to the registers step s has just
-  // finished with (two fragment sets, used alternately), so every operand is requested two
-  // slabs of MFMA work before its use -- enough bytes in flight to cover an HBM miss.
-  // Vector memory operations retire in order, so "the copies of slab kt+1 have landed" is a
-  // count of the younger operations: the 8 fragment loads of slab kt-1's steps, the 4 copies
-  // of slab kt+2 and the 8 fragment loads of slab kt's steps -- vmcnt(20) -- and the
-  // scheduling fences keep exactly that order.  Slabs past the end refetch the last one
-  // instead of branching.
-  // s_waitcnt vmcnt(n), other counters untouched
-  constexpr int kWaitVm0 = 0x0F70, kWaitVm20 = kDrainWaits ? kWaitVm0 : 0x4F74;
-  const int nk = Kdim / kPfBK;
-  bf16x8 bfrag[2][2][4];
-  stage_slab(0, 0);
-  stage_slab(min(1, nk - 1), 1);
-  __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-  for (int st = 0; st < 2; ++st)
-#pragma unroll
-    for (int ni = 0; ni < 2; ++ni)
-#pragma unroll
-      for (int s = 0; s < 4; ++s)
-        bfrag[st][ni][s] =
-            *reinterpret_cast<const bf16x8*>(bptr[ni] + static_cast<size_t>(min(st, nk - 1)) * 1024 + s * 128);
-  __builtin_amdgcn_sched_barrier(0);
-  __builtin_amdgcn_s_waitcnt(kWaitVm20);
-  __syncthreads();
-
-  const int fsw = ((fc >> 1) & 7) ^ ((fc & 1) << 2);
-  const int a_row = fc * kPfRowBytes, a_x = (fg ^ fsw) << 4;
-  int cur = 0, nxt2 = 2;  // buffer of slab kt, buffer of slab kt+2
-  auto slab = [&](auto stage_c, int kt) {
-    constexpr int st = decltype(stage_c)::value;
-    const int kt2 = min(kt + 2, nk - 1);
-    stage_slab(kt2, nxt2);
-    __builtin_amdgcn_sched_barrier(kPfSchedMask);
-    const uint8_t* la = lds[cur] + a_row;
-#pragma unroll
-    for (int s = 0; s < 4; ++s) {
-      bf16x8 fa[4];
-#pragma unroll
-      for (int mi = 0; mi < 4; ++mi)
-        fa[mi] = *reinterpret_cast<const bf16x8*>(la + mi * 32 * kPfRowBytes + (a_x ^ (s << 5)));
-#pragma unroll
-      for (int mi = 0; mi < 4; ++mi)
-#pragma unroll
-        for (int ni = 0; ni < 2; ++ni)
-          acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfrag[st][ni][s], fa[mi], acc[mi][ni], 0, 0, 0);
-      __builtin_amdgcn_sched_barrier(kPfSchedMask);
-#pragma unroll
+  // The tile's rows are processed in sub-tiles of 32 (one MFMA row block); a segment's last
+  // tile is specialised on how many of them hold rows, so that a ragged tail costs the MFMAs,
+  // LDS reads and stores of its own sub-tiles only.
+  auto body = [&](auto nmi_c) {
+    constexpr int NMI = decltype(nmi_c)::value;
+    f32x16 acc[NMI][2];
+  #pragma unroll
+    for (int mi = 0; mi < NMI; ++mi)
+  #pragma unroll
       for (int ni = 0; ni < 2; ++ni)
-        bfrag[st][ni][s] = *reinterpret_cast<const bf16x8*>(bptr[ni] + static_cast<size_t>(kt2) * 1024 + s * 128);
-      __builtin_amdgcn_sched_barrier(kPfSchedMask);
-    }
+  #pragma unroll
+        for (int v = 0; v < 16; ++v) acc[mi][ni][v] = 0.f;
+
+    // Pipeline: while slab kt is multiplied, the activation rows of slab kt+2 travel to the
+    // third LDS buffer and the weight fragments of slab kt+2 to the registers step s has just
+    // finished with (two fragment sets, used alternately), so every operand is requested two
+    // slabs of MFMA work before its use -- enough bytes in flight to cover an HBM miss.
+    // Vector memory operations retire in order, so "the copies of slab kt+1 have landed" is a
+    // count of the younger operations: the 8 fragment loads of slab kt-1's steps, the 4 copies
+    // of slab kt+2 and the 8 fragment loads of slab kt's steps -- vmcnt(20) -- and the
+    // scheduling fences keep exactly that order.  Slabs past the end refetch the last one
+    // instead of branching.
+    // s_waitcnt vmcnt(n), other counters untouched
+    constexpr int kWaitVm0 = 0x0F70, kWaitVm20 = kDrainWaits ? kWaitVm0 : 0x4F74;
+    const int nk = Kdim / kPfBK;
+    bf16x8 bfrag[2][2][4];
+    stage_slab(0, 0);
+    stage_slab(min(1, nk - 1), 1);
+    __builtin_amdgcn_sched_barrier(0);
+  #pragma unroll
+    for (int st = 0; st < 2; ++st)
+  #pragma unroll
+      for (int ni = 0; ni < 2; ++ni)
+  #pragma unroll
+        for (int s = 0; s < 4; ++s)
+          bfrag[st][ni][s] =
+              *reinterpret_cast<const bf16x8*>(bptr[ni] + static_cast<size_t>(min(st, nk - 1)) * 1024 + s * 128);
+    __builtin_amdgcn_sched_barrier(0);
     __builtin_amdgcn_s_waitcnt(kWaitVm20);
     __syncthreads();
-    cur = (cur == kPfStages - 1) ? 0 : cur + 1;
-    nxt2 = (nxt2 == kPfStages - 1) ? 0 : nxt2 + 1;
-  };
-  // Slabs go in pairs with no branch inside the loop: a conditional second slab would give the
-  // loop head two different pictures of the outstanding fragment loads, and the waits the
-  // compiler puts before each MFMA would then assume the shorter one (eight loads behind
-  // instead of sixteen), i.e. drain the loads issued for the slab after next.
-  int kt = 0;
-  for (; kt + 2 <= nk; kt += 2) {
-    slab(std::integral_constant<int, 0>{}, kt);
-    slab(std::integral_constant<int, 1>{}, kt + 1);
-  }
-  if (kt < nk) slab(std::integral_constant<int, 0>{}, kt);
-  __builtin_amdgcn_s_waitcnt(kWaitVm0);  // no copy may land in LDS after the epilogue starts to reuse it
-  __syncthreads();
 
-  // ---- epilogue ----------------------------------------------------------------
-  // The product was formed as W * X^T, so a lane holds one row m (= 32*mi + fc) and, per
-  // accumulator quad i, four consecutive output columns 8*i + 4*fg + j: eight bytes of
-  // bf16 that go to the wave's private staging area in LDS (free now: every wave is past
-  // the last barrier of the k loop) as one write.  The area holds a 128-row x 32-column
-  // tile, rows of 64 bytes with the 16-byte chunks swizzled by row; it is read back a row
-  // quarter per lane and stored with 16-byte writes, 64 contiguous bytes per row.
-  uint8_t* st = &lds[0][0] + wave * (kPfBM * 64);
-  float sc[4];
-#pragma unroll
-  for (int mi = 0; mi < 4; ++mi) sc[mi] = kGateUp ? 1.f : s_scale[mi * 32 + fc];
-#pragma unroll
-  for (int pass = 0; pass < (kGateUp ? 1 : 2); ++pass) {
-    if (pass) __syncthreads();  // staging rows are reused
-#pragma unroll
-    for (int mi = 0; mi < 4; ++mi) {
-      const int m = mi * 32 + fc;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        float v[4];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          if (kGateUp) {
-            const float g = round_bf16(acc[mi][0][4 * i + j]);
-            const float u = round_bf16(acc[mi][1][4 * i + j]);
-            v[j] = round_bf16(silu_f32(g)) * u;
-          } else {
-            v[j] = round_bf16(acc[mi][pass][4 * i + j]) * sc[mi];
+    const int fsw = ((fc >> 1) & 7) ^ ((fc & 1) << 2);
+    const int a_row = fc * kPfRowBytes, a_x = (fg ^ fsw) << 4;
+    int cur = 0, nxt2 = 2;  // buffer of slab kt, buffer of slab kt+2
+    auto slab = [&](auto stage_c, int kt) {
+      constexpr int st = decltype(stage_c)::value;
+      const int kt2 = min(kt + 2, nk - 1);
+      stage_slab(kt2, nxt2);
+      __builtin_amdgcn_sched_barrier(kPfSchedMask);
+      const uint8_t* la = lds[cur] + a_row;
+  #pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        bf16x8 fa[NMI];
+  #pragma unroll
+        for (int mi = 0; mi < NMI; ++mi)
+          fa[mi] = *reinterpret_cast<const bf16x8*>(la + mi * 32 * kPfRowBytes + (a_x ^ (s << 5)));
+  #pragma unroll
+        for (int mi = 0; mi < NMI; ++mi)
+  #pragma unroll
+          for (int ni = 0; ni < 2; ++ni)
+            acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfrag[st][ni][s], fa[mi], acc[mi][ni], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(kPfSchedMask);
+  #pragma unroll
+        for (int ni = 0; ni < 2; ++ni)
+          bfrag[st][ni][s] = *reinterpret_cast<const bf16x8*>(bptr[ni] + static_cast<size_t>(kt2) * 1024 + s * 128);
+        __builtin_amdgcn_sched_barrier(kPfSchedMask);
+      }
+      __builtin_amdgcn_s_waitcnt(kWaitVm20);
+      __syncthreads();
+      cur = (cur == kPfStages - 1) ? 0 : cur + 1;
+      nxt2 = (nxt2 == kPfStages - 1) ? 0 : nxt2 + 1;
+    };
+    // Slabs go in pairs with no branch inside the loop: a conditional second slab would give the
+    // loop head two different pictures of the outstanding fragment loads, and the waits the
+    // compiler puts before each MFMA would then assume the shorter one (eight loads behind
+    // instead of sixteen), i.e. drain the loads issued for the slab after next.
+    int kt = 0;
+    for (; kt + 2 <= nk; kt += 2) {
+      slab(std::integral_constant<int, 0>{}, kt);
+      slab(std::integral_constant<int, 1>{}, kt + 1);
+    }
+    if (kt < nk) slab(std::integral_constant<int, 0>{}, kt);
+    __builtin_amdgcn_s_waitcnt(kWaitVm0);  // no copy may land in LDS after the epilogue starts to reuse it
+    __syncthreads();
+
+    // ---- epilogue ----------------------------------------------------------------
+    // The product was formed as W * X^T, so a lane holds one row m (= 32*mi + fc) and, per
+    // accumulator quad i, four consecutive output columns 8*i + 4*fg + j: eight bytes of
+    // bf16 that go to the wave's private staging area in LDS (free now: every wave is past
+    // the last barrier of the k loop) as one write.  The area holds a 128-row x 32-column
+    // tile, rows of 64 bytes with the 16-byte chunks swizzled by row; it is read back a row
+    // quarter per lane and stored with 16-byte writes, 64 contiguous bytes per row.
+    uint8_t* st = &lds[0][0] + wave * (kPfBM * 64);
+    float sc[NMI];
+  #pragma unroll
+    for (int mi = 0; mi < NMI; ++mi) sc[mi] = kGateUp ? 1.f : s_scale[mi * 32 + fc];
+  #pragma unroll
+    for (int pass = 0; pass < (kGateUp ? 1 : 2); ++pass) {
+      if (pass) __syncthreads();  // staging rows are reused
+  #pragma unroll
+      for (int mi = 0; mi < NMI; ++mi) {
+        const int m = mi * 32 + fc;
+  #pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          float v[4];
+  #pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            if (kGateUp) {
+              const float g = round_bf16(acc[mi][0][4 * i + j]);
+              const float u = round_bf16(acc[mi][1][4 * i + j]);
+              v[j] = round_bf16(silu_f32(g)) * u;
+            } else {
+              v[j] = round_bf16(acc[mi][pass][4 * i + j]) * sc[mi];
+            }
           }
+          uint2 pk;
+          pk.x = f32x2_to_bf16x2_bits(v[0], v[1]);
+          pk.y = f32x2_to_bf16x2_bits(v[2], v[3]);
+          const int chunk = i ^ ((m >> 1) & 3);
+          *reinterpret_cast<uint2*>(st + m * 64 + chunk * 16 + fg * 8) = pk;
         }
-        uint2 pk;
-        pk.x = f32x2_to_bf16x2_bits(v[0], v[1]);
-        pk.y = f32x2_to_bf16x2_bits(v[2], v[3]);
-        const int chunk = i ^ ((m >> 1) & 3);
-        *reinterpret_cast<uint2*>(st + m * 64 + chunk * 16 + fg * 8) = pk;
+      }
+      __syncthreads();
+      const int ncol0 = kGateUp ? (n0 + wave * 32) : (n0 + wave * 64 + pass * 32);
+  #pragma unroll
+      for (int it = 0; it < 2 * NMI; ++it) {
+        const int m = it * 16 + (lane >> 2), q = lane & 3;
+        const uint4 val = *reinterpret_cast<const uint4*>(st + m * 64 + (q ^ ((m >> 1) & 3)) * 16);
+        const int n = ncol0 + q * 8;
+        if (m < M && n + 8 <= Ndim)
+          *reinterpret_cast<uint4*>(a.out + static_cast<size_t>(r0 + m) * Ndim + n) = val;
       }
     }
-    __syncthreads();
-    const int ncol0 = kGateUp ? (n0 + wave * 32) : (n0 + wave * 64 + pass * 32);
-#pragma unroll
-    for (int it = 0; it < 8; ++it) {
-      const int m = it * 16 + (lane >> 2), q = lane & 3;
-      const uint4 val = *reinterpret_cast<const uint4*>(st + m * 64 + (q ^ ((m >> 1) & 3)) * 16);
-      const int n = ncol0 + q * 8;
-      if (m < M && n + 8 <= Ndim)
-        *reinterpret_cast<uint4*>(a.out + static_cast<size_t>(r0 + m) * Ndim + n) = val;
-    }
+  };
+  switch ((M + 31) >> 5) {
+    case 1: body(std::integral_constant<int, 1>{}); break;
+    case 2: body(std::integral_constant<int, 2>{}); break;
+    case 3: body(std::integral_constant<int, 3>{}); break;
+    default: body(std::integral_constant<int, 4>{}); break;
   }
 }
 
