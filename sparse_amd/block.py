@@ -394,6 +394,29 @@ class DistributedSparseMoeBlock(nn.Module):
             DistributedSparseMoeBlock._shared_streams[key] = st
         return st
 
+    # ------------------------------------------------------------------ segment timing
+    def _segment_timing_on(self) -> bool:
+        """``SPARSE_EXPERT_TIMING=1``, read per call like the reference does (:14656)."""
+        return self.metrics is not None and os.environ.get("SPARSE_EXPERT_TIMING", "0").strip().lower() in (
+            "1", "true", "yes", "on")
+
+    def _timed_segment(self, name: str, fn, on: Optional[bool] = None):
+        """``_timed_segment`` (utils/eval_core.py:14655-14676): the segment between two events
+        on the compute stream, waited for at once, added to ``metrics.moe_<name>_ms``.  Timing
+        serialises the layer, so the block runs its one-stream, one-kernel-per-segment form
+        while it is on; the values do not change."""
+        if not (self._segment_timing_on() if on is None else on):
+            return fn()
+        start, end = ops.Event(timing=True), ops.Event(timing=True)
+        start.record()
+        out = fn()
+        end.record()
+        torch.cuda.current_stream().synchronize()
+        field = {"router": "moe_router_ms", "expert": "moe_expert_ms", "shared": "moe_shared_ms"}[name]
+        setattr(self.metrics, field, float(getattr(self.metrics, field, 0.0)) + start.elapsed_ms(end))
+        self.metrics.moe_timing_calls = int(getattr(self.metrics, "moe_timing_calls", 0)) + 1
+        return out
+
     # ------------------------------------------------------------------ routing
     def _route(self, x: torch.Tensor, ws: _Workspace, after_logits=None) -> torch.Tensor:
         """Router logits (+ shared gate), fused softmax/top-k, permutation (:9519-9595).
@@ -571,13 +594,14 @@ class DistributedSparseMoeBlock(nn.Module):
             rs_job = self._rs_begin(x, S, ws) if self._next_layer_rs_feature_mode() == "hidden" else None
 
         shared_gate = ws.shared_gate if self.shared_gate_weight is not None else None
+        timing = self._segment_timing_on()
         fused = (self.residency is None and self.shared_weights is not None and self.dtype == torch.bfloat16
-                 and T <= ops.DECODE_MAX_TOKENS)
+                 and T <= ops.DECODE_MAX_TOKENS and not timing)
         # Prefill-size batches: the shared expert needs only x and the shared gate, so it runs
         # on a second stream from the moment the logits kernel is queued, beside top-k,
         # permutation, tile map and the first routed tiles, and is joined before combine.
         side = (self._shared_stream() if self.shared_weights is not None and not fused and self.overlap_shared
-                and x.is_cuda and T > ops.DECODE_MAX_TOKENS else None)
+                and x.is_cuda and T > ops.DECODE_MAX_TOKENS and not timing else None)
 
         # Whether the shared expert's down projection is left as partial sums for the combine
         # step depends on the call's size and dtype only, never on where the routed experts
@@ -601,7 +625,11 @@ class DistributedSparseMoeBlock(nn.Module):
             with torch.cuda.stream(side):
                 ops.shared_expert(x, gw, uw, dw, shared_gate, ws.shared_inter, ws.shared_out)
 
-        if from_cache:
+        if timing:
+            # router, then (below) routed experts, then the shared expert: the reference's order
+            logits = self._timed_segment("router", lambda: (self._route_from_cache(x, ws) if from_cache
+                                                            else self._route(x, ws)), on=True)
+        elif from_cache:
             logits = self._route_from_cache(x, ws)
             run_shared()
         else:
@@ -612,34 +640,41 @@ class DistributedSparseMoeBlock(nn.Module):
 
         out = torch.empty((T, H), device=x.device, dtype=self.dtype)
         combined = False
-        if fused and split_shared and self.fold_combine:
-            # small decode call, everything resident: the down projection's launch also combines
-            ops.moe_ffn_decode_combine(self._experts_desc, x, ws.topv, ws.perm, ws.segs_dev, ws.inter, ws.parts,
-                                       self.shared_weights, shared_gate, ws.shared_inter, ws.split_ws, out)
-            combined = True
-        elif fused:
-            ops.moe_ffn_decode(self._experts_desc, x, ws.topv, ws.perm, ws.segs_dev, ws.inter, ws.parts,
-                               self.shared_weights, shared_gate, ws.shared_inter, ws.shared_out, ws.split_ws)
-        elif self.residency is None:
-            ops.grouped_swiglu(self._experts_desc, x, ws.topv, ws.perm, ws.segs_dev, ws.inter, ws.parts)
-        else:
-            ws.host_offsets.copy_(ws.perm.seg_offsets, non_blocking=True)
-            torch.cuda.current_stream().synchronize()
-            if rs_job is not None:
-                self._rs_finish(rs_job, ws)
-            off = ws.host_offsets.tolist()
-            segments = [(e, off[e + 1] - off[e]) for e in range(self.num_experts) if off[e + 1] > off[e]]
-            res = self.residency
-            res.phase, res.call_id = str(SparseContext.current_phase), int(SparseContext.runtime_call_id)
-            res.stage = self._current_stage(S)
-            self._backend.bind(x, ws)
-            if staged:
-                staging.seal(self, int(SparseContext.runtime_call_id))
-            try:
-                self.last_executor = res.execute(segments)
-            finally:
+
+        def run_experts() -> None:
+            nonlocal combined, rs_job
+            if fused and split_shared and self.fold_combine:
+                # small decode call, everything resident: the down projection's launch also combines
+                ops.moe_ffn_decode_combine(self._experts_desc, x, ws.topv, ws.perm, ws.segs_dev, ws.inter, ws.parts,
+                                           self.shared_weights, shared_gate, ws.shared_inter, ws.split_ws, out)
+                combined = True
+            elif fused:
+                ops.moe_ffn_decode(self._experts_desc, x, ws.topv, ws.perm, ws.segs_dev, ws.inter, ws.parts,
+                                   self.shared_weights, shared_gate, ws.shared_inter, ws.shared_out, ws.split_ws)
+            elif self.residency is None:
+                ops.grouped_swiglu(self._experts_desc, x, ws.topv, ws.perm, ws.segs_dev, ws.inter, ws.parts)
+            else:
+                ws.host_offsets.copy_(ws.perm.seg_offsets, non_blocking=True)
+                torch.cuda.current_stream().synchronize()
+                if rs_job is not None:
+                    self._rs_finish(rs_job, ws)
+                off = ws.host_offsets.tolist()
+                segments = [(e, off[e + 1] - off[e]) for e in range(self.num_experts) if off[e + 1] > off[e]]
+                res = self.residency
+                res.phase, res.call_id = str(SparseContext.current_phase), int(SparseContext.runtime_call_id)
+                res.stage = self._current_stage(S)
+                self._backend.bind(x, ws)
                 if staged:
-                    staging.settle(self)
+                    staging.seal(self, int(SparseContext.runtime_call_id))
+                try:
+                    self.last_executor = res.execute(segments)
+                finally:
+                    if staged:
+                        staging.settle(self)
+
+        self._timed_segment("expert", run_experts, on=timing)
+        if timing:
+            self._timed_segment("shared", run_shared, on=True)
         if self.residency is None and rs_job is not None:
             torch.cuda.current_stream().synchronize()
             self._rs_finish(rs_job, ws)

@@ -41,6 +41,12 @@ class Metrics:
     prefetch_budget_positive_count: int = 0
     rs_next_layer_pred_calls: int = 0
     rs_mlp_calls: int = 0
+    # device time of the three segments of a layer call, accumulated while
+    # SPARSE_EXPERT_TIMING=1 (utils/eval_core.py:1837-1840, :14655-14676)
+    moe_router_ms: float = 0.0
+    moe_expert_ms: float = 0.0
+    moe_shared_ms: float = 0.0
+    moe_timing_calls: int = 0
     counters: Dict[str, float] = field(default_factory=dict)
     # (kind, layer, expert) in issue order: kind in hit | prefetch_hit | miss
     events: Optional[List[Tuple[str, int, int]]] = None

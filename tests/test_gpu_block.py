@@ -348,6 +348,34 @@ def test_combine_folded_into_the_down_projection_gives_the_same_bits(device, sha
     assert int(ws.split_ws[off:].view(torch.int32).abs().sum().item()) == 0
 
 
+@pytest.mark.parametrize("T", [8, 300])
+def test_segment_timing_counters(device, monkeypatch, T):
+    """``SPARSE_EXPERT_TIMING=1`` (utils/eval_core.py:14655-14676): router, routed experts and
+    shared expert are timed one after the other into ``moe_{router,expert,shared}_ms``; the
+    output keeps its bits; without the switch nothing is counted."""
+    from sparse_amd.context import Metrics
+    from sparse_amd.synthetic import QWEN, make_hidden
+    metrics = Metrics()
+    _mlp, blk = _build(QWEN, torch.bfloat16, device, seed=5, metrics=metrics)
+    H = QWEN["hidden"]
+    x = make_hidden(T, H, torch.bfloat16, seed=77).view(T, 1, H).to(device)
+    want, want_logits = blk(x)
+    torch.cuda.synchronize()
+    assert metrics.moe_timing_calls == 0 and metrics.moe_expert_ms == 0.0
+    monkeypatch.setenv("SPARSE_EXPERT_TIMING", "1")
+    for _ in range(2):
+        got, got_logits = blk(x)
+    torch.cuda.synchronize()
+    assert torch.equal(got, want) and torch.equal(got_logits, want_logits)
+    assert metrics.moe_timing_calls == 6
+    assert metrics.moe_router_ms > 0 and metrics.moe_expert_ms > 0 and metrics.moe_shared_ms > 0
+    assert metrics.moe_router_ms + metrics.moe_expert_ms + metrics.moe_shared_ms < 1000
+    monkeypatch.delenv("SPARSE_EXPERT_TIMING")
+    again, _ = blk(x)
+    torch.cuda.synchronize()
+    assert torch.equal(again, want) and metrics.moe_timing_calls == 6
+
+
 @pytest.mark.parametrize("T", [1, 8, 32, 96])
 def test_decode_stack_in_a_hip_graph_replays_like_eager(device, T):
     """The decode path of a small stack captured into a HIP graph (one-launch router, fused FFN
