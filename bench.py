@@ -130,14 +130,23 @@ def decode_workload(blocks, shape, batch, steps, warmup, dtype, device, use_grap
     stats, mean_u = instrumented_pass(blocks, inputs, min(steps, 16))
     H, I, Is, K = shape["hidden"], shape["inter"], shape["shared_inter"], shape["top_k"]
     es = 2
-    # algorithmic bytes of one fused gate/up launch: the gate and up matrices of every
-    # distinct routed expert and of the shared expert, the token rows in, the products out
-    gu_bytes = mean_u * 2 * I * H * es + 2 * Is * H * es + batch * H * es + batch * K * I * es + batch * Is * es
+    from sparse_amd import ops
+    # calls of up to 16 tokens compute the shared expert's gate and up projections inside the
+    # routing launch; larger ones inside the gate/up launch
+    shared_in_route = bool(blocks[0].route_with_shared and blocks[0].gate_packed is not None
+                           and batch <= ops.ROUTE_PACKED_MAX_TOKENS and Is % 32 == 0)
+    shared_up_bytes = 2 * Is * H * es + batch * Is * es
+    # algorithmic bytes of one gate/up launch: the gate and up matrices of every distinct routed
+    # expert (and of the shared expert when they run here), the token rows in, the products out
+    gu_bytes = mean_u * 2 * I * H * es + batch * H * es + batch * K * I * es + (0 if shared_in_route else shared_up_bytes)
+    rt_bytes = 64 * H * es + batch * H * es + (shared_up_bytes if shared_in_route else 0)
     dn_bytes = mean_u * I * H * es + Is * H * es + batch * K * I * es + batch * Is * es + (batch * K + batch) * H * es
     gu_ms, gu_n, gu_name = stats["decode_gateup"]
     dn_ms, dn_n, _ = stats["decode_down"]
+    rt_ms, rt_n, _ = stats.get("route_decode", (0.0, 0, ""))
     gu_avg_s = gu_ms / max(1, gu_n) / 1e3
     dn_avg_s = dn_ms / max(1, dn_n) / 1e3
+    rt_avg_s = rt_ms / max(1, rt_n) / 1e3
     layer_bytes = mean_u * 3 * I * H * es + 3 * Is * H * es + shape["num_experts"] * H * es + H * es + \
         2 * batch * H * es
     ms_per_step = wall / steps * 1e3
@@ -149,6 +158,8 @@ def decode_workload(blocks, shape, batch, steps, warmup, dtype, device, use_grap
                     gbps=gu_bytes / gu_avg_s / 1e9 if gu_avg_s else 0.0),
         down=dict(launches=dn_n, avg_us=dn_avg_s * 1e6, bytes_per_launch=dn_bytes,
                   gbps=dn_bytes / dn_avg_s / 1e9 if dn_avg_s else 0.0),
+        route=dict(launches=rt_n, avg_us=rt_avg_s * 1e6, bytes_per_launch=rt_bytes,
+                   gbps=rt_bytes / rt_avg_s / 1e9 if rt_avg_s else 0.0, shared_gate_up_inside=shared_in_route),
         kernels_us={k: (v[0] / max(1, v[1]) * 1e3) for k, v in stats.items() if v[1]},
         graph=bool(use_graph),
     )
@@ -589,6 +600,7 @@ def main():
         "cpu_baseline": cpu,
         "step_hbm_frac": main_res["step_hbm_frac"],
         "kernels_us": main_res["kernels_us"],
+        "launches": {"gateup": main_res["gateup"], "down": main_res["down"], "route": main_res["route"]},
         "extra": extra,
     }
     print(json.dumps(line))

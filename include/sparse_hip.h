@@ -223,6 +223,26 @@ int sparse_hip_route_decode_packed(const void* x_dev, const void* gate_packed_de
                                    void* shared_gate_dev, void* topv_dev, int64_t* topi_dev, int32_t* perm_dev,
                                    int32_t* inv_perm_dev, int32_t* seg_offsets_dev, int32_t* active_eids_dev,
                                    int32_t* n_active_dev, void* stream);
+/* The same routing, and in the same launch the shared expert's gate and up projections with
+ * SiLU*up (which need the token rows only): shared_inter_dev [T, Is] = SiLU(x Wg^T) * (x Wu^T),
+ * rounded like the expert kernels round it.  Routing is one workgroup's work; the rest of the
+ * device reads the two matrices meanwhile instead of idling.  shared_gate_w_dev / shared_up_w_dev
+ * are [Is, H] in the tiled layout (sparse_hip_tile_weight), Is a multiple of 32.  The expert
+ * kernels are then called without these two matrices (NULL) and take shared_inter_dev as it is.
+ * Routing results are those of sparse_hip_route_decode_packed bit for bit.  No counterpart in
+ * the reference, whose block computes router and shared expert one after the other
+ * (utils/eval_core.py:16488, :16522-16525).
+ * sparse_hip_shared_gate_up is the shared expert's half alone (same kernel code, same bits),
+ * for a call that routes some other way; T <= SPARSE_HIP_ROUTE_PACKED_MAX_TOKENS, H % 64 == 0. */
+int sparse_hip_shared_gate_up(const void* x_dev, const void* shared_gate_w_dev, const void* shared_up_w_dev, int T,
+                              int H, int Is, void* shared_inter_dev, void* stream);
+int sparse_hip_route_decode_packed_shared(const void* x_dev, const void* gate_packed_dev, int has_shared_gate,
+                                          int logits_dtype, int T, int H, int E, int K, int renorm,
+                                          void* logits_dev, void* shared_gate_dev, void* topv_dev,
+                                          int64_t* topi_dev, int32_t* perm_dev, int32_t* inv_perm_dev,
+                                          int32_t* seg_offsets_dev, int32_t* active_eids_dev, int32_t* n_active_dev,
+                                          const void* shared_gate_w_dev, const void* shared_up_w_dev, int Is,
+                                          void* shared_inter_dev, void* stream);
 
 /* ---- A4/A6: grouped SwiGLU expert FFN -------------------------------------- */
 
@@ -265,7 +285,9 @@ int sparse_hip_grouped_swiglu_prefill(const sparse_hip_experts* experts, const v
  * dtype) -- `_shared_expert_forward` (utils/eval_core.py:9455-9463).
  * gate_s, up_s [Is,H], down_s [H,Is] (tiled); inter_ws [T,Is]; shared [T,H].
  * Uses the decode kernels when T <= SPARSE_HIP_DECODE_MAX_TOKENS, the prefill
- * kernels otherwise.
+ * kernels otherwise.  For a bf16 call of at most SPARSE_HIP_DECODE_MAX_TOKENS tokens gate_w_dev
+ * and up_w_dev may both be NULL: inter_ws then already holds act(gate_s x) * up_s x
+ * (sparse_hip_shared_gate_up) and only the down projection runs.
  */
 int sparse_hip_shared_expert(const void* x_dev, const void* gate_w_dev, const void* up_w_dev,
                              const void* down_w_dev, const void* shared_gate_dev, int dtype,
@@ -287,6 +309,9 @@ int sparse_hip_shared_expert(const void* x_dev, const void* gate_w_dev, const vo
  * fp32 partial sums [parts][T][H], and sparse_hip_combine_split finishes them (adds them in
  * their order, rounds, applies the shared gate) while it combines -- the same rounding steps
  * as the one-workgroup form, with the fp32 sum grouped differently.
+ * `sh_gate_w_dev` and `sh_up_w_dev` may both be NULL: `sh_inter_ws_dev` then already holds the
+ * shared expert's SiLU(gate x) * (up x) (sparse_hip_route_decode_packed_shared computes it beside
+ * the routing) and only the routed experts' gate/up projections run here.
  */
 size_t sparse_hip_decode_split_ws_bytes(int T, int H);
 int sparse_hip_decode_split_parts(int Is);

@@ -69,6 +69,10 @@ SIGNATURES = {
         _i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "sparse_hip_route_decode_packed": (
         _i, [_vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "sparse_hip_route_decode_packed_shared": (
+        _i, [_vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp,
+             _vp]),
+    "sparse_hip_shared_gate_up": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp, _vp]),
     "sparse_hip_permute_ws_bytes": (_sz, [_i, _i, _i]),
     "sparse_hip_permute_build": (_i, [_vp, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "sparse_hip_permute_build_static": (_i, [_vp, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp]),

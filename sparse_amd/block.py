@@ -286,6 +286,10 @@ class DistributedSparseMoeBlock(nn.Module):
         self.metrics = metrics if metrics is not None else Metrics()
         # all-resident decode calls of up to 16 tokens: combine inside the down projection's launch
         # (SPARSE_HIP_FOLD_COMBINE=0 keeps the separate combine launch; same bits either way)
+        self.route_with_shared = str(os.environ.get("SPARSE_HIP_ROUTE_WITH_SHARED", "1")).strip().lower() not in (
+            "0", "false", "no", "off")
+        self._shared_up_wanted = False      # forward: the call's expert launches can take a ready shared_inter
+        self._shared_inter_ready = False    # _route: this call's routing launch has filled it
         self.fold_combine = str(os.environ.get("SPARSE_HIP_FOLD_COMBINE", "1")).strip().lower() not in (
             "", "0", "false", "no", "off")
         # prefill-size batches run the shared expert on a second stream beside the routing
@@ -428,8 +432,13 @@ class DistributedSparseMoeBlock(nn.Module):
         shared_gate = ws.shared_gate if self.shared_gate_weight is not None else None
         one_launch = self.routed_scaling_factor == 1.0 and self.n_group == 1
         if self.gate_packed is not None and x.shape[0] <= ops.ROUTE_PACKED_MAX_TOKENS and one_launch:
+            # the routing launch also runs the shared expert's gate and up projections where it can
+            beside = self._shared_up_wanted
             ops.route_decode_packed(x, self.gate_packed, self.num_experts, self.shared_gate_weight is not None,
-                                    self.top_k, self.norm_topk_prob, logits, shared_gate, ws.topv, ws.topi, ws.perm)
+                                    self.top_k, self.norm_topk_prob, logits, shared_gate, ws.topv, ws.topi, ws.perm,
+                                    shared_up=(self.shared_weights[0], self.shared_weights[1], ws.shared_inter)
+                                    if beside else None)
+            self._shared_inter_ready = bool(beside)
             after_logits()
             return logits
         if x.shape[0] <= ops.DECODE_MAX_TOKENS and one_launch:
@@ -607,6 +616,20 @@ class DistributedSparseMoeBlock(nn.Module):
         # step depends on the call's size and dtype only, never on where the routed experts
         # live: an offloaded layer must give the bits of the all-resident one.
         split_shared = self.shared_weights is not None and ws.split_ws is not None
+        # Calls of up to 16 tokens compute the shared expert's gate and up projections with the
+        # 16-wavefront kernel, beside the routing when this call routes with the packed router,
+        # alone otherwise: the same code, so the same bits, wherever it runs.
+        shared_up_alone = (self.shared_weights is not None and self.dtype == torch.bfloat16 and x.is_cuda
+                           and self.route_with_shared and T <= ops.ROUTE_PACKED_MAX_TOKENS
+                           and self.shared_inter_size % 32 == 0 and H % 64 == 0)
+        self._shared_up_wanted = shared_up_alone and not timing
+        self._shared_inter_ready = False
+
+        def shared_inter_ready() -> bool:
+            if shared_up_alone and not self._shared_inter_ready:
+                ops.shared_gate_up(x, self.shared_weights[0], self.shared_weights[1], ws.shared_inter)
+                self._shared_inter_ready = True
+            return self._shared_inter_ready
 
         def run_shared() -> None:
             if self.shared_weights is None or fused:
@@ -616,10 +639,12 @@ class DistributedSparseMoeBlock(nn.Module):
                 # the fused decode entry point with no routed segment: the shared expert alone,
                 # in the same split form the all-resident call uses
                 ops.moe_ffn_decode(self._experts_desc, x, ws.topv, ws.perm, _NO_SEGMENTS(), ws.inter, ws.parts,
-                                   self.shared_weights, shared_gate, ws.shared_inter, ws.shared_out, ws.split_ws)
+                                   self.shared_weights, shared_gate, ws.shared_inter, ws.shared_out, ws.split_ws,
+                                   shared_inter_ready=shared_inter_ready())
                 return
             if side is None:
-                ops.shared_expert(x, gw, uw, dw, shared_gate, ws.shared_inter, ws.shared_out)
+                ops.shared_expert(x, gw, uw, dw, shared_gate, ws.shared_inter, ws.shared_out,
+                                  inter_ready=shared_inter_ready())
                 return
             side.wait_stream(torch.cuda.current_stream())
             with torch.cuda.stream(side):
@@ -646,11 +671,13 @@ class DistributedSparseMoeBlock(nn.Module):
             if fused and split_shared and self.fold_combine:
                 # small decode call, everything resident: the down projection's launch also combines
                 ops.moe_ffn_decode_combine(self._experts_desc, x, ws.topv, ws.perm, ws.segs_dev, ws.inter, ws.parts,
-                                           self.shared_weights, shared_gate, ws.shared_inter, ws.split_ws, out)
+                                           self.shared_weights, shared_gate, ws.shared_inter, ws.split_ws, out,
+                                           shared_inter_ready=shared_inter_ready())
                 combined = True
             elif fused:
                 ops.moe_ffn_decode(self._experts_desc, x, ws.topv, ws.perm, ws.segs_dev, ws.inter, ws.parts,
-                                   self.shared_weights, shared_gate, ws.shared_inter, ws.shared_out, ws.split_ws)
+                                   self.shared_weights, shared_gate, ws.shared_inter, ws.shared_out, ws.split_ws,
+                                   shared_inter_ready=shared_inter_ready())
             elif self.residency is None:
                 ops.grouped_swiglu(self._experts_desc, x, ws.topv, ws.perm, ws.segs_dev, ws.inter, ws.parts)
             else:

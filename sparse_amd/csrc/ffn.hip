@@ -129,8 +129,9 @@ int sparse_hip_moe_ffn_decode(const sparse_hip_experts* experts, const void* x_d
   SP_REQUIRE(T <= SPARSE_HIP_DECODE_MAX_TOKENS, "moe_ffn_decode: T=%d exceeds %d", T,
              SPARSE_HIP_DECODE_MAX_TOKENS);
   SP_REQUIRE(Is > 0 && Is % 64 == 0, "moe_ffn_decode: Is=%d must be a positive multiple of 64", Is);
-  SP_REQUIRE(sh_gate_w_dev && sh_up_w_dev && sh_down_w_dev && sh_inter_ws_dev && shared_dev,
-             "moe_ffn_decode: NULL shared-expert pointer");
+  SP_REQUIRE(sh_down_w_dev && sh_inter_ws_dev && shared_dev, "moe_ffn_decode: NULL shared-expert pointer");
+  SP_REQUIRE((sh_gate_w_dev == nullptr) == (sh_up_w_dev == nullptr),
+             "moe_ffn_decode: shared gate and up projections are given together or not at all");
   SP_REQUIRE(((reinterpret_cast<uintptr_t>(sh_gate_w_dev) | reinterpret_cast<uintptr_t>(sh_up_w_dev) |
                reinterpret_cast<uintptr_t>(sh_down_w_dev) | reinterpret_cast<uintptr_t>(sh_inter_ws_dev) |
                reinterpret_cast<uintptr_t>(shared_dev) | reinterpret_cast<uintptr_t>(split_ws_dev)) &
@@ -156,8 +157,10 @@ int sparse_hip_moe_ffn_decode_combine(const sparse_hip_experts* experts, const v
   SP_REQUIRE(Is > 0 && Is % 64 == 0, "moe_ffn_decode_combine: Is=%d must be a positive multiple of 64", Is);
   SP_REQUIRE(decode_split_parts(Is) > 1,
              "moe_ffn_decode_combine: Is=%d cannot be cut into parts; use sparse_hip_moe_ffn_decode + sparse_hip_combine", Is);
-  SP_REQUIRE(sh_gate_w_dev && sh_up_w_dev && sh_down_w_dev && sh_inter_ws_dev && split_ws_dev && inv_perm_dev && out_dev,
+  SP_REQUIRE(sh_down_w_dev && sh_inter_ws_dev && split_ws_dev && inv_perm_dev && out_dev,
              "moe_ffn_decode_combine: NULL pointer");
+  SP_REQUIRE((sh_gate_w_dev == nullptr) == (sh_up_w_dev == nullptr),
+             "moe_ffn_decode_combine: shared gate and up projections are given together or not at all");
   SP_REQUIRE(((reinterpret_cast<uintptr_t>(sh_gate_w_dev) | reinterpret_cast<uintptr_t>(sh_up_w_dev) |
                reinterpret_cast<uintptr_t>(sh_down_w_dev) | reinterpret_cast<uintptr_t>(sh_inter_ws_dev) |
                reinterpret_cast<uintptr_t>(out_dev) | reinterpret_cast<uintptr_t>(split_ws_dev)) &
@@ -188,8 +191,11 @@ int sparse_hip_shared_expert(const void* x_dev, const void* gate_w_dev, const vo
   SP_REQUIRE(T >= 1, "shared_expert: T=%d must be >= 1", T);
   SP_REQUIRE(H > 0 && H % 64 == 0 && Is > 0 && Is % 64 == 0,
              "shared_expert: H=%d and Is=%d must be positive multiples of 64", H, Is);
-  SP_REQUIRE(x_dev && gate_w_dev && up_w_dev && down_w_dev && inter_ws_dev && shared_dev,
-             "shared_expert: NULL pointer");
+  SP_REQUIRE(x_dev && down_w_dev && inter_ws_dev && shared_dev, "shared_expert: NULL pointer");
+  SP_REQUIRE((gate_w_dev == nullptr) == (up_w_dev == nullptr),
+             "shared_expert: gate and up projections are given together or not at all");
+  SP_REQUIRE(gate_w_dev != nullptr || (dtype == SPARSE_HIP_BF16 && T <= SPARSE_HIP_DECODE_MAX_TOKENS),
+             "shared_expert: only a bf16 call of up to %d tokens can take a ready inter_ws", SPARSE_HIP_DECODE_MAX_TOKENS);
   SP_REQUIRE(((reinterpret_cast<uintptr_t>(x_dev) | reinterpret_cast<uintptr_t>(gate_w_dev) |
                reinterpret_cast<uintptr_t>(up_w_dev) | reinterpret_cast<uintptr_t>(down_w_dev) |
                reinterpret_cast<uintptr_t>(inter_ws_dev) | reinterpret_cast<uintptr_t>(shared_dev)) &

@@ -497,7 +497,7 @@ constexpr int kRpTok = SPARSE_HIP_ROUTE_PACKED_MAX_TOKENS;
 static_assert(kRpTok == kRouteWaves && SPARSE_HIP_ROUTE_PACKED_ROWS == kRlRows, "one wavefront per token, four 16-row groups");
 
 template <typename TL>
-__global__ __launch_bounds__(kRouteThreads) void route_decode_packed_kernel(const RouteArgs a) {
+__device__ __forceinline__ void route_packed_block(const RouteArgs& a) {
   __shared__ float part[kRouteWaves / 2][kRpTok][kRlPad];
   __shared__ float s_logit[kRpTok][kRlRows];
   __shared__ int64_t s_topi[kRpTok * SPARSE_HIP_MAX_TOPK];
@@ -585,6 +585,117 @@ __global__ __launch_bounds__(kRouteThreads) void route_decode_packed_kernel(cons
   }
   __syncthreads();
   permute_small_block(s_topi, T, a.K, E, a.perm, a.inv_perm, a.seg_offsets, a.active_eids, a.n_active);
+}
+
+template <typename TL>
+__global__ __launch_bounds__(kRouteThreads) void route_decode_packed_kernel(const RouteArgs a) {
+  route_packed_block<TL>(a);
+}
+
+// ---------------------------------------------------------------------------
+// The same routing workgroup, and beside it -- routing is one workgroup's work and leaves the
+// memory system idle -- the shared expert's gate and up projections with SiLU*up, which need
+// the token rows only: workgroup 1 + j computes rows 32 j .. 32 j + 31 of both matrices for
+// all (at most 16) tokens.  Its 16 wavefronts cut the reduction into 64-wide slices dealt
+// round-robin and request every slice they own before the first MFMA, so the whole of the two
+// matrices is in flight at once; the 16 partial tiles meet in LDS and are added in wavefront
+// order.  Operand layouts, the tiled weight format and the epilogue's roundings are those of
+// the decode expert kernel (swiglu_decode.hip).
+// ---------------------------------------------------------------------------
+struct SharedUpArgs {
+  const uint16_t* gate_w;   // [Is, H] tiled
+  const uint16_t* up_w;     // [Is, H] tiled
+  const uint16_t* x;        // [T, H]
+  uint16_t* inter;          // [T, Is]: silu(gate x) * (up x)
+  int32_t T, H, Is;
+};
+
+constexpr int kSuRows = 32;   // output rows per workgroup: two 16-row MFMA tiles
+
+__device__ __forceinline__ void shared_gateup_block(const SharedUpArgs& s, int tile) {
+  __shared__ f32x4 red[kRouteWaves][4][64];   // [wavefront][2 * row tile + matrix][lane]
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int r = lane & 15, q = lane >> 4;
+  const int H = s.H, ND = H >> 6;
+  const size_t group_stride = static_cast<size_t>(16) * H;
+  const uint16_t* wt[2] = {s.gate_w + static_cast<size_t>(tile * 2) * group_stride + lane * 8,
+                           s.up_w + static_cast<size_t>(tile * 2) * group_stride + lane * 8};
+  // token column r (columns past T read token 0: their products are never stored)
+  const uint16_t* brow = s.x + static_cast<size_t>(r < s.T ? r : 0) * H + (q << 4);
+  f32x4 acc[2][2];   // [row tile][matrix]
+#pragma unroll
+  for (int tl = 0; tl < 2; ++tl)
+#pragma unroll
+    for (int m = 0; m < 2; ++m) acc[tl][m] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int d0 = wave; d0 < ND; d0 += 2 * kRouteWaves) {
+    const int d1 = d0 + kRouteWaves;           // this wavefront's next slice, if there is one
+    const int dd[2] = {d0, d1 < ND ? d1 : d0};
+    bf16x8 b[2][2], w[2][2][2][2];             // [slice][k half], [slice][row tile][matrix][k half]
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      b[j][0] = *reinterpret_cast<const bf16x8*>(brow + (dd[j] << 6));
+      b[j][1] = *reinterpret_cast<const bf16x8*>(brow + (dd[j] << 6) + 8);
+#pragma unroll
+      for (int tl = 0; tl < 2; ++tl)
+#pragma unroll
+        for (int m = 0; m < 2; ++m) {
+          const uint16_t* p = wt[m] + tl * group_stride + (static_cast<size_t>(dd[j]) << 10);
+          w[j][tl][m][0] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(p));
+          w[j][tl][m][1] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(p + 512));
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);          // all 20 loads in flight before the first MFMA
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      if (j == 1 && d1 >= ND) break;
+#pragma unroll
+      for (int tl = 0; tl < 2; ++tl)
+#pragma unroll
+        for (int m = 0; m < 2; ++m) {
+          acc[tl][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[j][tl][m][0], b[j][0], acc[tl][m], 0, 0, 0);
+          acc[tl][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[j][tl][m][1], b[j][1], acc[tl][m], 0, 0, 0);
+        }
+    }
+  }
+#pragma unroll
+  for (int tl = 0; tl < 2; ++tl)
+#pragma unroll
+    for (int m = 0; m < 2; ++m) red[wave][tl * 2 + m][lane] = acc[tl][m];
+  __syncthreads();
+  // wavefront tl finishes row tile tl: lane (r, q) holds rows 4 q .. 4 q + 3 of token r
+  if (wave < 2 && r < s.T) {
+    const int tl = wave;
+    f32x4 g = red[0][tl * 2][lane], u = red[0][tl * 2 + 1][lane];
+#pragma unroll
+    for (int w2 = 1; w2 < kRouteWaves; ++w2) {
+      g += red[w2][tl * 2][lane];
+      u += red[w2][tl * 2 + 1][lane];
+    }
+    uint16_t o[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float gv = round_bf16(g[j]), uv = round_bf16(u[j]);
+      o[j] = f32_to_bf16_bits(round_bf16(silu_f32(gv)) * uv);
+    }
+    uint2 pk;
+    pk.x = static_cast<uint32_t>(o[0]) | (static_cast<uint32_t>(o[1]) << 16);
+    pk.y = static_cast<uint32_t>(o[2]) | (static_cast<uint32_t>(o[3]) << 16);
+    *reinterpret_cast<uint2*>(s.inter + static_cast<size_t>(r) * s.Is + tile * kSuRows + tl * 16 + q * 4) = pk;
+  }
+}
+
+// the shared expert's half alone, for callers that route some other way
+__global__ __launch_bounds__(kRouteThreads) void shared_gateup_kernel(const SharedUpArgs s) {
+  shared_gateup_block(s, static_cast<int>(blockIdx.x));
+}
+
+template <typename TL>
+__global__ __launch_bounds__(kRouteThreads) void route_packed_shared_kernel(const RouteArgs a, const SharedUpArgs s) {
+  if (blockIdx.x == 0) {
+    route_packed_block<TL>(a);
+  } else {
+    shared_gateup_block(s, static_cast<int>(blockIdx.x) - 1);
+  }
 }
 
 template <typename T, typename TL>
@@ -726,11 +837,10 @@ int sparse_hip_route_decode(const void* x_dev, const void* wg_dev, const void* w
   return launch_route_decode<uint16_t, uint16_t>(a, st);
 }
 
-int sparse_hip_route_decode_packed(const void* x_dev, const void* gate_packed_dev, int has_shared_gate,
-                                   int logits_dtype, int T, int H, int E, int K, int renorm, void* logits_dev,
-                                   void* shared_gate_dev, void* topv_dev, int64_t* topi_dev, int32_t* perm_dev,
-                                   int32_t* inv_perm_dev, int32_t* seg_offsets_dev, int32_t* active_eids_dev,
-                                   int32_t* n_active_dev, void* stream) {
+static int route_packed_impl(const void* x_dev, const void* gate_packed_dev, int has_shared_gate, int logits_dtype, int T,
+                             int H, int E, int K, int renorm, void* logits_dev, void* shared_gate_dev, void* topv_dev,
+                             int64_t* topi_dev, int32_t* perm_dev, int32_t* inv_perm_dev, int32_t* seg_offsets_dev,
+                             int32_t* active_eids_dev, int32_t* n_active_dev, const SharedUpArgs* shared, void* stream) {
   SP_REQUIRE(logits_dtype == SPARSE_HIP_BF16 || logits_dtype == SPARSE_HIP_F32,
              "route_decode_packed: logits_dtype must be bf16 or fp32");
   SP_REQUIRE(T >= 1 && T <= SPARSE_HIP_ROUTE_PACKED_MAX_TOKENS, "route_decode_packed: T=%d outside [1,%d]", T,
@@ -750,6 +860,16 @@ int sparse_hip_route_decode_packed(const void* x_dev, const void* gate_packed_de
                  T,        H,               E,               K,               renorm,          has_shared_gate ? 1 : 0};
   hipStream_t st = as_stream(stream);
   ProfScope prof(SPARSE_HIP_K_ROUTE_DECODE, st);
+  if (shared != nullptr) {
+    const dim3 grid(1 + shared->Is / kSuRows);
+    if (logits_dtype == SPARSE_HIP_F32) {
+      hipLaunchKernelGGL((route_packed_shared_kernel<float>), grid, dim3(kRouteThreads), 0, st, a, *shared);
+    } else {
+      hipLaunchKernelGGL((route_packed_shared_kernel<uint16_t>), grid, dim3(kRouteThreads), 0, st, a, *shared);
+    }
+    SP_LAUNCH_CHECK("route_packed_shared_kernel");
+    return SPARSE_HIP_OK;
+  }
   if (logits_dtype == SPARSE_HIP_F32) {
     hipLaunchKernelGGL((route_decode_packed_kernel<float>), dim3(1), dim3(kRouteThreads), 0, st, a);
   } else {
@@ -757,6 +877,48 @@ int sparse_hip_route_decode_packed(const void* x_dev, const void* gate_packed_de
   }
   SP_LAUNCH_CHECK("route_decode_packed_kernel");
   return SPARSE_HIP_OK;
+}
+
+int sparse_hip_route_decode_packed(const void* x_dev, const void* gate_packed_dev, int has_shared_gate,
+                                   int logits_dtype, int T, int H, int E, int K, int renorm, void* logits_dev,
+                                   void* shared_gate_dev, void* topv_dev, int64_t* topi_dev, int32_t* perm_dev,
+                                   int32_t* inv_perm_dev, int32_t* seg_offsets_dev, int32_t* active_eids_dev,
+                                   int32_t* n_active_dev, void* stream) {
+  return route_packed_impl(x_dev, gate_packed_dev, has_shared_gate, logits_dtype, T, H, E, K, renorm, logits_dev,
+                           shared_gate_dev, topv_dev, topi_dev, perm_dev, inv_perm_dev, seg_offsets_dev,
+                           active_eids_dev, n_active_dev, nullptr, stream);
+}
+
+int sparse_hip_shared_gate_up(const void* x_dev, const void* shared_gate_w_dev, const void* shared_up_w_dev, int T,
+                              int H, int Is, void* shared_inter_dev, void* stream) {
+  SP_REQUIRE(x_dev && shared_gate_w_dev && shared_up_w_dev && shared_inter_dev, "shared_gate_up: NULL pointer");
+  SP_REQUIRE(T >= 1 && T <= SPARSE_HIP_ROUTE_PACKED_MAX_TOKENS, "shared_gate_up: T=%d outside [1,%d]", T,
+             SPARSE_HIP_ROUTE_PACKED_MAX_TOKENS);
+  SP_REQUIRE(H > 0 && H % 64 == 0, "shared_gate_up: H=%d must be a positive multiple of 64", H);
+  SP_REQUIRE(Is > 0 && Is % kSuRows == 0, "shared_gate_up: Is=%d must be a positive multiple of %d", Is, kSuRows);
+  SharedUpArgs s = {static_cast<const uint16_t*>(shared_gate_w_dev), static_cast<const uint16_t*>(shared_up_w_dev),
+                    static_cast<const uint16_t*>(x_dev), static_cast<uint16_t*>(shared_inter_dev), T, H, Is};
+  hipStream_t st = as_stream(stream);
+  hipLaunchKernelGGL(shared_gateup_kernel, dim3(Is / kSuRows), dim3(kRouteThreads), 0, st, s);
+  SP_LAUNCH_CHECK("shared_gateup_kernel");
+  return SPARSE_HIP_OK;
+}
+
+int sparse_hip_route_decode_packed_shared(const void* x_dev, const void* gate_packed_dev, int has_shared_gate,
+                                          int logits_dtype, int T, int H, int E, int K, int renorm,
+                                          void* logits_dev, void* shared_gate_dev, void* topv_dev,
+                                          int64_t* topi_dev, int32_t* perm_dev, int32_t* inv_perm_dev,
+                                          int32_t* seg_offsets_dev, int32_t* active_eids_dev, int32_t* n_active_dev,
+                                          const void* shared_gate_w_dev, const void* shared_up_w_dev, int Is,
+                                          void* shared_inter_dev, void* stream) {
+  SP_REQUIRE(shared_gate_w_dev && shared_up_w_dev && shared_inter_dev, "route_decode_packed_shared: NULL pointer");
+  SP_REQUIRE(Is > 0 && Is % kSuRows == 0, "route_decode_packed_shared: Is=%d must be a positive multiple of %d", Is,
+             kSuRows);
+  SharedUpArgs s = {static_cast<const uint16_t*>(shared_gate_w_dev), static_cast<const uint16_t*>(shared_up_w_dev),
+                    static_cast<const uint16_t*>(x_dev), static_cast<uint16_t*>(shared_inter_dev), T, H, Is};
+  return route_packed_impl(x_dev, gate_packed_dev, has_shared_gate, logits_dtype, T, H, E, K, renorm, logits_dev,
+                           shared_gate_dev, topv_dev, topi_dev, perm_dev, inv_perm_dev, seg_offsets_dev,
+                           active_eids_dev, n_active_dev, &s, stream);
 }
 
 }  // extern "C"

@@ -505,7 +505,8 @@ int decode_fused_bf16(const sparse_hip_experts* ex, const void* x, const void* t
   a.out_s = static_cast<uint16_t*>(sh_inter_ws);
   a.Kdim_s = static_cast<int32_t>(H);
   a.Ndim_s = Is;
-  a.tiles_s = Is / kDecRows;
+  // no gate / up matrices: sh_inter_ws already holds the shared expert's SiLU(gate x) * (up x)
+  a.tiles_s = sh_gate_w != nullptr ? Is / kDecRows : 0;
   int rc = launch_decode<true>(a, segs->n, st);
   if (rc != SPARSE_HIP_OK) return rc;
   // down
@@ -563,8 +564,10 @@ int decode_shared_bf16(const void* x, const void* gate_w, const void* up_w, cons
   a.Kdim_s = H;
   a.Ndim_s = Is;
   a.tiles_s = Is / kDecRows;
-  int rc = launch_decode<true>(a, 0, st);
-  if (rc != SPARSE_HIP_OK) return rc;
+  if (gate_w != nullptr) {  // else inter_ws already holds SiLU(gate x) * (up x)
+    int rc = launch_decode<true>(a, 0, st);
+    if (rc != SPARSE_HIP_OK) return rc;
+  }
   a.w_s = static_cast<const uint16_t*>(down_w);
   a.w2_s = nullptr;
   a.act_s = static_cast<const uint16_t*>(inter_ws);

@@ -191,9 +191,11 @@ def pack_router_gate(wg: torch.Tensor, wsg: Optional[torch.Tensor]) -> Optional[
 
 def route_decode_packed(x: torch.Tensor, gate_packed: torch.Tensor, num_experts: int, has_shared_gate: bool, k: int,
                         renorm: bool, logits: torch.Tensor, shared_gate: Optional[torch.Tensor], topv: torch.Tensor,
-                        topi: torch.Tensor, perm: Permutation) -> None:
+                        topi: torch.Tensor, perm: Permutation, shared_up=None) -> None:
     """Router logits + top-k + permutation of up to 16 bf16 tokens by one workgroup, on the
-    matrix ``pack_router_gate`` made."""
+    matrix ``pack_router_gate`` made.  ``shared_up = (gate_w, up_w, inter_out)``: the same launch
+    also computes the shared expert's SiLU(gate x) * (up x) into ``inter_out [T, Is]`` (tiled
+    weights ``[Is, H]``, Is a multiple of 32), on the part of the device routing leaves idle."""
     lib = _lib.load()
     T, H = x.shape
     E = int(num_experts)
@@ -204,12 +206,32 @@ def route_decode_packed(x: torch.Tensor, gate_packed: torch.Tensor, num_experts:
     _need(topi, "topi", torch.int64, (T, k))
     if has_shared_gate:
         _need(shared_gate, "shared gate logits", x.dtype, (T,))
-    rc = lib.sparse_hip_route_decode_packed(_ptr(x), _ptr(gate_packed), int(bool(has_shared_gate)),
-                                            dtype_code(logits.dtype), T, H, E, int(k), int(bool(renorm)),
-                                            _ptr(logits), _ptr(shared_gate), _ptr(topv), _ptr(topi),
-                                            _ptr(perm.perm), _ptr(perm.inv_perm), _ptr(perm.seg_offsets),
-                                            _ptr(perm.active_eids), _ptr(perm.n_active), _stream())
-    _lib.check(rc, "sparse_hip_route_decode_packed")
+    common = (_ptr(x), _ptr(gate_packed), int(bool(has_shared_gate)), dtype_code(logits.dtype), T, H, E, int(k),
+              int(bool(renorm)), _ptr(logits), _ptr(shared_gate), _ptr(topv), _ptr(topi), _ptr(perm.perm),
+              _ptr(perm.inv_perm), _ptr(perm.seg_offsets), _ptr(perm.active_eids), _ptr(perm.n_active))
+    if shared_up is None:
+        _lib.check(lib.sparse_hip_route_decode_packed(*common, _stream()), "sparse_hip_route_decode_packed")
+        return
+    gw, uw, inter = shared_up
+    Is = int(gw.shape[0])
+    _need(gw, "shared gate_proj", x.dtype, (Is, H))
+    _need(uw, "shared up_proj", x.dtype, (Is, H))
+    _need(inter, "shared inter_ws", x.dtype, (T, Is))
+    _lib.check(lib.sparse_hip_route_decode_packed_shared(*common, _ptr(gw), _ptr(uw), Is, _ptr(inter), _stream()),
+               "sparse_hip_route_decode_packed_shared")
+
+
+def shared_gate_up(x: torch.Tensor, gate_w: torch.Tensor, up_w: torch.Tensor, inter_out: torch.Tensor) -> None:
+    """The shared expert's SiLU(gate x) * (up x) for up to 16 bf16 tokens, by the kernel code
+    ``route_decode_packed(shared_up=...)`` runs beside the routing (same bits)."""
+    T, H = x.shape
+    Is = int(gate_w.shape[0])
+    _need(x, "x", torch.bfloat16)
+    _need(gate_w, "shared gate_proj", x.dtype, (Is, H))
+    _need(up_w, "shared up_proj", x.dtype, (Is, H))
+    _need(inter_out, "shared inter_ws", x.dtype, (T, Is))
+    _lib.check(_lib.load().sparse_hip_shared_gate_up(_ptr(x), _ptr(gate_w), _ptr(up_w), T, H, Is, _ptr(inter_out),
+                                                     _stream()), "sparse_hip_shared_gate_up")
 
 
 # --------------------------------------------------------------------------- experts
@@ -290,7 +312,10 @@ def prefill_tile_ws(T: int, K: int, num_segments: int, hidden: int, inter: int, 
 
 
 def shared_expert(x: torch.Tensor, gate_w: torch.Tensor, up_w: torch.Tensor, down_w: torch.Tensor,
-                  shared_gate: Optional[torch.Tensor], inter_ws: torch.Tensor, out: torch.Tensor) -> None:
+                  shared_gate: Optional[torch.Tensor], inter_ws: torch.Tensor, out: torch.Tensor,
+                  inter_ready: bool = False) -> None:
+    """The shared expert.  ``inter_ready``: ``inter_ws`` already holds SiLU(gate x) * (up x)
+    (bf16 calls of up to 32 tokens), only the down projection runs."""
     lib = _lib.load()
     T, H = x.shape
     Is = gate_w.shape[0]
@@ -304,7 +329,8 @@ def shared_expert(x: torch.Tensor, gate_w: torch.Tensor, up_w: torch.Tensor, dow
         _need(shared_gate, "shared gate logits", x.dtype)
         if shared_gate.numel() != T:
             raise ValueError("shared gate logits must hold T elements")
-    rc = lib.sparse_hip_shared_expert(_ptr(x), _ptr(gate_w), _ptr(up_w), _ptr(down_w), _ptr(shared_gate),
+    rc = lib.sparse_hip_shared_expert(_ptr(x), None if inter_ready else _ptr(gate_w),
+                                      None if inter_ready else _ptr(up_w), _ptr(down_w), _ptr(shared_gate),
                                       dtype_code(x.dtype), T, H, Is, _ptr(inter_ws), _ptr(out), _stream())
     _lib.check(rc, "sparse_hip_shared_expert")
 
@@ -449,10 +475,12 @@ def profile_read() -> dict:
 def moe_ffn_decode(experts: Experts, x: torch.Tensor, topv: torch.Tensor, perm: Permutation, segs: SegList,
                    inter_ws: torch.Tensor, parts: torch.Tensor, shared_w, shared_gate: Optional[torch.Tensor],
                    shared_inter_ws: torch.Tensor, shared_out: torch.Tensor,
-                   split_ws: Optional[torch.Tensor] = None) -> None:
+                   split_ws: Optional[torch.Tensor] = None, shared_inter_ready: bool = False) -> None:
     """Routed experts + shared expert of a decode call in one launch pair (bf16, T <= 32).
     ``split_ws`` (from ``decode_split_workspace``) lets the shared down projection spread its
-    long reduction over four workgroups per tile."""
+    long reduction over four workgroups per tile.  ``shared_inter_ready``: ``shared_inter_ws``
+    already holds the shared expert's SiLU(gate x) * (up x) (``route_decode_packed`` computed it
+    beside the routing), so its gate and up projections are not run again."""
     lib = _lib.load()
     T, H = x.shape
     K = topv.shape[1]
@@ -473,8 +501,9 @@ def moe_ffn_decode(experts: Experts, x: torch.Tensor, topv: torch.Tensor, perm: 
             raise ValueError("split workspace is too small for this T and H")
     rc = lib.sparse_hip_moe_ffn_decode(C.byref(experts), _ptr(x), _ptr(topv), _ptr(perm.perm),
                                        _ptr(perm.seg_offsets), C.byref(segs), T, K, _ptr(inter_ws), _ptr(parts),
-                                       _ptr(gw), _ptr(uw), _ptr(dw), _ptr(shared_gate), Is, _ptr(shared_inter_ws),
-                                       _ptr(shared_out), _ptr(split_ws), _stream())
+                                       None if shared_inter_ready else _ptr(gw),
+                                       None if shared_inter_ready else _ptr(uw), _ptr(dw), _ptr(shared_gate), Is,
+                                       _ptr(shared_inter_ws), _ptr(shared_out), _ptr(split_ws), _stream())
     _lib.check(rc, "sparse_hip_moe_ffn_decode")
 
 
@@ -489,7 +518,8 @@ def decode_split_workspace(T: int, H: int, device) -> torch.Tensor:
 
 def moe_ffn_decode_combine(experts: Experts, x: torch.Tensor, topv: torch.Tensor, perm: Permutation, segs: SegList,
                            inter_ws: torch.Tensor, parts: torch.Tensor, shared_w, shared_gate: Optional[torch.Tensor],
-                           shared_inter_ws: torch.Tensor, split_ws: torch.Tensor, out: torch.Tensor) -> None:
+                           shared_inter_ws: torch.Tensor, split_ws: torch.Tensor, out: torch.Tensor,
+                           shared_inter_ready: bool = False) -> None:
     """``moe_ffn_decode`` with the combine step folded into the down projection's launch:
     writes the layer's expert output ``out [T,H]`` (routed sum + shared expert)."""
     lib = _lib.load()
@@ -511,7 +541,8 @@ def moe_ffn_decode_combine(experts: Experts, x: torch.Tensor, topv: torch.Tensor
         raise ValueError("split workspace is too small for this T and H")
     rc = lib.sparse_hip_moe_ffn_decode_combine(
         C.byref(experts), _ptr(x), _ptr(topv), _ptr(perm.perm), _ptr(perm.inv_perm), _ptr(perm.seg_offsets),
-        C.byref(segs), T, K, _ptr(inter_ws), _ptr(parts), _ptr(gw), _ptr(uw), _ptr(dw), _ptr(shared_gate), Is,
+        C.byref(segs), T, K, _ptr(inter_ws), _ptr(parts), None if shared_inter_ready else _ptr(gw),
+        None if shared_inter_ready else _ptr(uw), _ptr(dw), _ptr(shared_gate), Is,
         _ptr(shared_inter_ws), _ptr(split_ws), _ptr(out), _stream())
     _lib.check(rc, "sparse_hip_moe_ffn_decode_combine")
 

@@ -264,6 +264,64 @@ def test_route_decode_packed_shapes(device, T, H, E, K, shared_gate, renorm, ldt
         assert torch.equal(topi.cpu(), ref_i)
 
 
+@pytest.mark.parametrize("T,H,E,K,Is", [(1, 2048, 60, 4, 5632), (8, 2048, 60, 4, 5632), (16, 2048, 63, 6, 2816),
+                                        (5, 192, 15, 3, 96), (13, 4096, 62, 2, 64), (7, 4160, 33, 4, 32)])
+def test_route_decode_packed_with_the_shared_gate_up_beside_it(device, T, H, E, K, Is):
+    """The routing launch that also computes the shared expert's SiLU(gate x) * (up x): routing
+    results bit for bit those of the routing-only launch; the activation equal to fp32 linear
+    algebra rounded the way the expert kernels round (gate and up to bf16, SiLU to bf16, the
+    product to bf16) within two bf16 steps (a sum that lands on the other side of a rounding
+    boundary moves gate or up by one step each), and to what the decode expert kernel writes for
+    the same weights within the same bound (their fp32 sums are grouped differently); H from three
+    64-wide blocks to more than two per wavefront, T up to the launch's 16 tokens."""
+    from sparse_amd.weights import tile_weight
+    ops = _ops()
+    dtype = torch.bfloat16
+    layer = make_layer(H, E, 64, K, Is=Is, shared_gate=True, dtype=dtype, seed=71 + T, std=0.05)
+    packed = ops.pack_router_gate(layer["gate_w"].to(device), layer["shared_gate_w"].to(device))
+    gw, uw = (tile_weight(w.to(device)).reshape(w.shape).contiguous() for w in layer["shared"][:2])
+    x = make_hidden(T, H, dtype, seed=500 + T)
+    xd = x.to(device)
+
+    def route(shared_up):
+        logits = torch.empty(T, E, dtype=dtype, device=device)
+        sg = torch.empty(T, dtype=dtype, device=device)
+        topv = torch.empty(T, K, dtype=dtype, device=device)
+        topi = torch.empty(T, K, dtype=torch.int64, device=device)
+        perm = ops.Permutation(T, K, E, device)
+        ops.route_decode_packed(xd, packed, E, True, K, False, logits, sg, topv, topi, perm, shared_up=shared_up)
+        torch.cuda.synchronize()
+        return logits, sg, topv, topi, perm
+
+    inter = torch.full((T, Is), float("nan"), dtype=dtype, device=device)
+    a, b = route(None), route((gw, uw, inter))
+    for u, v in zip(a[:4], b[:4]):
+        assert torch.equal(u, v)
+    for name in ("perm", "inv_perm", "seg_offsets", "n_active"):
+        assert torch.equal(getattr(a[4], name), getattr(b[4], name)), name
+    g = torch.nn.functional.linear(x.float(), layer["shared"][0].float()).to(dtype).float()
+    u = torch.nn.functional.linear(x.float(), layer["shared"][1].float()).to(dtype).float()
+    want = (torch.nn.functional.silu(g).to(dtype).float() * u).to(dtype)
+    got = inter.cpu()
+    assert not torch.isnan(got.float()).any()
+    torch.testing.assert_close(got.float(), want.float(), rtol=2 ** -6, atol=1e-3)
+    assert float(((got.float() - want.float()).abs() <= want.float().abs() * 2 ** -7 + 1e-3).float().mean()) > 0.995
+    alone = torch.empty_like(inter)
+    ops.shared_gate_up(xd, gw, uw, alone)       # the same kernel code without the routing
+    torch.cuda.synchronize()
+    assert torch.equal(alone, inter)
+    if Is % 64:
+        return      # the expert kernels' down projection needs Is in 64-wide blocks
+    # the decode expert kernel on the same weights
+    dw = tile_weight(layer["shared"][2].to(device)).reshape(H, Is).contiguous()
+    old_inter = torch.empty((T, Is), dtype=dtype, device=device)
+    old_out = torch.empty((T, H), dtype=dtype, device=device)
+    ops.shared_expert(xd, gw, uw, dw, a[1], old_inter, old_out)
+    torch.cuda.synchronize()
+    torch.testing.assert_close(got.float(), old_inter.cpu().float(), rtol=2 ** -6, atol=1e-3)
+    assert float((got == old_inter.cpu()).float().mean()) > 0.97
+
+
 def test_pack_router_gate_declines_what_does_not_fit():
     from sparse_amd import ops
     wg = torch.zeros(64, 128, dtype=torch.bfloat16)
