@@ -38,6 +38,7 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
+MFMA_PEAK_CLOCK_MHZ = 2400.0   # the clock the published MFMA rate is quoted at
 
 
 def build_stack(shape, dtype, device, offload="gpu", seed0=0, **kw):
@@ -175,6 +176,16 @@ def prefill_workload(shape, tokens, steps, warmup, dtype, device):
         blk.overlap_shared = False
     wall_serial = time_steps(blocks, inputs, 1, steps, use_graph=False)
     stats, _ = instrumented_pass(blocks, inputs, min(steps, 2))
+    # the clock the compute units really run at under this load (each workgroup of the FFN kernel
+    # reads the shader clock and the constant 100 MHz clock at its first and last instruction)
+    from sparse_amd import ops
+    clk = torch.zeros(2, dtype=torch.int64, device=device)
+    ops.prefill_clock_probe(clk)
+    try:
+        time_steps(blocks, inputs, 0, 2, use_graph=False)
+    finally:
+        ops.prefill_clock_probe(None)
+    clock_mhz = ops.prefill_shader_clock_mhz(clk)
     H, I, Is, K, E = shape["hidden"], shape["inter"], shape["shared_inter"], shape["top_k"], shape["num_experts"]
     flops_layer = 2.0 * tokens * K * 3 * H * I + 2.0 * tokens * 3 * H * Is + 2.0 * tokens * H * E
     gu_ms, gu_n, gu_name = stats["prefill_gateup"]
@@ -189,6 +200,11 @@ def prefill_workload(shape, tokens, steps, warmup, dtype, device):
         ms_per_step_one_stream=wall_serial / steps * 1e3,
         layer_tflops=flops_layer * len(blocks) / (ms_per_step / 1e3) / 1e12,
         mfma_frac=flops_layer * len(blocks) / (ms_per_step / 1e3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
+        # busy compute units' average shader clock during the FFN launches, and the fraction of the
+        # MFMA rate that clock allows (the published peak assumes MFMA_PEAK_CLOCK_MHZ)
+        ffn_shader_clock_mhz=clock_mhz,
+        mfma_frac_at_clock=(flops_layer * len(blocks) / (ms_per_step / 1e3) / 1e12
+                            / (MFMA_BF16_PEAK_TFLOPS * clock_mhz / MFMA_PEAK_CLOCK_MHZ)) if clock_mhz else None,
         gateup=dict(kernel=gu_name, launches=gu_n, est_routed_avg_us=gu_routed_s * 1e6,
                     tflops=gu_flops / gu_routed_s / 1e12 if gu_routed_s else 0.0),
         kernels_us={k: (v[0] / max(1, v[1]) * 1e3) for k, v in stats.items() if v[1]},

@@ -447,6 +447,14 @@ int sparse_hip_profile_read(int kernel, double* total_ms_out, int64_t* launches_
  * between the two means the counted waits no longer match the code the compiler produced.
  * Process-wide; returns the previous setting. */
 int sparse_hip_prefill_drain_waits(int on);
+/* Measurement aid with no counterpart in the reference: the clock the matrix cores really run
+ * at while the prefill-size expert FFN executes.  While `counters_dev` (two uint64 in device
+ * memory, zeroed by the caller) is set, every workgroup of that kernel adds the shader-clock
+ * cycles between its first and its last instruction to counters_dev[0] and the ticks of the
+ * constant 100 MHz clock over the same interval to counters_dev[1]; 100 MHz x [0] / [1] is
+ * the average shader clock of a busy compute unit, which under a power cap is well below the
+ * peak clock the published MFMA rate assumes.  NULL turns it off.  Process-wide. */
+int sparse_hip_prefill_clock_probe(void* counters_dev);
 /* Name of the __global__ function behind a kernel id (as rocprofv3 prints it, without
  * template arguments). */
 const char* sparse_hip_kernel_name(int kernel);

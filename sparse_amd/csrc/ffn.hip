@@ -19,6 +19,7 @@ int prefill_routed_bf16(const sparse_hip_experts*, const void*, const void*, con
                         const sparse_hip_seglist*, int, int, void*, void*, void*, hipStream_t);
 size_t prefill_ws_bytes(int, int, int, int, int);
 int prefill_set_drain_waits(int);
+void prefill_set_clock_probe(void*);
 int prefill_shared_bf16(const void*, const void*, const void*, const void*, const void*, int, int, int, void*,
                         void*, hipStream_t);
 template <typename T>
@@ -73,6 +74,11 @@ using namespace sparse;
 extern "C" {
 
 int sparse_hip_prefill_drain_waits(int on) { return prefill_set_drain_waits(on); }
+
+int sparse_hip_prefill_clock_probe(void* counters_dev) {
+  prefill_set_clock_probe(counters_dev);
+  return SPARSE_HIP_OK;
+}
 
 size_t sparse_hip_prefill_ws_bytes(int T, int K, int num_segments, int H, int I) {
   if (T <= 0 || K <= 0 || num_segments < 0 || H <= 0 || I <= 0) return 0;

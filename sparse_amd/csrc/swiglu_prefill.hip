@@ -74,6 +74,7 @@ struct PrefillArgs {
   const uint16_t* w_s;
   const uint16_t* w2_s;
   const uint16_t* gate_s;
+  unsigned long long* clk;  // clock probe: [0] += shader-clock cycles, [1] += 100 MHz ticks per workgroup; may be null
 };
 
 struct PfMapArgs {
@@ -145,6 +146,8 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_ffn_kernel(const Prefil
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63;
   const int fc = lane & 31, fg = lane >> 5;
+  const long long clk_c0 = clock64();
+  const unsigned long long clk_t0 = wall_clock64();
 
   // ---- which tile (XCD-aware order) ----------------------------------------------
   // The real tile count is split evenly over the XCDs (the grid is sized for the worst
@@ -379,9 +382,18 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_ffn_kernel(const Prefil
     case 3: body(std::integral_constant<int, 3>{}); break;
     default: body(std::integral_constant<int, 4>{}); break;
   }
+  if (a.clk != nullptr && tid == 0) {
+    atomicAdd(&a.clk[0], static_cast<unsigned long long>(clock64() - clk_c0));
+    atomicAdd(&a.clk[1], wall_clock64() - clk_t0);
+  }
 }
 
 static std::atomic<int> g_prefill_drain_waits{0};
+static std::atomic<unsigned long long*> g_prefill_clock{nullptr};
+
+void prefill_set_clock_probe(void* counters_dev) {
+  g_prefill_clock.store(static_cast<unsigned long long*>(counters_dev));
+}
 
 int prefill_set_drain_waits(int on) { return g_prefill_drain_waits.exchange(on ? 1 : 0); }
 
@@ -392,6 +404,7 @@ static int launch_prefill(PrefillArgs& a, int max_mtiles, hipStream_t st) {
   if (grid == 0) return SPARSE_HIP_OK;
   SP_REQUIRE(grid < (1ll << 31), "prefill_ffn: grid too large");
   ProfScope prof(kGateUp ? SPARSE_HIP_K_PREFILL_GATEUP : SPARSE_HIP_K_PREFILL_DOWN, st);
+  a.clk = g_prefill_clock.load(std::memory_order_relaxed);
   if (g_prefill_drain_waits.load(std::memory_order_relaxed))
     hipLaunchKernelGGL((prefill_ffn_kernel<kGateUp, true>), dim3(static_cast<unsigned>(grid)), dim3(kPfThreads), 0,
                        st, a);

@@ -472,6 +472,21 @@ def profile_read() -> dict:
     return out
 
 
+def prefill_clock_probe(counters: Optional[torch.Tensor]) -> None:
+    """Point the prefill-size FFN kernel's clock probe at ``counters`` (two int64 in device memory, which
+    the caller zeroes: [0] collects shader-clock cycles, [1] ticks of the constant 100 MHz clock, summed
+    over workgroups), or switch it off with ``None``.  A measurement aid; the reference has no such thing."""
+    if counters is not None:
+        _need(counters, "counters", torch.int64, (2,))
+    _lib.check(_lib.load().sparse_hip_prefill_clock_probe(_ptr(counters)), "sparse_hip_prefill_clock_probe")
+
+
+def prefill_shader_clock_mhz(counters: torch.Tensor) -> float:
+    """Average shader clock of a busy compute unit over the launches the probe has seen."""
+    cyc, ticks = (int(v) for v in counters.tolist())
+    return 100.0 * cyc / ticks if ticks else 0.0
+
+
 def moe_ffn_decode(experts: Experts, x: torch.Tensor, topv: torch.Tensor, perm: Permutation, segs: SegList,
                    inter_ws: torch.Tensor, parts: torch.Tensor, shared_w, shared_gate: Optional[torch.Tensor],
                    shared_inter_ws: torch.Tensor, shared_out: torch.Tensor,

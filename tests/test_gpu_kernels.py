@@ -472,6 +472,33 @@ def test_prefill_counted_waits_equal_full_drains(device, H, E, I, K, T):
     assert float(fast[0].float().abs().max()) > 0
 
 
+def test_prefill_clock_probe_reads_a_plausible_clock_and_changes_nothing(device):
+    """The probe adds up, per workgroup of the prefill FFN kernel, shader-clock cycles and ticks of the
+    constant 100 MHz clock: their ratio is a clock between the part's idle and peak clocks, both
+    counters grow with every launch, and the kernel's output is the same with and without it."""
+    ops = _ops()
+    H, E, I, K, T = 512, 12, 256, 4, 600
+    layer = make_layer(H, E, I, K, dtype=torch.bfloat16, seed=71)
+    x = make_hidden(T, H, torch.bfloat16, seed=72)
+    topv, topi = _routing(layer, x)
+    plain, _, _ = _run_routed(ops, layer, x, topv, topi, device, decode=False)
+    clk = torch.zeros(2, dtype=torch.int64, device=device)
+    ops.prefill_clock_probe(clk)
+    try:
+        probed, _, _ = _run_routed(ops, layer, x, topv, topi, device, decode=False)
+        first = clk.tolist()
+        _run_routed(ops, layer, x, topv, topi, device, decode=False)
+        second = clk.tolist()
+    finally:
+        ops.prefill_clock_probe(None)
+    assert torch.equal(plain, probed)
+    assert first[0] > 0 and first[1] > 0 and second[0] > first[0] and second[1] > first[1]
+    assert 100.0 < ops.prefill_shader_clock_mhz(clk) < 3000.0
+    _run_routed(ops, layer, x, topv, topi, device, decode=False)
+    torch.cuda.synchronize()
+    assert clk.tolist() == second   # switched off: nothing is added any more
+
+
 @pytest.mark.parametrize("T,decode", [(8, True), (128, False)])
 def test_ffn_fp32_matches_oracle(device, T, decode):
     ops = _ops()
