@@ -115,6 +115,12 @@ class RefConfig:
         self.epipe_decode_rs_commit = True
         self.epipe_decode_no_rs_commit = True
         self.epipe_stream_all = False                 # this build's addition, see RefLayer.execute
+        self.epipe_shadow = False                     # :4940
+        self.epipe_prefill_shadow = False             # :5008
+        self.epipe_prefill_multistage_shadow = False  # :5009
+        self.epipe_prefill_multistage_max_n = 4       # :5010
+        self.epipe_prefill_no_touch_ready = False     # :5018
+        self.epipe_rs_demand_stage_threshold_ms = 0.0  # :4988
         for k, v in kw.items():
             if not hasattr(self, k):
                 raise ValueError(f"unknown option {k}")
@@ -146,6 +152,7 @@ class RefLayer:
         self.phase, self.call_id, self.stage = "none", -1, "decode"
         self.trace: List[Tuple] = []
         self.counters: Dict[str, int] = {}
+        self.observed_exposed_ms = 0.0   # what the reference's metrics would hold; the caller sets it
         # cost-aware local policy (utils/lightweight_policy.py), off unless a test sets it:
         # dict(costs=..., expert_bytes=..., window_ms=0.0, ready_ms=0.0, feedback=True, prefetch=True)
         self.policy: Optional[Dict[str, Any]] = None
@@ -227,15 +234,20 @@ class RefLayer:
 
     # ---- prefill side cache (:5637-5720) -----------------------------------------------
     def extra_enabled(self) -> bool:
-        return self.extra.capacity > 0 and bool(self.cfg.epipe_prefill_enable)
+        """:5636-5644."""
+        c = self.cfg
+        return self.extra.capacity > 0 and bool(
+            c.epipe_prefill_enable or c.epipe_prefill_shadow or c.epipe_prefill_multistage_shadow)
 
     def _extra_readable(self) -> bool:
         return self.extra_enabled() and not (self.stage == "decode"
                                              and not self.cfg.epipe_prefill_extra_cache_decode_read)
 
-    def extra_get(self, eid: int) -> bool:
+    def extra_get(self, eid: int, touch: bool = True) -> bool:
         """A payload found in the side cache counts as an ordinary hit (:5687-5704)."""
-        if not self._extra_readable() or self.extra.get(eid) is None:
+        if not self._extra_readable():
+            return False
+        if (self.extra.get(eid) if touch else self.extra.peek(eid)) is None:
             return False
         self.trace.append(("hit", eid))
         self._count("epipe_prefill_extra_cache_hit_count")
@@ -270,12 +282,41 @@ class RefLayer:
         """:5585-5598."""
         c = self.cfg
         if self.stage == "prefill":
-            return bool(c.epipe_prefill_enable)
+            return bool(c.epipe_prefill_enable or c.epipe_prefill_shadow or c.epipe_prefill_multistage_shadow)
         if self.stage == "decode":
             if c.planner_mode == "rs_prefetch":
                 return bool(c.epipe_enable and c.epipe_decode_rs_mode not in ("off", "disabled"))
-            return bool(c.epipe_enable)
+            return bool(c.epipe_enable or c.epipe_shadow)
         return False
+
+    def shadow_for_stage(self) -> bool:
+        """:11890-11894, :12906-12910."""
+        c = self.cfg
+        return bool(c.epipe_shadow if self.stage == "decode"
+                    else (c.epipe_prefill_shadow or c.epipe_prefill_multistage_shadow))
+
+    def record_multistage_shadow(self, ready: Sequence[Segment], missing: Sequence[Segment]) -> None:
+        """:5738-5778."""
+        c = self.cfg
+        if self.stage != "prefill" or not c.epipe_prefill_multistage_shadow:
+            return
+        ready_items = sum(n for _, n in ready)
+        self._count("epipe_prefill_multistage_shadow_count")
+        self._count("epipe_prefill_multistage_ready_expert_count", len(ready))
+        self._count("epipe_prefill_multistage_missing_expert_count", len(missing))
+        self._count("epipe_prefill_multistage_ready_item_count", ready_items)
+        self._count("epipe_prefill_multistage_missing_item_count", sum(n for _, n in missing))
+        if not missing:
+            return
+        ranked = sorted(((n, self.expert_bytes) for _, n in missing), key=lambda x: x[0], reverse=True)
+        top = ranked[:min(max(1, int(c.epipe_prefill_multistage_max_n)), len(ranked))]
+        self._count("epipe_prefill_multistage_top_missing_item_count_sum", sum(x[0] for x in top))
+        self._count("epipe_prefill_multistage_est_expert_h2d_bytes", sum(x[1] for x in top))
+        self._count("epipe_prefill_multistage_est_ready_compute_items", ready_items)
+        for n in (1, 2, 4):
+            if int(c.epipe_prefill_multistage_max_n) >= n:
+                self._count(f"epipe_prefill_multistage_est_hidden_h2d_items_n{n}",
+                            sum(x[0] for x in ranked[:min(n, len(ranked))]))
 
     def execute(self, segments: Sequence[Segment]) -> str:
         """Executor choice of ``_execute_local_recv_groups`` :13264-13357."""
@@ -322,12 +363,27 @@ class RefLayer:
     def epipe_upfront_scan(self, segments: Sequence[Segment]) -> Optional[str]:
         """:11867-12167."""
         c = self.cfg
-        if not (c.epipe_enable if self.stage == "decode" else c.epipe_prefill_enable):
+        enabled = bool(c.epipe_enable if self.stage == "decode" else c.epipe_prefill_enable)
+        shadow = self.shadow_for_stage()
+        if not (enabled or shadow):
             return None
         ready = [s for s in segments if self.contains_no_touch(s[0])]
         missing = [s for s in segments if not self.contains_no_touch(s[0])]
         ready_items = sum(n for _, n in ready)
         free = max(0, self.cache.capacity - len(self.cache.resident_ids()))
+        self.record_multistage_shadow(ready, missing)
+        if shadow and not enabled:   # :11919-11932
+            self._count("epipe_shadow_count")
+            self._count("epipe_ready_expert_count", len(ready))
+            self._count("epipe_missing_expert_count", len(missing))
+            self._count("epipe_ready_item_count", ready_items)
+            self._count("epipe_missing_item_count", sum(n for _, n in missing))
+            self._count("epipe_missing_h2d_bytes_est", len(missing) * self.expert_bytes)
+            if free > 0:
+                self._count("epipe_cache_free_slot_count", free)
+            elif missing and c.epipe_transient_staging:
+                self._count("epipe_cache_full_staged_count")
+            return None
         if len(ready) < c.epipe_min_ready_experts or ready_items < c.epipe_min_ready_items:
             self._count("epipe_fallback_no_ready")
             return None
@@ -346,11 +402,22 @@ class RefLayer:
         if c.epipe_sort_ready_by_work:
             order.sort(key=lambda s: s[1], reverse=True)
         for eid, _ in order:
-            self.compute(eid)
+            # :12020-12031: with the no-touch switch a prefill call reads the ready payload itself
+            have = (self.stage == "prefill" and c.epipe_prefill_no_touch_ready
+                    and self.ready_payload_for_compute(eid))
+            self.compute(eid, have_payload=bool(have))
         self.trace.append(("wait", staged))
         self.trace.append(("miss", staged))
         if self.stage != "prefill":
             self.on_demand_access(staged)
+        for name, n in (("epipe_staged_missing_count", 1), ("epipe_enabled_count", 1), ("epipe_staged_expert_count", 1),
+                        ("epipe_no_evict_count", 1), ("epipe_ready_expert_count", len(ready)),
+                        ("epipe_missing_expert_count", len(missing)), ("epipe_ready_item_count", ready_items),
+                        ("epipe_missing_item_count", sum(n for _, n in missing)),
+                        ("epipe_missing_h2d_bytes_est", len(missing) * self.expert_bytes)):   # :12065-12074
+            self._count(name, n)
+        if free > 0:
+            self._count("epipe_cache_free_slot_count", free)
         if can_insert:
             if len(self.cache.resident_ids()) < self.cache.capacity:
                 if self.stage == "prefill":
@@ -358,8 +425,9 @@ class RefLayer:
                 self.cache_put_guarded(staged, transient=self.stage == "prefill" and c.epipe_prefill_mark_transient)
             else:
                 use_transient = True
-        if use_transient and self.stage == "prefill":
-            self.extra_store(staged)
+        if use_transient and not (self.stage == "prefill" and self.extra_store(staged)):   # :12101-12108
+            self._count("epipe_cache_full_staged_count")
+            self._count("epipe_transient_payload_count")
         self.compute(staged, have_payload=True)
         for eid, _ in missing[1:]:
             self.compute(eid)
@@ -377,8 +445,16 @@ class RefLayer:
         return True
 
     def demand_gate_can_open(self) -> bool:
-        """:5880-5893 (the exposed-stall threshold is zero by default, so only the force flag opens it)."""
-        return bool(self._handle_demand() and self.cfg.epipe_rs_force_demand_stage)
+        """:5880-5893.  ``observed_exposed_ms`` stands for max(sampled, measured) exposed demand-copy ms
+        of the decode phase, which the reference reads from its metrics."""
+        if not self._handle_demand():
+            return False
+        if self.cfg.epipe_rs_force_demand_stage:
+            return True
+        threshold = float(self.cfg.epipe_rs_demand_stage_threshold_ms)
+        if threshold <= 0.0:
+            return False
+        return float(self.observed_exposed_ms) > threshold
 
     def _residual_present(self, segments: Sequence[Segment]) -> bool:
         for eid, _ in segments:
@@ -587,10 +663,11 @@ class RefLayer:
     def ready_payload_for_compute(self, eid: int) -> bool:
         """:11672-11698: cache first (touching, counted as a hit, waiting a pending copy),
         then the prefill side cache (touching, not counted)."""
-        if self.cache.get(eid) is not None:
+        no_touch = self.stage == "prefill" and bool(self.cfg.epipe_prefill_no_touch_ready)
+        if (self.cache.peek(eid) if no_touch else self.cache.get(eid)) is not None:
             self.record_cached_use(eid, wait=True)
             return True
-        return self.extra_get(eid)
+        return self.extra_get(eid, touch=not no_touch)
 
     def epipe_miss_triggered(self, segments: Sequence[Segment]) -> Optional[str]:
         """:12845-13154.  Walk the segments in ascending expert id; at the first miss look
@@ -599,7 +676,9 @@ class RefLayer:
         Later misses of the same call take the ordinary demand path."""
         c = self.cfg
         stage, rs_active = self.stage, c.planner_mode == "rs_prefetch"
-        if not (c.epipe_prefill_enable if stage == "prefill" else c.epipe_enable):
+        enabled = bool(c.epipe_prefill_enable if stage == "prefill" else c.epipe_enable)
+        shadow = self.shadow_for_stage()
+        if not (enabled or shadow):
             return None
         if stage == "decode" and rs_active and c.epipe_decode_rs_mode == "off":
             return None
@@ -623,6 +702,13 @@ class RefLayer:
             ahead = [j for j in range(i + 1, min(len(segments), i + 1 + int(c.epipe_lookahead_experts)))
                      if j not in done and self.contains_no_touch(segments[j][0])]
             ready_items = sum(segments[j][1] for j in ahead)
+            if shadow and not enabled:   # :12982-12991
+                if ahead:
+                    self._count("epipe_prefill_shadow_opportunity_count" if stage == "prefill" else "epipe_shadow_count")
+                self._count("epipe_lookahead_ready_group_count", len(ahead))
+                self._count("epipe_lookahead_ready_item_count", ready_items)
+                self.compute(eid)
+                continue
             if not ahead:
                 self._count("epipe_fallback_no_ready_lookahead")
                 self.compute(eid)
@@ -640,6 +726,8 @@ class RefLayer:
             if stage != "prefill":
                 self.on_demand_access(eid)
             free = max(0, self.cache.capacity - len(self.cache.resident_ids()))
+            if free > 0:
+                self._count("epipe_cache_free_slot_count", free)
             if stage == "prefill":
                 commit_allowed, mark = bool(c.epipe_prefill_commit), bool(c.epipe_prefill_mark_transient)
             elif rs_active:
@@ -651,8 +739,16 @@ class RefLayer:
                 self.on_demand_access(eid)
             if insert:
                 self.cache_put_guarded(eid, transient=mark)
-            elif stage == "prefill":
-                self.extra_store(eid)
+            elif not (stage == "prefill" and self.extra_store(eid)):   # :13121-13130
+                if free <= 0:
+                    self._count("epipe_cache_full_staged_count")
+                self._count("epipe_transient_payload_count")
+            for name, n in (("epipe_enabled_count", 1), ("epipe_staged_missing_count", 1), ("epipe_staged_expert_count", 1),
+                            ("epipe_ready_expert_count", len(ahead)), ("epipe_ready_item_count", ready_items),
+                            ("epipe_lookahead_ready_group_count", len(ahead)),
+                            ("epipe_lookahead_ready_item_count", ready_items), ("epipe_missing_expert_count", 1),
+                            ("epipe_missing_item_count", _rows), ("epipe_missing_h2d_bytes_est", self.expert_bytes)):
+                self._count(name, n)   # :13132-13142
             self.compute(eid, have_payload=True)
             staged_once = True
         return "epipe_miss_triggered"

@@ -173,7 +173,8 @@ class _HipBackend(Backend):
                                 stream, ev)
         if timed:
             end.record(stream)
-            blk.metrics.pending_events.append((start, end, f"{lane}_h2d_ms", blk.layer_idx))
+            stage = blk.residency.stage if blk.residency is not None else "none"
+            blk.metrics.pending_events.append((start, end, f"{lane}_h2d_ms", blk.layer_idx, stage))
         return ev
 
     def event_done(self, event) -> bool:

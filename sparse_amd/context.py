@@ -47,13 +47,18 @@ class Metrics:
     moe_expert_ms: float = 0.0
     moe_shared_ms: float = 0.0
     moe_timing_calls: int = 0
+    # ms the compute lane spent in demand copies during decode (reference :1764-1766): filled from the
+    # timed copies by `harvest_timings`; the RS executors' demand stage reads it against
+    # SPARSE_EPIPE_RS_DEMAND_STAGE_THRESHOLD_MS
+    demand_h2d_exposed_decode_ms: float = 0.0
+    sampled_demand_h2d_exposed_decode_ms: float = 0.0
     counters: Dict[str, float] = field(default_factory=dict)
     # (kind, layer, expert) in issue order: kind in hit | prefetch_hit | miss
     events: Optional[List[Tuple[str, int, int]]] = None
     # when set, every expert upload is bracketed by a timing event pair on its lane
     time_copies: bool = False
-    # deferred timing: (start_event, end_event, tag, layer)
-    pending_events: List[Tuple[Any, Any, str, int]] = field(default_factory=list)
+    # deferred timing: (start_event, end_event, tag, layer[, stage])
+    pending_events: List[Tuple[Any, ...]] = field(default_factory=list)
     timings_ms: Dict[str, float] = field(default_factory=dict)
     timings_n: Dict[str, int] = field(default_factory=dict)
 
@@ -66,9 +71,12 @@ class Metrics:
 
     def harvest_timings(self) -> Dict[str, float]:
         """Read deferred event pairs (call after a device synchronisation)."""
-        for start, end, tag, _layer in self.pending_events:
-            self.timings_ms[tag] = self.timings_ms.get(tag, 0.0) + start.elapsed_ms(end)
+        for start, end, tag, _layer, *rest in self.pending_events:
+            ms = start.elapsed_ms(end)
+            self.timings_ms[tag] = self.timings_ms.get(tag, 0.0) + ms
             self.timings_n[tag] = self.timings_n.get(tag, 0) + 1
+            if tag == "compute_h2d_ms" and rest and rest[0] == "decode":
+                self.demand_h2d_exposed_decode_ms += ms
         self.pending_events.clear()
         return self.timings_ms
 

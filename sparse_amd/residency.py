@@ -100,6 +100,17 @@ class ResidencyConfig:
     # event, after the resident segments.  Cache events, eviction order and final contents are
     # those of the one-staged-expert executors; only lanes and waits change.
     epipe_stream_all: bool = False
+    # counting-only variants (reference :4940, :5008-5010): the executors classify ready / missing
+    # experts and count what EPIPE could have done, then leave the call to the demand path
+    epipe_shadow: bool = False
+    epipe_prefill_shadow: bool = False
+    epipe_prefill_multistage_shadow: bool = False
+    epipe_prefill_multistage_max_n: int = 4
+    # prefill: ready experts are read without moving them in the LRU (reference :5018)
+    epipe_prefill_no_touch_ready: bool = False
+    # the demand stage of the RS executors opens once the exposed demand-copy time seen so far
+    # exceeds this many ms (reference :4988, :5880-5893); 0: only `epipe_rs_force_demand_stage` opens it
+    epipe_rs_demand_stage_threshold_ms: float = 0.0
     epipe_min_ready_experts: int = 1
     epipe_min_ready_items: int = 1
     epipe_min_missing_experts: int = 1
@@ -169,6 +180,12 @@ class ResidencyConfig:
         c.epipe_transient_staging = _env_flag("SPARSE_EPIPE_TRANSIENT_STAGING", "1")
         c.epipe_max_staged_experts = _env_int("SPARSE_EPIPE_MAX_STAGED_EXPERTS", 1)
         c.epipe_stream_all = _env_flag("SPARSE_HIP_EPIPE_STREAM_ALL", "0")
+        c.epipe_shadow = _env_flag("SPARSE_EPIPE_SHADOW", "0")
+        c.epipe_prefill_shadow = _env_flag("SPARSE_EPIPE_PREFILL_SHADOW", "0")
+        c.epipe_prefill_multistage_shadow = _env_flag("SPARSE_EPIPE_PREFILL_MULTI_STAGE_SHADOW", "0")
+        c.epipe_prefill_multistage_max_n = max(1, _env_int("SPARSE_EPIPE_PREFILL_MULTI_STAGE_MAX_N", 4))
+        c.epipe_prefill_no_touch_ready = _env_flag("SPARSE_EPIPE_PREFILL_NO_TOUCH_READY", "0")
+        c.epipe_rs_demand_stage_threshold_ms = max(0.0, _env_float("SPARSE_EPIPE_RS_DEMAND_STAGE_THRESHOLD_MS", 0.0))
         c.epipe_sort_ready_by_work = _env_flag("SPARSE_EPIPE_SORT_READY_BY_WORK", "0")
         # the prefill policy sets the defaults of commit and transient mark (reference :5007-5016)
         policy = str(os.environ.get("SPARSE_EPIPE_PREFILL_POLICY", "deferred_lru_commit")
@@ -497,17 +514,19 @@ class LayerResidency:
 
     # ---- prefill side cache (reference :5637-5720) ------------------------------------
     def _extra_enabled(self) -> bool:
-        return self.extra_cache.capacity > 0 and bool(self.cfg.epipe_prefill_enable)
+        cfg = self.cfg   # reference :5636-5644
+        return self.extra_cache.capacity > 0 and bool(
+            cfg.epipe_prefill_enable or cfg.epipe_prefill_shadow or cfg.epipe_prefill_multistage_shadow)
 
     def _extra_readable(self) -> bool:
         return self._extra_enabled() and not (self.stage == "decode"
                                               and not self.cfg.epipe_prefill_extra_cache_decode_read)
 
-    def _extra_get(self, eid: int) -> Optional[int]:
+    def _extra_get(self, eid: int, touch: bool = True) -> Optional[int]:
         """Slot of an expert staged during prefill; finding it counts as an ordinary hit."""
         if not self._extra_readable():
             return None
-        slot = self.extra_cache.get(eid)
+        slot = self.extra_cache.get(eid) if touch else self.extra_cache.peek(eid)
         if slot is not None:
             self._event("hit", eid)
             self.metrics.bump("epipe_prefill_extra_cache_hit_count")
@@ -589,14 +608,45 @@ class LayerResidency:
         return name
 
     def _epipe_stage_enabled(self) -> bool:
-        """Reference :5585-5598 (shadow modes are not built)."""
+        """Reference :5585-5598."""
+        cfg = self.cfg
         if self.stage == "prefill":
-            return bool(self.cfg.epipe_prefill_enable)
+            return bool(cfg.epipe_prefill_enable or cfg.epipe_prefill_shadow or cfg.epipe_prefill_multistage_shadow)
         if self.stage == "decode":
-            if self.cfg.planner_mode == "rs_prefetch":
-                return bool(self.cfg.epipe_enable and self.cfg.epipe_decode_rs_mode not in ("off", "disabled"))
-            return bool(self.cfg.epipe_enable)
+            if cfg.planner_mode == "rs_prefetch":
+                return bool(cfg.epipe_enable and cfg.epipe_decode_rs_mode not in ("off", "disabled"))
+            return bool(cfg.epipe_enable or cfg.epipe_shadow)
         return False
+
+    def _shadow_for_stage(self) -> bool:
+        cfg = self.cfg
+        if self.stage == "decode":
+            return bool(cfg.epipe_shadow)
+        return bool(cfg.epipe_prefill_shadow or cfg.epipe_prefill_multistage_shadow)
+
+    def _record_multistage_shadow(self, ready: Sequence[Segment], missing: Sequence[Segment]) -> None:
+        """What staging the n largest missing experts of a prefill call at once would have moved and
+        hidden (reference :5738-5778); counters only."""
+        cfg, m = self.cfg, self.metrics
+        if self.stage != "prefill" or not cfg.epipe_prefill_multistage_shadow:
+            return
+        ready_items = sum(r for _, r in ready)
+        m.bump("epipe_prefill_multistage_shadow_count")
+        m.bump("epipe_prefill_multistage_ready_expert_count", len(ready))
+        m.bump("epipe_prefill_multistage_missing_expert_count", len(missing))
+        m.bump("epipe_prefill_multistage_ready_item_count", ready_items)
+        m.bump("epipe_prefill_multistage_missing_item_count", sum(r for _, r in missing))
+        if not missing:
+            return
+        ranked = sorted((int(r) for _, r in missing), reverse=True)   # stable: equal sizes keep segment order
+        max_n = max(1, int(cfg.epipe_prefill_multistage_max_n))
+        top = ranked[:min(max_n, len(ranked))]
+        m.bump("epipe_prefill_multistage_top_missing_item_count_sum", sum(top))
+        m.bump("epipe_prefill_multistage_est_expert_h2d_bytes", len(top) * self.expert_bytes)
+        m.bump("epipe_prefill_multistage_est_ready_compute_items", ready_items)
+        for n in (1, 2, 4):
+            if max_n >= n:
+                m.bump(f"epipe_prefill_multistage_est_hidden_h2d_items_n{n}", sum(ranked[:min(n, len(ranked))]))
 
     def _contains_no_touch(self, eid: int) -> bool:
         """Reference :5815-5851."""
@@ -616,12 +666,26 @@ class LayerResidency:
         cfg, m = self.cfg, self.metrics
         stage = self.stage
         enabled = bool(cfg.epipe_enable if stage == "decode" else cfg.epipe_prefill_enable)
-        if not enabled:
+        shadow = self._shadow_for_stage()
+        if not (enabled or shadow):
             return None
         ready = [s for s in segments if self._contains_no_touch(s[0])]
         missing = [s for s in segments if not self._contains_no_touch(s[0])]
         ready_items = sum(r for _, r in ready)
         free_cache_slots = max(0, self.cache.capacity - len(self.cache))
+        self._record_multistage_shadow(ready, missing)
+        if shadow and not enabled:      # reference :11919-11932: count the opportunity, execute nothing
+            m.bump("epipe_shadow_count")
+            m.bump("epipe_ready_expert_count", len(ready))
+            m.bump("epipe_missing_expert_count", len(missing))
+            m.bump("epipe_ready_item_count", ready_items)
+            m.bump("epipe_missing_item_count", sum(r for _, r in missing))
+            m.bump("epipe_missing_h2d_bytes_est", len(missing) * self.expert_bytes)
+            if free_cache_slots > 0:
+                m.bump("epipe_cache_free_slot_count", free_cache_slots)
+            elif missing and cfg.epipe_transient_staging:
+                m.bump("epipe_cache_full_staged_count")
+            return None
         if not cfg.epipe_no_evict:
             raise NotImplementedError("SPARSE_EPIPE_NO_EVICT=0 is not implemented in EPIPE-Lite.")
         if cfg.epipe_max_staged_experts != 1:
@@ -650,7 +714,11 @@ class LayerResidency:
         if cfg.epipe_sort_ready_by_work:
             ready_order.sort(key=lambda s: s[1], reverse=True)
         for eid, _rows in ready_order:
-            self._compute(eid)
+            # prefill with `epipe_prefill_no_touch_ready`: the ready expert is read where it lies, its
+            # place in the LRU unchanged (reference :12020-12021, :11672-11698)
+            ready_slot = (self._ready_slot_for_compute(eid)
+                          if stage == "prefill" and cfg.epipe_prefill_no_touch_ready else None)
+            self._compute(eid, ready_slot)
         # the ready batch must be on the device before the compute lane waits the copy
         self.flush()
         self.backend.wait_event(stage_event, "compute")
@@ -660,6 +728,15 @@ class LayerResidency:
         m.demand_h2d_bytes += self.expert_bytes
         m.bump("epipe_staged_missing_count")
         m.bump("epipe_enabled_count")
+        m.bump("epipe_staged_expert_count")
+        m.bump("epipe_no_evict_count")
+        m.bump("epipe_ready_expert_count", len(ready))
+        m.bump("epipe_missing_expert_count", len(missing))
+        m.bump("epipe_ready_item_count", ready_items)
+        m.bump("epipe_missing_item_count", sum(r for _, r in missing))
+        m.bump("epipe_missing_h2d_bytes_est", len(missing) * self.expert_bytes)
+        if free_cache_slots > 0:
+            m.bump("epipe_cache_free_slot_count", free_cache_slots)
         kept = False  # does some cache keep the staged slot alive after this call?
         if can_insert:
             if len(self.cache) < self.cache.capacity:
@@ -677,6 +754,8 @@ class LayerResidency:
             if use_transient and stage == "prefill":
                 kept = self._extra_store(staged_eid, slot)
             if not kept:
+                if use_transient:
+                    m.bump("epipe_cache_full_staged_count")
                 m.bump("epipe_transient_payload_count")
                 self._retired.append(slot)  # back to the pool once this batch is launched
         for eid, _rows in missing[1:]:
@@ -697,8 +776,19 @@ class LayerResidency:
         return ev
 
     def _demand_gate_can_open(self) -> bool:
-        """Reference :5880-5893; the exposed-stall threshold variant is not built."""
-        return bool(self._handle_demand() and self.cfg.epipe_rs_force_demand_stage)
+        """Reference :5880-5893: forced open, or open once the exposed demand-copy time of the decode
+        phase (as far as the metrics have it: sampled or measured, whichever is larger) exceeds the
+        threshold."""
+        if not self._handle_demand():
+            return False
+        if self.cfg.epipe_rs_force_demand_stage:
+            return True
+        threshold = float(self.cfg.epipe_rs_demand_stage_threshold_ms)
+        if threshold <= 0.0:
+            return False
+        observed = max(float(getattr(self.metrics, "sampled_demand_h2d_exposed_decode_ms", 0.0)),
+                       float(getattr(self.metrics, "demand_h2d_exposed_decode_ms", 0.0)))
+        return observed > threshold
 
     def _handle_late(self) -> bool:
         """``demand_only`` switches the handling of late prefetches off (reference :4975-4984)."""
@@ -866,7 +956,7 @@ class LayerResidency:
         return slot, self._upload(eid, slot, "epipe")
 
     def _finish_staged(self, eid: int, slot: int, stage_event: Any, commit: bool, transient: bool = False,
-                       to_extra: bool = False) -> None:
+                       to_extra: bool = False) -> bool:
         """Wait a staged copy on the compute lane, queue the expert, and either commit its
         slot to the cache, hand it to the prefill side cache, or let it go after the batch."""
         m = self.metrics
@@ -885,6 +975,7 @@ class LayerResidency:
             self._retired.append(slot)
         m.bump("epipe_enabled_count")
         m.bump("epipe_staged_missing_count")
+        return kept
 
     # ---- EPIPE on top of RS prefetch: bounded ready buffer (reference :12514-12843) -----
     def _epipe_rs_buffered(self, segments: Sequence[Segment]) -> Optional[str]:
@@ -988,11 +1079,12 @@ class LayerResidency:
     def _ready_slot_for_compute(self, eid: int) -> Optional[int]:
         """Reference :11672-11698: the cache first (touched, counted as a hit, a pending copy
         waited for), then the prefill side cache (touched, not counted)."""
-        slot = self.cache.get(eid)
+        no_touch = self.stage == "prefill" and self.cfg.epipe_prefill_no_touch_ready
+        slot = self.cache.peek(eid) if no_touch else self.cache.get(eid)
         if slot is not None:
             self._record_cached_use(eid, wait_prefetch=True)
             return slot
-        return self._extra_get(eid)
+        return self._extra_get(eid, touch=not no_touch)
 
     def _epipe_miss_triggered(self, segments: Sequence[Segment]) -> Optional[str]:
         """Walk the segments in ascending expert id; at the first miss look a few segments
@@ -1001,7 +1093,9 @@ class LayerResidency:
         the call take the ordinary demand path."""
         cfg, m = self.cfg, self.metrics
         stage, rs_active = self.stage, cfg.planner_mode == "rs_prefetch"
-        if not (cfg.epipe_prefill_enable if stage == "prefill" else cfg.epipe_enable):
+        enabled = bool(cfg.epipe_prefill_enable if stage == "prefill" else cfg.epipe_enable)
+        shadow = self._shadow_for_stage()
+        if not (enabled or shadow):
             return None
         mode = cfg.epipe_decode_rs_mode
         if stage == "decode" and rs_active and mode == "off":
@@ -1027,6 +1121,13 @@ class LayerResidency:
             ahead = [j for j in range(i + 1, min(len(segments), i + 1 + int(cfg.epipe_lookahead_experts)))
                      if j not in done and self._contains_no_touch(segments[j][0])]
             ready_items = sum(segments[j][1] for j in ahead)
+            if shadow and not enabled:   # reference :12982-12991: count the opportunity, take the demand path
+                if ahead:
+                    m.bump("epipe_prefill_shadow_opportunity_count" if stage == "prefill" else "epipe_shadow_count")
+                m.bump("epipe_lookahead_ready_group_count", len(ahead))
+                m.bump("epipe_lookahead_ready_item_count", ready_items)
+                self._compute(eid)
+                continue
             if not ahead:
                 self._fallback("epipe_fallback_no_ready_lookahead")
                 self._compute(eid)
@@ -1048,6 +1149,8 @@ class LayerResidency:
             if stage != "prefill":
                 self._on_demand_access(eid)
             free_cache_slots = max(0, self.cache.capacity - len(self.cache))
+            if free_cache_slots > 0:
+                m.bump("epipe_cache_free_slot_count", free_cache_slots)
             if stage == "prefill":
                 commit_allowed, mark = bool(cfg.epipe_prefill_commit), bool(cfg.epipe_prefill_mark_transient)
             elif rs_active:
@@ -1058,7 +1161,18 @@ class LayerResidency:
                           and (free_cache_slots > 0 or not cfg.epipe_no_evict))
             if stage == "prefill" and insert:
                 self._on_demand_access(eid)
-            self._finish_staged(eid, slot, stage_event, insert, transient=mark, to_extra=stage == "prefill")
+            kept = self._finish_staged(eid, slot, stage_event, insert, transient=mark, to_extra=stage == "prefill")
+            if not kept and free_cache_slots <= 0:
+                m.bump("epipe_cache_full_staged_count")
+            # reference :13132-13142
+            m.bump("epipe_staged_expert_count")
+            m.bump("epipe_ready_expert_count", len(ahead))
+            m.bump("epipe_ready_item_count", ready_items)
+            m.bump("epipe_lookahead_ready_group_count", len(ahead))
+            m.bump("epipe_lookahead_ready_item_count", ready_items)
+            m.bump("epipe_missing_expert_count")
+            m.bump("epipe_missing_item_count", _rows)
+            m.bump("epipe_missing_h2d_bytes_est", self.expert_bytes)
             staged_once = True
         return "epipe_miss_triggered"
 

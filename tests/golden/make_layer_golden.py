@@ -63,7 +63,7 @@ METHODS = (
     "_epipe_rs_demand_stage_gate_can_open", "_epipe_rs_demand_stage_gate_open",
     "_epipe_prefill_extra_cache_enabled", "_epipe_prefill_extra_cache_store", "_epipe_prefill_extra_cache_get",
     "_epipe_prefill_extra_cache_contains", "_epipe_prefill_extra_cache_resident_count",
-    "_epipe_prefill_extra_cache_clear",
+    "_epipe_prefill_extra_cache_clear", "_epipe_record_prefill_multistage_shadow",
     "_try_execute_local_recv_groups_epipe", "_try_execute_local_recv_groups_epipe_rs_residual_scan",
     "_try_execute_local_recv_groups_epipe_rs_buffered", "_try_execute_local_recv_groups_epipe_miss_triggered",
     # RS prefetch cycle, budget, plan, admission
@@ -259,7 +259,7 @@ class StubBlock:
         late_only = cfg["epipe_decode_rs_mode"] == "late_only"
         demand_only = cfg["epipe_decode_rs_mode"] == "demand_only"
         for name, value in dict(
-            _epipe_enable=cfg["epipe_enable"], _epipe_shadow=False, _epipe_mode=cfg["epipe_mode"],
+            _epipe_enable=cfg["epipe_enable"], _epipe_shadow=cfg["epipe_shadow"], _epipe_mode=cfg["epipe_mode"],
             _epipe_decode_with_rs_mode=cfg["epipe_decode_rs_mode"], _epipe_decode_only=True,
             _epipe_no_evict=cfg["epipe_no_evict"], _epipe_transient_staging=cfg["epipe_transient_staging"],
             _epipe_max_staged_experts=cfg["epipe_max_staged_experts"], _epipe_min_free_mb=0.0,
@@ -276,7 +276,8 @@ class StubBlock:
             _epipe_rs_handle_demand_miss=cfg["epipe_rs_handle_demand_miss"] and not late_only,
             _epipe_rs_demand_commit=cfg["epipe_rs_demand_commit"],
             _epipe_rs_force_demand_stage=cfg["epipe_rs_force_demand_stage"],
-            _epipe_rs_demand_stage_threshold_ms=0.0, _epipe_rs_rolling_gate=cfg["epipe_rs_rolling_gate"],
+            _epipe_rs_demand_stage_threshold_ms=cfg["epipe_rs_demand_stage_threshold_ms"],
+            _epipe_rs_rolling_gate=cfg["epipe_rs_rolling_gate"],
             _epipe_rs_gate_window=cfg["epipe_rs_gate_window"],
             _epipe_rs_gate_min_triggers=cfg["epipe_rs_gate_min_triggers"],
             _epipe_rs_gate_skip_steps=cfg["epipe_rs_gate_skip_steps"], _epipe_stage_first_missing_only=True,
@@ -286,9 +287,12 @@ class StubBlock:
             _epipe_deferred_lru_commit=cfg["epipe_deferred_lru_commit"],
             _epipe_decode_rs_commit=cfg["epipe_decode_rs_commit"],
             _epipe_decode_no_rs_commit=cfg["epipe_decode_no_rs_commit"],
-            _epipe_prefill_enable=cfg["epipe_prefill_enable"], _epipe_prefill_shadow=False,
-            _epipe_prefill_multistage_shadow=False, _epipe_prefill_commit=cfg["epipe_prefill_commit"],
-            _epipe_prefill_mark_transient=cfg["epipe_prefill_mark_transient"], _epipe_prefill_no_touch_ready=False,
+            _epipe_prefill_enable=cfg["epipe_prefill_enable"], _epipe_prefill_shadow=cfg["epipe_prefill_shadow"],
+            _epipe_prefill_multistage_shadow=cfg["epipe_prefill_multistage_shadow"],
+            _epipe_prefill_multistage_max_n=cfg["epipe_prefill_multistage_max_n"],
+            _epipe_prefill_commit=cfg["epipe_prefill_commit"],
+            _epipe_prefill_mark_transient=cfg["epipe_prefill_mark_transient"],
+            _epipe_prefill_no_touch_ready=cfg["epipe_prefill_no_touch_ready"],
             _epipe_timing=False, _epipe_debug_counters=False, _epipe_validate_output=False,
             _epipe_prefill_extra_cache_decode_read=cfg["epipe_prefill_extra_cache_decode_read"],
             _epipe_prefill_extra_cache_clear_at_decode=cfg["epipe_prefill_extra_cache_clear_at_decode"],
@@ -313,6 +317,10 @@ class StubBlock:
         raise AttributeError(name)
 
     # ---- what the device / harness would provide --------------------------------------------
+    def _record_epipe_counter(self, name: str, value: int = 1) -> None:
+        counts = self.__dict__.setdefault("_counts", {})
+        counts[str(name)] = counts.get(str(name), 0) + int(value)
+
     def _record_cache_hit(self, is_prefetch_hit: bool = False) -> None:
         self._rec.trace.append(("prefetch_hit" if is_prefetch_hit else "hit",))
 
@@ -491,6 +499,9 @@ def run_case(method: str, kw: Dict[str, Any]) -> Dict[str, Any]:
         rec.seed, rec.late_rate, rec.pending_copy = kw["seed"], kw["late_rate"], None
         ns, compute, torch_mod = extract(rec, env, context)
         blocks.append(StubBlock(ns, torch_mod, rec, compute, layer, cfg, kw["E"], kw["K"], env))
+        if kw.get("observed_exposed_ms"):
+            # what the harness's metrics would hold once demand copies of the decode phase were timed
+            blocks[-1].metrics.demand_h2d_exposed_decode_ms = float(kw["observed_exposed_ms"])
         recs.append(rec)
     costs = kw.get("policy_costs")
     if costs:
@@ -583,7 +594,24 @@ def run_case(method: str, kw: Dict[str, Any]) -> Dict[str, Any]:
             plans=None if dense else [x[1] for x in t if x[0] == "plan"],
             residents=[int(e) for e in blk._cache.resident_ids()],
             extra=[int(e) for e in blk._epipe_prefill_extra_cache.resident_ids()]))
+        if kw.get("counters"):
+            counts = blk.__dict__.get("_counts", {})
+            expect[-1]["counters"] = {name: int(counts.get(name, 0)) for name in kw["counters"]}
     return dict(method=method, kw=kw, steps=steps, executors=executors, expect=expect)
+
+
+SHADOW_COUNTERS = [
+    "epipe_shadow_count", "epipe_prefill_shadow_opportunity_count", "epipe_ready_expert_count",
+    "epipe_missing_expert_count", "epipe_ready_item_count", "epipe_missing_item_count",
+    "epipe_missing_h2d_bytes_est", "epipe_cache_free_slot_count", "epipe_cache_full_staged_count",
+    "epipe_lookahead_ready_group_count", "epipe_lookahead_ready_item_count",
+    "epipe_prefill_multistage_shadow_count", "epipe_prefill_multistage_ready_expert_count",
+    "epipe_prefill_multistage_missing_expert_count", "epipe_prefill_multistage_ready_item_count",
+    "epipe_prefill_multistage_missing_item_count", "epipe_prefill_multistage_top_missing_item_count_sum",
+    "epipe_prefill_multistage_est_expert_h2d_bytes", "epipe_prefill_multistage_est_ready_compute_items",
+    "epipe_prefill_multistage_est_hidden_h2d_items_n1", "epipe_prefill_multistage_est_hidden_h2d_items_n2",
+    "epipe_prefill_multistage_est_hidden_h2d_items_n4",
+]
 
 
 def cases() -> List[Tuple[str, Dict[str, Any]]]:
@@ -662,6 +690,42 @@ def cases() -> List[Tuple[str, Dict[str, Any]]]:
         c("rs-epipe", late_rate=0.4, policy_costs=POLICY_COSTS, seed=24),
         c("sparse", late_rate=0.3, T=8, capacity=6, policy_costs=POLICY_COSTS, seed=25),
         c("rs", policy_costs=POLICY_COSTS, seed=26),
+        # counting-only (shadow) variants: classify, count, leave the call to the demand path
+        c("epipe", overrides=dict(epipe_enable=False, epipe_shadow=True), seed=50, counters=SHADOW_COUNTERS),
+        c("epipe", capacity=2, T=8, overrides=dict(epipe_enable=False, epipe_shadow=True, epipe_transient_staging=False),
+          seed=51, counters=SHADOW_COUNTERS),
+        c("epipe", prefill_steps=5, capacity=8, T=2, overrides=dict(epipe_prefill_shadow=True), seed=52,
+          counters=SHADOW_COUNTERS),
+        c("epipe", prefill_steps=6, capacity=6, T=8,
+          overrides=dict(epipe_prefill_enable=True, epipe_prefill_multistage_shadow=True,
+                         epipe_prefill_multistage_max_n=2), seed=53, counters=SHADOW_COUNTERS),
+        c("rr", prefill_steps=6, capacity=6, T=8,
+          overrides=dict(epipe_prefill_multistage_shadow=True, epipe_prefill_extra_cache_slots=2), seed=54,
+          counters=SHADOW_COUNTERS),
+        c("epipe", overrides=dict(mt, epipe_enable=False, epipe_shadow=True), seed=55, counters=SHADOW_COUNTERS),
+        c("epipe", prefill_steps=5, capacity=6, T=8,
+          overrides=dict(mt, epipe_prefill_shadow=True, epipe_prefill_lookahead_min_ready_items=1), seed=56,
+          counters=SHADOW_COUNTERS),
+        # prefill reads ready experts without moving them in the LRU
+        c("epipe", prefill_steps=6, capacity=6, T=8,
+          overrides=dict(epipe_prefill_enable=True, epipe_prefill_no_touch_ready=True), seed=57),
+        c("epipe", prefill_steps=6, capacity=6, T=8,
+          overrides=dict(epipe_prefill_enable=True, epipe_prefill_no_touch_ready=True, epipe_prefill_commit=False,
+                         epipe_prefill_extra_cache_slots=2), seed=58),
+        c("epipe", prefill_steps=6, capacity=6, T=8,
+          overrides=dict(mt, epipe_prefill_enable=True, epipe_prefill_no_touch_ready=True,
+                         epipe_prefill_lookahead_min_ready_items=1, epipe_prefill_commit=False,
+                         epipe_prefill_extra_cache_slots=2), seed=59),
+        # the demand stage behind the exposed-stall threshold instead of the force flag
+        c("rs-epipe", late_rate=0.3, overrides=dict(epipe_rs_force_demand_stage=False,
+                                                    epipe_rs_demand_stage_threshold_ms=1.0),
+          observed_exposed_ms=5.0, seed=60),
+        c("rs-epipe", late_rate=0.3, overrides=dict(epipe_rs_force_demand_stage=False,
+                                                    epipe_rs_demand_stage_threshold_ms=1.0),
+          observed_exposed_ms=0.5, seed=60),
+        c("rs-epipe", late_rate=0.3, overrides=dict(epipe_decode_rs_mode="buffered", epipe_rs_force_demand_stage=False,
+                                                    epipe_rs_demand_stage_threshold_ms=2.0),
+          observed_exposed_ms=2.5, seed=61),
         # tiered cache under the same state machine
         c("rr", capacity=8, E=24, T=8, overrides=dict(cache_policy="tiered"), seed=21),
         c("rs", capacity=8, E=24, T=8, top_m=4, overrides=dict(cache_policy="tiered", prefetch_reserved=1), seed=22),

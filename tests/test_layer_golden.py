@@ -53,11 +53,14 @@ def replay(case, which):
 
     lays, backs, mets = [], [], []
     for l in range(kw["layers"]):
+        observed = float(kw.get("observed_exposed_ms") or 0.0)   # exposed demand-copy ms the metrics hold
         if which == "oracle":
             lay = RefLayer(l, kw["E"], kw["K"], to_ref_config(cfg), copy_done=copy_done(l))
             lay.expert_bytes = 100
+            lay.observed_exposed_ms = observed
         else:
             lay, be, m = product_layer(cfg, E=kw["E"], K=kw["K"], copy_done=copy_done(l), layer=l)
+            m.demand_h2d_exposed_decode_ms = observed
             backs.append(be)
             mets.append(m)
         lays.append(lay)
@@ -136,6 +139,9 @@ def replay(case, which):
         out.append(dict(events=[k for k, _e in events], h2d=[[lane, e] for _h, lane, e in h2d], compute=compute,
                         waits=[e for _w, e in waits], side_waits=side, plans=plans[l],
                         residents=lay.cache.resident_ids(), extra=extra))
+        if kw.get("counters"):
+            counts = lay.counters if which == "oracle" else mets[l].counters
+            out[-1]["counters"] = {name: int(counts.get(name, 0)) for name in kw["counters"]}
     return out, executors
 
 
@@ -149,6 +155,8 @@ def test_replay_matches_the_reference(case, which):
             if w[key] is None:
                 continue        # the reference's own scheduling function keeps no record of its plans
             assert g[key] == w[key], f"layer {l}: {key} differs from the reference"
+        if "counters" in w:
+            assert g["counters"] == w["counters"], f"layer {l}: counters differ from the reference"
 
 
 def test_fixture_covers_every_executor_and_feature():
@@ -160,3 +168,11 @@ def test_fixture_covers_every_executor_and_feature():
     assert any(e["plans"] for c in CASES for e in c["expect"])
     assert sum(1 for c in CASES if c["kw"].get("dense")) >= 5
     assert sum(len(e["events"]) for c in CASES for e in c["expect"]) > 10000
+    # the counting-only variants did count, the no-touch switch and the stall threshold are in
+    shadow = [c for c in CASES if c["kw"].get("counters")]
+    assert len(shadow) >= 7
+    for name in ("epipe_shadow_count", "epipe_prefill_shadow_opportunity_count", "epipe_lookahead_ready_item_count",
+                 "epipe_prefill_multistage_est_hidden_h2d_items_n2", "epipe_cache_full_staged_count"):
+        assert any(e["counters"][name] > 0 for c in shadow for e in c["expect"]), name
+    assert any(c["kw"]["overrides"].get("epipe_prefill_no_touch_ready") for c in CASES)
+    assert sum(1 for c in CASES if c["kw"].get("observed_exposed_ms")) >= 3
