@@ -25,7 +25,9 @@
  *     loads; row-major rows 4 KB apart would pile onto the same HBM channels.
  *     `sparse_hip_tile_weight` converts.  The router gate matrix `wg` and the shared
  *     gate vector stay row-major.
- *   - dtype codes: SPARSE_HIP_F32 = 0, SPARSE_HIP_BF16 = 1.
+ *   - dtype codes: SPARSE_HIP_F32 = 0, SPARSE_HIP_BF16 = 1, SPARSE_HIP_F16 = 2 (IEEE half, the
+ *     dtype of the reference's formal runs, scripts/run/run_case.sh:199).  Wherever this file says
+ *     bf16 for a kernel's 16-bit path, fp16 takes the same kernel with its own conversions and MFMA.
  */
 #ifndef SPARSE_HIP_H
 #define SPARSE_HIP_H
@@ -41,6 +43,7 @@ extern "C" {
 
 #define SPARSE_HIP_F32 0
 #define SPARSE_HIP_BF16 1
+#define SPARSE_HIP_F16 2
 
 #define SPARSE_HIP_OK 0
 #define SPARSE_HIP_EINVAL (-1)   /* bad argument (shape, dtype, alignment, NULL) */
@@ -82,7 +85,7 @@ typedef struct sparse_hip_experts {
   int32_t num_experts;             /* E */
   int32_t hidden;                  /* H */
   int32_t inter;                   /* I */
-  int32_t dtype;                   /* SPARSE_HIP_F32 | SPARSE_HIP_BF16 */
+  int32_t dtype;                   /* SPARSE_HIP_F32 | SPARSE_HIP_BF16 | SPARSE_HIP_F16 */
 } sparse_hip_experts;
 
 /*

@@ -12,6 +12,7 @@ LIB_PATH = Path(__file__).resolve().parent / "csrc" / "libsparse_hip.so"
 
 F32 = 0
 BF16 = 1
+F16 = 2
 MAX_EXPERTS = 256
 MAX_TOPK = 16
 DECODE_MAX_TOKENS = 32

@@ -279,8 +279,8 @@ class DistributedSparseMoeBlock(nn.Module):
         self.cache_policy = str(cache_policy).lower()
         if self.cache_policy not in ("lru", "lfu", "tiered"):
             raise ValueError(f"cache_policy must be lru|lfu|tiered, got {self.cache_policy}")
-        if self.dtype not in (torch.bfloat16, torch.float32):
-            raise ValueError(f"dtype must be bfloat16 or float32, got {self.dtype}")
+        if self.dtype not in (torch.bfloat16, torch.float16, torch.float32):
+            raise ValueError(f"dtype must be bfloat16, float16 or float32, got {self.dtype}")
         self.rs_group = int(rs_group)
         self.rs_prob_to_logit_eps = float(rs_prob_to_logit_eps)
         self.prefetch_top_m = int(prefetch_top_m)
@@ -605,7 +605,7 @@ class DistributedSparseMoeBlock(nn.Module):
 
         shared_gate = ws.shared_gate if self.shared_gate_weight is not None else None
         timing = self._segment_timing_on()
-        fused = (self.residency is None and self.shared_weights is not None and self.dtype == torch.bfloat16
+        fused = (self.residency is None and self.shared_weights is not None and self.dtype in ops.HALF_DTYPES
                  and T <= ops.DECODE_MAX_TOKENS and not timing)
         # Prefill-size batches: the shared expert needs only x and the shared gate, so it runs
         # on a second stream from the moment the logits kernel is queued, beside top-k,

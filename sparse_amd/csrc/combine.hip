@@ -148,6 +148,10 @@ extern "C" int sparse_hip_combine(const void* parts_dev, const int32_t* inv_perm
     hipLaunchKernelGGL((combine_kernel<uint16_t>), grid, dim3(kCombThreads), 0, as_stream(stream),
                        static_cast<const uint16_t*>(parts_dev), inv_perm_dev,
                        static_cast<const uint16_t*>(shared_dev), K, H, static_cast<uint16_t*>(out_dev));
+  } else if (dtype == SPARSE_HIP_F16) {
+    hipLaunchKernelGGL((combine_kernel<f16_t>), grid, dim3(kCombThreads), 0, as_stream(stream),
+                       static_cast<const f16_t*>(parts_dev), inv_perm_dev, static_cast<const f16_t*>(shared_dev), K, H,
+                       static_cast<f16_t*>(out_dev));
   } else {
     hipLaunchKernelGGL((combine_kernel<float>), grid, dim3(kCombThreads), 0, as_stream(stream),
                        static_cast<const float*>(parts_dev), inv_perm_dev, static_cast<const float*>(shared_dev),

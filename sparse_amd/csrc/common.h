@@ -48,11 +48,16 @@ struct ProfScope {
 };
 
 inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
-inline size_t elem_size(int dtype) { return dtype == SPARSE_HIP_BF16 ? 2 : 4; }
-inline bool valid_dtype(int dtype) { return dtype == SPARSE_HIP_F32 || dtype == SPARSE_HIP_BF16; }
+inline size_t elem_size(int dtype) { return dtype == SPARSE_HIP_F32 ? 4 : 2; }
+inline bool valid_dtype(int dtype) {
+  return dtype == SPARSE_HIP_F32 || dtype == SPARSE_HIP_BF16 || dtype == SPARSE_HIP_F16;
+}
+inline bool is_16bit(int dtype) { return dtype == SPARSE_HIP_BF16 || dtype == SPARSE_HIP_F16; }
 
 // ---- vector types -----------------------------------------------------------
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef _Float16 f16_t;  // IEEE half: the storage tag of fp16 tensors (bf16 tensors are tagged uint16_t)
+typedef __attribute__((__vector_size__(8 * sizeof(_Float16)))) _Float16 f16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16;
 
@@ -96,6 +101,53 @@ struct Elem<uint16_t> {
   __device__ static __forceinline__ void store(uint16_t* p, float v) { *p = f32_to_bf16_bits(v); }
   __device__ static __forceinline__ float round(float v) { return round_bf16(v); }
 };
+
+// IEEE half: round-to-nearest-even conversions in hardware, as torch's.
+template <>
+struct Elem<f16_t> {
+  static constexpr int dtype = SPARSE_HIP_F16;
+  __device__ static __forceinline__ float load(const f16_t* p) { return static_cast<float>(*p); }
+  __device__ static __forceinline__ void store(f16_t* p, float v) { *p = static_cast<f16_t>(v); }
+  __device__ static __forceinline__ float round(float v) { return static_cast<float>(static_cast<f16_t>(v)); }
+};
+
+// The two 16-bit formats as the MFMA kernels see them: tensors are raw uint16_t there, and a format is
+// its conversions plus its matrix instruction.  Operand fragments are 16 bytes either way (bf16x8 is the
+// carrier type; the fp16 instruction takes the same bits as f16x8).
+struct Bf16 {
+  static constexpr int dtype = SPARSE_HIP_BF16;
+  __device__ static __forceinline__ float from_bits(uint16_t b) { return bf16_bits_to_f32(b); }
+  __device__ static __forceinline__ uint16_t bits(float f) { return f32_to_bf16_bits(f); }
+  __device__ static __forceinline__ float round(float f) { return round_bf16(f); }
+  __device__ static __forceinline__ uint32_t pack2(float lo, float hi) { return f32x2_to_bf16x2_bits(lo, hi); }
+  __device__ static __forceinline__ f32x4 mfma16(bf16x8 a, bf16x8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  }
+  __device__ static __forceinline__ f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+};
+struct Fp16 {
+  static constexpr int dtype = SPARSE_HIP_F16;
+  __device__ static __forceinline__ float from_bits(uint16_t b) {
+    return static_cast<float>(__builtin_bit_cast(f16_t, b));
+  }
+  __device__ static __forceinline__ uint16_t bits(float f) { return __builtin_bit_cast(uint16_t, static_cast<f16_t>(f)); }
+  __device__ static __forceinline__ float round(float f) { return static_cast<float>(static_cast<f16_t>(f)); }
+  __device__ static __forceinline__ uint32_t pack2(float lo, float hi) {
+    return static_cast<uint32_t>(bits(lo)) | (static_cast<uint32_t>(bits(hi)) << 16);
+  }
+  __device__ static __forceinline__ f32x4 mfma16(bf16x8 a, bf16x8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  }
+  __device__ static __forceinline__ f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  }
+};
+// storage tag -> format
+template <typename T> struct FormatOf;
+template <> struct FormatOf<uint16_t> { typedef Bf16 type; };
+template <> struct FormatOf<f16_t> { typedef Fp16 type; };
 
 // SiLU and sigmoid evaluated in fp32, as ATen does for reduced-precision inputs.  SiLU runs
 // once per intermediate element, so it uses the hardware exp2 and reciprocal (a few fp32

@@ -7,7 +7,7 @@ namespace sparse {
 
 int decode_routed_bf16(const sparse_hip_experts*, const void*, const void*, const int32_t*, const int32_t*,
                        const sparse_hip_seglist*, int, int, void*, void*, hipStream_t);
-int decode_shared_bf16(const void*, const void*, const void*, const void*, const void*, int, int, int, void*,
+int decode_shared_bf16(const void*, const void*, const void*, const void*, const void*, int, int, int, int, void*,
                        void*, hipStream_t);
 int decode_fused_bf16(const sparse_hip_experts*, const void*, const void*, const int32_t*, const int32_t*,
                       const sparse_hip_seglist*, int, int, void*, void*, const void*, const void*, const void*,
@@ -20,7 +20,7 @@ int prefill_routed_bf16(const sparse_hip_experts*, const void*, const void*, con
 size_t prefill_ws_bytes(int, int, int, int, int);
 int prefill_set_drain_waits(int);
 void prefill_set_clock_probe(void*);
-int prefill_shared_bf16(const void*, const void*, const void*, const void*, const void*, int, int, int, void*,
+int prefill_shared_bf16(const void*, const void*, const void*, const void*, const void*, int, int, int, int, void*,
                         void*, hipStream_t);
 template <typename T>
 int tiled_routed(const sparse_hip_experts*, const void*, const void*, const int32_t*, const int32_t*,
@@ -96,7 +96,7 @@ int sparse_hip_grouped_swiglu_decode(const sparse_hip_experts* experts, const vo
              T, SPARSE_HIP_DECODE_MAX_TOKENS);
   if (segs->n == 0) return SPARSE_HIP_OK;
   hipStream_t st = as_stream(stream);
-  if (experts->dtype == SPARSE_HIP_BF16)
+  if (is_16bit(experts->dtype))
     return decode_routed_bf16(experts, x_dev, topv_dev, perm_dev, seg_offsets_dev, segs, T, K, inter_ws_dev,
                               parts_dev, st);
   return tiled_routed<float>(experts, x_dev, topv_dev, perm_dev, seg_offsets_dev, segs, T, K, inter_ws_dev,
@@ -112,7 +112,7 @@ int sparse_hip_grouped_swiglu_prefill(const sparse_hip_experts* experts, const v
   if (rc != SPARSE_HIP_OK) return rc;
   if (segs->n == 0) return SPARSE_HIP_OK;
   hipStream_t st = as_stream(stream);
-  if (experts->dtype == SPARSE_HIP_BF16) {
+  if (is_16bit(experts->dtype)) {
     SP_REQUIRE(tile_ws_dev != nullptr && (reinterpret_cast<uintptr_t>(tile_ws_dev) & 15) == 0,
                "grouped_swiglu_prefill: tile workspace is NULL or not 16-byte aligned");
     return prefill_routed_bf16(experts, x_dev, topv_dev, perm_dev, seg_offsets_dev, segs, T, K, inter_ws_dev,
@@ -131,7 +131,10 @@ int sparse_hip_moe_ffn_decode(const sparse_hip_experts* experts, const void* x_d
   int rc = check_routed("moe_ffn_decode", experts, x_dev, topv_dev, perm_dev, seg_offsets_dev, segs, T, K,
                         inter_ws_dev, parts_dev);
   if (rc != SPARSE_HIP_OK) return rc;
-  SP_REQUIRE(experts->dtype == SPARSE_HIP_BF16, "moe_ffn_decode: bf16 only; use the separate entry points");
+  SP_REQUIRE(is_16bit(experts->dtype), "moe_ffn_decode: bf16 / fp16 only; use the separate entry points");
+  SP_REQUIRE(experts->dtype == SPARSE_HIP_BF16 || split_ws_dev == nullptr,
+             "moe_ffn_decode: the split shared projection is finished by sparse_hip_combine_split, which is bf16 only; "
+             "pass split_ws_dev = NULL for fp16 or call sparse_hip_moe_ffn_decode_combine");
   SP_REQUIRE(T <= SPARSE_HIP_DECODE_MAX_TOKENS, "moe_ffn_decode: T=%d exceeds %d", T,
              SPARSE_HIP_DECODE_MAX_TOKENS);
   SP_REQUIRE(Is > 0 && Is % 64 == 0, "moe_ffn_decode: Is=%d must be a positive multiple of 64", Is);
@@ -157,7 +160,7 @@ int sparse_hip_moe_ffn_decode_combine(const sparse_hip_experts* experts, const v
   int rc = check_routed("moe_ffn_decode_combine", experts, x_dev, topv_dev, perm_dev, seg_offsets_dev, segs, T, K,
                         inter_ws_dev, parts_dev);
   if (rc != SPARSE_HIP_OK) return rc;
-  SP_REQUIRE(experts->dtype == SPARSE_HIP_BF16, "moe_ffn_decode_combine: bf16 only");
+  SP_REQUIRE(is_16bit(experts->dtype), "moe_ffn_decode_combine: bf16 / fp16 only");
   SP_REQUIRE(T <= SPARSE_HIP_DECODE_MAX_TOKENS, "moe_ffn_decode_combine: T=%d exceeds %d", T,
              SPARSE_HIP_DECODE_MAX_TOKENS);
   SP_REQUIRE(Is > 0 && Is % 64 == 0, "moe_ffn_decode_combine: Is=%d must be a positive multiple of 64", Is);
@@ -200,20 +203,20 @@ int sparse_hip_shared_expert(const void* x_dev, const void* gate_w_dev, const vo
   SP_REQUIRE(x_dev && down_w_dev && inter_ws_dev && shared_dev, "shared_expert: NULL pointer");
   SP_REQUIRE((gate_w_dev == nullptr) == (up_w_dev == nullptr),
              "shared_expert: gate and up projections are given together or not at all");
-  SP_REQUIRE(gate_w_dev != nullptr || (dtype == SPARSE_HIP_BF16 && T <= SPARSE_HIP_DECODE_MAX_TOKENS),
-             "shared_expert: only a bf16 call of up to %d tokens can take a ready inter_ws", SPARSE_HIP_DECODE_MAX_TOKENS);
+  SP_REQUIRE(gate_w_dev != nullptr || (is_16bit(dtype) && T <= SPARSE_HIP_DECODE_MAX_TOKENS),
+             "shared_expert: only a 16-bit call of up to %d tokens can take a ready inter_ws", SPARSE_HIP_DECODE_MAX_TOKENS);
   SP_REQUIRE(((reinterpret_cast<uintptr_t>(x_dev) | reinterpret_cast<uintptr_t>(gate_w_dev) |
                reinterpret_cast<uintptr_t>(up_w_dev) | reinterpret_cast<uintptr_t>(down_w_dev) |
                reinterpret_cast<uintptr_t>(inter_ws_dev) | reinterpret_cast<uintptr_t>(shared_dev)) &
               15) == 0,
              "shared_expert: pointers must be 16-byte aligned");
   hipStream_t st = as_stream(stream);
-  if (dtype == SPARSE_HIP_BF16) {
+  if (is_16bit(dtype)) {
     if (T <= SPARSE_HIP_DECODE_MAX_TOKENS)
-      return decode_shared_bf16(x_dev, gate_w_dev, up_w_dev, down_w_dev, shared_gate_dev, T, H, Is, inter_ws_dev,
-                                shared_dev, st);
-    return prefill_shared_bf16(x_dev, gate_w_dev, up_w_dev, down_w_dev, shared_gate_dev, T, H, Is, inter_ws_dev,
-                               shared_dev, st);
+      return decode_shared_bf16(x_dev, gate_w_dev, up_w_dev, down_w_dev, shared_gate_dev, dtype, T, H, Is,
+                                inter_ws_dev, shared_dev, st);
+    return prefill_shared_bf16(x_dev, gate_w_dev, up_w_dev, down_w_dev, shared_gate_dev, dtype, T, H, Is,
+                               inter_ws_dev, shared_dev, st);
   }
   return tiled_shared<float>(x_dev, gate_w_dev, up_w_dev, down_w_dev, shared_gate_dev, T, H, Is, inter_ws_dev,
                              shared_dev, st);

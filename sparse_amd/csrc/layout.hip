@@ -46,7 +46,7 @@ int sparse_hip_tile_weight(const void* src_dev, void* dst_dev, int rows, int col
   const size_t n = static_cast<size_t>(rows) * cols;
   const unsigned grid = static_cast<unsigned>((n + 255) / 256);
   hipStream_t st = as_stream(stream);
-  if (dtype == SPARSE_HIP_BF16) {
+  if (is_16bit(dtype)) {
     if (to_tiled)
       hipLaunchKernelGGL((tile_weight_kernel<uint16_t, true>), dim3(grid), dim3(256), 0, st,
                          static_cast<const uint16_t*>(src_dev), static_cast<uint16_t*>(dst_dev), rows, cols);

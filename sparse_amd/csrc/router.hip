@@ -39,6 +39,15 @@ struct Raw8<uint16_t> {
     v[6] = __uint_as_float(a.w << 16); v[7] = __uint_as_float(a.w & 0xffff0000u);
   }
 };
+template <>
+struct Raw8<f16_t> {
+  f16x8 a;
+  __device__ __forceinline__ void load(const f16_t* p) { a = *reinterpret_cast<const f16x8*>(p); }
+  __device__ __forceinline__ void widen(float (&v)[8]) const {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = static_cast<float>(a[j]);
+  }
+};
 template <typename T>
 __device__ __forceinline__ void load8(const T* p, float (&v)[8]) {
   Raw8<T> r;
@@ -114,7 +123,7 @@ constexpr int kRlTok = 16;
 constexpr int kRlRows = 64;   // gate rows per pass
 constexpr int kRlPad = 65;    // LDS row stride in floats
 
-template <typename TL>
+template <typename F, typename TL>
 __global__ __launch_bounds__(256) void router_logits_mfma_kernel(
     const uint16_t* __restrict__ x, const uint16_t* __restrict__ wg, const uint16_t* __restrict__ wsg, int Ttok,
     int H, int E, TL* __restrict__ logits, uint16_t* __restrict__ shared_gate) {
@@ -149,7 +158,7 @@ __global__ __launch_bounds__(256) void router_logits_mfma_kernel(
       for (int u = 0; u < 4; ++u)
 #pragma unroll
         for (int nt = 0; nt < 4; ++nt)
-          acc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[u], bv[u][nt], acc[nt], 0, 0, 0);
+          acc[nt] = F::mfma16(av[u], bv[u][nt], acc[nt]);
     }
     // D: lane holds gate row (column) nt*16 + r for tokens q*4 .. q*4+3
     if (row0 > 0) __syncthreads();
@@ -166,7 +175,7 @@ __global__ __launch_bounds__(256) void router_logits_mfma_kernel(
         if (row < E) {
           Elem<TL>::store(logits + static_cast<size_t>(t) * E + row, sum);
         } else {
-          shared_gate[t] = f32_to_bf16_bits(sum);
+          shared_gate[t] = F::bits(sum);
         }
       }
     }
@@ -704,7 +713,8 @@ static int launch_router_logits(const void* x, const void* wg, const void* wsg, 
   if constexpr (sizeof(T) == 2) {
     if (Ttok >= 64 && H % 512 == 0) {
       ProfScope prof(SPARSE_HIP_K_ROUTER_LOGITS, st);
-      hipLaunchKernelGGL((router_logits_mfma_kernel<TL>), dim3((Ttok + kRlTok - 1) / kRlTok), dim3(256), 0, st,
+      hipLaunchKernelGGL((router_logits_mfma_kernel<typename FormatOf<T>::type, TL>),
+                         dim3((Ttok + kRlTok - 1) / kRlTok), dim3(256), 0, st,
                          static_cast<const uint16_t*>(x), static_cast<const uint16_t*>(wg),
                          static_cast<const uint16_t*>(wsg), Ttok, H, E, static_cast<TL*>(logits),
                          static_cast<uint16_t*>(shared_gate));
@@ -761,6 +771,11 @@ int sparse_hip_router_logits(const void* x_dev, const void* wg_dev, const void* 
   hipStream_t st = as_stream(stream);
   if (dtype == SPARSE_HIP_F32)
     return launch_router_logits<float, float>(x_dev, wg_dev, wsg_dev, T, H, E, logits_dev, shared_gate_dev, st);
+  if (dtype == SPARSE_HIP_F16) {
+    if (logits_dtype == SPARSE_HIP_F32)
+      return launch_router_logits<f16_t, float>(x_dev, wg_dev, wsg_dev, T, H, E, logits_dev, shared_gate_dev, st);
+    return launch_router_logits<f16_t, f16_t>(x_dev, wg_dev, wsg_dev, T, H, E, logits_dev, shared_gate_dev, st);
+  }
   if (logits_dtype == SPARSE_HIP_F32)
     return launch_router_logits<uint16_t, float>(x_dev, wg_dev, wsg_dev, T, H, E, logits_dev, shared_gate_dev, st);
   return launch_router_logits<uint16_t, uint16_t>(x_dev, wg_dev, wsg_dev, T, H, E, logits_dev, shared_gate_dev, st);
@@ -787,12 +802,19 @@ int sparse_hip_gate_topk_grouped(const void* logits_dev, int logits_dtype, int T
   SP_REQUIRE(logits_dev && topv_dev && topi_dev, "gate_topk: NULL pointer");
   if (T == 0) return SPARSE_HIP_OK;
   hipStream_t st = as_stream(stream);
-  const bool lb = logits_dtype == SPARSE_HIP_BF16, ob = out_dtype == SPARSE_HIP_BF16;
+  SP_REQUIRE(!(is_16bit(logits_dtype) && is_16bit(out_dtype)) || logits_dtype == out_dtype,
+             "gate_topk: 16-bit logits and 16-bit weights must be of the same format");
   const int ng = (n_group > 1 && topk_group < n_group) ? n_group : 0;  // every group kept = plain top-k
-  if (lb && ob)
-    return launch_gate_topk<uint16_t, uint16_t>(logits_dev, T, E, K, renorm, topv_dev, topi_dev, st, ng, topk_group);
-  if (lb) return launch_gate_topk<uint16_t, float>(logits_dev, T, E, K, renorm, topv_dev, topi_dev, st, ng, topk_group);
-  if (ob) return launch_gate_topk<float, uint16_t>(logits_dev, T, E, K, renorm, topv_dev, topi_dev, st, ng, topk_group);
+#define SP_TOPK_CASE(LD, OD, TL, TO)                                                                          \
+  if (logits_dtype == (LD) && out_dtype == (OD))                                                              \
+    return launch_gate_topk<TL, TO>(logits_dev, T, E, K, renorm, topv_dev, topi_dev, st, ng, topk_group);
+  SP_TOPK_CASE(SPARSE_HIP_BF16, SPARSE_HIP_BF16, uint16_t, uint16_t)
+  SP_TOPK_CASE(SPARSE_HIP_BF16, SPARSE_HIP_F32, uint16_t, float)
+  SP_TOPK_CASE(SPARSE_HIP_F32, SPARSE_HIP_BF16, float, uint16_t)
+  SP_TOPK_CASE(SPARSE_HIP_F16, SPARSE_HIP_F16, f16_t, f16_t)
+  SP_TOPK_CASE(SPARSE_HIP_F16, SPARSE_HIP_F32, f16_t, float)
+  SP_TOPK_CASE(SPARSE_HIP_F32, SPARSE_HIP_F16, float, f16_t)
+#undef SP_TOPK_CASE
   return launch_gate_topk<float, float>(logits_dev, T, E, K, renorm, topv_dev, topi_dev, st, ng, topk_group);
 }
 
@@ -807,6 +829,8 @@ int sparse_hip_topk(const void* values_dev, int T, int E, int K, int renorm, int
   hipStream_t st = as_stream(stream);
   if (out_dtype == SPARSE_HIP_BF16)
     return launch_gate_topk<float, uint16_t>(values_dev, T, E, K, renorm, topv_dev, topi_dev, st, 0, 0, 0);
+  if (out_dtype == SPARSE_HIP_F16)
+    return launch_gate_topk<float, f16_t>(values_dev, T, E, K, renorm, topv_dev, topi_dev, st, 0, 0, 0);
   return launch_gate_topk<float, float>(values_dev, T, E, K, renorm, topv_dev, topi_dev, st, 0, 0, 0);
 }
 
@@ -833,6 +857,10 @@ int sparse_hip_route_decode(const void* x_dev, const void* wg_dev, const void* w
                  T,         H,            E,               K,               renorm,          0};
   hipStream_t st = as_stream(stream);
   if (dtype == SPARSE_HIP_F32) return launch_route_decode<float, float>(a, st);
+  if (dtype == SPARSE_HIP_F16) {
+    if (logits_dtype == SPARSE_HIP_F32) return launch_route_decode<f16_t, float>(a, st);
+    return launch_route_decode<f16_t, f16_t>(a, st);
+  }
   if (logits_dtype == SPARSE_HIP_F32) return launch_route_decode<uint16_t, float>(a, st);
   return launch_route_decode<uint16_t, uint16_t>(a, st);
 }

@@ -53,6 +53,7 @@ struct DecodeArgs {
   int32_t Ndim_s;
   int32_t tiles_s;
   int32_t T;
+  int32_t fp16;                 // 16-bit format of every tensor: 0 bfloat16, 1 IEEE half
   // shared down projection with its reduction cut into `split_s` parts, one workgroup each
   // (1 = not cut): fp32 partial sums [split_s][T][Ndim_s], finished by the combine step
   int32_t split_s;
@@ -87,7 +88,7 @@ __device__ __forceinline__ bf16x8 ld_stream_bf16x8(const uint16_t* p) {
   return __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(p));
 }
 
-template <bool kGateUp, int NT>
+template <typename F, bool kGateUp, int NT>
 __global__ __launch_bounds__(kDecThreads) void decode_ffn_kernel(const DecodeArgs a) {
   constexpr int NM = kGateUp ? 2 : 1;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -209,8 +210,8 @@ __global__ __launch_bounds__(kDecThreads) void decode_ffn_kernel(const DecodeArg
     _Pragma("unroll") for (int tl = 0; tl < kDecTiles; ++tl)                                                \
     _Pragma("unroll") for (int nt = 0; nt < NT; ++nt)                                                       \
     _Pragma("unroll") for (int m = 0; m < NM; ++m) {                                                        \
-      acc[m][tl][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(W[m][tl][0], B[nt][0], acc[m][tl][nt], 0, 0, 0); \
-      acc[m][tl][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(W[m][tl][1], B[nt][1], acc[m][tl][nt], 0, 0, 0); \
+      acc[m][tl][nt] = F::mfma16(W[m][tl][0], B[nt][0], acc[m][tl][nt]);                                \
+      acc[m][tl][nt] = F::mfma16(W[m][tl][1], B[nt][1], acc[m][tl][nt]);                                \
     }                                                                                                       \
   } while (0)
 
@@ -264,11 +265,11 @@ __global__ __launch_bounds__(kDecThreads) void decode_ffn_kernel(const DecodeArg
     if (!kGateUp) {
       if (is_shared) {
         if (a.gate_s != nullptr) {
-          scale = round_bf16(sigmoid_f32(bf16_bits_to_f32(a.gate_s[n])));
+          scale = F::round(sigmoid_f32(F::from_bits(a.gate_s[n])));
           has_scale = true;
         }
       } else {
-        scale = bf16_bits_to_f32(a.topv[a.perm[r0 + n]]);
+        scale = F::from_bits(a.topv[a.perm[r0 + n]]);
         has_scale = true;
       }
     }
@@ -277,14 +278,14 @@ __global__ __launch_bounds__(kDecThreads) void decode_ffn_kernel(const DecodeArg
     for (int j = 0; j < 4; ++j) {
       float v;
       if (kGateUp) {
-        const float g = round_bf16(s0[j]);
-        const float u = round_bf16(s1[j]);
-        v = round_bf16(silu_f32(g)) * u;
+        const float g = F::round(s0[j]);
+        const float u = F::round(s1[j]);
+        v = F::round(silu_f32(g)) * u;
       } else {
-        v = round_bf16(s0[j]);
+        v = F::round(s0[j]);
         if (has_scale) v = v * scale;
       }
-      o[j] = f32_to_bf16_bits(v);
+      o[j] = F::bits(v);
     }
     uint16_t* dst = is_shared ? a.out_s + static_cast<size_t>(n) * Ndim + orow
                               : a.out_r + static_cast<size_t>(r0 + n) * Ndim + orow;
@@ -378,7 +379,7 @@ __global__ __launch_bounds__(kDecThreads) void decode_ffn_kernel(const DecodeArg
         const uint64_t v = ld_device_u64(a.out_r + static_cast<size_t>(pos[k]) * H + h);
 #pragma unroll
         for (int j = 0; j < 4; ++j)
-          accv[j] = round_bf16(accv[j] + bf16_bits_to_f32(static_cast<uint16_t>(v >> (16 * j))));
+          accv[j] = F::round(accv[j] + F::from_bits(static_cast<uint16_t>(v >> (16 * j))));
       }
     }
     const size_t part_stride = static_cast<size_t>(Ttok) * H;
@@ -399,13 +400,13 @@ __global__ __launch_bounds__(kDecThreads) void decode_ffn_kernel(const DecodeArg
       sh[3] += __uint_as_float(static_cast<uint32_t>(hi >> 32));
     }
     const bool gated = a.gate_s != nullptr;
-    const float scale = gated ? round_bf16(sigmoid_f32(bf16_bits_to_f32(a.gate_s[t]))) : 1.f;
+    const float scale = gated ? F::round(sigmoid_f32(F::from_bits(a.gate_s[t]))) : 1.f;
     uint16_t o[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      float v = round_bf16(sh[j]);
+      float v = F::round(sh[j]);
       if (gated) v = v * scale;
-      o[j] = f32_to_bf16_bits(accv[j] + round_bf16(v));
+      o[j] = F::bits(accv[j] + F::round(v));
     }
     uint2 pk;
     pk.x = static_cast<uint32_t>(o[0]) | (static_cast<uint32_t>(o[1]) << 16);
@@ -419,29 +420,32 @@ static int launch_decode(const DecodeArgs& a, int n_seg, hipStream_t st) {
   const int grid = a.tiles_s * (kGateUp ? 1 : a.split_s) + n_seg * a.tiles_r;
   if (grid == 0) return SPARSE_HIP_OK;
   ProfScope prof(kGateUp ? SPARSE_HIP_K_DECODE_GATEUP : SPARSE_HIP_K_DECODE_DOWN, st, /*dispatch_events=*/true);
-  if (prof.active()) {  // profiling: the launch stamps the event pair with the dispatch's begin and end
-    if (a.T <= 16) {
-      hipExtLaunchKernelGGL((decode_ffn_kernel<kGateUp, 1>), dim3(grid), dim3(kDecThreads), 0, st, prof.start_,
-                            prof.stop_, 0, a);
-    } else {
-      hipExtLaunchKernelGGL((decode_ffn_kernel<kGateUp, 2>), dim3(grid), dim3(kDecThreads), 0, st, prof.start_,
-                            prof.stop_, 0, a);
-    }
-  } else if (a.T <= 16) {
-    hipLaunchKernelGGL((decode_ffn_kernel<kGateUp, 1>), dim3(grid), dim3(kDecThreads), 0, st, a);
+#define SP_DEC_LAUNCH(F, NT)                                                                                  \
+  do {                                                                                                       \
+    if (prof.active()) { /* profiling: the launch stamps the event pair with the dispatch's begin and end */ \
+      hipExtLaunchKernelGGL((decode_ffn_kernel<F, kGateUp, NT>), dim3(grid), dim3(kDecThreads), 0, st,       \
+                            prof.start_, prof.stop_, 0, a);                                                  \
+    } else {                                                                                                 \
+      hipLaunchKernelGGL((decode_ffn_kernel<F, kGateUp, NT>), dim3(grid), dim3(kDecThreads), 0, st, a);      \
+    }                                                                                                        \
+  } while (0)
+  if (a.fp16) {
+    if (a.T <= 16) SP_DEC_LAUNCH(Fp16, 1); else SP_DEC_LAUNCH(Fp16, 2);
   } else {
-    hipLaunchKernelGGL((decode_ffn_kernel<kGateUp, 2>), dim3(grid), dim3(kDecThreads), 0, st, a);
+    if (a.T <= 16) SP_DEC_LAUNCH(Bf16, 1); else SP_DEC_LAUNCH(Bf16, 2);
   }
+#undef SP_DEC_LAUNCH
   SP_LAUNCH_CHECK("decode_ffn_kernel");
   return SPARSE_HIP_OK;
 }
 
-// Routed experts, bf16.  Two launches: gate-up into inter_ws, down into parts.
+// Routed experts, 16-bit formats (the slab's dtype picks bfloat16 or IEEE half).  Two launches: gate-up into inter_ws, down into parts.
 int decode_routed_bf16(const sparse_hip_experts* ex, const void* x, const void* topv, const int32_t* perm,
                        const int32_t* seg_offsets, const sparse_hip_seglist* segs, int T, int K,
                        void* inter_ws, void* parts, hipStream_t st) {
   const uint64_t H = ex->hidden, I = ex->inter;
   DecodeArgs a = {};
+  a.fp16 = ex->dtype == SPARSE_HIP_F16;
   a.split_s = 1;
   a.slab = static_cast<const uint16_t*>(ex->slab_dev);
   a.slot_stride = ex->slot_stride / 2;
@@ -473,7 +477,7 @@ int decode_routed_bf16(const sparse_hip_experts* ex, const void* x, const void* 
   return launch_decode<false>(a, segs->n, st);
 }
 
-// Routed experts and the shared expert in one launch pair, bf16, T <= 32.  The shared
+// Routed experts and the shared expert in one launch pair, 16-bit formats, T <= 32.  The shared
 // expert's tiles lead the grid (largest, known amount of work), routed segments follow.
 int decode_fused_bf16(const sparse_hip_experts* ex, const void* x, const void* topv, const int32_t* perm,
                       const int32_t* seg_offsets, const sparse_hip_seglist* segs, int T, int K, void* inter_ws,
@@ -482,6 +486,7 @@ int decode_fused_bf16(const sparse_hip_experts* ex, const void* x, const void* t
                       const int32_t* inv_perm, void* final_out, hipStream_t st) {
   const uint64_t H = ex->hidden, I = ex->inter;
   DecodeArgs a = {};
+  a.fp16 = ex->dtype == SPARSE_HIP_F16;
   a.split_s = 1;
   a.slab = static_cast<const uint16_t*>(ex->slab_dev);
   a.slot_stride = ex->slot_stride / 2;
@@ -548,11 +553,12 @@ size_t decode_split_ws_bytes(int T, int H) {
 size_t decode_split_counter_offset(int T, int H) { return static_cast<size_t>(kDecSplit) * T * H * sizeof(float); }
 int decode_split_parts(int Is) { return (Is / 64) % kDecSplit == 0 ? kDecSplit : 1; }
 
-// Shared expert, bf16, T <= 32.
+// Shared expert, 16-bit formats, T <= 32.
 int decode_shared_bf16(const void* x, const void* gate_w, const void* up_w, const void* down_w,
-                       const void* shared_gate, int T, int H, int Is, void* inter_ws, void* shared_out,
+                       const void* shared_gate, int dtype, int T, int H, int Is, void* inter_ws, void* shared_out,
                        hipStream_t st) {
   DecodeArgs a = {};
+  a.fp16 = dtype == SPARSE_HIP_F16;
   a.split_s = 1;
   a.T = T;
   a.topk = 1;

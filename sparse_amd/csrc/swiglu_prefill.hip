@@ -74,6 +74,7 @@ struct PrefillArgs {
   const uint16_t* w_s;
   const uint16_t* w2_s;
   const uint16_t* gate_s;
+  int32_t fp16;             // 16-bit format of every tensor: 0 bfloat16, 1 IEEE half
   unsigned long long* clk;  // clock probe: [0] += shader-clock cycles, [1] += 100 MHz ticks per workgroup; may be null
 };
 
@@ -138,7 +139,7 @@ __global__ __launch_bounds__(256) void prefill_tile_map_kernel(const PfMapArgs a
 // kDrainWaits replaces the counted vector-memory waits of the k loop by full drains: slower,
 // and correct whatever else the compiler has in flight.  It exists to check the counted
 // waits: both variants must give the same bits.
-template <bool kGateUp, bool kDrainWaits>
+template <typename F, bool kGateUp, bool kDrainWaits>
 __global__ __launch_bounds__(kPfThreads, 2) void prefill_ffn_kernel(const PrefillArgs a) {
   __shared__ __attribute__((aligned(1024))) uint8_t lds[kPfStages][kPfLdsA];
   __shared__ float s_scale[kPfBM];
@@ -191,9 +192,9 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_ffn_kernel(const Prefil
     if (tid < M) {
       const int p = r0 + tid;
       if (a.shared) {
-        if (a.gate_s != nullptr) sc = round_bf16(sigmoid_f32(bf16_bits_to_f32(a.gate_s[p])));
+        if (a.gate_s != nullptr) sc = F::round(sigmoid_f32(F::from_bits(a.gate_s[p])));
       } else {
-        sc = bf16_bits_to_f32(a.topv[a.perm[p]]);
+        sc = F::from_bits(a.topv[a.perm[p]]);
       }
     }
     s_scale[tid] = sc;
@@ -302,7 +303,7 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_ffn_kernel(const Prefil
         for (int mi = 0; mi < NMI; ++mi)
   #pragma unroll
           for (int ni = 0; ni < 2; ++ni)
-            acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfrag[st][ni][s], fa[mi], acc[mi][ni], 0, 0, 0);
+            acc[mi][ni] = F::mfma32(bfrag[st][ni][s], fa[mi], acc[mi][ni]);
         __builtin_amdgcn_sched_barrier(kPfSchedMask);
   #pragma unroll
         for (int ni = 0; ni < 2; ++ni)
@@ -350,16 +351,16 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_ffn_kernel(const Prefil
   #pragma unroll
           for (int j = 0; j < 4; ++j) {
             if (kGateUp) {
-              const float g = round_bf16(acc[mi][0][4 * i + j]);
-              const float u = round_bf16(acc[mi][1][4 * i + j]);
-              v[j] = round_bf16(silu_f32(g)) * u;
+              const float g = F::round(acc[mi][0][4 * i + j]);
+              const float u = F::round(acc[mi][1][4 * i + j]);
+              v[j] = F::round(silu_f32(g)) * u;
             } else {
-              v[j] = round_bf16(acc[mi][pass][4 * i + j]) * sc[mi];
+              v[j] = F::round(acc[mi][pass][4 * i + j]) * sc[mi];
             }
           }
           uint2 pk;
-          pk.x = f32x2_to_bf16x2_bits(v[0], v[1]);
-          pk.y = f32x2_to_bf16x2_bits(v[2], v[3]);
+          pk.x = F::pack2(v[0], v[1]);
+          pk.y = F::pack2(v[2], v[3]);
           const int chunk = i ^ ((m >> 1) & 3);
           *reinterpret_cast<uint2*>(st + m * 64 + chunk * 16 + fg * 8) = pk;
         }
@@ -405,12 +406,15 @@ static int launch_prefill(PrefillArgs& a, int max_mtiles, hipStream_t st) {
   SP_REQUIRE(grid < (1ll << 31), "prefill_ffn: grid too large");
   ProfScope prof(kGateUp ? SPARSE_HIP_K_PREFILL_GATEUP : SPARSE_HIP_K_PREFILL_DOWN, st);
   a.clk = g_prefill_clock.load(std::memory_order_relaxed);
-  if (g_prefill_drain_waits.load(std::memory_order_relaxed))
-    hipLaunchKernelGGL((prefill_ffn_kernel<kGateUp, true>), dim3(static_cast<unsigned>(grid)), dim3(kPfThreads), 0,
-                       st, a);
-  else
-    hipLaunchKernelGGL((prefill_ffn_kernel<kGateUp, false>), dim3(static_cast<unsigned>(grid)), dim3(kPfThreads), 0,
-                       st, a);
+  const bool drain = g_prefill_drain_waits.load(std::memory_order_relaxed) != 0;
+#define SP_PF_LAUNCH(F, D) \
+  hipLaunchKernelGGL((prefill_ffn_kernel<F, kGateUp, D>), dim3(static_cast<unsigned>(grid)), dim3(kPfThreads), 0, st, a)
+  if (a.fp16) {
+    if (drain) SP_PF_LAUNCH(Fp16, true); else SP_PF_LAUNCH(Fp16, false);
+  } else {
+    if (drain) SP_PF_LAUNCH(Bf16, true); else SP_PF_LAUNCH(Bf16, false);
+  }
+#undef SP_PF_LAUNCH
   SP_LAUNCH_CHECK("prefill_ffn_kernel");
   return SPARSE_HIP_OK;
 }
@@ -453,6 +457,7 @@ int prefill_routed_bf16(const sparse_hip_experts* ex, const void* x, const void*
     SP_LAUNCH_CHECK("prefill_tile_map_kernel");
   }
   PrefillArgs a = {};
+  a.fp16 = ex->dtype == SPARSE_HIP_F16;
   a.slab = static_cast<const uint16_t*>(ex->slab_dev);
   a.slot_stride = ex->slot_stride / 2;
   a.perm = perm;
@@ -483,9 +488,10 @@ int prefill_routed_bf16(const sparse_hip_experts* ex, const void* x, const void*
 }
 
 int prefill_shared_bf16(const void* x, const void* gate_w, const void* up_w, const void* down_w,
-                        const void* shared_gate, int Ttok, int H, int Is, void* inter_ws, void* shared_out,
-                        hipStream_t st) {
+                        const void* shared_gate, int dtype, int Ttok, int H, int Is, void* inter_ws,
+                        void* shared_out, hipStream_t st) {
   PrefillArgs a = {};
+  a.fp16 = dtype == SPARSE_HIP_F16;
   a.shared = 1;
   a.T = Ttok;
   a.topk = 1;

@@ -193,7 +193,7 @@ def measure_costs(block: Any, batches: Sequence[int] = (1, 4, 8, 16, 32), repeat
         torch.cuda.synchronize()
         return start.elapsed_ms(end) / n
 
-    elem = 2 if block.dtype == torch.bfloat16 else 4
+    elem = 4 if block.dtype == torch.float32 else 2
     nbytes = int(expert_bytes) if expert_bytes else 3 * block.hidden_size * block.inter_size * elem
     host = ops.host_alloc(nbytes)
     try:

@@ -14,15 +14,26 @@ import torch
 
 from . import _lib
 from ._lru import LruTable
-from ._lib import BF16, F32, DECODE_MAX_TOKENS, Experts, SegList
+from ._lib import BF16, F16, F32, DECODE_MAX_TOKENS, Experts, SegList
 
 
 def dtype_code(dtype: torch.dtype) -> int:
     if dtype == torch.bfloat16:
         return BF16
+    if dtype == torch.float16:
+        return F16
     if dtype == torch.float32:
         return F32
-    raise ValueError(f"unsupported dtype {dtype}: the MoE kernels take bfloat16 or float32")
+    raise ValueError(f"unsupported dtype {dtype}: the MoE kernels take bfloat16, float16 or float32")
+
+
+HALF_DTYPES = (torch.bfloat16, torch.float16)   # the 16-bit formats of the MFMA kernels
+
+
+def _need_half(t: torch.Tensor, name: str) -> None:
+    _need(t, name)
+    if t.dtype not in HALF_DTYPES:
+        raise ValueError(f"{name} must be bfloat16 or float16, got {t.dtype}")
 
 
 def _stream() -> int:
@@ -491,7 +502,8 @@ def moe_ffn_decode(experts: Experts, x: torch.Tensor, topv: torch.Tensor, perm: 
                    inter_ws: torch.Tensor, parts: torch.Tensor, shared_w, shared_gate: Optional[torch.Tensor],
                    shared_inter_ws: torch.Tensor, shared_out: torch.Tensor,
                    split_ws: Optional[torch.Tensor] = None, shared_inter_ready: bool = False) -> None:
-    """Routed experts + shared expert of a decode call in one launch pair (bf16, T <= 32).
+    """Routed experts + shared expert of a decode call in one launch pair (bf16 or fp16, T <= 32;
+    ``split_ws`` with bf16 only, whose combine step finishes the split).
     ``split_ws`` (from ``decode_split_workspace``) lets the shared down projection spread its
     long reduction over four workgroups per tile.  ``shared_inter_ready``: ``shared_inter_ws``
     already holds the shared expert's SiLU(gate x) * (up x) (``route_decode_packed`` computed it
@@ -501,7 +513,7 @@ def moe_ffn_decode(experts: Experts, x: torch.Tensor, topv: torch.Tensor, perm: 
     K = topv.shape[1]
     gw, uw, dw = shared_w
     Is = gw.shape[0]
-    _need(x, "x", torch.bfloat16)
+    _need_half(x, "x")
     _need(topv, "topv", x.dtype, (T, K))
     _need(inter_ws, "inter_ws", x.dtype, (T * K, experts.inter))
     _need(parts, "parts", x.dtype, (T * K, H))
@@ -542,7 +554,7 @@ def moe_ffn_decode_combine(experts: Experts, x: torch.Tensor, topv: torch.Tensor
     K = topv.shape[1]
     gw, uw, dw = shared_w
     Is = gw.shape[0]
-    _need(x, "x", torch.bfloat16)
+    _need_half(x, "x")
     _need(topv, "topv", x.dtype, (T, K))
     _need(inter_ws, "inter_ws", x.dtype, (T * K, experts.inter))
     _need(parts, "parts", x.dtype, (T * K, H))

@@ -1,0 +1,211 @@
+"""GPU parity of the fp16 path (the reference's formal dtype, scripts/run/run_case.sh:199) against the CPU
+oracle run in fp16: the same kernels as bf16 with IEEE-half conversions and the fp16 MFMA.
+
+Indices and permutations bit for bit; values within rtol 5e-3 / atol 2e-3 (fp16 keeps 11 significant
+bits where bf16 keeps 8, so the bound is tighter than the bf16 one the north star states; what remains
+is the order of the fp32 sums before each rounding)."""
+import pytest
+import torch
+
+from oracle import ref_moe
+from tests.helpers import make_hidden, make_layer
+from tests.test_gpu_kernels import _ops, _routing, _run_routed
+
+pytestmark = pytest.mark.gpu
+
+F16 = torch.float16
+FP16_TOL = dict(rtol=5e-3, atol=2e-3)
+
+
+def _rel(a, b):
+    return float((a.float() - b.float()).abs().max() / b.float().abs().max())
+
+
+@pytest.mark.parametrize("T", [1, 8, 33, 128])
+def test_router_logits_fp16(device, T):
+    """T >= 64 takes the MFMA kernel, smaller calls the FMA one; logits in fp16 or fp32."""
+    ops = _ops()
+    layer = make_layer(2048, 60, 64, 4, Is=64, shared_gate=True, dtype=F16, seed=3)
+    x = make_hidden(T, 2048, F16, seed=4)
+    ref = torch.nn.functional.linear(x.float(), layer["gate_w"].float())
+    ref_sg = torch.nn.functional.linear(x.float(), layer["shared_gate_w"].float().reshape(1, -1)).reshape(-1)
+    logits, sg = ops.router_logits(x.to(device), layer["gate_w"].to(device), layer["shared_gate_w"].to(device))
+    assert logits.dtype == F16 and sg.dtype == F16
+    torch.testing.assert_close(logits.float().cpu(), ref, rtol=2e-3, atol=2e-3)
+    torch.testing.assert_close(sg.float().cpu(), ref_sg, rtol=2e-3, atol=2e-3)
+    l32, _ = ops.router_logits(x.to(device), layer["gate_w"].to(device), logits_dtype=torch.float32)
+    assert l32.dtype == torch.float32
+    torch.testing.assert_close(l32.cpu(), ref, rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("E,K", [(60, 4), (64, 6), (200, 8)])
+def test_gate_topk_fp16_logits_and_weights(device, E, K):
+    """Indices are a function of the logits alone (descending, then lower id), also where fp16 logits
+    tie around the K-th place; weights are the softmax probabilities rounded to fp16."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(E * 100 + K)
+    logits = (torch.randn(257, E, generator=g) * 2.0).to(F16)
+    srt = torch.sort(logits.float(), dim=-1, descending=True)
+    for t in range(0, 257, 3):
+        a, b = int(srt.indices[t, K - 1]), int(srt.indices[t, K])
+        logits[t, b] = logits[t, a]
+    probs = torch.softmax(logits, dim=-1, dtype=torch.float32)
+    ref_v, ref_i = ref_moe.topk_by_logit(logits, probs, K)
+    topv, topi = ops.gate_topk(logits.to(device), K, out_dtype=F16)
+    assert topv.dtype == F16
+    assert torch.equal(topi.cpu(), ref_i)
+    torch.testing.assert_close(topv.cpu().float(), ref_v.to(F16).float(), rtol=2e-3, atol=1e-6)
+    topv32, topi32 = ops.gate_topk(logits.to(device), K, out_dtype=torch.float32)
+    assert torch.equal(topi32.cpu(), ref_i)
+    torch.testing.assert_close(topv32.cpu(), ref_v.float(), rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.parametrize("T", [1, 8, 32])
+def test_route_decode_fp16_equals_the_three_separate_calls(device, T):
+    ops = _ops()
+    E, K, H = 60, 4, 2048
+    layer = make_layer(H, E, 64, K, Is=64, shared_gate=True, dtype=F16, seed=7)
+    wg, wsg = layer["gate_w"].to(device), layer["shared_gate_w"].to(device)
+    counter = torch.zeros(1, dtype=torch.int32, device=device)
+    for rep in range(2):
+        x = make_hidden(T, H, F16, seed=100 + rep).to(device)
+        logits_a, sg_a = ops.router_logits(x, wg, wsg)
+        logits_b, sg_b = torch.empty_like(logits_a), torch.empty_like(sg_a)
+        topv_b = torch.empty(T, K, dtype=F16, device=device)
+        topi_b = torch.empty(T, K, dtype=torch.int64, device=device)
+        perm_b = ops.Permutation(T, K, E, device)
+        ops.route_decode(x, wg, wsg, K, False, logits_b, sg_b, topv_b, topi_b, perm_b, counter)
+        torch.cuda.synchronize()
+        assert int(counter.item()) == 0
+        torch.testing.assert_close(logits_b.float(), logits_a.float(), rtol=1e-3, atol=1e-6)   # one fp16 ulp
+        torch.testing.assert_close(sg_b.float(), sg_a.float(), rtol=1e-3, atol=1e-6)
+        topv_a, topi_a = ops.gate_topk(logits_b, K, out_dtype=F16)
+        perm_a = ops.permute_build(topi_a, E)
+        torch.cuda.synchronize()
+        assert torch.equal(topv_a, topv_b) and torch.equal(topi_a, topi_b)
+        for name in ("perm", "inv_perm", "seg_offsets"):
+            assert torch.equal(getattr(perm_a, name), getattr(perm_b, name)), name
+
+
+@pytest.mark.parametrize("T", [1, 8, 17, 32])
+def test_decode_ffn_fp16_matches_oracle(device, T):
+    ops = _ops()
+    layer = make_layer(512, 12, 256, 4, dtype=F16, seed=11, std=0.05)
+    x = make_hidden(T, 512, F16, seed=12)
+    topv, topi = _routing(layer, x)
+    out, _, _ = _run_routed(ops, layer, x, topv, topi, device, decode=True)
+    ref = ref_moe.experts_world1_exact(x, topi, topv, layer["experts"])
+    torch.testing.assert_close(out.float(), ref.float(), **FP16_TOL)
+    assert _rel(out, ref) < 5e-3   # a bf16 instruction on fp16 bits, or a wrong mapping, gives O(1)
+
+
+@pytest.mark.parametrize("T", [40, 300])
+def test_prefill_ffn_fp16_matches_oracle(device, T):
+    ops = _ops()
+    layer = make_layer(512, 12, 256, 4, dtype=F16, seed=21, std=0.05)
+    x = make_hidden(T, 512, F16, seed=22)
+    topv, topi = _routing(layer, x)
+    out, _, _ = _run_routed(ops, layer, x, topv, topi, device, decode=False)
+    ref = ref_moe.experts_world1_exact(x, topi, topv, layer["experts"])
+    torch.testing.assert_close(out.float(), ref.float(), **FP16_TOL)
+    assert _rel(out, ref) < 5e-3
+
+
+def test_ffn_fp16_at_the_qwen_shape(device):
+    ops = _ops()
+    layer = make_layer(2048, 60, 1408, 4, dtype=F16, seed=0)
+    x = make_hidden(8, 2048, F16, seed=1000)
+    topv, topi = _routing(layer, x)
+    ref = ref_moe.experts_world1_exact(x, topi, topv, layer["experts"])
+    for decode in (True, False):
+        out, _, _ = _run_routed(ops, layer, x, topv, topi, device, decode=decode)
+        torch.testing.assert_close(out.float(), ref.float(), **FP16_TOL)
+        assert _rel(out, ref) < 5e-3
+
+
+@pytest.mark.parametrize("T", [8, 32, 200])
+@pytest.mark.parametrize("gated", [True, False])
+def test_shared_expert_fp16(device, T, gated):
+    ops = _ops()
+    layer = make_layer(512, 4, 64, 2, Is=384, shared_gate=gated, dtype=F16, seed=61, std=0.05)
+    x = make_hidden(T, 512, F16, seed=62)
+    ref = ref_moe.shared_expert_forward(x, layer["shared"], layer["shared_gate_w"])
+    xd = x.to(device)
+    sg = None
+    if gated:
+        _, sg = ops.router_logits(xd, layer["gate_w"].to(device), layer["shared_gate_w"].to(device))
+    from sparse_amd.weights import tile_weight
+    gw, uw, dw = (tile_weight(t).reshape(t.shape).contiguous().to(device) for t in layer["shared"])
+    inter = torch.empty((T, 384), device=device, dtype=F16)
+    out = torch.empty((T, 512), device=device, dtype=F16)
+    ops.shared_expert(xd, gw, uw, dw, sg, inter, out)
+    torch.testing.assert_close(out.cpu().float(), ref.float(), **FP16_TOL)
+
+
+def test_combine_fp16_is_the_ordered_sum(device):
+    ops = _ops()
+    T, K, H, E = 37, 4, 256, 20
+    g = torch.Generator().manual_seed(71)
+    topi = torch.topk(torch.rand(T, E, generator=g), K, dim=1).indices.to(torch.int64)
+    parts_tkh = (torch.randn(T, K, H, generator=g) * 3).to(F16)
+    shared = torch.randn(T, H, generator=g).to(F16)
+    ref = ref_moe.combine_expert_outputs(parts_tkh, topi) + shared
+    p = ops.permute_build(topi.to(device), E)
+    parts_sorted = parts_tkh.reshape(T * K, H)[p.perm.cpu().long()].contiguous().to(device)
+    out = torch.empty((T, H), device=device, dtype=F16)
+    ops.combine(parts_sorted, p, shared.to(device), T, K, out)
+    assert torch.equal(out.cpu(), ref)   # same adds in the same order: bit for bit
+
+
+SMALL_Q = dict(family="qwen_shared", hidden=512, num_experts=12, inter=256, top_k=4, shared_inter=384)
+SMALL_D = dict(family="deepseek_shared", hidden=512, num_experts=16, inter=256, top_k=6, shared_inter=512)
+
+
+def _check_block(shape, T, device, fused=False, seed=0):
+    from sparse_amd.synthetic import make_hidden as mk
+    from tests.helpers import oracle_layer
+    from tests.test_gpu_block import _build
+    mlp, blk = _build(shape, F16, device, seed=seed, fused=fused)
+    H = shape["hidden"]
+    x = mk(T, H, F16, seed=1000 + seed)
+    ret = blk(x.view(1, T, H).to(device))
+    torch.cuda.synchronize()
+    lay = oracle_layer(mlp)
+    ws = blk._workspace(T)
+    if lay["family"] == "qwen_shared":
+        out, logits = ret
+        logits = logits.cpu()
+        assert logits.dtype == F16
+    else:
+        out = ret
+        from sparse_amd import ops
+        logits, _ = ops.router_logits(x.to(device), blk.gate_weight, None, torch.float32)
+        logits = logits.cpu()
+    ref_out, ref_topv, ref_topi, _ = ref_moe.moe_forward(
+        x, lay["gate_w"], lay["experts"], shape["top_k"], lay["shared"], lay["shared_gate_w"],
+        family=lay["family"], router_logits=logits)
+    topi_dev = ws.topi.cpu()
+    if lay["family"] == "qwen_shared":
+        assert torch.equal(topi_dev, ref_topi), "expert indices differ on identical logits"
+    else:
+        assert torch.equal(torch.sort(topi_dev, 1).values, torch.sort(ref_topi, 1).values)
+    out = out.cpu().view(T, H)
+    assert out.dtype == F16
+    torch.testing.assert_close(out.float(), ref_out.float(), **FP16_TOL)
+    assert _rel(out, ref_out) < 5e-3
+
+
+@pytest.mark.parametrize("T", [1, 8, 32, 33, 130])
+def test_small_qwen_block_fp16(device, T):
+    _check_block(SMALL_Q, T, device)
+
+
+@pytest.mark.parametrize("T", [4, 200])
+def test_small_deepseek_block_fp16(device, T):
+    _check_block(SMALL_D, T, device, fused=True)
+
+
+def test_qwen_shape_fp16_decode_and_prefill(device):
+    from sparse_amd.synthetic import QWEN
+    for T in (8, 160):
+        _check_block(QWEN, T, device, seed=1)
