@@ -513,6 +513,7 @@ def main():
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--no-extra", action="store_true", help="skip batch 1/32 decode and the prefill workload")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-offload", action="store_true", help="skip the two offloaded workloads (the long legs)")
     ap.add_argument("--only-prefill", action="store_true", help="run just the prefill workload (for profiling)")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also launch a 256 MiB plain copy kernel a few times (yardstick for --pmc byte counters)")
@@ -564,7 +565,7 @@ def main():
     if not args.no_extra:
         extra["prefill_4k_deepseek"] = prefill_workload(DEEPSEEK, 4096, max(2, min(10, args.steps // 10)), 1, dtype,
                                                         device)
-    if not args.no_extra:
+    if not args.no_extra and not args.no_offload:
         # the offloaded configurations: rr and rs as the configuration states them (512 decode steps
         # from a cold cache), this build's other variants at 64 steps and labelled so; a failure
         # here (e.g. no pinned memory to be had) must not cost the main line
