@@ -373,6 +373,21 @@ int sparse_hip_combine_split(const void* parts_dev, const int32_t* inv_perm_dev,
                              int nparts, const void* shared_gate_dev, int T, int K, int H,
                              void* out_dev, void* stream);
 
+/* ---- A12: routing-scout predictor ------------------------------------------ */
+
+/*
+ * pred[T, E] = softmax(w2 relu(w1 float(x) + b1) + b2): the forward pass of the reference's
+ * `RoutingScoutMLP` in eval mode (utils/eval_core.py:3402-3417: Linear, BatchNorm1d, ReLU, Dropout,
+ * Linear, Softmax) as `_compute_and_schedule_next_layer_rs` runs it on the layer's input
+ * (:10916-10960, `rs_in = x.float()`), for a decode-size call (T <= SPARSE_HIP_DECODE_MAX_TOKENS).
+ * All parameters are fp32 and row-major; the caller folds the BatchNorm's running statistics and affine
+ * into w1 [D, H] and b1 [D] once, at load time (eval mode makes it a per-row scale and shift; Dropout is
+ * the identity).  x is [T, H] in `dtype`; hidden_ws_dev holds T * D floats; w2 is [E, D].  Two launches.
+ */
+int sparse_hip_rs_predict(const void* x_dev, int dtype, int T, int H, const float* w1_dev, const float* b1_dev,
+                          int D, const float* w2_dev, const float* b2_dev, int E, float* hidden_ws_dev,
+                          float* pred_dev, void* stream);
+
 /* ---- A11/A12/A13: expert residency ----------------------------------------- */
 
 /*

@@ -108,6 +108,7 @@ SIGNATURES = {
     "sparse_hip_host_free": (_i, [_vp]),
     "sparse_hip_tile_weight": (_i, [_vp, _vp, _i, _i, _i, _i, _vp]),
     "sparse_hip_calib_copy": (_i, [_vp, _vp, _sz, _vp]),
+    "sparse_hip_rs_predict": (_i, [_vp, _i, _i, _i, _vp, _vp, _i, _vp, _vp, _i, _vp, _vp, _vp]),
     "sparse_hip_prefill_drain_waits": (_i, [_i]),
     "sparse_hip_prefill_clock_probe": (_i, [_vp]),
     "sparse_hip_profile_enable": (_i, [_i]),

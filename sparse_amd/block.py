@@ -28,7 +28,7 @@ from . import ops
 from ._lru import LruTable
 from .context import DistEnv, Metrics, SparseContext
 from .residency import Backend, LayerResidency, ResidencyConfig
-from .rs import router_topk_feature, stable_topk, topk_for_planning
+from .rs import fused_scout, router_topk_feature, stable_topk, topk_for_planning
 from .weights import ExpertSlab, HostExpertArena, tile_weight
 
 
@@ -528,15 +528,21 @@ class DistributedSparseMoeBlock(nn.Module):
             policy = tres.light_policy
             here = policy.profile.cost(self.rank, self.layer_idx)
             policy.window_ms = here.compute(self.top_k, int(x.shape[0]) * self.top_k) + policy.cost.attention
-        rs_in = x.float()
         mode = self._next_layer_rs_feature_mode()
-        if mode == "hidden_router_topk":
-            if source is None:
-                return None
-            rs_in = torch.cat([rs_in, router_topk_feature(source[0], source[1], self.num_experts)], dim=-1)
-        elif mode != "hidden":
-            raise RuntimeError(f"Unsupported next-layer RS feature_mode={mode}")
-        pred = SparseContext.rs_bank[target](rs_in).to(torch.float32)
+        module = SparseContext.rs_bank[target]
+        fused = fused_scout(module, x) if mode == "hidden" else None
+        if fused is not None:
+            # decode-size call of the plain predictor: two HIP launches on the token rows as they are
+            pred = fused(x)
+        else:
+            rs_in = x.float()
+            if mode == "hidden_router_topk":
+                if source is None:
+                    return None
+                rs_in = torch.cat([rs_in, router_topk_feature(source[0], source[1], self.num_experts)], dim=-1)
+            elif mode != "hidden":
+                raise RuntimeError(f"Unsupported next-layer RS feature_mode={mode}")
+            pred = module(rs_in).to(torch.float32)
         self.metrics.rs_next_layer_pred_calls += 1
         self.metrics.rs_mlp_calls += 1
         if for_routing:

@@ -29,6 +29,7 @@ SOURCES = [
     "ffn_tiled.hip",
     "ffn.hip",
     "combine.hip",
+    "rs_predict.hip",
     "layout.hip",
 ]
 

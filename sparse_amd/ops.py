@@ -483,6 +483,31 @@ def profile_read() -> dict:
     return out
 
 
+def rs_predict(x: torch.Tensor, w1: torch.Tensor, b1: torch.Tensor, w2: torch.Tensor, b2: torch.Tensor,
+               hidden_ws: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Routing-scout forward pass of a decode-size call: ``softmax(w2 relu(w1 x + b1) + b2)`` in fp32, with
+    fp32 parameters whose BatchNorm is already folded into ``w1`` / ``b1``.  Returns ``pred [T, E]``."""
+    T, H = x.shape
+    D, E = w1.shape[0], w2.shape[0]
+    _need(x, "x")
+    _need(w1, "w1", torch.float32, (D, H))
+    _need(b1, "b1", torch.float32, (D,))
+    _need(w2, "w2", torch.float32, (E, D))
+    _need(b2, "b2", torch.float32, (E,))
+    if hidden_ws is None:
+        hidden_ws = torch.empty((T, D), device=x.device, dtype=torch.float32)
+    if out is None:
+        out = torch.empty((T, E), device=x.device, dtype=torch.float32)
+    _need(hidden_ws, "hidden workspace", torch.float32)
+    _need(out, "pred", torch.float32, (T, E))
+    if hidden_ws.numel() < T * D:
+        raise ValueError("hidden workspace is too small")
+    rc = _lib.load().sparse_hip_rs_predict(_ptr(x), dtype_code(x.dtype), T, H, _ptr(w1), _ptr(b1), D, _ptr(w2),
+                                           _ptr(b2), E, _ptr(hidden_ws), _ptr(out), _stream())
+    _lib.check(rc, "sparse_hip_rs_predict")
+    return out
+
+
 def prefill_clock_probe(counters: Optional[torch.Tensor]) -> None:
     """Point the prefill-size FFN kernel's clock probe at ``counters`` (two int64 in device memory, which
     the caller zeroes: [0] collects shader-clock cycles, [1] ticks of the constant 100 MHz clock, summed

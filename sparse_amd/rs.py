@@ -4,7 +4,9 @@
 the same name (utils/eval_core.py:3402-3417: Linear, BatchNorm1d, ReLU, Dropout(0.1),
 Linear, Softmax), so a bank trained for the reference (``rs_l{L}_inL{L-1}.pth`` payloads
 with a ``state_dict``, :3490-3550) loads into it unchanged.  Prediction runs on the device
-in fp32 through PyTorch; only its top-k leaves the device.
+in fp32: decode-size calls of the plain MLP through the two-launch HIP predictor (``FusedScout``,
+``sparse_hip_rs_predict``), everything else (the residual predictor, predictors that also read the
+routing, prefill-size calls) through PyTorch; only the top-k leaves the device.
 """
 from __future__ import annotations
 
@@ -33,6 +35,45 @@ class RoutingScoutMLP(nn.Module):
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         return self.mlp(x.reshape(-1, x.shape[-1]))
+
+
+class FusedScout:
+    """The parameters of a ``RoutingScoutMLP`` in eval mode as the HIP predictor kernel takes them: fp32,
+    row-major, the BatchNorm's running statistics and affine folded into the first Linear (eval mode makes
+    it a per-row scale and shift).  Built once per module (``fused_scout``); a module that is retrained or
+    moved afterwards must be fused again."""
+
+    def __init__(self, module: "RoutingScoutMLP") -> None:
+        lin1, bn, lin2 = module.mlp[0], module.mlp[1], module.mlp[4]
+        with torch.no_grad():
+            scale = bn.weight.float() / torch.sqrt(bn.running_var.float() + bn.eps)
+            self.w1 = (lin1.weight.float() * scale[:, None]).contiguous()
+            self.b1 = ((lin1.bias.float() - bn.running_mean.float()) * scale + bn.bias.float()).contiguous()
+            self.w2 = lin2.weight.float().contiguous()
+            self.b2 = lin2.bias.float().contiguous()
+        self.input_dim, self.hidden_dim, self.num_experts = self.w1.shape[1], self.w1.shape[0], self.w2.shape[0]
+
+    def __call__(self, x: torch.Tensor) -> torch.Tensor:
+        from . import ops
+        return ops.rs_predict(x.contiguous(), self.w1, self.b1, self.w2, self.b2)
+
+
+def fused_scout(module: Any, x: torch.Tensor) -> Optional[FusedScout]:
+    """The fused form of ``module`` for a call on ``x [T, H]``, or None where the HIP predictor does not
+    apply (another predictor class, training mode, host tensors, more tokens than a decode call, shapes
+    the kernel does not take); cached on the module."""
+    if not (isinstance(module, RoutingScoutMLP) and not module.training and x.is_cuda and x.dim() == 2):
+        return None
+    if x.shape[0] > _lib.DECODE_MAX_TOKENS or x.shape[1] % 8:
+        return None
+    fused = getattr(module, "_sparse_fused", None)
+    if fused is None or fused.w1.device != x.device:
+        lin1 = module.mlp[0]
+        if lin1.weight.device != x.device or lin1.out_features % 4 or module.mlp[4].out_features > _lib.MAX_EXPERTS:
+            return None
+        fused = FusedScout(module)
+        object.__setattr__(module, "_sparse_fused", fused)
+    return fused if fused.input_dim == x.shape[1] else None
 
 
 class _ResidualUnit(nn.Module):

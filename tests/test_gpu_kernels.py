@@ -499,6 +499,45 @@ def test_prefill_clock_probe_reads_a_plausible_clock_and_changes_nothing(device)
     assert clk.tolist() == second   # switched off: nothing is added any more
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("T", [1, 8, 32])
+def test_rs_predictor_kernel_matches_the_module(device, dtype, T):
+    """The two-launch HIP forward pass of the routing-scout MLP (BatchNorm folded into the first Linear)
+    against the PyTorch module in eval mode on ``x.float()``, with running statistics and affine
+    parameters that are not the identity; probabilities within fp32 summation-order noise, and the
+    planner's top-8 equal wherever the ninth probability is not within that noise of the eighth."""
+    from sparse_amd.rs import RoutingScoutMLP, fused_scout, stable_topk
+    ops = _ops()
+    H, E, D = 2048, 60, 512
+    torch.manual_seed(5)
+    mod = RoutingScoutMLP(H, E, hidden_dim=D)
+    bn = mod.mlp[1]
+    with torch.no_grad():
+        bn.running_mean.copy_(torch.randn(D) * 0.3)
+        bn.running_var.copy_(torch.rand(D) * 2 + 0.25)
+        bn.weight.copy_(torch.rand(D) + 0.5)
+        bn.bias.copy_(torch.randn(D) * 0.2)
+        mod.mlp[4].weight.mul_(4.0)          # spread the output distribution
+    mod = mod.eval().to(device)
+    x = make_hidden(T, H, dtype, seed=81).to(device)
+    with torch.no_grad():
+        ref = mod(x.float())
+    fused = fused_scout(mod, x)
+    assert fused is not None and fused_scout(mod, x) is fused          # built once, cached on the module
+    pred = fused(x)
+    assert pred.dtype == torch.float32 and tuple(pred.shape) == (T, E)
+    torch.testing.assert_close(pred, ref, rtol=2e-4, atol=1e-7)
+    torch.testing.assert_close(pred.sum(-1), torch.ones(T, device=device), rtol=1e-5, atol=1e-5)
+    v_ref, i_ref = stable_topk(ref, 9)
+    _, i_dev = stable_topk(pred, 8)
+    clear = (v_ref[:, 7] - v_ref[:, 8]) > 1e-4 * v_ref[:, 7]
+    assert bool(clear.any())
+    assert torch.equal(torch.sort(i_dev[clear], 1).values, torch.sort(i_ref[clear, :8], 1).values)
+    # what the kernel does not take falls back to the module: training mode, prefill-size calls
+    assert fused_scout(mod, make_hidden(40, H, dtype, seed=82).to(device)) is None
+    assert fused_scout(mod.train(), x) is None
+
+
 @pytest.mark.parametrize("T,decode", [(8, True), (128, False)])
 def test_ffn_fp32_matches_oracle(device, T, decode):
     ops = _ops()
