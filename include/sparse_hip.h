@@ -473,8 +473,9 @@ int sparse_hip_prefill_drain_waits(int on);
  * the average shader clock of a busy compute unit, which under a power cap is well below the
  * peak clock the published MFMA rate assumes.  NULL turns it off.  Process-wide. */
 int sparse_hip_prefill_clock_probe(void* counters_dev);
-/* Name of the __global__ function behind a kernel id (as rocprofv3 prints it, without
- * template arguments). */
+/* Name of the __global__ function behind a kernel id (as rocprofv3 prints it, with the template
+ * arguments that tell the kernels of one family apart: F stands for the 16-bit format, sparse::Bf16 or
+ * sparse::Fp16; the tile-count arguments that follow are left out). */
 const char* sparse_hip_kernel_name(int kernel);
 
 #ifdef __cplusplus

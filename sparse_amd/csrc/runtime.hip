@@ -208,8 +208,8 @@ int sparse_hip_profile_read(int kernel, double* total_ms_out, int64_t* launches_
 
 const char* sparse_hip_kernel_name(int kernel) {
   static const char* names[SPARSE_HIP_K_COUNT] = {
-      "router_logits_kernel", "gate_topk_kernel",   "permute_scatter_kernel", "decode_ffn_kernel<true>",
-      "decode_ffn_kernel<false>", "prefill_ffn_kernel<true>", "prefill_ffn_kernel<false>",
+      "router_logits_kernel", "gate_topk_kernel",   "permute_scatter_kernel", "decode_ffn_kernel<F, true>",
+      "decode_ffn_kernel<F, false>", "prefill_ffn_kernel<F, true>", "prefill_ffn_kernel<F, false>",
       "ffn_tiled_kernel<gate_up>", "ffn_tiled_kernel<down>", "combine_kernel", "route_decode_kernel"};
   if (kernel < 0 || kernel >= SPARSE_HIP_K_COUNT) return "";
   return names[kernel];
