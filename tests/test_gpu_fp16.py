@@ -209,3 +209,19 @@ def test_qwen_shape_fp16_decode_and_prefill(device):
     from sparse_amd.synthetic import QWEN
     for T in (8, 160):
         _check_block(QWEN, T, device, seed=1)
+
+
+@pytest.mark.parametrize("method", ["rr", "rs-epipe"])
+def test_offloaded_fp16_stack_gives_the_resident_bits(device, method):
+    """Residency decides where the weights come from and in which order experts run, never the values:
+    an fp16 stack with 4 of 12 experts cached gives, bit for bit, what the all-resident fp16 stack gives,
+    over a prefill call and decode steps, with misses, prefetches and staged copies on the way."""
+    from tests.test_gpu_offload import _run, _stack
+    blocks, metrics = _stack(device, method, 4, 3, "cpu", dtype=F16)
+    got = _run(blocks, device, 7, 4, prefill_first=True, dtype=F16)
+    assert metrics.cache_miss_count > 0 and got[0].dtype == F16
+    resident, _ = _stack(device, method, 4, 3, "gpu", dtype=F16)
+    want = _run(resident, device, 7, 4, prefill_first=True, dtype=F16)
+    assert len(got) == len(want)
+    for i, (a, b) in enumerate(zip(got, want)):
+        assert torch.equal(a, b), f"call {i}: offloaded and resident outputs differ"

@@ -15,7 +15,8 @@ pytestmark = pytest.mark.gpu
 SHAPE = dict(family="qwen_shared", hidden=512, num_experts=12, inter=256, top_k=4, shared_inter=384, num_layers=3)
 
 
-def _stack(device, method, capacity, top_m, offload, seed0=0, shape=None, structured=False, **overrides):
+def _stack(device, method, capacity, top_m, offload, seed0=0, shape=None, structured=False, dtype=torch.bfloat16,
+           **overrides):
     """``shape``: the toy stack unless given.  ``structured``: skewed, co-activating routing
     (Zipf popularity + clusters of 4) written into the gates; the blocks then carry the
     structure the inputs must be drawn with as ``blocks[0].test_structure``."""
@@ -32,14 +33,14 @@ def _stack(device, method, capacity, top_m, offload, seed0=0, shape=None, struct
     blocks = []
     structure = None
     for layer in range(shape["num_layers"]):
-        mlp = make_mlp_block(shape, dtype=torch.bfloat16, seed=seed0 + layer, fused=shape is not SHAPE,
+        mlp = make_mlp_block(shape, dtype=dtype, seed=seed0 + layer, fused=shape is not SHAPE,
                              device=device if shape is not SHAPE else "cpu")
         if structured:
             structure = add_routing_structure(mlp, shape["num_experts"], seed=layer)
         cfg = residency_config(method, capacity, top_m, **overrides) if offload == "cpu" else None
         blocks.append(DistributedSparseMoeBlock(
             layer, mlp, None, DistEnv(0, 1, 0, device), num_layers=shape["num_layers"],
-            num_experts=shape["num_experts"], top_k=shape["top_k"], dtype=torch.bfloat16, expert_offload=offload,
+            num_experts=shape["num_experts"], top_k=shape["top_k"], dtype=dtype, expert_offload=offload,
             expert_cache=capacity, planner_mode=kw["planner_mode"] if offload == "cpu" else "none",
             prefetch_top_m=top_m, placement_mode=kw["placement_mode"], metrics=metrics, residency_config=cfg))
         del mlp
@@ -50,7 +51,8 @@ def _stack(device, method, capacity, top_m, offload, seed0=0, shape=None, struct
     return blocks, metrics
 
 
-def _run(blocks, device, steps, T, record=None, sync_prefetch=False, prefill_first=False, calls=None):
+def _run(blocks, device, steps, T, record=None, sync_prefetch=False, prefill_first=False, calls=None,
+         dtype=torch.bfloat16):
     """``calls``: explicit list of ``(phase, hidden [B,S,H] on the device)`` instead of the toy
     schedule of ``steps`` decode steps of ``T`` tokens."""
     from sparse_amd.block import _SideStreams
@@ -79,7 +81,7 @@ def _run(blocks, device, steps, T, record=None, sync_prefetch=False, prefill_fir
         for step in range(steps):
             prefill = prefill_first and step == 0
             n = 40 if prefill else T
-            x = make_hidden(n, SHAPE["hidden"], torch.bfloat16, seed=1000 + step).to(device)
+            x = make_hidden(n, SHAPE["hidden"], dtype, seed=1000 + step).to(device)
             calls.append(("prefill" if prefill else "decode", x.view(1, n, -1) if prefill else x.view(n, 1, -1)))
     for step, (phase, hid) in enumerate(calls):
         SparseContext.current_phase = phase
