@@ -2,9 +2,9 @@
 //
 // C[p, n] = sum_k A[p, k] * W[n, k] per expert segment.  A workgroup (4 waves) owns a
 // 128-row x 256-weight-row tile; wave w owns all 128 rows and 64 of the weight rows
-// (four by two 32x32x16 MFMA tiles, 128 accumulator registers).  For the gate/up
+// (eight by four 16x16x32 MFMA tiles, 128 accumulator registers).  For the gate/up
 // projection the 256 weight rows are 128 gate rows and the 128 matching up rows, and a
-// wave's two column tiles are the gate and the up tile of the same 32 neurons, so
+// wave's four 16-row groups are the gate groups and the up groups of the same 32 neurons, so
 // SiLU(gate)*up is a lane-local epilogue.
 //
 // The two operands take different roads.  Activation rows are shared by the four waves:
@@ -13,7 +13,7 @@
 // 16-byte fragment reads are bank-conflict free.
 // Weight rows are private to a wave: they go HBM/L2 -> registers directly in MFMA
 // B-operand order, which is exactly the order the tiled layout stores them in (a wave
-// load is four 256-byte runs), one slab ahead of the multiply.  LDS thus carries a third
+// load is one 1 KB run), two slabs ahead of the multiply.  LDS thus carries a third
 // of the bytes of a both-operands-through-LDS design, which is what bounds this shape.
 //
 // Which tile a workgroup owns is read from a map built by a one-workgroup kernel before
@@ -22,11 +22,16 @@
 // works through whole experts, m-tiles of one weight tile adjacent in time, which keeps a
 // weight tile in that XCD's L2 while it is reused.
 //
-// MFMA 32x32x16 bf16 operand layout (lane l, c = l & 31, g = l >> 5):
-//   A: row c, k = g*8 .. g*8+7     B: column c, k = g*8 .. g*8+7
-//   D: column c, rows 8*i + 4*g + j for register 4*i + j
-// The weights are passed as A and the activations as B, so D is the transposed output
-// tile: a lane owns one activation row and runs of four consecutive output columns.
+// MFMA 16x16x32 operand layout (lane l, r = l & 15, q = l >> 4):
+//   A: row r, eight k    B: column r, the same eight k    D: column r, rows 4*q + j for register j
+// The weights are passed as A and the activations as B, so D is the transposed output tile: a lane
+// owns one activation row and four consecutive output columns.  Which eight k a lane holds is free as
+// long as A and B agree; the tiled weight layout fixes it: half h of a 64-wide slab is the A operand
+// of one MFMA in lane order, lane (r, q) holding k = 16*q + 8*h + 0..7, i.e. the 16-byte chunk 2*q + h
+// of a 128-byte slab row, and the activation fragments are read from LDS in the same order.
+// (The 16x16x32 shape moves half the accumulator data per flop of the 32x32x16 one; with real operands
+// the part is power-capped in either, and a loop of this wavefront tile fed from LDS sustains 1.65
+// against 1.52 PFLOP/s.)
 #include <atomic>
 #include <type_traits>
 
@@ -146,7 +151,7 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_ffn_kernel(const Prefil
 
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63;
-  const int fc = lane & 31, fg = lane >> 5;
+  const int fr = lane & 15, fq = lane >> 4;
   const long long clk_c0 = clock64();
   const unsigned long long clk_t0 = wall_clock64();
 
@@ -203,9 +208,11 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_ffn_kernel(const Prefil
   // ---- activation loader: global -> LDS without passing through registers ----------
   // One wave instruction moves 64 sixteen-byte pieces to 1 KB of consecutive LDS (lane l
   // lands at byte 16*l), i.e. eight 128-byte rows of the slab; the lane chooses which
-  // piece of which row it fetches.  Row r keeps its chunk j at position j ^ f(r) with
-  // f(r) = ((r >> 1) & 7) ^ ((r & 1) << 2), which spreads the 16-byte fragment reads of
-  // 8 and of 16 consecutive rows over all banks.  Wave w owns rows 32w .. 32w+31.
+  // piece of which row it fetches.  Row r keeps its chunk j = 2q + h (the eight k values of
+  // MFMA lane group q in k half h) at position (q + 4h) ^ f(r) with
+  // f(r) = ((r >> 1) & 7) ^ ((r & 1) << 2): a fragment read (16 rows, the four q of one half)
+  // then takes the four clocks of a conflict-free one -- with the chunks in their natural order
+  // the same read measured 6.4.  Wave w owns rows 32w .. 32w+31.
   const uint16_t* dptr[4];
 #pragma unroll
   for (int it = 0; it < 4; ++it) {
@@ -213,7 +220,8 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_ffn_kernel(const Prefil
     const int p = r0 + min(row, M - 1);
     const size_t grow = (a.shared || !kGateUp) ? static_cast<size_t>(p) : static_cast<size_t>(a.perm[p] / a.topk);
     const int f = ((row >> 1) & 7) ^ ((row & 1) << 2);
-    dptr[it] = a.act + grow * Kdim + (((lane & 7) ^ f) << 3);
+    const int pos = (lane & 7) ^ f;                    // position q + 4h holds chunk 2q + h
+    dptr[it] = a.act + grow * Kdim + ((((pos & 3) << 1) | (pos >> 2)) << 3);
   }
   // Issued as inline assembly: the compiler would otherwise make every barrier wait for all
   // outstanding vector memory operations because one of them writes LDS, which is exactly
@@ -230,62 +238,62 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_ffn_kernel(const Prefil
   };
 
   // ---- weight fragments straight from the tiled layout ------------------------------
-  // lane = (kh, gsel, r16): row r16 of 16-row group gsel of the wave's 32 rows, k half kh.
-  // In a 2 KB block of 64 k, the 16 bytes of (k step s, half kh, row r16) sit at element
-  // kh*512 + (s*16 + r16)*8, so k inside step s is s*16 + kh*8 + j: the MFMA's own order.
-  const int r16 = lane & 15, gsel = (lane >> 4) & 1, kh = lane >> 5;
-  const uint16_t* bptr[2];
+  // The wavefront's 64 weight rows are four 16-row groups; in the tiled layout a group's 64-wide slab
+  // is 2 KB: the first KB is the A operand of the MFMA over its k half 0 in lane order, the second KB
+  // that of half 1.  Gate/up: groups 0, 1 are gate rows of 32 neurons, groups 2, 3 the up rows of the
+  // same neurons.
+  const uint16_t* wptr[4];
 #pragma unroll
-  for (int ni = 0; ni < 2; ++ni) {
-    const uint16_t* base = (kGateUp && ni == 1) ? w1 : w0;
-    int n = kGateUp ? (n0 + wave * 32) : (n0 + wave * 64 + ni * 32);
-    n = min(n + gsel * 16, Ndim - 16);
-    bptr[ni] = base + static_cast<size_t>(n >> 4) * 16 * Kdim + kh * 512 + r16 * 8;
+  for (int g = 0; g < 4; ++g) {
+    const uint16_t* base = (kGateUp && g >= 2) ? w1 : w0;
+    int n = kGateUp ? (n0 + wave * 32 + (g & 1) * 16) : (n0 + wave * 64 + g * 16);
+    n = min(n, Ndim - 16);
+    wptr[g] = base + static_cast<size_t>(n >> 4) * 16 * Kdim + lane * 8;
   }
 
   // The tile's rows are processed in sub-tiles of 32 (one MFMA row block); a segment's last
   // tile is specialised on how many of them hold rows, so that a ragged tail costs the MFMAs,
   // LDS reads and stores of its own sub-tiles only.
   auto body = [&](auto nmi_c) {
-    constexpr int NMI = decltype(nmi_c)::value;
-    f32x16 acc[NMI][2];
+    constexpr int NMI = decltype(nmi_c)::value;   // 32-row sub-tiles that hold rows
+    constexpr int NMT = 2 * NMI;                  // 16-row MFMA column tiles
+    f32x4 acc[NMT][4];
   #pragma unroll
-    for (int mi = 0; mi < NMI; ++mi)
+    for (int mt = 0; mt < NMT; ++mt)
   #pragma unroll
-      for (int ni = 0; ni < 2; ++ni)
-  #pragma unroll
-        for (int v = 0; v < 16; ++v) acc[mi][ni][v] = 0.f;
+      for (int g = 0; g < 4; ++g) acc[mt][g] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     // Pipeline: while slab kt is multiplied, the activation rows of slab kt+2 travel to the
-    // third LDS buffer and the weight fragments of slab kt+2 to the registers step s has just
+    // third LDS buffer and the weight fragments of slab kt+2 to the registers half h has just
     // finished with (two fragment sets, used alternately), so every operand is requested two
     // slabs of MFMA work before its use -- enough bytes in flight to cover an HBM miss.
     // Vector memory operations retire in order, so "the copies of slab kt+1 have landed" is a
-    // count of the younger operations: the 8 fragment loads of slab kt-1's steps, the 4 copies
-    // of slab kt+2 and the 8 fragment loads of slab kt's steps -- vmcnt(20) -- and the
+    // count of the younger operations: the 8 fragment loads of slab kt-1's halves, the 4 copies
+    // of slab kt+2 and the 8 fragment loads of slab kt's halves -- vmcnt(20) -- and the
     // scheduling fences keep exactly that order.  Slabs past the end refetch the last one
     // instead of branching.
     // s_waitcnt vmcnt(n), other counters untouched
     constexpr int kWaitVm0 = 0x0F70, kWaitVm20 = kDrainWaits ? kWaitVm0 : 0x4F74;
     const int nk = Kdim / kPfBK;
-    bf16x8 bfrag[2][2][4];
+    bf16x8 wfrag[2][2][4];   // [stage][k half][16-row group]
     stage_slab(0, 0);
     stage_slab(min(1, nk - 1), 1);
     __builtin_amdgcn_sched_barrier(0);
   #pragma unroll
     for (int st = 0; st < 2; ++st)
   #pragma unroll
-      for (int ni = 0; ni < 2; ++ni)
+      for (int h = 0; h < 2; ++h)
   #pragma unroll
-        for (int s = 0; s < 4; ++s)
-          bfrag[st][ni][s] =
-              *reinterpret_cast<const bf16x8*>(bptr[ni] + static_cast<size_t>(min(st, nk - 1)) * 1024 + s * 128);
+        for (int g = 0; g < 4; ++g)
+          wfrag[st][h][g] =
+              *reinterpret_cast<const bf16x8*>(wptr[g] + static_cast<size_t>(min(st, nk - 1)) * 1024 + h * 512);
     __builtin_amdgcn_sched_barrier(0);
     __builtin_amdgcn_s_waitcnt(kWaitVm20);
     __syncthreads();
 
-    const int fsw = ((fc >> 1) & 7) ^ ((fc & 1) << 2);
-    const int a_row = fc * kPfRowBytes, a_x = (fg ^ fsw) << 4;
+    // activation fragment of lane (r, q), tile mt, half h: row 16*mt + r, position (q + 4h) ^ f(r)
+    const int fsw = ((fr >> 1) & 7) ^ ((fr & 1) << 2);
+    const int a_row = fr * kPfRowBytes, a_x = (fq ^ fsw) << 4;
     int cur = 0, nxt2 = 2;  // buffer of slab kt, buffer of slab kt+2
     auto slab = [&](auto stage_c, int kt) {
       constexpr int st = decltype(stage_c)::value;
@@ -294,20 +302,23 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_ffn_kernel(const Prefil
       __builtin_amdgcn_sched_barrier(kPfSchedMask);
       const uint8_t* la = lds[cur] + a_row;
   #pragma unroll
-      for (int s = 0; s < 4; ++s) {
-        bf16x8 fa[NMI];
+      for (int h = 0; h < 2; ++h) {
   #pragma unroll
-        for (int mi = 0; mi < NMI; ++mi)
-          fa[mi] = *reinterpret_cast<const bf16x8*>(la + mi * 32 * kPfRowBytes + (a_x ^ (s << 5)));
+        for (int mb = 0; mb < NMT; mb += 4) {   // four activation fragments at a time
+          bf16x8 fa[4];
   #pragma unroll
-        for (int mi = 0; mi < NMI; ++mi)
+          for (int i = 0; i < 4; ++i)
+            fa[i] = *reinterpret_cast<const bf16x8*>(la + (mb + i) * 16 * kPfRowBytes + (a_x ^ (h << 6)));
   #pragma unroll
-          for (int ni = 0; ni < 2; ++ni)
-            acc[mi][ni] = F::mfma32(bfrag[st][ni][s], fa[mi], acc[mi][ni]);
+          for (int i = 0; i < 4; ++i)
+  #pragma unroll
+            for (int g = 0; g < 4; ++g)
+              acc[mb + i][g] = F::mfma16(wfrag[st][h][g], fa[i], acc[mb + i][g]);
+        }
         __builtin_amdgcn_sched_barrier(kPfSchedMask);
   #pragma unroll
-        for (int ni = 0; ni < 2; ++ni)
-          bfrag[st][ni][s] = *reinterpret_cast<const bf16x8*>(bptr[ni] + static_cast<size_t>(kt2) * 1024 + s * 128);
+        for (int g = 0; g < 4; ++g)
+          wfrag[st][h][g] = *reinterpret_cast<const bf16x8*>(wptr[g] + static_cast<size_t>(kt2) * 1024 + h * 512);
         __builtin_amdgcn_sched_barrier(kPfSchedMask);
       }
       __builtin_amdgcn_s_waitcnt(kWaitVm20);
@@ -329,40 +340,38 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_ffn_kernel(const Prefil
     __syncthreads();
 
     // ---- epilogue ----------------------------------------------------------------
-    // The product was formed as W * X^T, so a lane holds one row m (= 32*mi + fc) and, per
-    // accumulator quad i, four consecutive output columns 8*i + 4*fg + j: eight bytes of
-    // bf16 that go to the wave's private staging area in LDS (free now: every wave is past
-    // the last barrier of the k loop) as one write.  The area holds a 128-row x 32-column
-    // tile, rows of 64 bytes with the 16-byte chunks swizzled by row; it is read back a row
-    // quarter per lane and stored with 16-byte writes, 64 contiguous bytes per row.
+    // The product was formed as W * X^T, so a lane holds one row m (= 16*mt + fr) and, per 16-row
+    // weight group, four consecutive output columns 4*fq + j: eight bytes of 16-bit values that go
+    // to the wave's private staging area in LDS (free now: every wave is past the last barrier of
+    // the k loop) as one write.  The area holds a 128-row x 32-column tile, rows of 64 bytes with
+    // the 16-byte chunks swizzled by row; it is read back a row quarter per lane and stored with
+    // 16-byte writes, 64 contiguous bytes per row.
     uint8_t* st = &lds[0][0] + wave * (kPfBM * 64);
-    float sc[NMI];
-  #pragma unroll
-    for (int mi = 0; mi < NMI; ++mi) sc[mi] = kGateUp ? 1.f : s_scale[mi * 32 + fc];
   #pragma unroll
     for (int pass = 0; pass < (kGateUp ? 1 : 2); ++pass) {
       if (pass) __syncthreads();  // staging rows are reused
   #pragma unroll
-      for (int mi = 0; mi < NMI; ++mi) {
-        const int m = mi * 32 + fc;
+      for (int mt = 0; mt < NMT; ++mt) {
+        const int m = mt * 16 + fr;
+        const float sc = kGateUp ? 1.f : s_scale[m];
   #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int p = 0; p < 2; ++p) {   // the pass's two 16-column groups
           float v[4];
   #pragma unroll
           for (int j = 0; j < 4; ++j) {
             if (kGateUp) {
-              const float g = F::round(acc[mi][0][4 * i + j]);
-              const float u = F::round(acc[mi][1][4 * i + j]);
+              const float g = F::round(acc[mt][p][j]);
+              const float u = F::round(acc[mt][2 + p][j]);
               v[j] = F::round(silu_f32(g)) * u;
             } else {
-              v[j] = F::round(acc[mi][pass][4 * i + j]) * sc[mi];
+              v[j] = F::round(acc[mt][2 * pass + p][j]) * sc;
             }
           }
           uint2 pk;
           pk.x = F::pack2(v[0], v[1]);
           pk.y = F::pack2(v[2], v[3]);
-          const int chunk = i ^ ((m >> 1) & 3);
-          *reinterpret_cast<uint2*>(st + m * 64 + chunk * 16 + fg * 8) = pk;
+          const int chunk = (2 * p + (fq >> 1)) ^ ((m >> 1) & 3);
+          *reinterpret_cast<uint2*>(st + m * 64 + chunk * 16 + (fq & 1) * 8) = pk;
         }
       }
       __syncthreads();
