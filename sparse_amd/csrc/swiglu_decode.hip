@@ -190,13 +190,11 @@ __global__ __launch_bounds__(kDecThreads) void decode_ffn_kernel(const DecodeArg
   for (int nt = 0; nt < NT; ++nt)
     if (brow[nt] == nullptr) brow[nt] = bsafe;
 
+// (weights first: their addresses need the segment's slot only, the token rows' addresses wait for the
+// permutation entry as well, and the first weight loads should be in flight while that arrives)
 #define SP_DEC_LOAD(B, W, d)                                                             \
   do {                                                                                   \
     const int koff_ = (d) << 6;                                                          \
-    _Pragma("unroll") for (int nt = 0; nt < NT; ++nt) {                                  \
-      B[nt][0] = ld_bf16x8(brow[nt] + koff_ + (q << 4));                                 \
-      B[nt][1] = ld_bf16x8(brow[nt] + koff_ + (q << 4) + 8);                             \
-    }                                                                                    \
     _Pragma("unroll") for (int tl = 0; tl < kDecTiles; ++tl) {                           \
       const size_t o_ = tl * group_stride + (static_cast<size_t>(d) << 10);              \
       W[0][tl][0] = ld_stream_bf16x8(wt0 + o_);                                                 \
@@ -205,6 +203,10 @@ __global__ __launch_bounds__(kDecThreads) void decode_ffn_kernel(const DecodeArg
         W[NM - 1][tl][0] = ld_stream_bf16x8(wt1 + o_);                                          \
         W[NM - 1][tl][1] = ld_stream_bf16x8(wt1 + o_ + 512);                                    \
       }                                                                                  \
+    }                                                                                    \
+    _Pragma("unroll") for (int nt = 0; nt < NT; ++nt) {                                  \
+      B[nt][0] = ld_bf16x8(brow[nt] + koff_ + (q << 4));                                 \
+      B[nt][1] = ld_bf16x8(brow[nt] + koff_ + (q << 4) + 8);                             \
     }                                                                                    \
   } while (0)
 
