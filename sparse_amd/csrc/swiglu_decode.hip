@@ -348,6 +348,16 @@ __global__ __launch_bounds__(kDecThreads) void decode_ffn_kernel(const DecodeArg
     // expert) has written its rows through to memory; once its own writes are acknowledged it
     // counts itself in.  The last one finds everybody's rows in memory.
     __shared__ int s_last;
+    // thread -> (token, four columns); the arithmetic is that of the stand-alone combine step:
+    // K ordered adds rounded to bf16, then the shared expert finished from its parts.  Where the
+    // token's rows lie is read before the hand-off, so that the last workgroup's reads of them
+    // do not wait for it.
+    const int Ttok = a.T, K = a.topk, H = a.Ndim_s;
+    constexpr int kPerTok = kDecRows / 4;   // threads per token: four columns each
+    const int t = threadIdx.x / kPerTok, c4 = (threadIdx.x % kPerTok) * 4;
+    int32_t pos[SPARSE_HIP_MAX_TOPK];
+#pragma unroll
+    for (int k = 0; k < SPARSE_HIP_MAX_TOPK; ++k) pos[k] = (k < K && t < Ttok) ? a.inv_perm[t * K + k] : 0x7fffffff;
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wavefront's stores have been acknowledged
     __syncthreads();
     const int tile = row0 / kDecRows;
@@ -359,15 +369,7 @@ __global__ __launch_bounds__(kDecThreads) void decode_ffn_kernel(const DecodeArg
     }
     __syncthreads();
     if (!s_last) return;
-    // thread -> (token, four columns); the arithmetic is that of the stand-alone combine step:
-    // K ordered adds rounded to bf16, then the shared expert finished from its parts
-    const int Ttok = a.T, K = a.topk, H = a.Ndim_s;
-    constexpr int kPerTok = kDecRows / 4;   // threads per token: four columns each
-    const int t = threadIdx.x / kPerTok, c4 = (threadIdx.x % kPerTok) * 4;
     if (t >= Ttok) return;
-    int32_t pos[SPARSE_HIP_MAX_TOPK];
-#pragma unroll
-    for (int k = 0; k < SPARSE_HIP_MAX_TOPK; ++k) pos[k] = (k < K) ? a.inv_perm[t * K + k] : 0x7fffffff;
 #pragma unroll
     for (int i = 1; i < SPARSE_HIP_MAX_TOPK; ++i) {
 #pragma unroll
