@@ -515,6 +515,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-offload", action="store_true", help="skip the two offloaded workloads (the long legs)")
     ap.add_argument("--only-prefill", action="store_true", help="run just the prefill workload (for profiling)")
+    ap.add_argument("--only-decode", type=int, default=0, metavar="BATCH",
+                    help="run just the all-resident decode workload at this batch size (for profiling)")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also launch a 256 MiB plain copy kernel a few times (yardstick for --pmc byte counters)")
     ap.add_argument("--cached-decode", type=int, default=0, metavar="STEPS",
@@ -536,6 +538,11 @@ def main():
 
     if args.only_prefill:
         print(json.dumps(prefill_workload(DEEPSEEK, 4096, max(2, args.steps), args.warmup, dtype, device)))
+        return
+    if args.only_decode:
+        blocks = build_stack(QWEN, dtype, device)
+        print(json.dumps(decode_workload(blocks, QWEN, args.only_decode, args.steps, args.warmup, dtype, device,
+                                         not args.no_graph)))
         return
     if args.cached_decode:
         print(json.dumps({"cached_decode_qwen": cached_decode_workload(dtype, device, args.cached_decode)}))
