@@ -186,6 +186,12 @@ def prefill_workload(shape, tokens, steps, warmup, dtype, device):
     finally:
         ops.prefill_clock_probe(None)
     clock_mhz = ops.prefill_shader_clock_mhz(clk)
+    # what the matrix cores sustain on this box with nothing but the kernel's wavefront tile going on:
+    # operands in registers, and with the activation fragments read from LDS every k step
+    probe = {}
+    for name, from_lds in (("registers", False), ("lds_fragments", True)):
+        tf, mhz = ops.mfma_probe(from_lds, device=device)
+        probe[name] = {"tflops": tf, "clock_mhz": mhz, "frac_of_peak": tf / MFMA_BF16_PEAK_TFLOPS}
     H, I, Is, K, E = shape["hidden"], shape["inter"], shape["shared_inter"], shape["top_k"], shape["num_experts"]
     flops_layer = 2.0 * tokens * K * 3 * H * I + 2.0 * tokens * 3 * H * Is + 2.0 * tokens * H * E
     gu_ms, gu_n, gu_name = stats["prefill_gateup"]
@@ -205,6 +211,8 @@ def prefill_workload(shape, tokens, steps, warmup, dtype, device):
         ffn_shader_clock_mhz=clock_mhz,
         mfma_frac_at_clock=(flops_layer * len(blocks) / (ms_per_step / 1e3) / 1e12
                             / (MFMA_BF16_PEAK_TFLOPS * clock_mhz / MFMA_PEAK_CLOCK_MHZ)) if clock_mhz else None,
+        # a loop of the same MFMAs on the same wavefront tile and nothing else (sparse_hip_mfma_probe)
+        mfma_probe=probe,
         gateup=dict(kernel=gu_name, launches=gu_n, est_routed_avg_us=gu_routed_s * 1e6,
                     tflops=gu_flops / gu_routed_s / 1e12 if gu_routed_s else 0.0),
         kernels_us={k: (v[0] / max(1, v[1]) * 1e3) for k, v in stats.items() if v[1]},

@@ -473,6 +473,17 @@ int sparse_hip_prefill_drain_waits(int on);
  * the average shader clock of a busy compute unit, which under a power cap is well below the
  * peak clock the published MFMA rate assumes.  NULL turns it off.  Process-wide. */
 int sparse_hip_prefill_clock_probe(void* counters_dev);
+/* Measurement aid with no counterpart in the reference: what the matrix cores sustain on this part
+ * for the prefill kernel's wavefront tile with nothing else going on.  Launches, twice (the first
+ * untimed), one workgroup of eight wavefronts per compute unit, every wavefront multiplying a
+ * 128 x 64 tile as eight by four bf16 16x16x32 MFMA tiles, `iters` (even) k steps of 32 on
+ * pseudo-random operands held in registers (from_lds == 0) or with the eight activation fragments
+ * of every k step read from LDS, as the prefill kernel's inner loop reads them (from_lds != 0).
+ * `counters_dev`: 32 bytes of device memory, 8-byte aligned, which the call clears and uses.
+ * Returns the rate of the timed launch (HIP events on `stream`) in TFLOP/s and the average shader
+ * clock of the busy compute units in MHz.  Waits for the launch; not for use under graph capture. */
+int sparse_hip_mfma_probe(int from_lds, int iters, void* counters_dev, double* tflops_out, double* clock_mhz_out,
+                          void* stream);
 /* Name of the __global__ function behind a kernel id (as rocprofv3 prints it, with the template
  * arguments that tell the kernels of one family apart: F stands for the 16-bit format, sparse::Bf16 or
  * sparse::Fp16; the tile-count arguments that follow are left out). */

@@ -111,6 +111,7 @@ SIGNATURES = {
     "sparse_hip_rs_predict": (_i, [_vp, _i, _i, _i, _vp, _vp, _i, _vp, _vp, _i, _vp, _vp, _vp]),
     "sparse_hip_prefill_drain_waits": (_i, [_i]),
     "sparse_hip_prefill_clock_probe": (_i, [_vp]),
+    "sparse_hip_mfma_probe": (_i, [_i, _i, _vp, C.POINTER(C.c_double), C.POINTER(C.c_double), _vp]),
     "sparse_hip_profile_enable": (_i, [_i]),
     "sparse_hip_profile_reset": (_i, []),
     "sparse_hip_profile_read": (_i, [_i, C.POINTER(C.c_double), C.POINTER(C.c_int64)]),

@@ -31,6 +31,7 @@ SOURCES = [
     "combine.hip",
     "rs_predict.hip",
     "layout.hip",
+    "mfma_probe.hip",
 ]
 
 # Packed-fp32 VALU ops are switched off for the device pass; the host pass does not know

@@ -1,0 +1,130 @@
+// Measurement aid: the rate and the clock the matrix cores sustain on this part, for the wavefront tile of
+// the prefill expert kernel.  The published bf16 MFMA peak assumes the peak shader clock; under load the
+// part settles well below it, and how far depends on what else the loop does.  This probe runs nothing but
+// that loop: eight wavefronts per compute unit (two per SIMD, as the prefill kernel runs), every wavefront
+// multiplying a 128 x 64 tile (eight by four 16x16x32 tiles, 128 accumulator registers) over and over on
+// pseudo-random operands, with the activation fragments either held in registers or read from LDS on every
+// k step as the prefill kernel reads them.  No global memory traffic inside the loop.
+#include "common.h"
+
+namespace sparse {
+
+constexpr int kProbeThreads = 512;
+constexpr int kProbeLds = 64 * 1024;
+
+__device__ __forceinline__ uint32_t probe_hash(uint32_t v) {
+  v *= 2654435761u;
+  v ^= v >> 15;
+  v *= 2246822519u;
+  v ^= v >> 13;
+  return v;
+}
+
+// bf16 in (-2, 2) from a hash value
+__device__ __forceinline__ __bf16 probe_value(uint32_t h) {
+  return static_cast<__bf16>((static_cast<int>(h & 0xffff) - 32768) * (1.0f / 16384.0f));
+}
+
+template <bool kFromLds>
+__global__ __launch_bounds__(kProbeThreads, 1) void mfma_probe_kernel(int iters, unsigned long long* counters,
+                                                                     float* sink) {
+  __shared__ __attribute__((aligned(1024))) uint8_t lds[kProbeLds];
+  for (int i = threadIdx.x; i < kProbeLds / 2; i += kProbeThreads)
+    reinterpret_cast<__bf16*>(lds)[i] = probe_value(probe_hash(i + 977u * blockIdx.x));
+  __syncthreads();
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  bf16x8 w[2][4];   // weight fragments of two k steps, four 16-row groups
+#pragma unroll
+  for (int s = 0; s < 2; ++s)
+#pragma unroll
+    for (int g = 0; g < 4; ++g)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) w[s][g][j] = probe_value(probe_hash(threadIdx.x * 131u + (4 * s + g) * 17u + j)) * static_cast<__bf16>(0.01f);
+  // a fragment is 1 KB of consecutive LDS (lane l reads bytes 16 l .. 16 l + 15): conflict-free; the 64
+  // fragments of the buffer are taken in an order that differs from wavefront to wavefront
+  const uint8_t* la = lds + lane * 16;
+  const int rot = wave * 5;
+  bf16x8 fa[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) fa[i] = *reinterpret_cast<const bf16x8*>(la + ((i + rot) & 31) * 1024);
+  f32x4 acc[8][4];
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) acc[i][g] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  const long long c0 = clock64();
+  const unsigned long long t0 = wall_clock64();
+  for (int it = 0; it < iters; it += 2) {
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const bf16x8 cur = fa[i];
+        if (kFromLds)
+          fa[i] = *reinterpret_cast<const bf16x8*>(la + ((i + ((it + s) & 3) * 8 + rot) & 31) * 1024 + 32768 * ((it >> 2) & 1));
+#pragma unroll
+        for (int g = 0; g < 4; ++g) acc[i][g] = Bf16::mfma16(w[s][g], cur, acc[i][g]);
+      }
+    }
+  }
+  const long long c1 = clock64();
+  const unsigned long long t1 = wall_clock64();
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) s += acc[i][g][0] + acc[i][g][1] + acc[i][g][2] + acc[i][g][3];
+  if (s == 123.456f) sink[0] = s;   // keeps the loop alive
+  if (threadIdx.x == 0) {
+    atomicAdd(&counters[0], static_cast<unsigned long long>(c1 - c0));
+    atomicAdd(&counters[1], t1 - t0);
+  }
+}
+
+}  // namespace sparse
+
+using namespace sparse;
+
+extern "C" int sparse_hip_mfma_probe(int from_lds, int iters, void* counters_dev, double* tflops_out,
+                                     double* clock_mhz_out, void* stream) {
+  SP_REQUIRE(iters >= 2 && iters <= (1 << 22) && iters % 2 == 0, "mfma_probe: iters=%d must be even and in [2, 2^22]",
+             iters);
+  SP_REQUIRE(counters_dev && tflops_out && clock_mhz_out, "mfma_probe: NULL pointer");
+  SP_REQUIRE((reinterpret_cast<uintptr_t>(counters_dev) & 7) == 0, "mfma_probe: counters must be 8-byte aligned");
+  hipStream_t st = as_stream(stream);
+  int dev = 0, cus = 0;
+  SP_HIP(hipGetDevice(&dev));
+  SP_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+  SP_REQUIRE(cus > 0, "mfma_probe: device reports %d compute units", cus);
+  unsigned long long* counters = static_cast<unsigned long long*>(counters_dev);
+  float* sink = reinterpret_cast<float*>(counters + 2);
+  hipEvent_t e0 = nullptr, e1 = nullptr;
+  SP_HIP(hipEventCreate(&e0));
+  SP_HIP(hipEventCreate(&e1));
+  float ms = 0.f;
+  unsigned long long host[2] = {0, 0};
+  hipError_t err = hipSuccess;
+  // one untimed launch first: the clock settles within the first milliseconds of a load
+  for (int rep = 0; rep < 2 && err == hipSuccess; ++rep) {
+    err = hipMemsetAsync(counters, 0, 3 * sizeof(unsigned long long), st);
+    if (err == hipSuccess) err = hipEventRecord(e0, st);
+    if (err != hipSuccess) break;
+    if (from_lds)
+      hipLaunchKernelGGL((mfma_probe_kernel<true>), dim3(cus), dim3(kProbeThreads), 0, st, iters, counters, sink);
+    else
+      hipLaunchKernelGGL((mfma_probe_kernel<false>), dim3(cus), dim3(kProbeThreads), 0, st, iters, counters, sink);
+    err = hipGetLastError();
+    if (err == hipSuccess) err = hipEventRecord(e1, st);
+    if (err == hipSuccess) err = hipEventSynchronize(e1);
+    if (err == hipSuccess) err = hipEventElapsedTime(&ms, e0, e1);
+    if (err == hipSuccess) err = hipMemcpy(host, counters, sizeof(host), hipMemcpyDeviceToHost);
+  }
+  hipEventDestroy(e0);
+  hipEventDestroy(e1);
+  if (err != hipSuccess) return hip_fail(err, "mfma_probe");
+  const double flops = static_cast<double>(cus) * (kProbeThreads / 64) * iters * (2.0 * 128 * 64 * 32);
+  *tflops_out = ms > 0.f ? flops / (ms * 1e-3) / 1e12 : 0.0;
+  *clock_mhz_out = host[1] ? 100.0 * static_cast<double>(host[0]) / static_cast<double>(host[1]) : 0.0;
+  return SPARSE_HIP_OK;
+}

@@ -523,6 +523,18 @@ def prefill_shader_clock_mhz(counters: torch.Tensor) -> float:
     return 100.0 * cyc / ticks if ticks else 0.0
 
 
+def mfma_probe(from_lds: bool, iters: int = 20000, device="cuda:0") -> Tuple[float, float]:
+    """``(TFLOP/s, shader clock in MHz)`` of a loop of bf16 16x16x32 MFMAs on the prefill kernel's wavefront
+    tile, eight wavefronts per compute unit, operands in registers or (``from_lds``) with the activation
+    fragments read from LDS every k step.  A measurement aid; the reference has no such thing."""
+    counters = torch.zeros(4, dtype=torch.int64, device=device)
+    tflops, mhz = C.c_double(0.0), C.c_double(0.0)
+    with torch.cuda.device(counters.device):
+        _lib.check(_lib.load().sparse_hip_mfma_probe(int(bool(from_lds)), int(iters), _ptr(counters), C.byref(tflops),
+                                                     C.byref(mhz), _stream()), "sparse_hip_mfma_probe")
+    return float(tflops.value), float(mhz.value)
+
+
 def moe_ffn_decode(experts: Experts, x: torch.Tensor, topv: torch.Tensor, perm: Permutation, segs: SegList,
                    inter_ws: torch.Tensor, parts: torch.Tensor, shared_w, shared_gate: Optional[torch.Tensor],
                    shared_inter_ws: torch.Tensor, shared_out: torch.Tensor,

@@ -499,6 +499,21 @@ def test_prefill_clock_probe_reads_a_plausible_clock_and_changes_nothing(device)
     assert clk.tolist() == second   # switched off: nothing is added any more
 
 
+def test_mfma_probe_reports_a_rate_below_peak_and_a_plausible_clock(device):
+    """The probe's loop is nothing but MFMAs (and, in its second form, LDS fragment reads): its rate can
+    not exceed what 256 compute units deliver at the clock it measured (4096 flop per clock per unit), it
+    is a sizeable fraction of it, and bad arguments are rejected."""
+    ops = _ops()
+    cus = torch.cuda.get_device_properties(device).multi_processor_count
+    for from_lds in (False, True):
+        tflops, mhz = ops.mfma_probe(from_lds, iters=4000, device=device)
+        assert 100.0 < mhz < 3000.0
+        at_clock = cus * 4096 * mhz * 1e6 / 1e12
+        assert 0.5 * at_clock < tflops <= 1.02 * at_clock, (from_lds, tflops, mhz)
+    with pytest.raises(Exception):
+        ops.mfma_probe(False, iters=3, device=device)
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("T", [1, 8, 32])
 def test_rs_predictor_kernel_matches_the_module(device, dtype, T):
