@@ -418,6 +418,24 @@ def test_prefill_ffn_bf16_matches_oracle(device, T):
     assert (out.float() - ref.float()).abs().max() / ref.float().abs().max() < 2e-2
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("H,E,I,K,T", [(320, 6, 192, 2, 200), (576, 5, 448, 3, 333), (192, 4, 64, 2, 150),
+                                       (64, 3, 64, 1, 129)])
+def test_prefill_ffn_odd_shapes_match_oracle(device, dtype, H, E, I, K, T):
+    """Reduction lengths that are an odd number of 64-wide slabs (the k loop runs its slabs in pairs plus a
+    tail), output widths that end inside a workgroup's column tile or inside a wavefront's 16-row group
+    range, and segments that end inside a 32-row sub-tile."""
+    ops = _ops()
+    layer = make_layer(H, E, I, K, dtype=dtype, seed=41 + H, std=0.05)
+    x = make_hidden(T, H, dtype, seed=42 + T)
+    topv, topi = _routing(layer, x)
+    out, _, _ = _run_routed(ops, layer, x, topv, topi, device, decode=False)
+    ref = ref_moe.experts_world1_exact(x, topi, topv, layer["experts"])
+    tol = BF16_TOL if dtype == torch.bfloat16 else dict(rtol=5e-3, atol=2e-3)
+    torch.testing.assert_close(out.float(), ref.float(), **tol)
+    assert not torch.isnan(out.float()).any()
+
+
 def test_prefill_and_decode_kernels_agree(device):
     ops = _ops()
     layer = make_layer(512, 12, 256, 4, dtype=torch.bfloat16, seed=31, std=0.05)
