@@ -120,8 +120,8 @@ extern "C" int sparse_hip_mfma_probe(int from_lds, int iters, void* counters_dev
     if (err == hipSuccess) err = hipEventElapsedTime(&ms, e0, e1);
     if (err == hipSuccess) err = hipMemcpy(host, counters, sizeof(host), hipMemcpyDeviceToHost);
   }
-  hipEventDestroy(e0);
-  hipEventDestroy(e1);
+  (void)hipEventDestroy(e0);
+  (void)hipEventDestroy(e1);
   if (err != hipSuccess) return hip_fail(err, "mfma_probe");
   const double flops = static_cast<double>(cus) * (kProbeThreads / 64) * iters * (2.0 * 128 * 64 * 32);
   *tflops_out = ms > 0.f ? flops / (ms * 1e-3) / 1e12 : 0.0;

@@ -47,10 +47,6 @@ constexpr int kPfRowBytes = kPfBK * 2;  // LDS row of one k slab (16-byte chunks
 constexpr int kPfLdsA = kPfBM * kPfRowBytes;
 constexpr int kPfStages = 3;            // activation slabs resident in LDS
 constexpr int kPfXcds = 8;
-// Scheduling fence that vector/scalar ALU and LDS instructions may cross but global loads and MFMAs may
-// not: it keeps every prefetch where the loop puts it (the compiler otherwise sinks the
-// loads to the end of the slab, right in front of their first use).
-constexpr int kPfSchedMask = 0x2 | 0x4 | 0x80 | 0x100 | 0x200;
 
 struct PfTile {
   int32_t slot;  // weight slot of the segment's expert
@@ -270,7 +266,7 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_ffn_kernel(const Prefil
     // Vector memory operations retire in order, so "the copies of slab kt+1 have landed" is a
     // count of the younger operations: the 8 fragment loads of slab kt-1's halves, the 4 copies
     // of slab kt+2 and the 8 fragment loads of slab kt's halves -- vmcnt(20) -- and the
-    // scheduling fences keep exactly that order.  Slabs past the end refetch the last one
+    // scheduling fences keep exactly that order (copies, half 0, half 1 in every slab).  Slabs past the end refetch the last one
     // instead of branching.
     // s_waitcnt vmcnt(n), other counters untouched
     constexpr int kWaitVm0 = 0x0F70, kWaitVm20 = kDrainWaits ? kWaitVm0 : 0x4F74;
@@ -298,28 +294,53 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_ffn_kernel(const Prefil
     auto slab = [&](auto stage_c, int kt) {
       constexpr int st = decltype(stage_c)::value;
       const int kt2 = min(kt + 2, nk - 1);
-      stage_slab(kt2, nxt2);
-      __builtin_amdgcn_sched_barrier(kPfSchedMask);
       const uint8_t* la = lds[cur] + a_row;
+      // Activation fragments come from LDS two at a time (two 16-row tiles: eight MFMAs), and the next pair
+      // is requested before the current pair multiplies: a wavefront on its own then waits for an LDS read
+      // once per slab instead of once per pair.  The full fences keep that order (the compiler otherwise
+      // sinks every read to just in front of its first use).
+      constexpr int NP = NMT / 2, NB = 2 * NP;   // pairs per k half, pairs per slab
+      bf16x8 fa[2][2];
+      if (NP == 1) {   // one pair per half: the copies go first, so that every tile height issues its
+        stage_slab(kt2, nxt2);   // vector memory operations in the order the counted wait below assumes
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      auto rd = [&](int idx, bf16x8 (&f)[2]) __attribute__((always_inline)) {
+        const int h = idx / NP, mb = 2 * (idx % NP);
   #pragma unroll
-      for (int h = 0; h < 2; ++h) {
+        for (int i = 0; i < 2; ++i)
+          f[i] = *reinterpret_cast<const bf16x8*>(la + (mb + i) * 16 * kPfRowBytes + (a_x ^ (h << 6)));
+      };
+      rd(0, fa[0]);
   #pragma unroll
-        for (int mb = 0; mb < NMT; mb += 4) {   // four activation fragments at a time
-          bf16x8 fa[4];
+      for (int idx = 0; idx < NB; ++idx) {
+        const int h = idx / NP, mb = 2 * (idx % NP);
+        if (idx + 1 < NB) rd(idx + 1, fa[(idx + 1) & 1]);
+        __builtin_amdgcn_sched_barrier(0);    // the next pair's reads stay ahead of this pair's MFMAs
+        if (idx % NP != NP - 1) {
   #pragma unroll
-          for (int i = 0; i < 4; ++i)
-            fa[i] = *reinterpret_cast<const bf16x8*>(la + (mb + i) * 16 * kPfRowBytes + (a_x ^ (h << 6)));
-  #pragma unroll
-          for (int i = 0; i < 4; ++i)
+          for (int i = 0; i < 2; ++i)
   #pragma unroll
             for (int g = 0; g < 4; ++g)
-              acc[mb + i][g] = F::mfma16(wfrag[st][h][g], fa[i], acc[mb + i][g]);
-        }
-        __builtin_amdgcn_sched_barrier(kPfSchedMask);
+              acc[mb + i][g] = F::mfma16(wfrag[st][h][g], fa[idx & 1][i], acc[mb + i][g]);
+          __builtin_amdgcn_sched_barrier(0);
+        } else {
+          // last pair of the half: group by group, each group's fragment of slab kt+2 requested right behind
+          // its last MFMA, so that the four loads are spread over the pair instead of queueing behind it
   #pragma unroll
-        for (int g = 0; g < 4; ++g)
-          wfrag[st][h][g] = *reinterpret_cast<const bf16x8*>(wptr[g] + static_cast<size_t>(kt2) * 1024 + h * 512);
-        __builtin_amdgcn_sched_barrier(kPfSchedMask);
+          for (int g = 0; g < 4; ++g) {
+  #pragma unroll
+            for (int i = 0; i < 2; ++i)
+              acc[mb + i][g] = F::mfma16(wfrag[st][h][g], fa[idx & 1][i], acc[mb + i][g]);
+            __builtin_amdgcn_sched_barrier(0);
+            wfrag[st][h][g] = *reinterpret_cast<const bf16x8*>(wptr[g] + static_cast<size_t>(kt2) * 1024 + h * 512);
+            __builtin_amdgcn_sched_barrier(0);
+          }
+        }
+        if (NP > 1 && idx == 0) {   // the copies of slab kt+2 go out once the matrix pipe has work
+          stage_slab(kt2, nxt2);
+          __builtin_amdgcn_sched_barrier(0);
+        }
       }
       __builtin_amdgcn_s_waitcnt(kWaitVm20);
       __syncthreads();
