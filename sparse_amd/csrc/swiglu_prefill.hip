@@ -1,4 +1,4 @@
-// Prefill-time grouped SwiGLU expert FFN (bf16): the MFMA grouped-GEMM path.
+// Prefill-time grouped SwiGLU expert FFN (bf16 / fp16): the MFMA grouped-GEMM path.
 //
 // C[p, n] = sum_k A[p, k] * W[n, k] per expert segment.  A workgroup (4 waves) owns a
 // 128-row x 256-weight-row tile; wave w owns all 128 rows and 64 of the weight rows
@@ -12,7 +12,7 @@
 // two slabs ahead of the multiply, one barrier per slab, chunks swizzled by row so that
 // 16-byte fragment reads are bank-conflict free.
 // Weight rows are private to a wave: they go HBM/L2 -> registers directly in MFMA
-// B-operand order, which is exactly the order the tiled layout stores them in (a wave
+// A-operand order, which is exactly the order the tiled layout stores them in (a wave
 // load is one 1 KB run), two slabs ahead of the multiply.  LDS thus carries a third
 // of the bytes of a both-operands-through-LDS design, which is what bounds this shape.
 //
@@ -30,8 +30,8 @@
 // of one MFMA in lane order, lane (r, q) holding k = 16*q + 8*h + 0..7, i.e. the 16-byte chunk 2*q + h
 // of a 128-byte slab row, and the activation fragments are read from LDS in the same order.
 // (The 16x16x32 shape moves half the accumulator data per flop of the 32x32x16 one; with real operands
-// the part is power-capped in either, and a loop of this wavefront tile fed from LDS sustains 1.65
-// against 1.52 PFLOP/s.)
+// the part is power-capped in either, and a loop of this wavefront tile fed from LDS sustained 8 % more
+// with it.)
 #include <atomic>
 #include <type_traits>
 
