@@ -90,24 +90,22 @@ struct PfMapArgs {
   sparse_hip_seglist segs;
 };
 
-// One workgroup: segment s -> its m-tile count, exclusive scan, then every (segment,
-// column tile, m-tile) triple in that order; the rest of each map is marked idle.
+// One workgroup per column tile of each of the two maps (gate/up first): segment s -> its m-tile
+// count, scan (every workgroup does its own: 256 entries), then thread s writes the entries of
+// (segment s, this column tile, m-tile 0 ..) -- tiles in the order segment, column tile, m-tile.
+// The workgroups of column tile 0 also mark the rest of their map idle and write its tile count.
 __global__ __launch_bounds__(256) void prefill_tile_map_kernel(const PfMapArgs a) {
   __shared__ int32_t s_scan[SPARSE_HIP_MAX_EXPERTS];
-  __shared__ int32_t s_slot[SPARSE_HIP_MAX_EXPERTS];
-  __shared__ int32_t s_r0[SPARSE_HIP_MAX_EXPERTS];
-  __shared__ int32_t s_rows[SPARSE_HIP_MAX_EXPERTS];
   const int tid = threadIdx.x;
   int nseg = a.segs.n;
   if (a.segs.eids_dev != nullptr) nseg = min(nseg, a.segs.count_dev[0]);
-  int mt = 0;
+  int mt = 0, slot = 0, r0 = 0, rows = 0;
   if (tid < nseg) {
     const int e = (a.segs.eids_dev != nullptr) ? a.segs.eids_dev[tid] : a.segs.eids[tid];
-    const int b = a.seg_offsets[e], m = a.seg_offsets[e + 1] - b;
-    mt = (m + kPfBM - 1) / kPfBM;
-    s_slot[tid] = (a.segs.eids_dev != nullptr) ? a.expert_slot[e] : a.segs.slots[tid];
-    s_r0[tid] = b;
-    s_rows[tid] = m;
+    r0 = a.seg_offsets[e];
+    rows = a.seg_offsets[e + 1] - r0;
+    mt = (rows + kPfBM - 1) / kPfBM;
+    slot = (a.segs.eids_dev != nullptr) ? a.expert_slot[e] : a.segs.slots[tid];
   }
   s_scan[tid] = mt;
   __syncthreads();
@@ -118,20 +116,17 @@ __global__ __launch_bounds__(256) void prefill_tile_map_kernel(const PfMapArgs a
     __syncthreads();
   }
   const int total_mt = s_scan[255];
-#pragma unroll
-  for (int which = 0; which < 2; ++which) {
-    PfTile* map = which == 0 ? a.map_gu : a.map_dn;
-    const int nt = which == 0 ? a.ntiles_gu : a.ntiles_dn;
-    const int cap = which == 0 ? a.cap_gu : a.cap_dn;
-    if (tid < nseg && mt > 0) {
-      const int base = (s_scan[tid] - mt) * nt;
-      for (int bn = 0; bn < nt; ++bn)
-        for (int bm = 0; bm < mt; ++bm) {
-          const int idx = base + bn * mt + bm;
-          if (idx < cap)
-            map[idx] = PfTile{s_slot[tid], s_r0[tid] + bm * kPfBM, min(kPfBM, s_rows[tid] - bm * kPfBM), bn};
-        }
-    }
+  const int which = static_cast<int>(blockIdx.x) < a.ntiles_gu ? 0 : 1;
+  const int bn = which == 0 ? blockIdx.x : blockIdx.x - a.ntiles_gu;
+  PfTile* map = which == 0 ? a.map_gu : a.map_dn;
+  const int nt = which == 0 ? a.ntiles_gu : a.ntiles_dn;
+  const int cap = which == 0 ? a.cap_gu : a.cap_dn;
+  if (mt > 0) {
+    const int base = (s_scan[tid] - mt) * nt + bn * mt;
+    for (int bm = 0; bm < mt; ++bm)
+      if (base + bm < cap) map[base + bm] = PfTile{slot, r0 + bm * kPfBM, min(kPfBM, rows - bm * kPfBM), bn};
+  }
+  if (bn == 0) {
     for (int idx = total_mt * nt + tid; idx < cap; idx += 256) map[idx] = PfTile{0, 0, 0, 0};
     if (tid == 0) a.totals[which] = total_mt * nt;
   }
@@ -483,7 +478,7 @@ int prefill_routed_bf16(const sparse_hip_experts* ex, const void* x, const void*
     m.cap_gu = cap_gu;
     m.cap_dn = cap_dn;
     m.segs = *segs;
-    hipLaunchKernelGGL(prefill_tile_map_kernel, dim3(1), dim3(256), 0, st, m);
+    hipLaunchKernelGGL(prefill_tile_map_kernel, dim3(nt_gu + nt_dn), dim3(256), 0, st, m);
     SP_LAUNCH_CHECK("prefill_tile_map_kernel");
   }
   PrefillArgs a = {};
