@@ -34,3 +34,67 @@ def test_build_refuses_scratch_in_a_kernel_with_counted_waits():
 
 def test_every_guarded_source_is_built():
     assert set(build.NO_SCRATCH) <= set(build.SOURCES)
+
+
+def _hot_loops(asm: str, kernel_prefix: str):
+    """Basic blocks with at least 16 MFMAs of every function whose name starts with ``kernel_prefix``,
+    as lists of instruction mnemonics + operands."""
+    import re
+    loops, name, block = [], None, None
+    for line in asm.splitlines():
+        text = line.strip()
+        m = re.match(r"^(_Z\w+):", line)
+        if m:
+            name, block = m.group(1), None
+            continue
+        if line.startswith(".Lfunc_end"):
+            name, block = None, None
+            continue
+        if name is None or not name.startswith(kernel_prefix):
+            continue
+        if re.match(r"^\.LBB\d+_\d+:", line):
+            block = []
+            loops.append((name, block))
+            continue
+        if block is not None and text and not text.startswith((";", ".")):
+            block.append(text)
+    return [(n, b) for n, b in loops if sum(i.startswith("v_mfma") for i in b) >= 16]
+
+
+def test_prefill_k_loop_issues_its_vector_memory_operations_as_the_counted_wait_assumes(tmp_path):
+    """The prefill kernel waits for "all but the 20 newest" vector memory operations before the barrier that
+    closes a k slab.  That is exact only if every slab issues, in this order, the 4 LDS copies of the slab
+    after next and then 8 fragment loads, and nothing else that the counter counts (no scratch traffic, no
+    other global access).  Checked on the compiler's output for the counted-wait kernels."""
+    import re
+    import subprocess
+    hipcc = build._hipcc()
+    out = tmp_path / "prefill.s"
+    cmd = [hipcc, *[f for f in build.HIP_FLAGS if f not in ("-fPIC",)], f"-I{build.INCLUDE}", f"-I{build.CSRC}", "-S",
+           "--cuda-device-only", str(build.CSRC / "swiglu_prefill.hip"), "-o", str(out)]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    loops = _hot_loops(out.read_text(), "_ZN6sparse18prefill_ffn_kernel")
+    # counted-wait variants only: the last template argument (kDrainWaits) is false
+    loops = [(n, b) for n, b in loops if re.search(r"ELb[01]ELb0EEEv", n)]
+    assert len(loops) >= 8          # bf16 and fp16, gate/up and down, several tile heights each
+    slabs = 0
+    for name, block in loops:
+        segment = []
+        for ins in block:
+            if ins.startswith("s_barrier"):
+                vm = [i for i in segment if i.startswith(("global_", "scratch_", "buffer_", "flat_"))]
+                kinds = ["copy" if i.startswith("global_load_lds") else "frag" if i.startswith("global_load_dwordx4")
+                         else "other" for i in vm]
+                if kinds:           # (a block may begin in the middle of a slab: only whole slabs are judged)
+                    if len(kinds) == 12:
+                        assert kinds == ["copy"] * 4 + ["frag"] * 8, (name, kinds)
+                        waits = [i for i in segment if i.startswith("s_waitcnt") and "vmcnt" in i]
+                        assert waits and "vmcnt(20)" in waits[-1], (name, waits[-3:])
+                        slabs += 1
+                    else:
+                        assert "other" not in kinds, (name, kinds)
+                segment = []
+            else:
+                segment.append(ins)
+    assert slabs >= 8
