@@ -39,7 +39,7 @@
 extern "C" {
 #endif
 
-#define SPARSE_HIP_ABI_VERSION 1
+#define SPARSE_HIP_ABI_VERSION 2
 
 #define SPARSE_HIP_F32 0
 #define SPARSE_HIP_BF16 1
@@ -212,16 +212,17 @@ int sparse_hip_route_decode(const void* x_dev, const void* wg_dev, const void* w
 
 /*
  * The same routing step (utils/eval_core.py:9519-9520, :9590-9595, and the stable bucketing
- * of :13224-13243) for bf16 activations and at most SPARSE_HIP_ROUTE_PACKED_MAX_TOKENS tokens,
+ * of :13224-13243) for 16-bit activations (`dtype`: bf16 or fp16; `logits_dtype`: the same, or
+ * fp32) and at most SPARSE_HIP_ROUTE_PACKED_MAX_TOKENS tokens,
  * on a gate matrix packed ahead of time so that one workgroup streams it with contiguous
  * wave loads and finishes logits, top-k and permutation without waiting for another
- * workgroup: `gate_packed_dev` is a [SPARSE_HIP_ROUTE_PACKED_ROWS, H] bf16 matrix in the tiled
+ * workgroup: `gate_packed_dev` is a [SPARSE_HIP_ROUTE_PACKED_ROWS, H] matrix of that dtype in the tiled
  * layout (`sparse_hip_tile_weight` of the row-major matrix whose rows are the E gate rows,
  * then the shared-expert gate vector if `has_shared_gate`, then zero rows); H % 64 == 0 and
  * E + has_shared_gate <= SPARSE_HIP_ROUTE_PACKED_ROWS.  Outputs are those of
  * `sparse_hip_route_decode`; the logits differ from it only in the order of the fp32 sum.
  */
-int sparse_hip_route_decode_packed(const void* x_dev, const void* gate_packed_dev, int has_shared_gate,
+int sparse_hip_route_decode_packed(const void* x_dev, const void* gate_packed_dev, int has_shared_gate, int dtype,
                                    int logits_dtype, int T, int H, int E, int K, int renorm, void* logits_dev,
                                    void* shared_gate_dev, void* topv_dev, int64_t* topi_dev, int32_t* perm_dev,
                                    int32_t* inv_perm_dev, int32_t* seg_offsets_dev, int32_t* active_eids_dev,
@@ -237,10 +238,10 @@ int sparse_hip_route_decode_packed(const void* x_dev, const void* gate_packed_de
  * (utils/eval_core.py:16488, :16522-16525).
  * sparse_hip_shared_gate_up is the shared expert's half alone (same kernel code, same bits),
  * for a call that routes some other way; T <= SPARSE_HIP_ROUTE_PACKED_MAX_TOKENS, H % 64 == 0. */
-int sparse_hip_shared_gate_up(const void* x_dev, const void* shared_gate_w_dev, const void* shared_up_w_dev, int T,
-                              int H, int Is, void* shared_inter_dev, void* stream);
+int sparse_hip_shared_gate_up(const void* x_dev, const void* shared_gate_w_dev, const void* shared_up_w_dev, int dtype,
+                              int T, int H, int Is, void* shared_inter_dev, void* stream);
 int sparse_hip_route_decode_packed_shared(const void* x_dev, const void* gate_packed_dev, int has_shared_gate,
-                                          int logits_dtype, int T, int H, int E, int K, int renorm,
+                                          int dtype, int logits_dtype, int T, int H, int E, int K, int renorm,
                                           void* logits_dev, void* shared_gate_dev, void* topv_dev,
                                           int64_t* topi_dev, int32_t* perm_dev, int32_t* inv_perm_dev,
                                           int32_t* seg_offsets_dev, int32_t* active_eids_dev, int32_t* n_active_dev,
@@ -301,7 +302,7 @@ int sparse_hip_shared_expert(const void* x_dev, const void* gate_w_dev, const vo
  * Decode fast path: sparse_hip_grouped_swiglu_decode and sparse_hip_shared_expert of one
  * call in a single launch pair (gate/up of every routed segment and of the shared
  * expert, then all down projections), so the chip sees one fat stream of weights
- * instead of four thinner launches.  bf16 only, T <= SPARSE_HIP_DECODE_MAX_TOKENS.
+ * instead of four thinner launches.  bf16 or fp16 (the slab's dtype), T <= SPARSE_HIP_DECODE_MAX_TOKENS.
  * Arguments as in those two functions; `sh_*` are the shared expert's
  * (utils/eval_core.py:16520-16526).
  * `split_ws_dev` is NULL or a workspace of sparse_hip_decode_split_ws_bytes(T, H) bytes.  With
@@ -364,13 +365,13 @@ int sparse_hip_combine(const void* parts_dev, const int32_t* inv_perm_dev,
 
 /*
  * The same for a decode call whose shared expert was left as partial sums by
- * sparse_hip_moe_ffn_decode(split_ws_dev): shared[t] = bf16(bf16(sum of the `nparts` fp32
- * parts) * bf16(sigmoid(shared_gate[t]))) (no factor when `shared_gate_dev` is NULL) -- the
- * tail of `_shared_expert_forward` (utils/eval_core.py:9455-9463) -- added after the routed
- * parts as above.  bf16 only.
+ * sparse_hip_moe_ffn_decode(split_ws_dev): shared[t] = r(r(sum of the `nparts` fp32
+ * parts) * r(sigmoid(shared_gate[t]))) with r = rounding to `dtype` (no factor when
+ * `shared_gate_dev` is NULL) -- the tail of `_shared_expert_forward`
+ * (utils/eval_core.py:9455-9463) -- added after the routed parts as above.  bf16 or fp16.
  */
 int sparse_hip_combine_split(const void* parts_dev, const int32_t* inv_perm_dev, const void* split_ws_dev,
-                             int nparts, const void* shared_gate_dev, int T, int K, int H,
+                             int nparts, const void* shared_gate_dev, int dtype, int T, int K, int H,
                              void* out_dev, void* stream);
 
 /* ---- A12: routing-scout predictor ------------------------------------------ */

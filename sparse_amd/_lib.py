@@ -17,7 +17,7 @@ MAX_EXPERTS = 256
 MAX_TOPK = 16
 DECODE_MAX_TOKENS = 32
 ENOTREADY = 1
-ABI_VERSION = 1
+ABI_VERSION = 2
 PERMUTE_STATIC_MAX_TOKENS = 65536
 
 
@@ -69,11 +69,11 @@ SIGNATURES = {
     "sparse_hip_route_decode": (
         _i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "sparse_hip_route_decode_packed": (
-        _i, [_vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+        _i, [_vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "sparse_hip_route_decode_packed_shared": (
-        _i, [_vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp,
-             _vp]),
-    "sparse_hip_shared_gate_up": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp, _vp]),
+        _i, [_vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i,
+             _vp, _vp]),
+    "sparse_hip_shared_gate_up": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp]),
     "sparse_hip_permute_ws_bytes": (_sz, [_i, _i, _i]),
     "sparse_hip_permute_build": (_i, [_vp, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "sparse_hip_permute_build_static": (_i, [_vp, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp]),
@@ -91,7 +91,7 @@ SIGNATURES = {
     "sparse_hip_decode_split_counter_offset": (_sz, [_i, _i]),
     "sparse_hip_decode_split_ws_bytes": (_sz, [_i, _i]),
     "sparse_hip_decode_split_parts": (_i, [_i]),
-    "sparse_hip_combine_split": (_i, [_vp, _vp, _vp, _i, _vp, _i, _i, _i, _vp, _vp]),
+    "sparse_hip_combine_split": (_i, [_vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _vp, _vp]),
     "sparse_hip_shared_expert": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp, _vp]),
     "sparse_hip_combine": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp]),
     "sparse_hip_expert_upload_async": (_i, [_vp, _vp, _sz, _vp, _vp]),

@@ -95,7 +95,7 @@ class _Workspace:
         # sums here) that the combine step finishes; from 17 tokens on the routed experts are
         # enough work beside it and the extra reads of the combine step cost more than they save
         self.split_parts = (ops.decode_split_parts(Is) if Is and T <= 16
-                            and dtype == torch.bfloat16 and torch.device(device).type == "cuda" else 1)
+                            and dtype in ops.HALF_DTYPES and torch.device(device).type == "cuda" else 1)
         self.split_ws = ops.decode_split_workspace(T, H, device) if self.split_parts > 1 else None
         # host mirrors for the offloaded path (pinned, written by async D2H copies)
         self.host_offsets = torch.empty((E + 1,), dtype=torch.int32, pin_memory=True)
@@ -626,7 +626,7 @@ class DistributedSparseMoeBlock(nn.Module):
         # Calls of up to 16 tokens compute the shared expert's gate and up projections with the
         # 16-wavefront kernel, beside the routing when this call routes with the packed router,
         # alone otherwise: the same code, so the same bits, wherever it runs.
-        shared_up_alone = (self.shared_weights is not None and self.dtype == torch.bfloat16 and x.is_cuda
+        shared_up_alone = (self.shared_weights is not None and self.dtype in ops.HALF_DTYPES and x.is_cuda
                            and self.route_with_shared and T <= ops.ROUTE_PACKED_MAX_TOKENS
                            and self.shared_inter_size % 32 == 0 and H % 64 == 0)
         self._shared_up_wanted = shared_up_alone and not timing

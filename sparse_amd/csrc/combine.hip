@@ -57,9 +57,10 @@ __global__ __launch_bounds__(kCombThreads) void combine_kernel(const T* __restri
 // partial sums [nparts][T][H]: the shared value is bf16(bf16(p_0 + p_1 + ...) * bf16(sigmoid(
 // gate[t]))) (no factor without a gate), exactly what the one-workgroup down projection
 // stores, and is added after the routed parts.
+template <typename T16>
 __global__ __launch_bounds__(kCombThreads) void combine_split_kernel(
-    const uint16_t* __restrict__ parts, const int32_t* __restrict__ inv_perm, const float* __restrict__ sums,
-    int nparts, const uint16_t* __restrict__ gate, int T, int K, int H, uint16_t* __restrict__ out) {
+    const T16* __restrict__ parts, const int32_t* __restrict__ inv_perm, const float* __restrict__ sums,
+    int nparts, const T16* __restrict__ gate, int T, int K, int H, T16* __restrict__ out) {
   const int hb = (H / 8 + kCombThreads - 1) / kCombThreads;
   const int t = blockIdx.x / hb;
   const int h = ((blockIdx.x - t * hb) * kCombThreads + threadIdx.x) * 8;
@@ -84,9 +85,9 @@ __global__ __launch_bounds__(kCombThreads) void combine_split_kernel(
 #pragma unroll
   for (int k = 0; k < SPARSE_HIP_MAX_TOPK; ++k) {
     if (k < K) {
-      const uint16_t* row = parts + static_cast<size_t>(pos[k]) * H + h;
+      const T16* row = parts + static_cast<size_t>(pos[k]) * H + h;
 #pragma unroll
-      for (int j = 0; j < 8; ++j) acc[j] = Elem<uint16_t>::round(acc[j] + Elem<uint16_t>::load(row + j));
+      for (int j = 0; j < 8; ++j) acc[j] = Elem<T16>::round(acc[j] + Elem<T16>::load(row + j));
     }
   }
   const float* src = sums + static_cast<size_t>(t) * H + h;
@@ -99,16 +100,16 @@ __global__ __launch_bounds__(kCombThreads) void combine_split_kernel(
     for (int j = 0; j < 8; ++j) sh[j] += src[p * part_stride + j];
   }
   const bool gated = gate != nullptr;
-  const float scale = gated ? round_bf16(sigmoid_f32(bf16_bits_to_f32(gate[t]))) : 1.f;
+  const float scale = gated ? Elem<T16>::round(sigmoid_f32(Elem<T16>::load(gate + t))) : 1.f;
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
-    float v = round_bf16(sh[j]);
+    float v = Elem<T16>::round(sh[j]);
     if (gated) v = v * scale;
-    acc[j] = Elem<uint16_t>::round(acc[j] + round_bf16(v));
+    acc[j] = Elem<T16>::round(acc[j] + Elem<T16>::round(v));
   }
-  uint16_t* o = out + static_cast<size_t>(t) * H + h;
+  T16* o = out + static_cast<size_t>(t) * H + h;
 #pragma unroll
-  for (int j = 0; j < 8; ++j) Elem<uint16_t>::store(o + j, acc[j]);
+  for (int j = 0; j < 8; ++j) Elem<T16>::store(o + j, acc[j]);
 }
 
 }  // namespace sparse
@@ -116,8 +117,9 @@ __global__ __launch_bounds__(kCombThreads) void combine_split_kernel(
 using namespace sparse;
 
 extern "C" int sparse_hip_combine_split(const void* parts_dev, const int32_t* inv_perm_dev, const void* split_ws_dev,
-                                        int nparts, const void* shared_gate_dev, int T, int K, int H, void* out_dev,
-                                        void* stream) {
+                                        int nparts, const void* shared_gate_dev, int dtype, int T, int K, int H,
+                                        void* out_dev, void* stream) {
+  SP_REQUIRE(is_16bit(dtype), "combine_split: dtype must be bf16 or fp16");
   SP_REQUIRE(T >= 0 && H > 0 && H % 8 == 0, "combine_split: bad shape T=%d H=%d", T, H);
   SP_REQUIRE(K >= 1 && K <= SPARSE_HIP_MAX_TOPK, "combine_split: K=%d outside [1,%d]", K, SPARSE_HIP_MAX_TOPK);
   SP_REQUIRE(nparts >= 1 && nparts <= 16, "combine_split: nparts=%d outside [1,16]", nparts);
@@ -126,9 +128,17 @@ extern "C" int sparse_hip_combine_split(const void* parts_dev, const int32_t* in
   const int64_t nblk = static_cast<int64_t>((H / 8 + kCombThreads - 1) / kCombThreads) * T;
   SP_REQUIRE(nblk < (1ll << 31), "combine_split: grid too large");
   ProfScope prof(SPARSE_HIP_K_COMBINE, as_stream(stream));
-  hipLaunchKernelGGL(combine_split_kernel, dim3(static_cast<unsigned>(nblk)), dim3(kCombThreads), 0, as_stream(stream),
-                     static_cast<const uint16_t*>(parts_dev), inv_perm_dev, static_cast<const float*>(split_ws_dev),
-                     nparts, static_cast<const uint16_t*>(shared_gate_dev), T, K, H, static_cast<uint16_t*>(out_dev));
+  if (dtype == SPARSE_HIP_F16) {
+    hipLaunchKernelGGL((combine_split_kernel<f16_t>), dim3(static_cast<unsigned>(nblk)), dim3(kCombThreads), 0,
+                       as_stream(stream), static_cast<const f16_t*>(parts_dev), inv_perm_dev,
+                       static_cast<const float*>(split_ws_dev), nparts, static_cast<const f16_t*>(shared_gate_dev), T, K,
+                       H, static_cast<f16_t*>(out_dev));
+  } else {
+    hipLaunchKernelGGL((combine_split_kernel<uint16_t>), dim3(static_cast<unsigned>(nblk)), dim3(kCombThreads), 0,
+                       as_stream(stream), static_cast<const uint16_t*>(parts_dev), inv_perm_dev,
+                       static_cast<const float*>(split_ws_dev), nparts, static_cast<const uint16_t*>(shared_gate_dev), T,
+                       K, H, static_cast<uint16_t*>(out_dev));
+  }
   SP_LAUNCH_CHECK("combine_split_kernel");
   return SPARSE_HIP_OK;
 }

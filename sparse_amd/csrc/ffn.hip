@@ -132,9 +132,6 @@ int sparse_hip_moe_ffn_decode(const sparse_hip_experts* experts, const void* x_d
                         inter_ws_dev, parts_dev);
   if (rc != SPARSE_HIP_OK) return rc;
   SP_REQUIRE(is_16bit(experts->dtype), "moe_ffn_decode: bf16 / fp16 only; use the separate entry points");
-  SP_REQUIRE(experts->dtype == SPARSE_HIP_BF16 || split_ws_dev == nullptr,
-             "moe_ffn_decode: the split shared projection is finished by sparse_hip_combine_split, which is bf16 only; "
-             "pass split_ws_dev = NULL for fp16 or call sparse_hip_moe_ffn_decode_combine");
   SP_REQUIRE(T <= SPARSE_HIP_DECODE_MAX_TOKENS, "moe_ffn_decode: T=%d exceeds %d", T,
              SPARSE_HIP_DECODE_MAX_TOKENS);
   SP_REQUIRE(Is > 0 && Is % 64 == 0, "moe_ffn_decode: Is=%d must be a positive multiple of 64", Is);

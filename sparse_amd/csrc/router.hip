@@ -505,8 +505,9 @@ __global__ __launch_bounds__(kRouteThreads) void route_decode_kernel(const Route
 constexpr int kRpTok = SPARSE_HIP_ROUTE_PACKED_MAX_TOKENS;
 static_assert(kRpTok == kRouteWaves && SPARSE_HIP_ROUTE_PACKED_ROWS == kRlRows, "one wavefront per token, four 16-row groups");
 
-template <typename TL>
+template <typename T16, typename TL>
 __device__ __forceinline__ void route_packed_block(const RouteArgs& a) {
+  using F = typename FormatOf<T16>::type;
   __shared__ float part[kRouteWaves / 2][kRpTok][kRlPad];
   __shared__ float s_logit[kRpTok][kRlRows];
   __shared__ int64_t s_topi[kRpTok * SPARSE_HIP_MAX_TOPK];
@@ -543,7 +544,7 @@ __device__ __forceinline__ void route_packed_block(const RouteArgs& a) {
       for (int h = 0; h < 2; ++h)
 #pragma unroll
         for (int nt = 0; nt < 4; ++nt)
-          acc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[j][h], bv[j][nt][h], acc[nt], 0, 0, 0);
+          acc[nt] = F::mfma16(av[j][h], bv[j][nt][h], acc[nt]);
   }
   if (b < nblk) {
     const bf16x8 av0 = *reinterpret_cast<const bf16x8*>(xrow + b * 64);
@@ -551,8 +552,8 @@ __device__ __forceinline__ void route_packed_block(const RouteArgs& a) {
 #pragma unroll
     for (int nt = 0; nt < 4; ++nt) {
       const uint16_t* p = wt + nt * group_stride + static_cast<size_t>(b) * 1024;
-      acc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av0, *reinterpret_cast<const bf16x8*>(p), acc[nt], 0, 0, 0);
-      acc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av1, *reinterpret_cast<const bf16x8*>(p + 512), acc[nt], 0, 0, 0);
+      acc[nt] = F::mfma16(av0, *reinterpret_cast<const bf16x8*>(p), acc[nt]);
+      acc[nt] = F::mfma16(av1, *reinterpret_cast<const bf16x8*>(p + 512), acc[nt]);
     }
   }
   // D: lane holds gate row nt*16 + r for tokens q*4 .. q*4+3.  Wavefronts 8..15 hand their
@@ -581,24 +582,24 @@ __device__ __forceinline__ void route_packed_block(const RouteArgs& a) {
         Elem<TL>::store(static_cast<TL*>(a.logits) + static_cast<size_t>(tok) * E + col, sum);
         s_logit[tok][col] = Elem<TL>::round(sum);
       } else {
-        static_cast<uint16_t*>(a.shared_gate)[tok] = f32_to_bf16_bits(sum);
+        static_cast<uint16_t*>(a.shared_gate)[tok] = F::bits(sum);
       }
     }
   }
   __syncthreads();
   if (wave < T) {
-    const int sel = topk_token<float, uint16_t>(s_logit[wave], E, a.K, a.renorm,
-                                                static_cast<uint16_t*>(a.topv) + static_cast<size_t>(wave) * a.K,
-                                                a.topi + static_cast<size_t>(wave) * a.K, lane);
+    const int sel = topk_token<float, T16>(s_logit[wave], E, a.K, a.renorm,
+                                           static_cast<T16*>(a.topv) + static_cast<size_t>(wave) * a.K,
+                                           a.topi + static_cast<size_t>(wave) * a.K, lane);
     if (lane < a.K) s_topi[wave * a.K + lane] = static_cast<int64_t>(sel);
   }
   __syncthreads();
   permute_small_block(s_topi, T, a.K, E, a.perm, a.inv_perm, a.seg_offsets, a.active_eids, a.n_active);
 }
 
-template <typename TL>
+template <typename T16, typename TL>
 __global__ __launch_bounds__(kRouteThreads) void route_decode_packed_kernel(const RouteArgs a) {
-  route_packed_block<TL>(a);
+  route_packed_block<T16, TL>(a);
 }
 
 // ---------------------------------------------------------------------------
@@ -621,6 +622,7 @@ struct SharedUpArgs {
 
 constexpr int kSuRows = 32;   // output rows per workgroup: two 16-row MFMA tiles
 
+template <typename F>
 __device__ __forceinline__ void shared_gateup_block(const SharedUpArgs& s, int tile) {
   __shared__ f32x4 red[kRouteWaves][4][64];   // [wavefront][2 * row tile + matrix][lane]
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -661,8 +663,8 @@ __device__ __forceinline__ void shared_gateup_block(const SharedUpArgs& s, int t
       for (int tl = 0; tl < 2; ++tl)
 #pragma unroll
         for (int m = 0; m < 2; ++m) {
-          acc[tl][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[j][tl][m][0], b[j][0], acc[tl][m], 0, 0, 0);
-          acc[tl][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[j][tl][m][1], b[j][1], acc[tl][m], 0, 0, 0);
+          acc[tl][m] = F::mfma16(w[j][tl][m][0], b[j][0], acc[tl][m]);
+          acc[tl][m] = F::mfma16(w[j][tl][m][1], b[j][1], acc[tl][m]);
         }
     }
   }
@@ -683,8 +685,8 @@ __device__ __forceinline__ void shared_gateup_block(const SharedUpArgs& s, int t
     uint16_t o[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const float gv = round_bf16(g[j]), uv = round_bf16(u[j]);
-      o[j] = f32_to_bf16_bits(round_bf16(silu_f32(gv)) * uv);
+      const float gv = F::round(g[j]), uv = F::round(u[j]);
+      o[j] = F::bits(F::round(silu_f32(gv)) * uv);
     }
     uint2 pk;
     pk.x = static_cast<uint32_t>(o[0]) | (static_cast<uint32_t>(o[1]) << 16);
@@ -694,16 +696,17 @@ __device__ __forceinline__ void shared_gateup_block(const SharedUpArgs& s, int t
 }
 
 // the shared expert's half alone, for callers that route some other way
+template <typename F>
 __global__ __launch_bounds__(kRouteThreads) void shared_gateup_kernel(const SharedUpArgs s) {
-  shared_gateup_block(s, static_cast<int>(blockIdx.x));
+  shared_gateup_block<F>(s, static_cast<int>(blockIdx.x));
 }
 
-template <typename TL>
+template <typename T16, typename TL>
 __global__ __launch_bounds__(kRouteThreads) void route_packed_shared_kernel(const RouteArgs a, const SharedUpArgs s) {
   if (blockIdx.x == 0) {
-    route_packed_block<TL>(a);
+    route_packed_block<T16, TL>(a);
   } else {
-    shared_gateup_block(s, static_cast<int>(blockIdx.x) - 1);
+    shared_gateup_block<typename FormatOf<T16>::type>(s, static_cast<int>(blockIdx.x) - 1);
   }
 }
 
@@ -754,6 +757,16 @@ static int launch_route_decode(const RouteArgs& a, hipStream_t st) {
 }  // namespace sparse
 
 using namespace sparse;
+
+template <typename T16, typename TL>
+static void launch_route_packed(const RouteArgs& a, const SharedUpArgs* shared, hipStream_t st) {
+  if (shared != nullptr) {
+    const dim3 grid(1 + shared->Is / kSuRows);
+    hipLaunchKernelGGL((route_packed_shared_kernel<T16, TL>), grid, dim3(kRouteThreads), 0, st, a, *shared);
+  } else {
+    hipLaunchKernelGGL((route_decode_packed_kernel<T16, TL>), dim3(1), dim3(kRouteThreads), 0, st, a);
+  }
+}
 
 extern "C" {
 
@@ -865,12 +878,14 @@ int sparse_hip_route_decode(const void* x_dev, const void* wg_dev, const void* w
   return launch_route_decode<uint16_t, uint16_t>(a, st);
 }
 
-static int route_packed_impl(const void* x_dev, const void* gate_packed_dev, int has_shared_gate, int logits_dtype, int T,
-                             int H, int E, int K, int renorm, void* logits_dev, void* shared_gate_dev, void* topv_dev,
-                             int64_t* topi_dev, int32_t* perm_dev, int32_t* inv_perm_dev, int32_t* seg_offsets_dev,
-                             int32_t* active_eids_dev, int32_t* n_active_dev, const SharedUpArgs* shared, void* stream) {
-  SP_REQUIRE(logits_dtype == SPARSE_HIP_BF16 || logits_dtype == SPARSE_HIP_F32,
-             "route_decode_packed: logits_dtype must be bf16 or fp32");
+static int route_packed_impl(const void* x_dev, const void* gate_packed_dev, int has_shared_gate, int dtype,
+                             int logits_dtype, int T, int H, int E, int K, int renorm, void* logits_dev,
+                             void* shared_gate_dev, void* topv_dev, int64_t* topi_dev, int32_t* perm_dev,
+                             int32_t* inv_perm_dev, int32_t* seg_offsets_dev, int32_t* active_eids_dev,
+                             int32_t* n_active_dev, const SharedUpArgs* shared, void* stream) {
+  SP_REQUIRE(is_16bit(dtype), "route_decode_packed: dtype must be bf16 or fp16");
+  SP_REQUIRE(logits_dtype == dtype || logits_dtype == SPARSE_HIP_F32,
+             "route_decode_packed: logits_dtype must be the activations' dtype or fp32");
   SP_REQUIRE(T >= 1 && T <= SPARSE_HIP_ROUTE_PACKED_MAX_TOKENS, "route_decode_packed: T=%d outside [1,%d]", T,
              SPARSE_HIP_ROUTE_PACKED_MAX_TOKENS);
   SP_REQUIRE(H > 0 && H % 64 == 0, "route_decode_packed: H=%d must be a positive multiple of 64", H);
@@ -888,37 +903,29 @@ static int route_packed_impl(const void* x_dev, const void* gate_packed_dev, int
                  T,        H,               E,               K,               renorm,          has_shared_gate ? 1 : 0};
   hipStream_t st = as_stream(stream);
   ProfScope prof(SPARSE_HIP_K_ROUTE_DECODE, st);
-  if (shared != nullptr) {
-    const dim3 grid(1 + shared->Is / kSuRows);
-    if (logits_dtype == SPARSE_HIP_F32) {
-      hipLaunchKernelGGL((route_packed_shared_kernel<float>), grid, dim3(kRouteThreads), 0, st, a, *shared);
-    } else {
-      hipLaunchKernelGGL((route_packed_shared_kernel<uint16_t>), grid, dim3(kRouteThreads), 0, st, a, *shared);
-    }
-    SP_LAUNCH_CHECK("route_packed_shared_kernel");
-    return SPARSE_HIP_OK;
-  }
-  if (logits_dtype == SPARSE_HIP_F32) {
-    hipLaunchKernelGGL((route_decode_packed_kernel<float>), dim3(1), dim3(kRouteThreads), 0, st, a);
+  const bool wide_logits = logits_dtype == SPARSE_HIP_F32;
+  if (dtype == SPARSE_HIP_F16) {
+    if (wide_logits) launch_route_packed<f16_t, float>(a, shared, st); else launch_route_packed<f16_t, f16_t>(a, shared, st);
   } else {
-    hipLaunchKernelGGL((route_decode_packed_kernel<uint16_t>), dim3(1), dim3(kRouteThreads), 0, st, a);
+    if (wide_logits) launch_route_packed<uint16_t, float>(a, shared, st); else launch_route_packed<uint16_t, uint16_t>(a, shared, st);
   }
-  SP_LAUNCH_CHECK("route_decode_packed_kernel");
+  SP_LAUNCH_CHECK(shared != nullptr ? "route_packed_shared_kernel" : "route_decode_packed_kernel");
   return SPARSE_HIP_OK;
 }
 
-int sparse_hip_route_decode_packed(const void* x_dev, const void* gate_packed_dev, int has_shared_gate,
+int sparse_hip_route_decode_packed(const void* x_dev, const void* gate_packed_dev, int has_shared_gate, int dtype,
                                    int logits_dtype, int T, int H, int E, int K, int renorm, void* logits_dev,
                                    void* shared_gate_dev, void* topv_dev, int64_t* topi_dev, int32_t* perm_dev,
                                    int32_t* inv_perm_dev, int32_t* seg_offsets_dev, int32_t* active_eids_dev,
                                    int32_t* n_active_dev, void* stream) {
-  return route_packed_impl(x_dev, gate_packed_dev, has_shared_gate, logits_dtype, T, H, E, K, renorm, logits_dev,
-                           shared_gate_dev, topv_dev, topi_dev, perm_dev, inv_perm_dev, seg_offsets_dev,
+  return route_packed_impl(x_dev, gate_packed_dev, has_shared_gate, dtype, logits_dtype, T, H, E, K, renorm,
+                           logits_dev, shared_gate_dev, topv_dev, topi_dev, perm_dev, inv_perm_dev, seg_offsets_dev,
                            active_eids_dev, n_active_dev, nullptr, stream);
 }
 
-int sparse_hip_shared_gate_up(const void* x_dev, const void* shared_gate_w_dev, const void* shared_up_w_dev, int T,
-                              int H, int Is, void* shared_inter_dev, void* stream) {
+int sparse_hip_shared_gate_up(const void* x_dev, const void* shared_gate_w_dev, const void* shared_up_w_dev, int dtype,
+                              int T, int H, int Is, void* shared_inter_dev, void* stream) {
+  SP_REQUIRE(is_16bit(dtype), "shared_gate_up: dtype must be bf16 or fp16");
   SP_REQUIRE(x_dev && shared_gate_w_dev && shared_up_w_dev && shared_inter_dev, "shared_gate_up: NULL pointer");
   SP_REQUIRE(T >= 1 && T <= SPARSE_HIP_ROUTE_PACKED_MAX_TOKENS, "shared_gate_up: T=%d outside [1,%d]", T,
              SPARSE_HIP_ROUTE_PACKED_MAX_TOKENS);
@@ -927,13 +934,17 @@ int sparse_hip_shared_gate_up(const void* x_dev, const void* shared_gate_w_dev, 
   SharedUpArgs s = {static_cast<const uint16_t*>(shared_gate_w_dev), static_cast<const uint16_t*>(shared_up_w_dev),
                     static_cast<const uint16_t*>(x_dev), static_cast<uint16_t*>(shared_inter_dev), T, H, Is};
   hipStream_t st = as_stream(stream);
-  hipLaunchKernelGGL(shared_gateup_kernel, dim3(Is / kSuRows), dim3(kRouteThreads), 0, st, s);
+  if (dtype == SPARSE_HIP_F16) {
+    hipLaunchKernelGGL((shared_gateup_kernel<Fp16>), dim3(Is / kSuRows), dim3(kRouteThreads), 0, st, s);
+  } else {
+    hipLaunchKernelGGL((shared_gateup_kernel<Bf16>), dim3(Is / kSuRows), dim3(kRouteThreads), 0, st, s);
+  }
   SP_LAUNCH_CHECK("shared_gateup_kernel");
   return SPARSE_HIP_OK;
 }
 
 int sparse_hip_route_decode_packed_shared(const void* x_dev, const void* gate_packed_dev, int has_shared_gate,
-                                          int logits_dtype, int T, int H, int E, int K, int renorm,
+                                          int dtype, int logits_dtype, int T, int H, int E, int K, int renorm,
                                           void* logits_dev, void* shared_gate_dev, void* topv_dev,
                                           int64_t* topi_dev, int32_t* perm_dev, int32_t* inv_perm_dev,
                                           int32_t* seg_offsets_dev, int32_t* active_eids_dev, int32_t* n_active_dev,
@@ -944,8 +955,8 @@ int sparse_hip_route_decode_packed_shared(const void* x_dev, const void* gate_pa
              kSuRows);
   SharedUpArgs s = {static_cast<const uint16_t*>(shared_gate_w_dev), static_cast<const uint16_t*>(shared_up_w_dev),
                     static_cast<const uint16_t*>(x_dev), static_cast<uint16_t*>(shared_inter_dev), T, H, Is};
-  return route_packed_impl(x_dev, gate_packed_dev, has_shared_gate, logits_dtype, T, H, E, K, renorm, logits_dev,
-                           shared_gate_dev, topv_dev, topi_dev, perm_dev, inv_perm_dev, seg_offsets_dev,
+  return route_packed_impl(x_dev, gate_packed_dev, has_shared_gate, dtype, logits_dtype, T, H, E, K, renorm,
+                           logits_dev, shared_gate_dev, topv_dev, topi_dev, perm_dev, inv_perm_dev, seg_offsets_dev,
                            active_eids_dev, n_active_dev, &s, stream);
 }
 

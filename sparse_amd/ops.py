@@ -184,14 +184,14 @@ ROUTE_PACKED_ROWS = 64
 
 
 def pack_router_gate(wg: torch.Tensor, wsg: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
-    """The gate matrix ``route_decode_packed`` reads: 64 bf16 rows (the E gate rows, then the
-    shared-expert gate vector when there is one, then zeros) in the tiled weight layout,
-    flattened.  ``None`` when the shapes do not fit (more than 64 rows, H not a multiple of
-    64, not bf16): the caller then stays on ``route_decode``."""
+    """The gate matrix ``route_decode_packed`` reads: 64 rows of the weights' 16-bit dtype (the E
+    gate rows, then the shared-expert gate vector when there is one, then zeros) in the tiled
+    weight layout, flattened.  ``None`` when the shapes do not fit (more than 64 rows, H not a
+    multiple of 64, fp32): the caller then stays on ``route_decode``."""
     from .weights import tile_weight
     E, H = wg.shape
     rows = E + (1 if wsg is not None else 0)
-    if wg.dtype != torch.bfloat16 or H % 64 or rows > ROUTE_PACKED_ROWS:
+    if wg.dtype not in HALF_DTYPES or H % 64 or rows > ROUTE_PACKED_ROWS:
         return None
     full = torch.zeros((ROUTE_PACKED_ROWS, H), dtype=wg.dtype, device=wg.device)
     full[:E] = wg
@@ -203,21 +203,22 @@ def pack_router_gate(wg: torch.Tensor, wsg: Optional[torch.Tensor]) -> Optional[
 def route_decode_packed(x: torch.Tensor, gate_packed: torch.Tensor, num_experts: int, has_shared_gate: bool, k: int,
                         renorm: bool, logits: torch.Tensor, shared_gate: Optional[torch.Tensor], topv: torch.Tensor,
                         topi: torch.Tensor, perm: Permutation, shared_up=None) -> None:
-    """Router logits + top-k + permutation of up to 16 bf16 tokens by one workgroup, on the
+    """Router logits + top-k + permutation of up to 16 bf16 or fp16 tokens by one workgroup, on the
     matrix ``pack_router_gate`` made.  ``shared_up = (gate_w, up_w, inter_out)``: the same launch
     also computes the shared expert's SiLU(gate x) * (up x) into ``inter_out [T, Is]`` (tiled
     weights ``[Is, H]``, Is a multiple of 32), on the part of the device routing leaves idle."""
     lib = _lib.load()
     T, H = x.shape
     E = int(num_experts)
-    _need(x, "x", torch.bfloat16)
-    _need(gate_packed, "packed gate", torch.bfloat16, (ROUTE_PACKED_ROWS * H,))
+    _need_half(x, "x")
+    _need(gate_packed, "packed gate", x.dtype, (ROUTE_PACKED_ROWS * H,))
     _need(logits, "logits", None, (T, E))
     _need(topv, "topv", x.dtype, (T, k))
     _need(topi, "topi", torch.int64, (T, k))
     if has_shared_gate:
         _need(shared_gate, "shared gate logits", x.dtype, (T,))
-    common = (_ptr(x), _ptr(gate_packed), int(bool(has_shared_gate)), dtype_code(logits.dtype), T, H, E, int(k),
+    common = (_ptr(x), _ptr(gate_packed), int(bool(has_shared_gate)), dtype_code(x.dtype), dtype_code(logits.dtype),
+              T, H, E, int(k),
               int(bool(renorm)), _ptr(logits), _ptr(shared_gate), _ptr(topv), _ptr(topi), _ptr(perm.perm),
               _ptr(perm.inv_perm), _ptr(perm.seg_offsets), _ptr(perm.active_eids), _ptr(perm.n_active))
     if shared_up is None:
@@ -233,16 +234,16 @@ def route_decode_packed(x: torch.Tensor, gate_packed: torch.Tensor, num_experts:
 
 
 def shared_gate_up(x: torch.Tensor, gate_w: torch.Tensor, up_w: torch.Tensor, inter_out: torch.Tensor) -> None:
-    """The shared expert's SiLU(gate x) * (up x) for up to 16 bf16 tokens, by the kernel code
+    """The shared expert's SiLU(gate x) * (up x) for up to 16 bf16 or fp16 tokens, by the kernel code
     ``route_decode_packed(shared_up=...)`` runs beside the routing (same bits)."""
     T, H = x.shape
     Is = int(gate_w.shape[0])
-    _need(x, "x", torch.bfloat16)
+    _need_half(x, "x")
     _need(gate_w, "shared gate_proj", x.dtype, (Is, H))
     _need(up_w, "shared up_proj", x.dtype, (Is, H))
     _need(inter_out, "shared inter_ws", x.dtype, (T, Is))
-    _lib.check(_lib.load().sparse_hip_shared_gate_up(_ptr(x), _ptr(gate_w), _ptr(up_w), T, H, Is, _ptr(inter_out),
-                                                     _stream()), "sparse_hip_shared_gate_up")
+    _lib.check(_lib.load().sparse_hip_shared_gate_up(_ptr(x), _ptr(gate_w), _ptr(up_w), dtype_code(x.dtype), T, H, Is,
+                                                     _ptr(inter_out), _stream()), "sparse_hip_shared_gate_up")
 
 
 # --------------------------------------------------------------------------- experts
@@ -365,7 +366,8 @@ def combine_split(parts: torch.Tensor, perm: Permutation, split_ws: torch.Tensor
     partial sums in ``split_ws`` (``moe_ffn_decode(split_ws=...)``)."""
     lib = _lib.load()
     H = parts.shape[1]
-    _need(parts, "parts", torch.bfloat16, (T * K, H))
+    _need_half(parts, "parts")
+    _need(parts, "parts", parts.dtype, (T * K, H))
     _need(out, "out", parts.dtype, (T, H))
     _need(split_ws, "split workspace", torch.float32)
     if split_ws.numel() < int(nparts) * T * H:
@@ -373,7 +375,7 @@ def combine_split(parts: torch.Tensor, perm: Permutation, split_ws: torch.Tensor
     if shared_gate is not None:
         _need(shared_gate, "shared gate logits", parts.dtype, (T,))
     rc = lib.sparse_hip_combine_split(_ptr(parts), _ptr(perm.inv_perm), _ptr(split_ws), int(nparts), _ptr(shared_gate),
-                                      T, K, H, _ptr(out), _stream())
+                                      dtype_code(parts.dtype), T, K, H, _ptr(out), _stream())
     _lib.check(rc, "sparse_hip_combine_split")
 
 
@@ -539,8 +541,7 @@ def moe_ffn_decode(experts: Experts, x: torch.Tensor, topv: torch.Tensor, perm: 
                    inter_ws: torch.Tensor, parts: torch.Tensor, shared_w, shared_gate: Optional[torch.Tensor],
                    shared_inter_ws: torch.Tensor, shared_out: torch.Tensor,
                    split_ws: Optional[torch.Tensor] = None, shared_inter_ready: bool = False) -> None:
-    """Routed experts + shared expert of a decode call in one launch pair (bf16 or fp16, T <= 32;
-    ``split_ws`` with bf16 only, whose combine step finishes the split).
+    """Routed experts + shared expert of a decode call in one launch pair (bf16 or fp16, T <= 32).
     ``split_ws`` (from ``decode_split_workspace``) lets the shared down projection spread its
     long reduction over four workgroups per tile.  ``shared_inter_ready``: ``shared_inter_ws``
     already holds the shared expert's SiLU(gate x) * (up x) (``route_decode_packed`` computed it

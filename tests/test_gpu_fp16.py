@@ -87,6 +87,118 @@ def test_route_decode_fp16_equals_the_three_separate_calls(device, T):
             assert torch.equal(getattr(perm_a, name), getattr(perm_b, name)), name
 
 
+@pytest.mark.parametrize("ldt", [F16, torch.float32])
+@pytest.mark.parametrize("T,H,E,K,Is", [(1, 2048, 60, 4, 5632), (8, 2048, 60, 4, 5632), (16, 2048, 63, 6, 2816),
+                                        (5, 192, 15, 3, 96)])
+def test_route_decode_packed_fp16(device, T, H, E, K, Is, ldt):
+    """The one-workgroup router on the packed gate matrix in fp16, alone and with the shared expert's gate and up
+    projections beside it: logits against fp32 linear algebra, top-k and permutation bit for bit what gate_topk
+    and permute_build return on the logits it wrote, SiLU(gate x) * (up x) within the fp16 bound of fp32 linear
+    algebra rounded the way the expert kernels round, and the same bits from the stand-alone launch."""
+    from sparse_amd.weights import tile_weight
+    ops = _ops()
+    layer = make_layer(H, E, 64, K, Is=Is, shared_gate=True, dtype=F16, seed=23 + T, std=0.05)
+    packed = ops.pack_router_gate(layer["gate_w"].to(device), layer["shared_gate_w"].to(device))
+    assert packed is not None and packed.dtype == F16 and packed.numel() == 64 * H
+    gw, uw = (tile_weight(w.to(device)).reshape(w.shape).contiguous() for w in layer["shared"][:2])
+    x = make_hidden(T, H, F16, seed=400 + T)
+    xd = x.to(device)
+
+    def route(shared_up):
+        logits = torch.empty(T, E, dtype=ldt, device=device)
+        sg = torch.empty(T, dtype=F16, device=device)
+        topv = torch.empty(T, K, dtype=F16, device=device)
+        topi = torch.empty(T, K, dtype=torch.int64, device=device)
+        perm = ops.Permutation(T, K, E, device)
+        ops.route_decode_packed(xd, packed, E, True, K, False, logits, sg, topv, topi, perm, shared_up=shared_up)
+        torch.cuda.synchronize()
+        return logits, sg, topv, topi, perm
+
+    inter = torch.full((T, Is), float("nan"), dtype=F16, device=device)
+    a, b = route(None), route((gw, uw, inter))
+    for u, v in zip(a[:4], b[:4]):
+        assert torch.equal(u, v)
+    for name in ("perm", "inv_perm", "seg_offsets", "n_active"):
+        assert torch.equal(getattr(a[4], name), getattr(b[4], name)), name
+    logits, sg, topv, topi, perm = a
+    ref = torch.nn.functional.linear(x.float(), layer["gate_w"].float())
+    tol = dict(rtol=2e-3, atol=2e-3) if ldt == F16 else dict(rtol=1e-4, atol=1e-4)
+    torch.testing.assert_close(logits.float().cpu(), ref, **tol)
+    ref_sg = torch.nn.functional.linear(x.float(), layer["shared_gate_w"].float().reshape(1, -1)).reshape(-1)
+    torch.testing.assert_close(sg.float().cpu(), ref_sg, rtol=2e-3, atol=2e-3)
+    topv_a, topi_a = ops.gate_topk(logits, K, out_dtype=F16)
+    perm_a = ops.permute_build(topi_a, E)
+    torch.cuda.synchronize()
+    assert torch.equal(topv_a, topv) and torch.equal(topi_a, topi)
+    n = int(perm_a.n_active.item())
+    assert n == int(perm.n_active.item())
+    for name in ("perm", "inv_perm", "seg_offsets"):
+        assert torch.equal(getattr(perm_a, name), getattr(perm, name)), name
+    g = torch.nn.functional.linear(x.float(), layer["shared"][0].float()).to(F16).float()
+    u = torch.nn.functional.linear(x.float(), layer["shared"][1].float()).to(F16).float()
+    want = (torch.nn.functional.silu(g).to(F16).float() * u).to(F16)
+    got = inter.cpu()
+    assert not torch.isnan(got.float()).any()
+    torch.testing.assert_close(got.float(), want.float(), **FP16_TOL)
+    alone = torch.empty_like(inter)
+    ops.shared_gate_up(xd, gw, uw, alone)
+    torch.cuda.synchronize()
+    assert torch.equal(alone, inter)
+
+
+@pytest.mark.parametrize("T", [1, 8, 16])
+@pytest.mark.parametrize("gated", [True, False])
+def test_fused_decode_fp16_with_the_shared_reduction_split(device, T, gated):
+    """The fp16 decode launch pair with the shared expert's down projection left as fp32 partial sums: finished
+    by combine_split, and by the down launch itself (moe_ffn_decode_combine) with the same bits; routed parts
+    those of the one-workgroup form, the output within tolerance of the oracle."""
+    from sparse_amd.weights import ExpertSlab, tile_weight
+    ops = _ops()
+    H, E, I, K, Is = 512, 8, 128, 2, 1024
+    layer = make_layer(H, E, I, K, Is=Is, shared_gate=gated, dtype=F16, seed=81, std=0.05)
+    xc = make_hidden(T, H, F16, seed=82)
+    x = xc.to(device)
+    slab = ExpertSlab.resident(layer["experts"], H, I, F16, device)
+    experts = ops.make_experts(slab.data, slab.expert_slot, E, H, I)
+    logits, sg = ops.router_logits(x, layer["gate_w"].to(device), layer["shared_gate_w"].to(device) if gated else None)
+    topv, topi = ops.gate_topk(logits, K, out_dtype=F16)
+    perm = ops.permute_build(topi, E)
+    segs = ops.seglist_device(perm, min(E, T * K))
+    sw = tuple(tile_weight(t).reshape(t.shape).contiguous().to(device) for t in layer["shared"])
+    nparts = ops.decode_split_parts(Is)
+    ws = ops.decode_split_workspace(T, H, device)
+
+    def run(mode):
+        inter = torch.empty((T * K, I), device=device, dtype=F16)
+        parts = torch.empty((T * K, H), device=device, dtype=F16)
+        sh_inter = torch.empty((T, Is), device=device, dtype=F16)
+        sh_out = torch.empty((T, H), device=device, dtype=F16)
+        out = torch.full((T, H), float("nan"), device=device, dtype=F16)
+        if mode == "plain":
+            ops.moe_ffn_decode(experts, x, topv, perm, segs, inter, parts, sw, sg if gated else None, sh_inter, sh_out, None)
+            ops.combine(parts, perm, sh_out, T, K, out)
+        elif mode == "split":
+            ops.moe_ffn_decode(experts, x, topv, perm, segs, inter, parts, sw, sg if gated else None, sh_inter, sh_out, ws)
+            ops.combine_split(parts, perm, ws, nparts, sg if gated else None, T, K, out)
+        else:
+            ops.moe_ffn_decode_combine(experts, x, topv, perm, segs, inter, parts, sw, sg if gated else None, sh_inter,
+                                       ws, out)
+        torch.cuda.synchronize()
+        return parts, out
+
+    parts0, out0 = run("plain")
+    ref, _, _, _ = ref_moe.moe_forward(xc, layer["gate_w"], layer["experts"], K, layer["shared"], layer["shared_gate_w"],
+                                       router_logits=logits.cpu())
+    parts1, out1 = run("split")
+    parts2, out2 = run("fold")
+    assert torch.equal(parts1, parts0) and torch.equal(parts2, parts0)
+    assert not torch.isnan(out1.float()).any() and torch.equal(out1, out2)
+    torch.testing.assert_close(out1.float(), out0.float(), rtol=2e-3, atol=1e-6)   # two fp16 roundings apart at most
+    torch.testing.assert_close(out1.cpu().float(), ref.float(), **FP16_TOL)
+    _, again = run("fold")
+    assert torch.equal(again, out2)
+
+
 @pytest.mark.parametrize("T", [1, 8, 17, 32])
 def test_decode_ffn_fp16_matches_oracle(device, T):
     ops = _ops()
