@@ -59,7 +59,6 @@ typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef _Float16 f16_t;  // IEEE half: the storage tag of fp16 tensors (bf16 tensors are tagged uint16_t)
 typedef __attribute__((__vector_size__(8 * sizeof(_Float16)))) _Float16 f16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
-typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16;
 
 struct __attribute__((aligned(16))) u32x4 {
   uint32_t x, y, z, w;
@@ -123,9 +122,6 @@ struct Bf16 {
   __device__ static __forceinline__ f32x4 mfma16(bf16x8 a, bf16x8 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
   }
-  __device__ static __forceinline__ f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
-  }
 };
 struct Fp16 {
   static constexpr int dtype = SPARSE_HIP_F16;
@@ -139,9 +135,6 @@ struct Fp16 {
   }
   __device__ static __forceinline__ f32x4 mfma16(bf16x8 a, bf16x8 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
-  }
-  __device__ static __forceinline__ f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
   }
 };
 // storage tag -> format
