@@ -578,6 +578,9 @@ def main():
     _Workspace._cache.clear()
     torch.cuda.empty_cache()
     if not args.no_extra:
+        extra["prefill_4k_deepseek"] = prefill_workload(DEEPSEEK, 4096, max(2, min(10, args.steps // 10)), 1, dtype,
+                                                        device)
+    if not args.no_extra:
         # the same stack and step in fp16, the dtype of the reference's formal runs
         blocks16 = build_stack(QWEN, torch.float16, device)
         extra["decode_b8_fp16"] = decode_workload(blocks16, QWEN, 8, max(10, args.steps // 2), args.warmup,
@@ -585,9 +588,6 @@ def main():
         del blocks16
         _Workspace._cache.clear()
         torch.cuda.empty_cache()
-    if not args.no_extra:
-        extra["prefill_4k_deepseek"] = prefill_workload(DEEPSEEK, 4096, max(2, min(10, args.steps // 10)), 1, dtype,
-                                                        device)
     if not args.no_extra and not args.no_offload:
         # the offloaded configurations: rr and rs as the configuration states them (512 decode steps
         # from a cold cache), this build's other variants at 64 steps and labelled so; a failure
