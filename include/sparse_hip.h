@@ -299,6 +299,28 @@ int sparse_hip_shared_expert(const void* x_dev, const void* gate_w_dev, const vo
                              void* stream);
 
 /*
+ * Prefill fast path: sparse_hip_grouped_swiglu_prefill and sparse_hip_shared_expert of one call
+ * as two launches of persistent workgroups (every gate/up projection, then every down projection),
+ * bf16 or fp16, any T.  Tiles of the routed segments and of the shared expert sit in one set of
+ * queues (one per XCD, built on the device in `tile_ws_dev`); a workgroup takes tile after tile and
+ * requests the first operands of its next tile while it finishes the current one, so routed and
+ * shared work share one tail per launch and no tile but a workgroup's first pays a prologue.
+ * Results are bit-identical to the two separate calls.  Arguments as in those two functions
+ * (utils/eval_core.py:11700-11793 for the routed experts, :9455-9463 and :16520-16526 for the shared
+ * expert).  `sh_down_w_dev` NULL: no shared expert (the other sh_* arguments are ignored);
+ * segs->n == 0: the shared expert alone.  `tile_ws_dev`: 256-byte aligned workspace of
+ * sparse_hip_moe_ffn_prefill_ws_bytes(T, K, segs->n, H, I, Is) bytes (Is = 0 without a shared
+ * expert).  Calls that share a workspace must be ordered on one stream.
+ */
+size_t sparse_hip_moe_ffn_prefill_ws_bytes(int T, int K, int num_segments, int H, int I, int Is);
+int sparse_hip_moe_ffn_prefill(const sparse_hip_experts* experts, const void* x_dev, const void* topv_dev,
+                               const int32_t* perm_dev, const int32_t* seg_offsets_dev,
+                               const sparse_hip_seglist* segs, int T, int K, void* inter_ws_dev,
+                               void* parts_dev, const void* sh_gate_w_dev, const void* sh_up_w_dev,
+                               const void* sh_down_w_dev, const void* shared_gate_dev, int Is,
+                               void* sh_inter_ws_dev, void* shared_dev, void* tile_ws_dev, void* stream);
+
+/*
  * Decode fast path: sparse_hip_grouped_swiglu_decode and sparse_hip_shared_expert of one
  * call in a single launch pair (gate/up of every routed segment and of the shared
  * expert, then all down projections), so the chip sees one fat stream of weights
@@ -460,7 +482,7 @@ int sparse_hip_profile_enable(int on);
 int sparse_hip_profile_reset(void);
 int sparse_hip_profile_read(int kernel, double* total_ms_out, int64_t* launches_out);
 /* Checking aid with no counterpart in the reference: while on, the prefill-size expert FFN
- * (sparse_hip_moe_ffn_prefill, sparse_hip_shared_ffn at prefill sizes) runs the variant of its
+ * (sparse_hip_grouped_swiglu_prefill, sparse_hip_moe_ffn_prefill, sparse_hip_shared_expert at prefill sizes) runs the variant of its
  * kernel whose k loop drains every outstanding vector-memory operation where the normal one
  * waits for a counted number of them.  Same arithmetic, same bits, slower; a difference
  * between the two means the counted waits no longer match the code the compiler produced.

@@ -82,6 +82,10 @@ SIGNATURES = {
     "sparse_hip_prefill_ws_bytes": (_sz, [_i, _i, _i, _i, _i]),
     "sparse_hip_grouped_swiglu_prefill": (
         _i, [C.POINTER(Experts), _vp, _vp, _vp, _vp, C.POINTER(SegList), _i, _i, _vp, _vp, _vp, _vp]),
+    "sparse_hip_moe_ffn_prefill_ws_bytes": (_sz, [_i, _i, _i, _i, _i, _i]),
+    "sparse_hip_moe_ffn_prefill": (
+        _i, [C.POINTER(Experts), _vp, _vp, _vp, _vp, C.POINTER(SegList), _i, _i, _vp, _vp,
+             _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _vp]),
     "sparse_hip_moe_ffn_decode": (
         _i, [C.POINTER(Experts), _vp, _vp, _vp, _vp, C.POINTER(SegList), _i, _i, _vp, _vp,
              _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _vp]),

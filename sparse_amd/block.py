@@ -293,7 +293,11 @@ class DistributedSparseMoeBlock(nn.Module):
         self._shared_inter_ready = False    # _route: this call's routing launch has filled it
         self.fold_combine = str(os.environ.get("SPARSE_HIP_FOLD_COMBINE", "1")).strip().lower() not in (
             "", "0", "false", "no", "off")
-        # prefill-size batches run the shared expert on a second stream beside the routing
+        # all-resident prefill-size batches run routed and shared tiles in one launch per projection
+        # (SPARSE_HIP_MERGED_PREFILL=0: separate launches; same bits either way)
+        self.merged_prefill = str(os.environ.get("SPARSE_HIP_MERGED_PREFILL", "1")).strip().lower() not in (
+            "", "0", "false", "no", "off")
+        # ... and otherwise the shared expert on a second stream beside the routing
         self.overlap_shared = str(os.environ.get("SPARSE_HIP_OVERLAP_SHARED", "1")).strip().lower() not in (
             "", "0", "false", "no", "off")
 
@@ -616,8 +620,10 @@ class DistributedSparseMoeBlock(nn.Module):
         # Prefill-size batches: the shared expert needs only x and the shared gate, so it runs
         # on a second stream from the moment the logits kernel is queued, beside top-k,
         # permutation, tile map and the first routed tiles, and is joined before combine.
+        merged = (self.merged_prefill and self.residency is None and self.dtype in ops.HALF_DTYPES and x.is_cuda
+                  and T > ops.DECODE_MAX_TOKENS and not timing)
         side = (self._shared_stream() if self.shared_weights is not None and not fused and self.overlap_shared
-                and x.is_cuda and T > ops.DECODE_MAX_TOKENS and not timing else None)
+                and x.is_cuda and T > ops.DECODE_MAX_TOKENS and not timing and not merged else None)
 
         # Whether the shared expert's down projection is left as partial sums for the combine
         # step depends on the call's size and dtype only, never on where the routed experts
@@ -639,7 +645,7 @@ class DistributedSparseMoeBlock(nn.Module):
             return self._shared_inter_ready
 
         def run_shared() -> None:
-            if self.shared_weights is None or fused:
+            if self.shared_weights is None or fused or merged:
                 return
             gw, uw, dw = self.shared_weights
             if split_shared:
@@ -685,6 +691,9 @@ class DistributedSparseMoeBlock(nn.Module):
                 ops.moe_ffn_decode(self._experts_desc, x, ws.topv, ws.perm, ws.segs_dev, ws.inter, ws.parts,
                                    self.shared_weights, shared_gate, ws.shared_inter, ws.shared_out, ws.split_ws,
                                    shared_inter_ready=shared_inter_ready())
+            elif merged:
+                ops.moe_ffn_prefill(self._experts_desc, x, ws.topv, ws.perm, ws.segs_dev, ws.inter, ws.parts,
+                                    self.shared_weights, shared_gate, ws.shared_inter, ws.shared_out)
             elif self.residency is None:
                 ops.grouped_swiglu(self._experts_desc, x, ws.topv, ws.perm, ws.segs_dev, ws.inter, ws.parts)
             else:

@@ -26,6 +26,7 @@ SOURCES = [
     "permute.hip",
     "swiglu_decode.hip",
     "swiglu_prefill.hip",
+    "swiglu_prefill_merged.hip",
     "ffn_tiled.hip",
     "ffn.hip",
     "combine.hip",
@@ -49,7 +50,8 @@ HIP_FLAGS = [
 # Kernels whose pipelines wait for a *counted* number of vector-memory operations.  A register
 # spill adds scratch loads and stores to that count, so a build in which one of these kernels
 # uses scratch memory is refused.
-NO_SCRATCH = {"swiglu_prefill.hip": ("prefill_ffn_kernel",)}
+NO_SCRATCH = {"swiglu_prefill.hip": ("prefill_ffn_kernel",),
+              "swiglu_prefill_merged.hip": ("prefill_merged_kernel",)}
 RESOURCE_REMARKS = "-Rpass-analysis=kernel-resource-usage"
 
 

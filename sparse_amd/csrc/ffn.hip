@@ -18,6 +18,10 @@ int decode_split_parts(int);
 int prefill_routed_bf16(const sparse_hip_experts*, const void*, const void*, const int32_t*, const int32_t*,
                         const sparse_hip_seglist*, int, int, void*, void*, void*, hipStream_t);
 size_t prefill_ws_bytes(int, int, int, int, int);
+size_t prefill_merged_ws_bytes(int, int, int, int, int, int);
+int prefill_merged(const sparse_hip_experts*, const void*, const void*, const int32_t*, const int32_t*,
+                   const sparse_hip_seglist*, int, int, void*, void*, const void*, const void*, const void*,
+                   const void*, int, void*, void*, void*, hipStream_t);
 int prefill_set_drain_waits(int);
 void prefill_set_clock_probe(void*);
 int prefill_shared_bf16(const void*, const void*, const void*, const void*, const void*, int, int, int, int, void*,
@@ -120,6 +124,46 @@ int sparse_hip_grouped_swiglu_prefill(const sparse_hip_experts* experts, const v
   }
   return tiled_routed<float>(experts, x_dev, topv_dev, perm_dev, seg_offsets_dev, segs, T, K, inter_ws_dev,
                              parts_dev, st);
+}
+
+size_t sparse_hip_moe_ffn_prefill_ws_bytes(int T, int K, int num_segments, int H, int I, int Is) {
+  if (T <= 0 || K <= 0 || num_segments < 0 || H <= 0 || I <= 0 || Is < 0) return 0;
+  return prefill_merged_ws_bytes(T, K, num_segments, H, I, Is);
+}
+
+int sparse_hip_moe_ffn_prefill(const sparse_hip_experts* experts, const void* x_dev, const void* topv_dev,
+                               const int32_t* perm_dev, const int32_t* seg_offsets_dev,
+                               const sparse_hip_seglist* segs, int T, int K, void* inter_ws_dev, void* parts_dev,
+                               const void* sh_gate_w_dev, const void* sh_up_w_dev, const void* sh_down_w_dev,
+                               const void* shared_gate_dev, int Is, void* sh_inter_ws_dev, void* shared_dev,
+                               void* tile_ws_dev, void* stream) {
+  int rc = check_routed("moe_ffn_prefill", experts, x_dev, topv_dev, perm_dev, seg_offsets_dev, segs, T, K,
+                        inter_ws_dev, parts_dev);
+  if (rc != SPARSE_HIP_OK) return rc;
+  SP_REQUIRE(is_16bit(experts->dtype), "moe_ffn_prefill: bf16 / fp16 only; use the separate entry points");
+  const bool shared = sh_down_w_dev != nullptr;
+  if (shared) {
+    SP_REQUIRE(Is > 0 && Is % 64 == 0, "moe_ffn_prefill: Is=%d must be a positive multiple of 64", Is);
+    SP_REQUIRE(sh_gate_w_dev && sh_up_w_dev && sh_inter_ws_dev && shared_dev,
+               "moe_ffn_prefill: NULL shared-expert pointer");
+    SP_REQUIRE(((reinterpret_cast<uintptr_t>(sh_gate_w_dev) | reinterpret_cast<uintptr_t>(sh_up_w_dev) |
+                 reinterpret_cast<uintptr_t>(sh_down_w_dev) | reinterpret_cast<uintptr_t>(sh_inter_ws_dev) |
+                 reinterpret_cast<uintptr_t>(shared_dev)) &
+                15) == 0,
+               "moe_ffn_prefill: shared-expert pointers must be 16-byte aligned");
+  }
+  SP_REQUIRE(tile_ws_dev != nullptr && (reinterpret_cast<uintptr_t>(tile_ws_dev) & 255) == 0,
+             "moe_ffn_prefill: tile workspace is NULL or not 256-byte aligned");
+  // lane offsets into an activation matrix are 32-bit byte counts
+  const uint64_t widest = static_cast<uint64_t>(experts->hidden > experts->inter ? experts->hidden : experts->inter);
+  SP_REQUIRE(static_cast<uint64_t>(T) * K * widest * 2 < (1ull << 32) &&
+                 static_cast<uint64_t>(T) * (shared ? static_cast<uint64_t>(Is > experts->hidden ? Is : experts->hidden) : 1) * 2 < (1ull << 32),
+             "moe_ffn_prefill: T=%d is too large for 32-bit row offsets; split the call", T);
+  SP_REQUIRE(static_cast<uint64_t>(T) * K < (1ull << 32) / static_cast<uint64_t>(K), "moe_ffn_prefill: T*K too large");
+  if (segs->n == 0 && !shared) return SPARSE_HIP_OK;
+  return prefill_merged(experts, x_dev, topv_dev, perm_dev, seg_offsets_dev, segs, T, K, inter_ws_dev, parts_dev,
+                        sh_gate_w_dev, sh_up_w_dev, sh_down_w_dev, shared_gate_dev, Is, sh_inter_ws_dev,
+                        shared_dev, tile_ws_dev, as_stream(stream));
 }
 
 int sparse_hip_moe_ffn_decode(const sparse_hip_experts* experts, const void* x_dev, const void* topv_dev,

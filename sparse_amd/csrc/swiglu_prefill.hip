@@ -36,24 +36,10 @@
 #include <type_traits>
 
 #include "common.h"
+#include "prefill_tiles.h"
 
 namespace sparse {
 
-constexpr int kPfBM = 128;        // rows per tile
-constexpr int kPfBR = 256;        // weight rows per tile
-constexpr int kPfBK = 64;         // k slab
-constexpr int kPfThreads = 256;
-constexpr int kPfRowBytes = kPfBK * 2;  // LDS row of one k slab (16-byte chunks swizzled by row)
-constexpr int kPfLdsA = kPfBM * kPfRowBytes;
-constexpr int kPfStages = 3;            // activation slabs resident in LDS
-constexpr int kPfXcds = 8;
-
-struct PfTile {
-  int32_t slot;  // weight slot of the segment's expert
-  int32_t r0;    // first permuted row of the tile
-  int32_t rows;  // rows in the tile (0: idle workgroup)
-  int32_t bn;    // column tile
-};
 
 struct PrefillArgs {
   const uint16_t* slab;
@@ -414,8 +400,9 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_ffn_kernel(const Prefil
   }
 }
 
-static std::atomic<int> g_prefill_drain_waits{0};
-static std::atomic<unsigned long long*> g_prefill_clock{nullptr};
+// also read by the persistent-workgroup form of this kernel
+std::atomic<int> g_prefill_drain_waits{0};
+std::atomic<unsigned long long*> g_prefill_clock{nullptr};
 
 void prefill_set_clock_probe(void* counters_dev) {
   g_prefill_clock.store(static_cast<unsigned long long*>(counters_dev));

@@ -537,6 +537,56 @@ def mfma_probe(from_lds: bool, iters: int = 20000, device="cuda:0") -> Tuple[flo
     return float(tflops.value), float(mhz.value)
 
 
+def moe_ffn_prefill(experts: Experts, x: torch.Tensor, topv: torch.Tensor, perm: Permutation, segs: SegList,
+                    inter_ws: torch.Tensor, parts: torch.Tensor, shared_w=None,
+                    shared_gate: Optional[torch.Tensor] = None, shared_inter_ws: Optional[torch.Tensor] = None,
+                    shared_out: Optional[torch.Tensor] = None, tile_ws: Optional[torch.Tensor] = None) -> None:
+    """Routed experts + shared expert of a prefill-size call as one launch per projection (bf16 or
+    fp16): routed and shared tiles share the launches' tails.  ``shared_w`` None: routed experts only;
+    an empty ``segs``: the shared expert only.  Bit-identical to ``grouped_swiglu`` + ``shared_expert``."""
+    lib = _lib.load()
+    T, H = x.shape
+    K = topv.shape[1]
+    _need_half(x, "x")
+    _need(topv, "topv", x.dtype, (T, K))
+    _need(inter_ws, "inter_ws", x.dtype, (T * K, experts.inter))
+    _need(parts, "parts", x.dtype, (T * K, H))
+    if H != experts.hidden:
+        raise ValueError(f"x has hidden {H}, the expert slab has {experts.hidden}")
+    Is = 0
+    gw = uw = dw = None
+    if shared_w is not None:
+        gw, uw, dw = shared_w
+        Is = gw.shape[0]
+        _need(gw, "shared gate_proj", x.dtype, (Is, H))
+        _need(uw, "shared up_proj", x.dtype, (Is, H))
+        _need(dw, "shared down_proj", x.dtype, (H, Is))
+        _need(shared_inter_ws, "shared inter_ws", x.dtype, (T, Is))
+        _need(shared_out, "shared out", x.dtype, (T, H))
+        if shared_gate is not None:
+            _need(shared_gate, "shared gate logits", x.dtype)
+            if shared_gate.numel() != T:
+                raise ValueError("shared gate logits must hold T elements")
+    if tile_ws is None:
+        tile_ws = moe_ffn_prefill_ws(T, K, experts.num_experts, H, experts.inter, Is, x.device)
+    rc = lib.sparse_hip_moe_ffn_prefill(C.byref(experts), _ptr(x), _ptr(topv), _ptr(perm.perm),
+                                        _ptr(perm.seg_offsets), C.byref(segs), T, K, _ptr(inter_ws), _ptr(parts),
+                                        _ptr(gw), _ptr(uw), _ptr(dw), _ptr(shared_gate), Is,
+                                        _ptr(shared_inter_ws), _ptr(shared_out), _ptr(tile_ws), _stream())
+    _lib.check(rc, "sparse_hip_moe_ffn_prefill")
+
+
+def moe_ffn_prefill_ws(T: int, K: int, num_segments: int, hidden: int, inter: int, shared_inter: int,
+                       device) -> torch.Tensor:
+    """Tile-queue workspace of ``moe_ffn_prefill``, cached per shape (launches on one stream reuse it
+    in order)."""
+    def make() -> torch.Tensor:
+        nbytes = _lib.load().sparse_hip_moe_ffn_prefill_ws_bytes(T, K, num_segments, hidden, inter, shared_inter)
+        return torch.empty((max(256, nbytes),), device=device, dtype=torch.uint8)
+
+    return _TILE_WS.get_or_make(("merged", T, K, num_segments, hidden, inter, shared_inter, str(device)), make)
+
+
 def moe_ffn_decode(experts: Experts, x: torch.Tensor, topv: torch.Tensor, perm: Permutation, segs: SegList,
                    inter_ws: torch.Tensor, parts: torch.Tensor, shared_w, shared_gate: Optional[torch.Tensor],
                    shared_inter_ws: torch.Tensor, shared_out: torch.Tensor,
