@@ -358,9 +358,10 @@ int sparse_hip_moe_ffn_decode(const sparse_hip_experts* experts, const void* x_d
  * (utils/eval_core.py:16520-16526, :14690-14721, :523-538, :9455-9463).  Needs
  * sparse_hip_decode_split_parts(Is) > 1.  `split_ws_dev` holds
  * sparse_hip_decode_split_ws_bytes(T, H) bytes: the partial sums, then, from
- * sparse_hip_decode_split_counter_offset(T, H) on, one int32 counter per tile, which must be
- * zero before the first call; every call leaves them zero.  Calls that share a workspace must
- * not overlap.  `parts_dev` is written as by sparse_hip_moe_ffn_decode.
+ * sparse_hip_decode_split_counter_offset(T, H) on, one int32 counter per tile.  The call's first
+ * launch puts the counters to zero, so the workspace may hold anything before (an earlier call with
+ * another T, a call that did not finish); a finished call leaves them at zero.  Calls that share a
+ * workspace must not overlap.  `parts_dev` is written as by sparse_hip_moe_ffn_decode.
  */
 size_t sparse_hip_decode_split_counter_offset(int T, int H);
 int sparse_hip_moe_ffn_decode_combine(const sparse_hip_experts* experts, const void* x_dev, const void* topv_dev,

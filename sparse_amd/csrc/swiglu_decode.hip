@@ -61,7 +61,12 @@ struct DecodeArgs {
   // combine folded into the down projection (needs split_s > 1): the workgroup that finishes a
   // 32-column tile last, counted per tile in `tile_counters`, sums that tile's columns of
   // every token over its K routed rows and the shared expert and writes `final_out`
-  int32_t* tile_counters;       // [Ndim / kDecRows], zero between launches; NULL: no combine here
+  int32_t* tile_counters;       // [Ndim / kDecRows], zero when the launch starts; NULL: no combine here
+  // gate/up launch of a call whose down launch combines: the counters to put to zero, so that the call
+  // does not depend on what an earlier call (another token count on the same workspace, a launch that
+  // did not finish) left there
+  int32_t* clear_counters;
+  int32_t n_clear;
   const int32_t* inv_perm;      // [T*K]
   uint16_t* final_out;          // [T, Ndim]
   sparse_hip_seglist segs;
@@ -96,6 +101,8 @@ __global__ __launch_bounds__(kDecThreads) void decode_ffn_kernel(const DecodeArg
   constexpr int kDecTiles = TL, kDecRows = TL * 16;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int r = lane & 15, q = lane >> 4;
+  if (kGateUp && a.clear_counters != nullptr && blockIdx.x == 0)   // before any workgroup of this launch can return
+    for (int i = threadIdx.x; i < a.n_clear; i += kDecThreads) a.clear_counters[i] = 0;
 
   // ---- which tile of which matrix ------------------------------------------
   const int split = kGateUp ? 1 : a.split_s;
@@ -423,6 +430,10 @@ __global__ __launch_bounds__(kDecThreads) void decode_ffn_kernel(const DecodeArg
   }
 }
 
+__global__ void decode_clear_kernel(int32_t* p, int n) {
+  for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) p[i] = 0;
+}
+
 template <bool kGateUp>
 static int launch_decode(const DecodeArgs& a0, int n_seg, hipStream_t st) {
   // A gate/up launch of up to 16 tokens whose 32-row workgroups would not all be resident at once (four
@@ -440,7 +451,13 @@ static int launch_decode(const DecodeArgs& a0, int n_seg, hipStream_t st) {
     a.tiles_s *= kDecTilesMax;
   }
   const int grid = a.tiles_s * (kGateUp ? 1 : a.split_s) + n_seg * a.tiles_r;
-  if (grid == 0) return SPARSE_HIP_OK;
+  if (grid == 0) {
+    if (kGateUp && a.clear_counters != nullptr) {   // nothing to project, but the counters are still this launch's job
+      hipLaunchKernelGGL(decode_clear_kernel, dim3(1), dim3(256), 0, st, a.clear_counters, a.n_clear);
+      SP_LAUNCH_CHECK("decode_clear_kernel");
+    }
+    return SPARSE_HIP_OK;
+  }
   ProfScope prof(kGateUp ? SPARSE_HIP_K_DECODE_GATEUP : SPARSE_HIP_K_DECODE_DOWN, st, /*dispatch_events=*/true);
 #define SP_DEC_LAUNCH(F, NT, TL)                                                                              \
   do {                                                                                                       \
@@ -499,6 +516,8 @@ int decode_routed_bf16(const sparse_hip_experts* ex, const void* x, const void* 
   return launch_decode<false>(a, segs->n, st);
 }
 
+size_t decode_split_counter_offset(int T, int H);
+
 // Routed experts and the shared expert in one launch pair, 16-bit formats, T <= 32.  The shared
 // expert's tiles lead the grid (largest, known amount of work), routed segments follow.
 int decode_fused_bf16(const sparse_hip_experts* ex, const void* x, const void* topv, const int32_t* perm,
@@ -534,8 +553,14 @@ int decode_fused_bf16(const sparse_hip_experts* ex, const void* x, const void* t
   a.Ndim_s = Is;
   // no gate / up matrices: sh_inter_ws already holds the shared expert's SiLU(gate x) * (up x)
   a.tiles_s = sh_gate_w != nullptr ? Is / kDecRowsMax : 0;
+  const bool split = split_ws != nullptr && (Is / 64) % kDecSplit == 0;
+  if (split && final_out != nullptr) {   // the down launch below combines: its arrival counters start at zero
+    a.clear_counters = reinterpret_cast<int32_t*>(static_cast<uint8_t*>(split_ws) + decode_split_counter_offset(T, static_cast<int>(H)));
+    a.n_clear = (static_cast<int>(H) + 15) / 16;
+  }
   int rc = launch_decode<true>(a, segs->n, st);
   if (rc != SPARSE_HIP_OK) return rc;
+  a.clear_counters = nullptr;
   // down
   a.mat_offset = 2 * I * H;
   a.mat2_offset = 0;
@@ -556,7 +581,7 @@ int decode_fused_bf16(const sparse_hip_experts* ex, const void* x, const void* t
   // The shared down projection reduces over Is, several times the routed experts' I: as one
   // workgroup per tile it would still be streaming when everything else has finished.  With a
   // workspace it is cut into kDecSplit parts whose fp32 sums the combine step adds up.
-  if (split_ws != nullptr && (Is / 64) % kDecSplit == 0) {
+  if (split) {
     a.split_s = kDecSplit;
     a.split_sums = static_cast<float*>(split_ws);
     if (final_out != nullptr) {  // the per-tile arrival counters follow the partial sums in the workspace

@@ -188,3 +188,28 @@ def test_workspace_tables_are_bounded():
     from sparse_amd import ops
     from sparse_amd.block import _Workspace
     assert isinstance(_Workspace._cache, LruTable) and isinstance(ops._TILE_WS, LruTable)
+
+
+def test_workspace_used_under_graph_capture_is_never_dropped():
+    """A captured graph holds raw pointers into a workspace and no reference: an entry that was
+    looked up while the stream was capturing stays, whatever else is used afterwards."""
+    from sparse_amd._lru import LruTable
+    capturing = [False]
+    table = LruTable(2, capturing=lambda: capturing[0])
+    table.get_or_make("a", object)
+    capturing[0] = True
+    held = table.get_or_make("graph", object)          # looked up during capture: pinned
+    assert table.get_or_make("a", lambda: pytest.fail("held")) is not None and table.pinned() == {"graph", "a"}
+    capturing[0] = False
+    for key in range(10):                                # eager shapes come and go
+        table.get_or_make(key, object)
+    assert "graph" in table and "a" in table
+    assert table.get_or_make("graph", lambda: pytest.fail("a pinned entry was dropped")) is held
+    # pinned entries do not count against the limit: the two most recent eager shapes are still there
+    assert [k for k in table.keys() if k not in ("graph", "a")] == [8, 9]
+    table.pin(9)
+    table.get_or_make(10, object)
+    table.get_or_make(11, object)
+    assert 9 in table and 8 not in table
+    table.clear()
+    assert len(table) == 0 and table.pinned() == set()

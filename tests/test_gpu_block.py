@@ -421,3 +421,27 @@ def test_decode_stack_in_a_hip_graph_replays_like_eager(device, T):
         torch.cuda.synchronize()
         for got, ref in zip(captured, want):
             assert torch.equal(got, ref), (T, i)
+
+
+def test_folded_combine_does_not_depend_on_what_the_workspace_held(device):
+    """The arrival counters of the folded combine sit behind the partial sums, at an offset that depends
+    on the token count.  A workspace sized and used for 16 tokens, then reused for 3, puts the counters
+    of the second call on top of stale partial sums -- and a workspace may hold anything at all before its
+    first call.  Every call clears its own counters first, so both give the bits of the separate combine."""
+    from sparse_amd import ops
+    from sparse_amd.synthetic import make_hidden
+    shape = dict(family="qwen_shared", hidden=512, num_experts=12, inter=256, top_k=4, shared_inter=1024)
+    _mlp, blk = _build(shape, torch.bfloat16, device, seed=3)
+    H, K = shape["hidden"], shape["top_k"]
+    big = ops.decode_split_workspace(16, H, device)
+    big.view(torch.int32).fill_(0x7F7F7F7F)          # garbage, also where any counter could be
+    for i, T in enumerate((16, 3, 16, 1)):
+        x = make_hidden(T, H, torch.bfloat16, seed=4100 + i).view(T, 1, H).to(device)
+        blk.fold_combine = False
+        want, _ = blk(x)                                # routes, and leaves topv / perm of this call in ws
+        ws = blk._workspace(T)
+        got = torch.empty_like(want).view(T, H)
+        ops.moe_ffn_decode_combine(blk._experts_desc, x.view(T, H), ws.topv, ws.perm, ws.segs_dev, ws.inter,
+                                   ws.parts, blk.shared_weights, ws.shared_gate, ws.shared_inter, big, got)
+        torch.cuda.synchronize()
+        assert torch.equal(got.view_as(want), want), f"T={T}"
