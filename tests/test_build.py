@@ -61,20 +61,23 @@ def _hot_loops(asm: str, kernel_prefix: str):
     return [(n, b) for n, b in loops if sum(i.startswith("v_mfma") for i in b) >= 16]
 
 
-def test_prefill_k_loop_issues_its_vector_memory_operations_as_the_counted_wait_assumes(tmp_path):
+@pytest.mark.parametrize("source,prefix", [("swiglu_prefill.hip", "_ZN6sparse18prefill_ffn_kernel"),
+                                           ("swiglu_prefill_merged.hip", "_ZN6sparse21prefill_merged_kernel")])
+def test_prefill_k_loop_issues_its_vector_memory_operations_as_the_counted_wait_assumes(tmp_path, source, prefix):
     """The prefill kernel waits for "all but the 20 newest" vector memory operations before the barrier that
     closes a k slab.  That is exact only if every slab issues, in this order, the 4 LDS copies of the slab
     after next and then 8 fragment loads, and nothing else that the counter counts (no scratch traffic, no
-    other global access).  Checked on the compiler's output for the counted-wait kernels."""
+    other global access).  Checked on the compiler's output for the counted-wait kernels
+    (the one-tile-per-workgroup form and the merged routed + shared form)."""
     import re
     import subprocess
     hipcc = build._hipcc()
     out = tmp_path / "prefill.s"
     cmd = [hipcc, *[f for f in build.HIP_FLAGS if f not in ("-fPIC",)], f"-I{build.INCLUDE}", f"-I{build.CSRC}", "-S",
-           "--cuda-device-only", str(build.CSRC / "swiglu_prefill.hip"), "-o", str(out)]
+           "--cuda-device-only", str(build.CSRC / source), "-o", str(out)]
     proc = subprocess.run(cmd, capture_output=True, text=True)
     assert proc.returncode == 0, proc.stderr[-2000:]
-    loops = _hot_loops(out.read_text(), "_ZN6sparse18prefill_ffn_kernel")
+    loops = _hot_loops(out.read_text(), prefix)
     # counted-wait variants only: the last template argument (kDrainWaits) is false
     loops = [(n, b) for n, b in loops if re.search(r"ELb[01]ELb0EEEv", n)]
     assert len(loops) >= 8          # bf16 and fp16, gate/up and down, several tile heights each

@@ -442,6 +442,38 @@ def test_folded_combine_does_not_depend_on_what_the_workspace_held(device):
         ws = blk._workspace(T)
         got = torch.empty_like(want).view(T, H)
         ops.moe_ffn_decode_combine(blk._experts_desc, x.view(T, H), ws.topv, ws.perm, ws.segs_dev, ws.inter,
-                                   ws.parts, blk.shared_weights, ws.shared_gate, ws.shared_inter, big, got)
+                                   ws.parts, blk.shared_weights, ws.shared_gate, ws.shared_inter, big, got,
+                                   shared_inter_ready=True)   # the routing launch of blk(x) left it there
         torch.cuda.synchronize()
         assert torch.equal(got.view_as(want), want), f"T={T}"
+
+
+@pytest.mark.parametrize("T", [17, 24, 32])
+def test_folded_combine_above_sixteen_tokens_through_the_c_entry(device, T):
+    """The block folds the combine only for calls of up to 16 tokens; the entry point takes up to 32.
+    Against the split down projection followed by the separate combine launch: the same bits."""
+    from sparse_amd import ops
+    from sparse_amd.synthetic import make_hidden
+    shape = dict(family="qwen_shared", hidden=512, num_experts=12, inter=256, top_k=4, shared_inter=1024)
+    _mlp, blk = _build(shape, torch.bfloat16, device, seed=7)
+    H, K = shape["hidden"], shape["top_k"]
+    split_ws = ops.decode_split_workspace(T, H, device)
+    nparts = ops.decode_split_parts(shape["shared_inter"])
+    assert nparts > 1
+    for i in range(3):
+        x = make_hidden(T, H, torch.bfloat16, seed=4200 + i).view(T, 1, H).to(device)
+        blk(x)                                          # routing of this call stays in the workspace
+        ws = blk._workspace(T)
+        x2 = x.view(T, H)
+        # (both calls compute the shared expert's gate and up projections themselves, the same way)
+        ops.moe_ffn_decode(blk._experts_desc, x2, ws.topv, ws.perm, ws.segs_dev, ws.inter, ws.parts,
+                           blk.shared_weights, ws.shared_gate, ws.shared_inter, ws.shared_out, split_ws)
+        want = torch.empty((T, H), device=device, dtype=torch.bfloat16)
+        ops.combine_split(ws.parts, ws.perm, split_ws, nparts, ws.shared_gate, T, K, want)
+        parts_a = ws.parts.clone()
+        got = torch.empty_like(want)
+        ops.moe_ffn_decode_combine(blk._experts_desc, x2, ws.topv, ws.perm, ws.segs_dev, ws.inter, ws.parts,
+                                   blk.shared_weights, ws.shared_gate, ws.shared_inter, split_ws, got)
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), f"call {i}"
+        assert torch.equal(parts_a, ws.parts)

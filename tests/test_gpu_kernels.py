@@ -623,6 +623,92 @@ def test_tile_weight_kernel_matches_host_packing(device, dtype):
 
 
 # ------------------------------------------------------------------ shared expert + combine
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("H,E,I,K,Is,T,gated", [
+    (512, 12, 256, 4, 384, 300, True),        # 8 / 4 / 6 k slabs, ragged segments
+    (2048, 60, 1408, 4, 5632, 700, True),     # the Qwen shape
+    (2048, 64, 1408, 6, 2816, 1100, False),   # the DeepSeek shape: more tiles than one round of the grid
+    (320, 6, 192, 2, 448, 200, False),        # odd slab counts (5, 3, 7), column tiles that end inside a group
+    (64, 3, 64, 1, 64, 129, True),            # one slab, one column tile, K = 1
+])
+def test_merged_prefill_equals_the_separate_calls(device, dtype, H, E, I, K, Is, T, gated):
+    """Routed experts and shared expert of a prefill-size call as one launch per projection
+    (``sparse_hip_moe_ffn_prefill``) against ``grouped_swiglu`` + ``shared_expert``: the same bits in the
+    routed rows, the routed intermediate, the shared intermediate and the shared output; with the routed
+    experts alone and with the shared expert alone; counted waits against full drains."""
+    from sparse_amd import _lib
+    from sparse_amd.weights import ExpertSlab, tile_weight
+    ops = _ops()
+    lib = _lib.load()
+    layer = make_layer(H, E, I, K, Is=Is, shared_gate=gated, dtype=dtype, seed=71 + H, std=0.05)
+    x = make_hidden(T, H, dtype, seed=72 + T)
+    g = torch.Generator().manual_seed(73)
+    popularity = 1.0 / torch.arange(1, E + 1, dtype=torch.float32) ** 1.1
+    if E > 3:
+        popularity[E - 1] = 0.0                                               # an expert nobody routes to
+    topi = torch.multinomial(popularity.expand(T, E), K, replacement=False, generator=g)
+    topv = torch.rand(T, K, generator=g).to(dtype)
+    slab = ExpertSlab.resident(layer["experts"], H, I, dtype, device)
+    ex = ops.make_experts(slab.data, slab.expert_slot, E, H, I)
+    xd, tvd = x.to(device), topv.to(device)
+    perm = ops.permute_build(topi.to(device), E)
+    segs = ops.seglist_device(perm, min(E, T * K))
+    gw, uw, dw = (tile_weight(t.to(device)).reshape(t.shape).contiguous() for t in layer["shared"])
+    sg = None
+    if gated:
+        sg = torch.nn.functional.linear(x.float(), layer["shared_gate_w"].float().reshape(1, -1)).reshape(-1)
+        sg = sg.to(dtype).to(device)
+
+    def fresh():
+        return (torch.zeros((T * K, I), device=device, dtype=dtype), torch.zeros((T * K, H), device=device, dtype=dtype),
+                torch.zeros((T, Is), device=device, dtype=dtype), torch.zeros((T, H), device=device, dtype=dtype))
+
+    want = fresh()
+    ops.grouped_swiglu(ex, xd, tvd, perm, segs, want[0], want[1], decode=False)
+    ops.shared_expert(xd, gw, uw, dw, sg, want[2], want[3])
+    names = ("routed intermediate", "routed rows", "shared intermediate", "shared output")
+
+    def merged(shared=True, routed=True):
+        got = fresh()
+        ops.moe_ffn_prefill(ex, xd, tvd, perm, segs if routed else ops.seglist_host([], []), got[0], got[1],
+                            (gw, uw, dw) if shared else None, sg, got[2] if shared else None,
+                            got[3] if shared else None)
+        torch.cuda.synchronize()
+        return got
+
+    got = merged()
+    for a, b, what in zip(got, want, names):
+        assert torch.equal(a, b), what
+    assert float(got[1].float().abs().max()) > 0 and float(got[3].float().abs().max()) > 0
+    only_routed = merged(shared=False)
+    assert torch.equal(only_routed[0], want[0]) and torch.equal(only_routed[1], want[1])
+    assert int(only_routed[3].abs().sum()) == 0
+    only_shared = merged(routed=False)
+    assert torch.equal(only_shared[2], want[2]) and torch.equal(only_shared[3], want[3])
+    assert int(only_shared[1].abs().sum()) == 0
+    assert lib.sparse_hip_prefill_drain_waits(1) == 0
+    try:
+        safe = merged()
+    finally:
+        assert lib.sparse_hip_prefill_drain_waits(0) == 1
+    for a, b, what in zip(safe, want, names):
+        assert torch.equal(a, b), f"{what}: counted waits and full drains differ"
+
+
+def test_merged_prefill_rejects_bad_arguments(device):
+    ops = _ops()
+    from sparse_amd._lib import SparseHipError
+    from sparse_amd.weights import ExpertSlab
+    layer = make_layer(128, 4, 64, 2, Is=64, dtype=torch.float32, seed=5)
+    slab = ExpertSlab.resident(layer["experts"], 128, 64, torch.float32, device)
+    ex = ops.make_experts(slab.data, slab.expert_slot, 4, 128, 64)
+    x = make_hidden(40, 128, torch.float32).to(device)
+    with pytest.raises((SparseHipError, ValueError)):       # fp32 takes the separate entry points
+        perm = ops.permute_build(torch.zeros((40, 2), dtype=torch.int64, device=device), 4)
+        ops.moe_ffn_prefill(ex, x, torch.ones((40, 2), device=device), perm, ops.seglist_device(perm, 4),
+                            torch.zeros((80, 64), device=device), torch.zeros((80, 128), device=device))
+
 @pytest.mark.parametrize("dtype,T", [(torch.bfloat16, 8), (torch.bfloat16, 32), (torch.bfloat16, 200),
                                      (torch.bfloat16, 2048), (torch.bfloat16, 2500),   # XCDs own bands of M-tiles
                                      (torch.float32, 8), (torch.float32, 100)])
