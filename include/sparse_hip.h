@@ -39,7 +39,7 @@
 extern "C" {
 #endif
 
-#define SPARSE_HIP_ABI_VERSION 2
+#define SPARSE_HIP_ABI_VERSION 3
 
 #define SPARSE_HIP_F32 0
 #define SPARSE_HIP_BF16 1
@@ -144,6 +144,27 @@ int sparse_hip_gate_topk(const void* logits_dev, int logits_dtype, int T, int E,
 int sparse_hip_gate_topk_grouped(const void* logits_dev, int logits_dtype, int T, int E, int K,
                                  int renorm, int n_group, int topk_group, int out_dtype,
                                  void* topv_dev, int64_t* topi_dev, void* stream);
+
+/*
+ * The same with the two things the DeepSeek branch of `_routing_router` does after the gate
+ * (utils/eval_core.py:9503-9517, :9490-9499) in the same launch: the weights are multiplied by the
+ * gate's routed scaling factor `scale` in fp32 before their one rounding to `out_dtype` (as the gate
+ * module multiplies before the reference casts), and, where `pseudo_logits_dev` [T,E] fp32 is not
+ * NULL, it receives -inf everywhere but at the selected experts, which hold
+ * log(max(weight as rounded, 1e-12)).  scale == 1 and NULL give sparse_hip_gate_topk_grouped.
+ */
+int sparse_hip_gate_topk_scaled(const void* logits_dev, int logits_dtype, int T, int E, int K,
+                                int renorm, int n_group, int topk_group, float scale, int out_dtype,
+                                void* topv_dev, int64_t* topi_dev, float* pseudo_logits_dev, void* stream);
+
+/*
+ * Pseudo logits of a routing that is given rather than computed: out [T,E] fp32 = `fill` everywhere
+ * but at topi[t, k], which holds log(max(topv[t, k], eps)) -- what `_routing_for_execute` returns when
+ * a layer executes its predecessor's prediction (utils/eval_core.py:11137-11155, fill -1e9, eps from the
+ * block's rs_prob_to_logit_eps) and what :9490-9499 builds (fill -inf, eps 1e-12).  topv in `dtype`.
+ */
+int sparse_hip_pseudo_logits(const void* topv_dev, int dtype, const int64_t* topi_dev, int T, int K, int E,
+                             float eps, float fill, float* out_dev, void* stream);
 
 /*
  * Top-K of each row of given probabilities, no softmax: values descending, ties to the lower
@@ -403,7 +424,8 @@ int sparse_hip_combine_split(const void* parts_dev, const int32_t* inv_perm_dev,
  * pred[T, E] = softmax(w2 relu(w1 float(x) + b1) + b2): the forward pass of the reference's
  * `RoutingScoutMLP` in eval mode (utils/eval_core.py:3402-3417: Linear, BatchNorm1d, ReLU, Dropout,
  * Linear, Softmax) as `_compute_and_schedule_next_layer_rs` runs it on the layer's input
- * (:10916-10960, `rs_in = x.float()`), for a decode-size call (T <= SPARSE_HIP_DECODE_MAX_TOKENS).
+ * (:10916-10960, `rs_in = x.float()`), for any number of token rows (a workgroup takes
+ * SPARSE_HIP_DECODE_MAX_TOKENS of them).
  * All parameters are fp32 and row-major; the caller folds the BatchNorm's running statistics and affine
  * into w1 [D, H] and b1 [D] once, at load time (eval mode makes it a per-row scale and shift; Dropout is
  * the identity).  x is [T, H] in `dtype`; hidden_ws_dev holds T * D floats; w2 is [E, D].  Two launches.
@@ -411,6 +433,31 @@ int sparse_hip_combine_split(const void* parts_dev, const int32_t* inv_perm_dev,
 int sparse_hip_rs_predict(const void* x_dev, int dtype, int T, int H, const float* w1_dev, const float* b1_dev,
                           int D, const float* w2_dev, const float* b2_dev, int E, float* hidden_ws_dev,
                           float* pred_dev, void* stream);
+
+/*
+ * The pieces of the deeper predictor, `RoutingScoutResidualMLP` in eval mode
+ * (utils/eval_core.py:3419-3461: LayerNorm, Linear, GELU; units of x + Linear(GELU(Linear(LayerNorm(x))));
+ * LayerNorm, Linear, softmax) and of predictors that also read the layer's routing (:10903-10914), which
+ * the host strings together; fp32 arithmetic and fp32 row-major parameters throughout.
+ *
+ * sparse_hip_rs_dense:     out[T, D] = act(x[T, H] w[D, H]^T + b[D]) (+ residual[T, D] when not NULL), with
+ *                          act 0 = none, 1 = ReLU, 2 = GELU in its exact (erf) form; x in `dtype`, H a
+ *                          multiple of 8 (pad rows and weight columns with zeros otherwise).
+ * sparse_hip_rs_layernorm: out[t, :H] = (x[t, :H] - mean) / sqrt(var + eps) * gamma + beta with the biased
+ *                          variance, as nn.LayerNorm; rows of x are ld_in elements apart, rows of out
+ *                          ld_out, and out[t, H:ld_out] is set to zero.
+ * sparse_hip_rs_features:  out[t, :] = [ float(x[t, :H]) | feat[t, :E] | zeros up to ld ], where feat holds
+ *                          the token's K routing weights divided by max(their sum, 1e-12) at its K expert
+ *                          ids (`idx`/`w` of :10903-10908; ids outside [0, E) are skipped).
+ * sparse_hip_rs_softmax:   out[t, :] = softmax(in[t, :E]).
+ */
+int sparse_hip_rs_dense(const void* x_dev, int dtype, int T, int H, const float* w_dev, const float* b_dev, int D,
+                        int act, const float* residual_dev, float* out_dev, void* stream);
+int sparse_hip_rs_layernorm(const void* x_dev, int dtype, int T, int H, int ld_in, int ld_out,
+                            const float* gamma_dev, const float* beta_dev, float eps, float* out_dev, void* stream);
+int sparse_hip_rs_features(const void* x_dev, int dtype, int T, int H, const int32_t* topi_dev,
+                           const void* topv_dev, int K, int E, int ld, float* out_dev, void* stream);
+int sparse_hip_rs_softmax(const float* in_dev, int T, int E, float* out_dev, void* stream);
 
 /* ---- A11/A12/A13: expert residency ----------------------------------------- */
 

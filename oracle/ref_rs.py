@@ -7,6 +7,12 @@ import this.
 as identity, Linear, Softmax) in numpy float32.  Pinned by closed form against
 ``torch.nn`` layers with the same parameters (tests/test_residency.py).
 
+``routing_scout_residual_forward`` restates ``RoutingScoutResidualMLP.forward`` in eval mode
+(utils/eval_core.py:3419-3461: LayerNorm, Linear, GELU; units ``x + Linear(GELU(Linear(LayerNorm(x))))``;
+LayerNorm, Linear, softmax) in numpy float32.  Pinned against ``torch.nn.LayerNorm`` / ``nn.GELU`` /
+``nn.Linear`` stacks holding the same parameters, and by hand-made cases (a unit whose second Linear is
+zero is the identity; constant rows normalise to the LayerNorm's bias) in tests/test_rs_fused.py.
+
 ``select_candidates`` restates utils/rs_staging.py:97-118, the staging adapter's scoring
 (the same formula as utils/eval_core.py:10104-10106).  Pinned by the reference's own
 known-answer tests, tests/test_rs_staging.py:147-150 and :308-312.
@@ -28,6 +34,35 @@ def routing_scout_forward(x: np.ndarray, w1, b1, bn_weight, bn_bias, bn_mean, bn
     h = (h - bn_mean) / np.sqrt(np.asarray(bn_var, np.float32) + eps) * bn_weight + bn_bias
     h = np.maximum(h, 0.0)
     z = h @ np.asarray(w2, np.float32).T + np.asarray(b2, np.float32)
+    z = z - z.max(axis=-1, keepdims=True)
+    e = np.exp(z)
+    return (e / e.sum(axis=-1, keepdims=True)).astype(np.float32)
+
+
+def _layer_norm(x: np.ndarray, weight, bias, eps: float) -> np.ndarray:
+    mean = x.mean(axis=-1, keepdims=True, dtype=np.float32)
+    var = np.square(x - mean).mean(axis=-1, keepdims=True, dtype=np.float32)      # biased, as nn.LayerNorm
+    return ((x - mean) / np.sqrt(var + np.float32(eps)) * np.asarray(weight, np.float32)
+            + np.asarray(bias, np.float32)).astype(np.float32)
+
+
+def _gelu(x: np.ndarray) -> np.ndarray:
+    from scipy.special import erf
+    return (0.5 * x * (1.0 + erf(x.astype(np.float64) / np.sqrt(2.0)))).astype(np.float32)    # nn.GELU's default
+
+
+def _linear(x: np.ndarray, weight, bias) -> np.ndarray:
+    return (x @ np.asarray(weight, np.float32).T + np.asarray(bias, np.float32)).astype(np.float32)
+
+
+def routing_scout_residual_forward(x: np.ndarray, stem, units, out_norm, head, eps: float = 1e-5) -> np.ndarray:
+    """``stem = (ln_weight, ln_bias, w, b)``; ``units`` = list of ``(ln_weight, ln_bias, w_up, b_up, w_down,
+    b_down)``; ``out_norm = (ln_weight, ln_bias)``; ``head = (w, b)``.  Returns ``[T, E]`` probabilities."""
+    h = np.asarray(x, np.float32)
+    h = _gelu(_linear(_layer_norm(h, stem[0], stem[1], eps), stem[2], stem[3]))
+    for ln_w, ln_b, w_up, b_up, w_down, b_down in units:
+        h = (h + _linear(_gelu(_linear(_layer_norm(h, ln_w, ln_b, eps), w_up, b_up)), w_down, b_down)).astype(np.float32)
+    z = _linear(_layer_norm(h, out_norm[0], out_norm[1], eps), head[0], head[1])
     z = z - z.max(axis=-1, keepdims=True)
     e = np.exp(z)
     return (e / e.sum(axis=-1, keepdims=True)).astype(np.float32)

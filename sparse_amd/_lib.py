@@ -17,7 +17,7 @@ MAX_EXPERTS = 256
 MAX_TOPK = 16
 DECODE_MAX_TOKENS = 32
 ENOTREADY = 1
-ABI_VERSION = 2
+ABI_VERSION = 3
 PERMUTE_STATIC_MAX_TOKENS = 65536
 
 
@@ -65,6 +65,8 @@ SIGNATURES = {
     "sparse_hip_router_logits": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _vp, _vp]),
     "sparse_hip_gate_topk": (_i, [_vp, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp]),
     "sparse_hip_gate_topk_grouped": (_i, [_vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp]),
+    "sparse_hip_gate_topk_scaled": (_i, [_vp, _i, _i, _i, _i, _i, _i, _i, C.c_float, _i, _vp, _vp, _vp, _vp]),
+    "sparse_hip_pseudo_logits": (_i, [_vp, _i, _vp, _i, _i, _i, C.c_float, C.c_float, _vp, _vp]),
     "sparse_hip_topk": (_i, [_vp, _i, _i, _i, _i, _i, _vp, _vp, _vp]),
     "sparse_hip_route_decode": (
         _i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
@@ -113,6 +115,10 @@ SIGNATURES = {
     "sparse_hip_tile_weight": (_i, [_vp, _vp, _i, _i, _i, _i, _vp]),
     "sparse_hip_calib_copy": (_i, [_vp, _vp, _sz, _vp]),
     "sparse_hip_rs_predict": (_i, [_vp, _i, _i, _i, _vp, _vp, _i, _vp, _vp, _i, _vp, _vp, _vp]),
+    "sparse_hip_rs_dense": (_i, [_vp, _i, _i, _i, _vp, _vp, _i, _i, _vp, _vp, _vp]),
+    "sparse_hip_rs_layernorm": (_i, [_vp, _i, _i, _i, _i, _i, _vp, _vp, C.c_float, _vp, _vp]),
+    "sparse_hip_rs_features": (_i, [_vp, _i, _i, _i, _vp, _vp, _i, _i, _i, _vp, _vp]),
+    "sparse_hip_rs_softmax": (_i, [_vp, _i, _i, _vp, _vp]),
     "sparse_hip_prefill_drain_waits": (_i, [_i]),
     "sparse_hip_prefill_clock_probe": (_i, [_vp]),
     "sparse_hip_mfma_probe": (_i, [_i, _i, _vp, C.POINTER(C.c_double), C.POINTER(C.c_double), _vp]),

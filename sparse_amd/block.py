@@ -274,6 +274,17 @@ class DistributedSparseMoeBlock(nn.Module):
             raise NotImplementedError(f"oracle_mode={oracle_mode} (record / replay traces) is not built")
         self.oracle_mode = "none"
         self.expert_offload = str(expert_offload)
+        # Read and validated as the reference does (:4795-4798).  Both settings are satisfied by
+        # construction here: "fixed64" asks for a prefill summation order that does not depend on where a
+        # row sits in its expert's batch or on how many rows that batch has, per-row decode granularity for
+        # the same of a decode call -- the prefill-size kernels and the decode-size kernels each reduce every
+        # output element over k in one fixed order (64-wide slabs in sequence, the same MFMA sequence inside
+        # a slab), whatever the row's position and whoever shares its tile.
+        self._native_decode_granularity = str(os.environ.get("SPARSE_EP_NATIVE_DECODE_GRANULARITY", "0")).strip().lower() \
+            not in ("0", "false", "no", "off")
+        self._prefill_expert_math = str(os.environ.get("SPARSE_PREFILL_EXPERT_MATH", "native")).strip().lower()
+        if self._prefill_expert_math not in ("native", "fixed64"):
+            raise ValueError("SPARSE_PREFILL_EXPERT_MATH must be native or fixed64")
         if self.expert_offload not in ("cpu", "gpu"):
             raise ValueError(f"expert_offload must be cpu|gpu, got {self.expert_offload}")
         self.cache_policy = str(cache_policy).lower()
@@ -454,10 +465,10 @@ class DistributedSparseMoeBlock(nn.Module):
         ops.router_logits(x, self.gate_weight, self.shared_gate_weight, self.logits_dtype, out=logits,
                           shared_gate_out=shared_gate)
         after_logits()
+        # the routed scaling factor multiplies in fp32 inside the top-k launch, before the one rounding to
+        # the activation dtype, as the gate module does before the reference's cast (:9509-9513)
         ops.gate_topk(logits, self.top_k, self.norm_topk_prob, out_dtype=self.dtype, topv=ws.topv, topi=ws.topi,
-                      n_group=self.n_group, topk_group=self.topk_group)
-        if self.routed_scaling_factor != 1.0:
-            ws.topv.mul_(self.routed_scaling_factor)
+                      n_group=self.n_group, topk_group=self.topk_group, scale=self.routed_scaling_factor)
         ops.permute_build(ws.topi, self.num_experts, out=ws.perm)
         return logits
 
@@ -476,17 +487,14 @@ class DistributedSparseMoeBlock(nn.Module):
             # the shared expert's gate comes out of the router-logits kernel; the logits are unused
             ops.router_logits(x, self.gate_weight, self.shared_gate_weight, self.logits_dtype,
                               shared_gate_out=ws.shared_gate)
-        logits = torch.full((T, self.num_experts), -1e9, device=x.device, dtype=torch.float32)
-        logits.scatter_(1, ws.topi, ws.topv.float().clamp_min(self.rs_prob_to_logit_eps).log())
-        return logits
+        return ops.pseudo_logits(ws.topv, ws.topi, self.num_experts, eps=self.rs_prob_to_logit_eps, fill=-1e9)
 
     def _routing_router(self, x: torch.Tensor):
         """``(topv, topi, router_logits)`` like the reference's method (:9502-9595)."""
         ws = self._workspace(int(x.shape[0]))
         logits = self._route(x.contiguous(), ws)
         if self.moe_family == "deepseek_shared":
-            logits = torch.full_like(logits, float("-inf"), dtype=torch.float32)
-            logits.scatter_(1, ws.topi, ws.topv.float().clamp_min(1e-12).log())
+            logits = ops.pseudo_logits(ws.topv, ws.topi, self.num_experts, eps=1e-12, fill=float("-inf"))
         return ws.topv, ws.topi, logits
 
     # ------------------------------------------------------------------ RS prefetch
@@ -534,18 +542,19 @@ class DistributedSparseMoeBlock(nn.Module):
             policy.window_ms = here.compute(self.top_k, int(x.shape[0]) * self.top_k) + policy.cost.attention
         mode = self._next_layer_rs_feature_mode()
         module = SparseContext.rs_bank[target]
-        fused = fused_scout(module, x) if mode == "hidden" else None
+        if mode not in ("hidden", "hidden_router_topk"):
+            raise RuntimeError(f"Unsupported next-layer RS feature_mode={mode}")
+        if mode == "hidden_router_topk" and source is None:
+            return None
+        fused = fused_scout(module, x, mode, self.num_experts)
         if fused is not None:
-            # decode-size call of the plain predictor: two HIP launches on the token rows as they are
-            pred = fused(x)
+            # HIP predictor on the token rows as they are (after one launch that appends the routing
+            # columns, for predictors that read them)
+            pred = fused(x if mode == "hidden" else ops.rs_features(x, source[0], source[1], self.num_experts))
         else:
             rs_in = x.float()
             if mode == "hidden_router_topk":
-                if source is None:
-                    return None
                 rs_in = torch.cat([rs_in, router_topk_feature(source[0], source[1], self.num_experts)], dim=-1)
-            elif mode != "hidden":
-                raise RuntimeError(f"Unsupported next-layer RS feature_mode={mode}")
             pred = module(rs_in).to(torch.float32)
         self.metrics.rs_next_layer_pred_calls += 1
         self.metrics.rs_mlp_calls += 1

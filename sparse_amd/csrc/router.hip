@@ -199,7 +199,8 @@ constexpr int kTopkNV = SPARSE_HIP_MAX_EXPERTS / 64;
 template <typename TL, typename TO>
 __device__ __forceinline__ int topk_token(const TL* __restrict__ row, int E, int K, int renorm,
                                           TO* __restrict__ topv_row, int64_t* __restrict__ topi_row, int lane,
-                                          int n_group = 0, int topk_group = 0, bool softmax = true) {
+                                          int n_group = 0, int topk_group = 0, bool softmax = true,
+                                          float scale = 1.f, float* __restrict__ pseudo_row = nullptr) {
   float key[kTopkNV];  // what is ranked: the logit (-inf once masked by the group limit)
   unsigned alive = 0u;  // bit j: expert lane + 64*j exists and has not been selected yet
   float m = -INFINITY;
@@ -281,11 +282,21 @@ __device__ __forceinline__ int topk_token(const TL* __restrict__ row, int E, int
     }
     sum_sel += pv;
   }
+  if (pseudo_row != nullptr) {
+    // pseudo logits (utils/eval_core.py:9490-9499): -inf everywhere but at the selected experts
+#pragma unroll
+    for (int j = 0; j < kTopkNV; ++j)
+      if (lane + 64 * j < E) pseudo_row[lane + 64 * j] = -INFINITY;
+  }
   if (lane < K) {
     float v = sel_v;
     if (renorm) v = v / fmaxf(sum_sel, 1e-12f);
+    v *= scale;   // the routed scaling factor, applied in fp32 before the one rounding to the output type
     Elem<TO>::store(topv_row + lane, v);
     topi_row[lane] = static_cast<int64_t>(sel_i);
+    // ... where they hold the log of the weight as the layer will use it (rounded), clamped at 1e-12;
+    // a lane's stores to one address keep their order
+    if (pseudo_row != nullptr) pseudo_row[sel_i] = logf(fmaxf(Elem<TO>::round(v), 1e-12f));
   }
   return sel_i;  // lane r < K: the r-th selected expert
 }
@@ -293,11 +304,32 @@ __device__ __forceinline__ int topk_token(const TL* __restrict__ row, int E, int
 template <typename TL, typename TO>
 __global__ __launch_bounds__(kTopkWaves * 64) void gate_topk_kernel(
     const TL* __restrict__ logits, int Ttok, int E, int K, int renorm, TO* __restrict__ topv,
-    int64_t* __restrict__ topi, int n_group, int topk_group, int softmax) {
+    int64_t* __restrict__ topi, int n_group, int topk_group, int softmax, float scale, float* __restrict__ pseudo) {
   const int t = blockIdx.x * kTopkWaves + (threadIdx.x >> 6);
   if (t >= Ttok) return;
   topk_token<TL, TO>(logits + static_cast<size_t>(t) * E, E, K, renorm, topv + static_cast<size_t>(t) * K,
-                     topi + static_cast<size_t>(t) * K, threadIdx.x & 63, n_group, topk_group, softmax != 0);
+                     topi + static_cast<size_t>(t) * K, threadIdx.x & 63, n_group, topk_group, softmax != 0, scale,
+                     pseudo != nullptr ? pseudo + static_cast<size_t>(t) * E : nullptr);
+}
+
+// Pseudo logits of a routing that was not computed here (utils/eval_core.py:11137-11155, the replayed
+// prediction of the previous layer): `fill` everywhere but at the K given experts of a token, which hold
+// log(max(weight, eps)).  One wavefront per token.
+template <typename TV>
+__global__ __launch_bounds__(kTopkWaves * 64) void pseudo_logits_kernel(const TV* __restrict__ topv,
+                                                                        const int64_t* __restrict__ topi, int Ttok,
+                                                                        int K, int E, float eps, float fill,
+                                                                        float* __restrict__ out) {
+  const int t = blockIdx.x * kTopkWaves + (threadIdx.x >> 6);
+  if (t >= Ttok) return;
+  const int lane = threadIdx.x & 63;
+  float* row = out + static_cast<size_t>(t) * E;
+  for (int e = lane; e < E; e += 64) {
+    float v = fill;
+    for (int k = 0; k < K; ++k)   // (the last slot that names an expert wins, as a scatter in slot order would have it)
+      if (topi[static_cast<size_t>(t) * K + k] == e) v = logf(fmaxf(Elem<TV>::load(topv + static_cast<size_t>(t) * K + k), eps));
+    row[e] = v;
+  }
 }
 
 // ---------------------------------------------------------------------------
@@ -736,12 +768,13 @@ static int launch_router_logits(const void* x, const void* wg, const void* wsg, 
 
 template <typename TL, typename TO>
 static int launch_gate_topk(const void* logits, int Ttok, int E, int K, int renorm, void* topv,
-                            int64_t* topi, hipStream_t st, int n_group = 0, int topk_group = 0, int softmax = 1) {
+                            int64_t* topi, hipStream_t st, int n_group = 0, int topk_group = 0, int softmax = 1,
+                            float scale = 1.f, float* pseudo = nullptr) {
   dim3 grid((Ttok + kTopkWaves - 1) / kTopkWaves);
   ProfScope prof(SPARSE_HIP_K_GATE_TOPK, st);
   hipLaunchKernelGGL((gate_topk_kernel<TL, TO>), grid, dim3(kTopkWaves * 64), 0, st,
                      static_cast<const TL*>(logits), Ttok, E, K, renorm, static_cast<TO*>(topv), topi, n_group,
-                     topk_group, softmax);
+                     topk_group, softmax, scale, pseudo);
   SP_LAUNCH_CHECK("gate_topk_kernel");
   return SPARSE_HIP_OK;
 }
@@ -803,6 +836,14 @@ int sparse_hip_gate_topk(const void* logits_dev, int logits_dtype, int T, int E,
 int sparse_hip_gate_topk_grouped(const void* logits_dev, int logits_dtype, int T, int E, int K, int renorm,
                                  int n_group, int topk_group, int out_dtype, void* topv_dev, int64_t* topi_dev,
                                  void* stream) {
+  return sparse_hip_gate_topk_scaled(logits_dev, logits_dtype, T, E, K, renorm, n_group, topk_group, 1.0f, out_dtype,
+                                     topv_dev, topi_dev, nullptr, stream);
+}
+
+int sparse_hip_gate_topk_scaled(const void* logits_dev, int logits_dtype, int T, int E, int K, int renorm,
+                                int n_group, int topk_group, float scale, int out_dtype, void* topv_dev,
+                                int64_t* topi_dev, float* pseudo_logits_dev, void* stream) {
+  SP_REQUIRE(scale == scale && scale > 0.f, "gate_topk: scale must be positive");
   SP_REQUIRE(valid_dtype(logits_dtype) && valid_dtype(out_dtype), "gate_topk: unknown dtype");
   SP_REQUIRE(n_group >= 1 && n_group <= 64 && E % n_group == 0, "gate_topk: n_group=%d must divide E=%d and be <= 64",
              n_group, E);
@@ -820,7 +861,8 @@ int sparse_hip_gate_topk_grouped(const void* logits_dev, int logits_dtype, int T
   const int ng = (n_group > 1 && topk_group < n_group) ? n_group : 0;  // every group kept = plain top-k
 #define SP_TOPK_CASE(LD, OD, TL, TO)                                                                          \
   if (logits_dtype == (LD) && out_dtype == (OD))                                                              \
-    return launch_gate_topk<TL, TO>(logits_dev, T, E, K, renorm, topv_dev, topi_dev, st, ng, topk_group);
+    return launch_gate_topk<TL, TO>(logits_dev, T, E, K, renorm, topv_dev, topi_dev, st, ng, topk_group, 1, scale, \
+                                    pseudo_logits_dev);
   SP_TOPK_CASE(SPARSE_HIP_BF16, SPARSE_HIP_BF16, uint16_t, uint16_t)
   SP_TOPK_CASE(SPARSE_HIP_BF16, SPARSE_HIP_F32, uint16_t, float)
   SP_TOPK_CASE(SPARSE_HIP_F32, SPARSE_HIP_BF16, float, uint16_t)
@@ -828,7 +870,33 @@ int sparse_hip_gate_topk_grouped(const void* logits_dev, int logits_dtype, int T
   SP_TOPK_CASE(SPARSE_HIP_F16, SPARSE_HIP_F32, f16_t, float)
   SP_TOPK_CASE(SPARSE_HIP_F32, SPARSE_HIP_F16, float, f16_t)
 #undef SP_TOPK_CASE
-  return launch_gate_topk<float, float>(logits_dev, T, E, K, renorm, topv_dev, topi_dev, st, ng, topk_group);
+  return launch_gate_topk<float, float>(logits_dev, T, E, K, renorm, topv_dev, topi_dev, st, ng, topk_group, 1, scale,
+                                        pseudo_logits_dev);
+}
+
+int sparse_hip_pseudo_logits(const void* topv_dev, int dtype, const int64_t* topi_dev, int T, int K, int E, float eps,
+                             float fill, float* out_dev, void* stream) {
+  SP_REQUIRE(valid_dtype(dtype), "pseudo_logits: unknown dtype %d", dtype);
+  SP_REQUIRE(T >= 0, "pseudo_logits: T=%d", T);
+  SP_REQUIRE(E >= 1 && K >= 1 && K <= SPARSE_HIP_MAX_TOPK, "pseudo_logits: E=%d, K=%d (K at most %d)", E, K,
+             SPARSE_HIP_MAX_TOPK);
+  SP_REQUIRE(eps > 0.f, "pseudo_logits: eps must be positive");
+  SP_REQUIRE(topv_dev && topi_dev && out_dev, "pseudo_logits: NULL pointer");
+  if (T == 0) return SPARSE_HIP_OK;
+  hipStream_t st = as_stream(stream);
+  dim3 grid((T + kTopkWaves - 1) / kTopkWaves);
+  if (dtype == SPARSE_HIP_F32) {
+    hipLaunchKernelGGL((pseudo_logits_kernel<float>), grid, dim3(kTopkWaves * 64), 0, st,
+                       static_cast<const float*>(topv_dev), topi_dev, T, K, E, eps, fill, out_dev);
+  } else if (dtype == SPARSE_HIP_F16) {
+    hipLaunchKernelGGL((pseudo_logits_kernel<f16_t>), grid, dim3(kTopkWaves * 64), 0, st,
+                       static_cast<const f16_t*>(topv_dev), topi_dev, T, K, E, eps, fill, out_dev);
+  } else {
+    hipLaunchKernelGGL((pseudo_logits_kernel<uint16_t>), grid, dim3(kTopkWaves * 64), 0, st,
+                       static_cast<const uint16_t*>(topv_dev), topi_dev, T, K, E, eps, fill, out_dev);
+  }
+  SP_LAUNCH_CHECK("pseudo_logits_kernel");
+  return SPARSE_HIP_OK;
 }
 
 int sparse_hip_topk(const void* values_dev, int T, int E, int K, int renorm, int out_dtype, void* topv_dev,

@@ -84,10 +84,13 @@ def router_logits(x: torch.Tensor, wg: torch.Tensor, wsg: Optional[torch.Tensor]
 
 def gate_topk(logits: torch.Tensor, k: int, renorm: bool = False, out_dtype: Optional[torch.dtype] = None,
               topv: Optional[torch.Tensor] = None, topi: Optional[torch.Tensor] = None,
-              n_group: int = 1, topk_group: int = 1):
+              n_group: int = 1, topk_group: int = 1, scale: float = 1.0,
+              pseudo_logits: Optional[torch.Tensor] = None):
     """Fused softmax(fp32) + top-k: returns ``(topv [T,k] out_dtype, topi [T,k] int64)``.
     With ``n_group > 1`` only experts of the ``topk_group`` best groups keep their probability
-    (DeepSeek-V2's group-limited selection); the others enter the top-k with 0."""
+    (DeepSeek-V2's group-limited selection); the others enter the top-k with 0.  ``scale`` (the
+    gate's routed scaling factor) multiplies the weights in fp32 before they are rounded;
+    ``pseudo_logits`` [T,E] fp32, if given, receives -inf except log(weight) at the selected experts."""
     lib = _lib.load()
     _need(logits, "logits")
     T, E = logits.shape
@@ -98,11 +101,30 @@ def gate_topk(logits: torch.Tensor, k: int, renorm: bool = False, out_dtype: Opt
         topi = torch.empty((T, k), device=logits.device, dtype=torch.int64)
     _need(topv, "topv", odt, (T, k))
     _need(topi, "topi", torch.int64, (T, k))
-    rc = lib.sparse_hip_gate_topk_grouped(_ptr(logits), dtype_code(logits.dtype), T, E, int(k), int(bool(renorm)),
-                                          int(n_group), int(topk_group), dtype_code(odt), _ptr(topv), _ptr(topi),
-                                          _stream())
-    _lib.check(rc, "sparse_hip_gate_topk_grouped")
+    if pseudo_logits is not None:
+        _need(pseudo_logits, "pseudo logits", torch.float32, (T, E))
+    rc = lib.sparse_hip_gate_topk_scaled(_ptr(logits), dtype_code(logits.dtype), T, E, int(k), int(bool(renorm)),
+                                         int(n_group), int(topk_group), float(scale), dtype_code(odt), _ptr(topv),
+                                         _ptr(topi), _ptr(pseudo_logits), _stream())
+    _lib.check(rc, "sparse_hip_gate_topk_scaled")
     return topv, topi
+
+
+def pseudo_logits(topv: torch.Tensor, topi: torch.Tensor, num_experts: int, eps: float = 1e-12,
+                  fill: float = float("-inf"), out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``out [T,E]`` fp32 = ``fill`` except ``log(max(topv, eps))`` at ``topi`` (utils/eval_core.py:9490-9499,
+    :11137-11155)."""
+    lib = _lib.load()
+    _need(topv, "topv")
+    T, K = topv.shape
+    _need(topi, "topi", torch.int64, (T, K))
+    if out is None:
+        out = torch.empty((T, int(num_experts)), device=topv.device, dtype=torch.float32)
+    _need(out, "pseudo logits", torch.float32, (T, int(num_experts)))
+    rc = lib.sparse_hip_pseudo_logits(_ptr(topv), dtype_code(topv.dtype), _ptr(topi), T, K, int(num_experts),
+                                      float(eps), float(fill), _ptr(out), _stream())
+    _lib.check(rc, "sparse_hip_pseudo_logits")
+    return out
 
 
 def topk_values(values: torch.Tensor, k: int, renorm: bool = False, out_dtype: Optional[torch.dtype] = None,
@@ -487,8 +509,8 @@ def profile_read() -> dict:
 
 def rs_predict(x: torch.Tensor, w1: torch.Tensor, b1: torch.Tensor, w2: torch.Tensor, b2: torch.Tensor,
                hidden_ws: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """Routing-scout forward pass of a decode-size call: ``softmax(w2 relu(w1 x + b1) + b2)`` in fp32, with
-    fp32 parameters whose BatchNorm is already folded into ``w1`` / ``b1``.  Returns ``pred [T, E]``."""
+    """Routing-scout forward pass: ``softmax(w2 relu(w1 x + b1) + b2)`` in fp32, with fp32 parameters
+    whose BatchNorm is already folded into ``w1`` / ``b1``.  Returns ``pred [T, E]``."""
     T, H = x.shape
     D, E = w1.shape[0], w2.shape[0]
     _need(x, "x")
@@ -507,6 +529,82 @@ def rs_predict(x: torch.Tensor, w1: torch.Tensor, b1: torch.Tensor, w2: torch.Te
     rc = _lib.load().sparse_hip_rs_predict(_ptr(x), dtype_code(x.dtype), T, H, _ptr(w1), _ptr(b1), D, _ptr(w2),
                                            _ptr(b2), E, _ptr(hidden_ws), _ptr(out), _stream())
     _lib.check(rc, "sparse_hip_rs_predict")
+    return out
+
+
+RS_ACT = {"none": 0, "relu": 1, "gelu": 2}
+
+
+def rs_dense(x: torch.Tensor, w: torch.Tensor, b: torch.Tensor, act: str = "none",
+             residual: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``act(x w^T + b) (+ residual)`` in fp32: one Linear of a routing-scout predictor with the
+    activation and the residual connection that follow it.  ``x [T, H]`` in any supported dtype, fp32
+    parameters, fp32 result ``[T, D]``."""
+    T, H = x.shape
+    D = w.shape[0]
+    _need(x, "x")
+    _need(w, "w", torch.float32, (D, H))
+    _need(b, "b", torch.float32, (D,))
+    if residual is not None:
+        _need(residual, "residual", torch.float32, (T, D))
+    if out is None:
+        out = torch.empty((T, D), device=x.device, dtype=torch.float32)
+    _need(out, "out", torch.float32, (T, D))
+    rc = _lib.load().sparse_hip_rs_dense(_ptr(x), dtype_code(x.dtype), T, H, _ptr(w), _ptr(b), D, RS_ACT[act],
+                                         _ptr(residual) if residual is not None else None, _ptr(out), _stream())
+    _lib.check(rc, "sparse_hip_rs_dense")
+    return out
+
+
+def rs_layernorm(x: torch.Tensor, gamma: torch.Tensor, beta: torch.Tensor, eps: float, width: Optional[int] = None,
+                 out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """LayerNorm over the first ``width`` columns of ``x [T, ld_in]`` (all of them by default) into fp32
+    rows ``out [T, ld_out]`` (as wide as ``x`` by default); columns past ``width`` come out zero."""
+    T, ld_in = x.shape
+    H = ld_in if width is None else int(width)
+    _need(x, "x")
+    _need(gamma, "gamma", torch.float32, (H,))
+    _need(beta, "beta", torch.float32, (H,))
+    if out is None:
+        out = torch.empty((T, ld_in), device=x.device, dtype=torch.float32)
+    _need(out, "out", torch.float32)
+    if out.dim() != 2 or out.shape[0] != T:
+        raise ValueError("out must be [T, ld_out]")
+    rc = _lib.load().sparse_hip_rs_layernorm(_ptr(x), dtype_code(x.dtype), T, H, ld_in, int(out.shape[1]),
+                                             _ptr(gamma), _ptr(beta), float(eps), _ptr(out), _stream())
+    _lib.check(rc, "sparse_hip_rs_layernorm")
+    return out
+
+
+def rs_features(x: torch.Tensor, topi: torch.Tensor, topv: torch.Tensor, num_experts: int,
+                out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``[float(x) | routing weights rescaled to sum 1 at the chosen experts | zero padding]`` as fp32
+    rows whose length is H + E rounded up to a multiple of 8: what a predictor of the
+    ``hidden_router_topk`` kind reads."""
+    T, H = x.shape
+    K, E = int(topi.shape[1]), int(num_experts)
+    ld = (H + E + 7) // 8 * 8
+    _need(x, "x")
+    _need(topi, "topi", torch.int32, (T, K))
+    _need(topv, "topv", x.dtype, (T, K))
+    if out is None:
+        out = torch.empty((T, ld), device=x.device, dtype=torch.float32)
+    _need(out, "out", torch.float32, (T, ld))
+    rc = _lib.load().sparse_hip_rs_features(_ptr(x), dtype_code(x.dtype), T, H, _ptr(topi), _ptr(topv), K, E, ld,
+                                            _ptr(out), _stream())
+    _lib.check(rc, "sparse_hip_rs_features")
+    return out
+
+
+def rs_softmax(logits: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Row softmax of fp32 ``logits [T, E]``."""
+    T, E = logits.shape
+    _need(logits, "logits", torch.float32)
+    if out is None:
+        out = torch.empty_like(logits)
+    _need(out, "out", torch.float32, (T, E))
+    rc = _lib.load().sparse_hip_rs_softmax(_ptr(logits), T, E, _ptr(out), _stream())
+    _lib.check(rc, "sparse_hip_rs_softmax")
     return out
 
 

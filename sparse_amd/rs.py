@@ -4,9 +4,11 @@
 the same name (utils/eval_core.py:3402-3417: Linear, BatchNorm1d, ReLU, Dropout(0.1),
 Linear, Softmax), so a bank trained for the reference (``rs_l{L}_inL{L-1}.pth`` payloads
 with a ``state_dict``, :3490-3550) loads into it unchanged.  Prediction runs on the device
-in fp32: decode-size calls of the plain MLP through the two-launch HIP predictor (``FusedScout``,
-``sparse_hip_rs_predict``), everything else (the residual predictor, predictors that also read the
-routing, prefill-size calls) through PyTorch; only the top-k leaves the device.
+in fp32 through the HIP predictor kernels, at any token count: the plain MLP in two launches
+(``FusedScout``, ``sparse_hip_rs_predict``), the residual predictor as a chain of LayerNorm and dense
+launches (``FusedResidualScout``), predictors that also read the routing after one launch that lays
+their input rows out; only the top-k leaves the device.  The ``nn.Module`` classes hold the parameters
+(and run on host tensors, in training, and for shapes the kernels do not take).
 """
 from __future__ import annotations
 
@@ -37,6 +39,16 @@ class RoutingScoutMLP(nn.Module):
         return self.mlp(x.reshape(-1, x.shape[-1]))
 
 
+def _padded_columns(w: torch.Tensor) -> torch.Tensor:
+    """``w [D, H]`` as fp32 with zero columns appended up to a multiple of 8 (the dense kernel reads rows
+    eight values at a time; an input row padded with zeros the same way gives the same products)."""
+    w = w.detach().float()
+    pad = -w.shape[1] % 8
+    if pad:
+        w = torch.cat([w, w.new_zeros((w.shape[0], pad))], dim=1)
+    return w.contiguous()
+
+
 class FusedScout:
     """The parameters of a ``RoutingScoutMLP`` in eval mode as the HIP predictor kernel takes them: fp32,
     row-major, the BatchNorm's running statistics and affine folded into the first Linear (eval mode makes
@@ -47,33 +59,90 @@ class FusedScout:
         lin1, bn, lin2 = module.mlp[0], module.mlp[1], module.mlp[4]
         with torch.no_grad():
             scale = bn.weight.float() / torch.sqrt(bn.running_var.float() + bn.eps)
-            self.w1 = (lin1.weight.float() * scale[:, None]).contiguous()
+            self.w1 = _padded_columns(lin1.weight.float() * scale[:, None])
             self.b1 = ((lin1.bias.float() - bn.running_mean.float()) * scale + bn.bias.float()).contiguous()
             self.w2 = lin2.weight.float().contiguous()
             self.b2 = lin2.bias.float().contiguous()
-        self.input_dim, self.hidden_dim, self.num_experts = self.w1.shape[1], self.w1.shape[0], self.w2.shape[0]
+        self.input_dim, self.hidden_dim, self.num_experts = lin1.in_features, self.w1.shape[0], self.w2.shape[0]
+        self.device = self.w1.device
 
     def __call__(self, x: torch.Tensor) -> torch.Tensor:
+        """``x [T, input_dim rounded up to a multiple of 8]``, in the activations' dtype or fp32."""
         from . import ops
-        return ops.rs_predict(x.contiguous(), self.w1, self.b1, self.w2, self.b2)
+        return ops.rs_predict(x, self.w1, self.b1, self.w2, self.b2)
 
 
-def fused_scout(module: Any, x: torch.Tensor) -> Optional[FusedScout]:
-    """The fused form of ``module`` for a call on ``x [T, H]``, or None where the HIP predictor does not
-    apply (another predictor class, training mode, host tensors, more tokens than a decode call, shapes
-    the kernel does not take); cached on the module."""
-    if not (isinstance(module, RoutingScoutMLP) and not module.training and x.is_cuda and x.dim() == 2):
+class FusedResidualScout:
+    """The parameters of a ``RoutingScoutResidualMLP`` in eval mode (Dropout is the identity) as the HIP
+    kernels take them, and the launch chain: LayerNorm, dense + GELU; per unit LayerNorm, dense + GELU,
+    dense + residual; LayerNorm, dense, softmax."""
+
+    def __init__(self, module: "RoutingScoutResidualMLP") -> None:
+        f = lambda t: t.detach().float().contiguous()
+        norm, lin = module.input[0], module.input[1]
+        self.stem = (f(norm.weight), f(norm.bias), float(norm.eps), _padded_columns(lin.weight), f(lin.bias))
+        self.units = []
+        for unit in module.blocks:
+            n, up, down = unit.net[0], unit.net[1], unit.net[4]
+            self.units.append((f(n.weight), f(n.bias), float(n.eps), f(up.weight), f(up.bias), f(down.weight),
+                               f(down.bias)))
+        self.out_norm = (f(module.out_norm.weight), f(module.out_norm.bias), float(module.out_norm.eps))
+        self.head = (f(module.head.weight), f(module.head.bias))
+        self.input_dim, self.hidden_dim, self.num_experts = lin.in_features, lin.out_features, module.head.out_features
+        self.device = self.head[0].device
+
+    def __call__(self, x: torch.Tensor) -> torch.Tensor:
+        """``x [T, input_dim rounded up to a multiple of 8]``, in the activations' dtype or fp32."""
+        from . import ops
+        T = x.shape[0]
+        gamma, beta, eps, w, b = self.stem
+        new = lambda width: torch.empty((T, width), device=x.device, dtype=torch.float32)
+        normed = ops.rs_layernorm(x, gamma, beta, eps, width=self.input_dim)
+        h = ops.rs_dense(normed, w, b, act="gelu")
+        if self.units:
+            normed, wide, other = new(self.hidden_dim), new(2 * self.hidden_dim), new(self.hidden_dim)
+        for gamma, beta, eps, w_up, b_up, w_down, b_down in self.units:
+            ops.rs_layernorm(h, gamma, beta, eps, out=normed)
+            ops.rs_dense(normed, w_up, b_up, act="gelu", out=wide)
+            ops.rs_dense(wide, w_down, b_down, residual=h, out=other)
+            h, other = other, h
+        gamma, beta, eps = self.out_norm
+        normed = ops.rs_layernorm(h, gamma, beta, eps)
+        return ops.rs_softmax(ops.rs_dense(normed, self.head[0], self.head[1]))
+
+
+def fused_scout(module: Any, x: torch.Tensor, mode: str = "hidden", num_experts: int = 0):
+    """The HIP form of the predictor ``module`` for a call on ``x [T, H]`` with input kind ``mode``
+    (``hidden``: the token rows; ``hidden_router_topk``: the token rows followed by ``num_experts``
+    routing-weight columns), or None where the kernels do not apply (another class, training mode, host
+    tensors, parameters on another device, widths the kernels do not take); cached on the module."""
+    if not (isinstance(module, (RoutingScoutMLP, RoutingScoutResidualMLP)) and not module.training
+            and x.is_cuda and x.dim() == 2 and x.shape[0] >= 1):
         return None
-    if x.shape[0] > _lib.DECODE_MAX_TOKENS or x.shape[1] % 8:
+    if mode == "hidden":
+        width = x.shape[1]
+        if width % 8:
+            return None
+    elif mode == "hidden_router_topk":
+        width = x.shape[1] + int(num_experts)
+        if not 1 <= int(num_experts) <= _lib.MAX_EXPERTS:
+            return None
+    else:
         return None
     fused = getattr(module, "_sparse_fused", None)
-    if fused is None or fused.w1.device != x.device:
-        lin1 = module.mlp[0]
-        if lin1.weight.device != x.device or lin1.out_features % 4 or module.mlp[4].out_features > _lib.MAX_EXPERTS:
+    if fused is None or fused.device != x.device:
+        plain = isinstance(module, RoutingScoutMLP)
+        first = module.mlp[0] if plain else module.input[1]
+        last = module.mlp[4] if plain else module.head
+        if first.weight.device != x.device or last.out_features > _lib.MAX_EXPERTS:
             return None
-        fused = FusedScout(module)
+        if plain and first.out_features % 4:
+            return None
+        if not plain and first.out_features % 8:
+            return None
+        fused = FusedScout(module) if plain else FusedResidualScout(module)
         object.__setattr__(module, "_sparse_fused", fused)
-    return fused if fused.input_dim == x.shape[1] else None
+    return fused if fused.input_dim == width else None
 
 
 class _ResidualUnit(nn.Module):

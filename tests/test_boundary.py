@@ -213,3 +213,23 @@ def test_workspace_used_under_graph_capture_is_never_dropped():
     assert 9 in table and 8 not in table
     table.clear()
     assert len(table) == 0 and table.pinned() == set()
+
+
+def test_prefill_expert_math_is_validated_like_the_reference(monkeypatch):
+    """``SPARSE_PREFILL_EXPERT_MATH`` must be ``native`` or ``fixed64`` (utils/eval_core.py:4795-4798): anything
+    else is a ``ValueError`` of the constructor, before a weight is touched; both accepted values (and
+    ``SPARSE_EP_NATIVE_DECODE_GRANULARITY``) are read and recorded."""
+    import torch
+    from sparse_amd.context import DistEnv
+    from sparse_amd.synthetic import make_mlp_block
+    shape = dict(family="qwen_shared", hidden=64, num_experts=4, inter=64, top_k=2, shared_inter=64)
+    mlp = make_mlp_block(shape, dtype=torch.float32, seed=0)
+    env = DistEnv(0, 1, 0, torch.device("cpu"))
+    monkeypatch.setenv("SPARSE_PREFILL_EXPERT_MATH", "fixed32")
+    SparseContext.reset()
+    try:
+        with pytest.raises(ValueError, match="SPARSE_PREFILL_EXPERT_MATH must be native or fixed64"):
+            Block(0, mlp, None, env, num_layers=1, num_experts=4, top_k=2, dtype=torch.float32)
+        assert 0 not in SparseContext.layer_blocks
+    finally:
+        SparseContext.reset()

@@ -48,6 +48,39 @@ def test_gate_topk_matches_oracle(device, E, K, ldt):
                                atol=1e-6)
 
 
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("scale", [1.0, 2.5, 16.0])
+def test_gate_topk_scaling_factor_and_pseudo_logits(device, dt, scale):
+    """The DeepSeek branch after the gate (utils/eval_core.py:9503-9517, :9490-9499) inside the top-k
+    launch: weights times the routed scaling factor, multiplied in fp32 and rounded once (the oracle's
+    ``(topv * factor).to(dtype)``), and the pseudo logits: -inf but log(weight) at the chosen experts."""
+    ops = _ops()
+    E, K, T = 64, 6, 193
+    x = make_hidden(T, 128, dt, seed=5)
+    gate_w = (torch.randn(E, 128, generator=torch.Generator().manual_seed(6)) * 0.3).to(dt)
+    want_v, want_i, want_p = ref_moe.deepseek_router(x, gate_w, K, routed_scaling_factor=scale)
+    logits = torch.nn.functional.linear(x.float(), gate_w.float())
+    pseudo = torch.empty((T, E), device=device, dtype=torch.float32)
+    topv, topi = ops.gate_topk(logits.to(device), K, out_dtype=dt, scale=scale, pseudo_logits=pseudo)
+    assert torch.equal(topi.cpu(), want_i)
+    got_v = topv.cpu()
+    # one rounding of an fp32 product: at most the last bit of the output type apart from the oracle's
+    # (exp and the division differ in their last fp32 bits between host and device)
+    ulp = {torch.bfloat16: 2.0 ** -7, torch.float16: 2.0 ** -10, torch.float32: 2.0 ** -22}[dt]
+    assert float(((got_v.float() - want_v.float()).abs() / want_v.float().abs()).max()) <= ulp
+    assert (got_v == want_v).float().mean() > (0.9 if dt != torch.float32 else 0.0)
+    got_p = pseudo.cpu()
+    chosen = torch.zeros((T, E), dtype=torch.bool).scatter_(1, want_i, True)
+    assert torch.isneginf(got_p[~chosen]).all() and torch.isfinite(got_p[chosen]).all()
+    torch.testing.assert_close(got_p.gather(1, want_i), got_v.float().clamp_min(1e-12).log(), rtol=1e-5, atol=1e-6)
+    # the stand-alone kernel on the same weights, with the replay convention (-1e9, a larger eps)
+    again = ops.pseudo_logits(topv, topi, E, eps=1e-12, fill=float("-inf")).cpu()
+    assert torch.equal(again, got_p)
+    replay = ops.pseudo_logits(topv, topi, E, eps=0.05, fill=-1e9).cpu()
+    assert (replay[~chosen] == -1e9).all()
+    torch.testing.assert_close(replay.gather(1, want_i), got_v.float().clamp_min(0.05).log(), rtol=1e-5, atol=1e-6)
+
+
 @pytest.mark.parametrize("E,n_group,topk_group,K", [(16, 4, 2, 6), (160, 8, 3, 6), (256, 64, 5, 16), (64, 2, 1, 8),
                                                       (60, 6, 6, 4), (12, 4, 1, 5)])
 @pytest.mark.parametrize("ldt", [torch.float32, torch.bfloat16])
@@ -566,9 +599,146 @@ def test_rs_predictor_kernel_matches_the_module(device, dtype, T):
     clear = (v_ref[:, 7] - v_ref[:, 8]) > 1e-4 * v_ref[:, 7]
     assert bool(clear.any())
     assert torch.equal(torch.sort(i_dev[clear], 1).values, torch.sort(i_ref[clear, :8], 1).values)
-    # what the kernel does not take falls back to the module: training mode, prefill-size calls
-    assert fused_scout(mod, make_hidden(40, H, dtype, seed=82).to(device)) is None
+    # what the kernel does not take falls back to the module: training mode, widths off the 8-grid
     assert fused_scout(mod.train(), x) is None
+    assert fused_scout(mod.eval(), x[:, :H - 4].contiguous()) is None
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("T", [33, 100, 4096])
+def test_rs_predictor_kernel_at_prefill_sizes(device, dtype, T):
+    """The same two launches over blocks of 32 token rows: a prefill-size call against the numpy oracle of
+    the predictor (and through it the module), including a last block that is not full."""
+    from oracle import ref_rs
+    from sparse_amd.rs import RoutingScoutMLP, fused_scout
+    H, E, D = 512, 60, 256
+    torch.manual_seed(6)
+    mod = RoutingScoutMLP(H, E, hidden_dim=D)
+    bn = mod.mlp[1]
+    with torch.no_grad():
+        bn.running_mean.copy_(torch.randn(D) * 0.3)
+        bn.running_var.copy_(torch.rand(D) * 2 + 0.25)
+        bn.weight.copy_(torch.rand(D) + 0.5)
+        bn.bias.copy_(torch.randn(D) * 0.2)
+        mod.mlp[4].weight.mul_(4.0)
+    mod = mod.eval()
+    x = make_hidden(T, H, dtype, seed=83)
+    n = lambda t: t.detach().numpy()
+    want = ref_rs.routing_scout_forward(x.float().numpy(), n(mod.mlp[0].weight), n(mod.mlp[0].bias), n(bn.weight),
+                                        n(bn.bias), n(bn.running_mean), n(bn.running_var), n(mod.mlp[4].weight),
+                                        n(mod.mlp[4].bias), eps=bn.eps)
+    mod = mod.to(device)
+    fused = fused_scout(mod, x.to(device))
+    assert fused is not None
+    pred = fused(x.to(device))
+    assert tuple(pred.shape) == (T, E)
+    torch.testing.assert_close(pred.cpu(), torch.from_numpy(want), rtol=2e-4, atol=1e-7)
+
+
+def _residual_scout(H, E, D, layers, seed):
+    from sparse_amd.rs import RoutingScoutResidualMLP
+    torch.manual_seed(seed)
+    mod = RoutingScoutResidualMLP(H, E, hidden_dim=D, num_hidden_layers=layers)
+    with torch.no_grad():
+        for m in mod.modules():
+            if isinstance(m, torch.nn.LayerNorm):
+                m.weight.copy_(torch.rand_like(m.weight) + 0.5)
+                m.bias.copy_(torch.randn_like(m.bias) * 0.3)
+        mod.head.weight.mul_(4.0)
+    return mod.eval()
+
+
+def _residual_oracle(mod, rows):
+    from oracle import ref_rs
+    n = lambda t: t.detach().cpu().numpy()
+    stem = (n(mod.input[0].weight), n(mod.input[0].bias), n(mod.input[1].weight), n(mod.input[1].bias))
+    units = [(n(u.net[0].weight), n(u.net[0].bias), n(u.net[1].weight), n(u.net[1].bias), n(u.net[4].weight),
+              n(u.net[4].bias)) for u in mod.blocks]
+    return ref_rs.routing_scout_residual_forward(rows, stem, units, (n(mod.out_norm.weight), n(mod.out_norm.bias)),
+                                                 (n(mod.head.weight), n(mod.head.bias)), eps=mod.out_norm.eps)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("T,layers", [(1, 3), (8, 3), (32, 1), (40, 0), (300, 2)])
+def test_residual_rs_predictor_chain_matches_oracle(device, dtype, T, layers):
+    """The deeper predictor as a chain of LayerNorm, dense (+GELU, +residual) and softmax launches against
+    its numpy oracle on the widened token rows; fp32 arithmetic both sides, tolerance for summation order
+    (1e-3 relative on probabilities that pass through up to eight matrix products)."""
+    from sparse_amd.rs import FusedResidualScout, fused_scout
+    H, E, D = 512, 60, 128
+    mod = _residual_scout(H, E, D, layers, seed=7 + layers)
+    x = make_hidden(T, H, dtype, seed=84 + T)
+    want = _residual_oracle(mod, x.float().numpy())
+    mod = mod.to(device)
+    fused = fused_scout(mod, x.to(device))
+    assert isinstance(fused, FusedResidualScout) and fused_scout(mod, x.to(device)) is fused
+    pred = fused(x.to(device))
+    assert pred.dtype == torch.float32 and tuple(pred.shape) == (T, E)
+    torch.testing.assert_close(pred.cpu(), torch.from_numpy(want), rtol=1e-3, atol=1e-7)
+    torch.testing.assert_close(pred.sum(-1), torch.ones(T, device=device), rtol=1e-5, atol=1e-5)
+    with torch.no_grad():
+        torch.testing.assert_close(pred, mod(x.to(device).float()), rtol=1e-3, atol=1e-7)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("residual", [False, True])
+@pytest.mark.parametrize("T", [5, 70])
+def test_rs_predictors_that_read_the_routing(device, dtype, residual, T):
+    """``feature_mode = hidden_router_topk``: one launch lays out [x | routing-weight columns | padding]
+    (bit-exact against the oracle's feature rows: E = 60 makes the row length 572, padded to 576), and the
+    predictors run on those rows; against the oracle fed the oracle's own concatenation."""
+    from oracle import ref_rs
+    from sparse_amd.rs import RoutingScoutMLP, fused_scout
+    ops = _ops()
+    H, E, K, D = 512, 60, 4, 128
+    x = make_hidden(T, H, dtype, seed=90 + T)
+    g = torch.Generator().manual_seed(91 + T)
+    topi = torch.stack([torch.randperm(E, generator=g)[:K] for _ in range(T)]).to(torch.int32)
+    topv = torch.rand((T, K), generator=g).to(dtype)
+    if T > 1:
+        topv[1].zero_()                                             # a row whose weights sum to zero
+    feat = ref_rs.router_topk_feature(topi.numpy(), topv.float().numpy(), E)
+    rows = np.concatenate([x.float().numpy(), feat], axis=1)
+    got_rows = ops.rs_features(x.to(device), topi.to(device), topv.to(device), E)
+    assert tuple(got_rows.shape) == (T, 576)
+    assert np.array_equal(got_rows[:, :H + E].cpu().numpy(), rows) and not bool(got_rows[:, H + E:].any())
+    if residual:
+        mod = _residual_scout(H + E, E, D, 2, seed=12)
+        want = _residual_oracle(mod, rows)
+    else:
+        torch.manual_seed(13)
+        mod = RoutingScoutMLP(H + E, E, hidden_dim=D).eval()
+        bn = mod.mlp[1]
+        n = lambda t: t.detach().numpy()
+        want = ref_rs.routing_scout_forward(rows, n(mod.mlp[0].weight), n(mod.mlp[0].bias), n(bn.weight), n(bn.bias),
+                                            n(bn.running_mean), n(bn.running_var), n(mod.mlp[4].weight),
+                                            n(mod.mlp[4].bias), eps=bn.eps)
+    mod = mod.to(device)
+    assert fused_scout(mod, x.to(device)) is None                   # the wrong input kind for this module
+    fused = fused_scout(mod, x.to(device), "hidden_router_topk", E)
+    assert fused is not None
+    pred = fused(got_rows)
+    torch.testing.assert_close(pred.cpu(), torch.from_numpy(want), rtol=1e-3, atol=1e-7)
+
+
+def test_rs_building_blocks_reject_bad_arguments(device):
+    ops = _ops()
+    x = torch.zeros((4, 64), device=device)
+    w, b = torch.zeros((16, 64), device=device), torch.zeros(16, device=device)
+    with pytest.raises(Exception):
+        ops.rs_dense(x[:, :60].contiguous(), w[:, :60].contiguous(), b)          # width off the 8-grid
+    with pytest.raises(Exception):
+        ops.rs_dense(x, w, b, act="tanh")
+    with pytest.raises(Exception):
+        ops.rs_layernorm(x, torch.ones(64, device=device), torch.zeros(64, device=device), -1.0)
+    with pytest.raises(Exception):
+        ops.rs_layernorm(x, torch.ones(64, device=device), torch.zeros(64, device=device), 1e-5,
+                         out=torch.empty((4, 32), device=device))               # rows shorter than the width
+    with pytest.raises(Exception):
+        ops.rs_softmax(torch.zeros((2, 300), device=device))                    # more than 256 experts
+    with pytest.raises(Exception):
+        ops.rs_features(x.bfloat16(), torch.zeros((4, 2), device=device, dtype=torch.int32),
+                        torch.zeros((4, 2), device=device, dtype=torch.bfloat16), 300)
 
 
 @pytest.mark.parametrize("T,decode", [(8, True), (128, False)])
