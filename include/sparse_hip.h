@@ -455,7 +455,7 @@ int sparse_hip_rs_dense(const void* x_dev, int dtype, int T, int H, const float*
                         int act, const float* residual_dev, float* out_dev, void* stream);
 int sparse_hip_rs_layernorm(const void* x_dev, int dtype, int T, int H, int ld_in, int ld_out,
                             const float* gamma_dev, const float* beta_dev, float eps, float* out_dev, void* stream);
-int sparse_hip_rs_features(const void* x_dev, int dtype, int T, int H, const int32_t* topi_dev,
+int sparse_hip_rs_features(const void* x_dev, int dtype, int T, int H, const int64_t* topi_dev,
                            const void* topv_dev, int K, int E, int ld, float* out_dev, void* stream);
 int sparse_hip_rs_softmax(const float* in_dev, int T, int E, float* out_dev, void* stream);
 

@@ -131,7 +131,7 @@ __global__ __launch_bounds__(kRsThreads) void rs_layernorm_kernel(const T* __res
 // among E columns | zeros up to ld ], one workgroup per token.
 template <typename T>
 __global__ __launch_bounds__(kRsThreads) void rs_features_kernel(const T* __restrict__ x, int H,
-                                                                 const int32_t* __restrict__ topi,
+                                                                 const int64_t* __restrict__ topi,
                                                                  const T* __restrict__ topv, int K, int E, int ld,
                                                                  float* __restrict__ out) {
   const T* row = x + static_cast<size_t>(blockIdx.x) * H;
@@ -140,13 +140,13 @@ __global__ __launch_bounds__(kRsThreads) void rs_features_kernel(const T* __rest
   for (int h = H + threadIdx.x; h < ld; h += kRsThreads) orow[h] = 0.f;
   __syncthreads();
   if (threadIdx.x == 0) {
-    const int32_t* ti = topi + static_cast<size_t>(blockIdx.x) * K;
+    const int64_t* ti = topi + static_cast<size_t>(blockIdx.x) * K;
     const T* tv = topv + static_cast<size_t>(blockIdx.x) * K;
     float sum = 0.f;
     for (int k = 0; k < K; ++k) sum += Elem<T>::load(tv + k);
     sum = fmaxf(sum, 1e-12f);
     for (int k = 0; k < K; ++k) {
-      const int e = ti[k];
+      const int64_t e = ti[k];
       if (e >= 0 && e < E) orow[H + e] += Elem<T>::load(tv + k) / sum;
     }
   }
@@ -306,7 +306,7 @@ extern "C" int sparse_hip_rs_layernorm(const void* x_dev, int dtype, int T, int 
   return SPARSE_HIP_OK;
 }
 
-extern "C" int sparse_hip_rs_features(const void* x_dev, int dtype, int T, int H, const int32_t* topi_dev,
+extern "C" int sparse_hip_rs_features(const void* x_dev, int dtype, int T, int H, const int64_t* topi_dev,
                                       const void* topv_dev, int K, int E, int ld, float* out_dev, void* stream) {
   SP_REQUIRE(valid_dtype(dtype), "rs_features: unknown dtype %d", dtype);
   SP_REQUIRE(T >= 1 && H >= 1 && K >= 1, "rs_features: T=%d H=%d K=%d", T, H, K);

@@ -585,7 +585,7 @@ def rs_features(x: torch.Tensor, topi: torch.Tensor, topv: torch.Tensor, num_exp
     K, E = int(topi.shape[1]), int(num_experts)
     ld = (H + E + 7) // 8 * 8
     _need(x, "x")
-    _need(topi, "topi", torch.int32, (T, K))
+    _need(topi, "topi", torch.int64, (T, K))
     _need(topv, "topv", x.dtype, (T, K))
     if out is None:
         out = torch.empty((T, ld), device=x.device, dtype=torch.float32)
