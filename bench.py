@@ -166,6 +166,133 @@ def decode_workload(blocks, shape, batch, steps, warmup, dtype, device, use_grap
     )
 
 
+class GpuTelemetry:
+    """Socket power and shader clock of the GPU in use, sampled from host threads while a workload runs.
+    Power: the amdgpu driver's hwmon file (power1_average or power1_input, with power1_cap) every
+    ``period`` seconds.  Clock: hwmon freq1_input where the driver has it, else one `amd-smi metric` child
+    process per sample (a few a second; it also gives the power where the sysfs file is missing), averaged
+    over the XCDs.  What the box does not expose to this user is reported as missing, without figures."""
+
+    def __init__(self, device_index=0, period=0.01):
+        import glob
+        self.period, self.power, self.clock, self.note = period, [], [], None
+        self._stop, self._threads = None, []
+        self.hwmon = None
+        want = None
+        try:
+            p = torch.cuda.get_device_properties(device_index)
+            want = f"{p.pci_domain_id:04x}:{p.pci_bus_id:02x}:{p.pci_device_id:02x}"
+        except Exception:  # noqa: BLE001
+            pass
+        cards = []
+        for card in sorted(glob.glob("/sys/class/drm/card[0-9]*")):
+            if "-" in os.path.basename(card):
+                continue
+            hw = sorted(glob.glob(os.path.join(card, "device", "hwmon", "hwmon*")))
+            if hw:
+                cards.append((hw[0], os.path.realpath(os.path.join(card, "device"))))
+        match = [c for c in cards if want and want in c[1]]
+        pick = match[0] if match else (cards[0] if len(cards) == 1 else None)
+        if pick is not None:
+            self.hwmon = pick[0]
+        self.power_file = next((f for f in ("power1_average", "power1_input")
+                                if self.hwmon and (self._read(f) or "").isdigit()), None)
+        self.freq_file = "freq1_input" if self.hwmon and (self._read("freq1_input") or "").isdigit() else None
+        cap = self._read("power1_cap") if self.hwmon else None
+        self.cap_w = int(cap) / 1e6 if cap and cap.isdigit() else None
+        self.smi = None
+        if self.power_file is None or self.freq_file is None:
+            self.smi = self._amd_smi()
+        self.power_source = (f"sysfs {self.power_file}" if self.power_file
+                             else "amd-smi socket_power" if self.smi and self.smi[0] is not None else None)
+        self.clock_source = ("sysfs freq1_input" if self.freq_file
+                             else "amd-smi gfx clk, mean over XCDs" if self.smi and self.smi[1] is not None else None)
+        if not (self.power_source or self.clock_source):
+            self.note = (f"no readable power / clock source: {len(cards)} drm cards with hwmon, wanted PCI {want}, "
+                         "amd-smi metric gave nothing")
+
+    def _read(self, name):
+        try:
+            with open(os.path.join(self.hwmon, name)) as f:
+                return f.read().strip()
+        except OSError:
+            return None
+
+    @staticmethod
+    def _amd_smi():
+        import subprocess
+        try:
+            raw = subprocess.run(["amd-smi", "metric", "--power", "--clock", "--json"], capture_output=True,
+                                 text=True, timeout=10).stdout
+            data = json.loads(raw)
+        except Exception:  # noqa: BLE001
+            return None
+        if isinstance(data, dict):
+            data = data.get("gpu_data")
+        entry = data[0] if isinstance(data, list) and data else None
+        if not isinstance(entry, dict):
+            return None
+
+        def number(node):
+            node = node.get("value") if isinstance(node, dict) else node
+            return float(node) if isinstance(node, (int, float)) else None
+
+        power = number((entry.get("power") or {}).get("socket_power"))
+        gfx = [number(v.get("clk")) for k, v in (entry.get("clock") or {}).items()
+               if k.startswith("gfx") and isinstance(v, dict)]
+        gfx = [v for v in gfx if v is not None]
+        if power is None and not gfx:
+            return None
+        return (power, sum(gfx) / len(gfx) if gfx else None)
+
+    def __enter__(self):
+        import threading
+        self._stop = threading.Event()
+
+        def sysfs_loop():
+            while not self._stop.is_set():
+                if self.power_file:
+                    v = self._read(self.power_file)
+                    if v and v.isdigit():
+                        self.power.append(int(v) / 1e6)
+                if self.freq_file:
+                    v = self._read(self.freq_file)
+                    if v and v.isdigit():
+                        self.clock.append(int(v) / 1e6)
+                self._stop.wait(self.period)
+
+        def smi_loop():
+            while not self._stop.is_set():
+                got = self._amd_smi()
+                if got is not None:
+                    if self.power_file is None and got[0] is not None:
+                        self.power.append(got[0])
+                    if self.freq_file is None and got[1] is not None:
+                        self.clock.append(got[1])
+                self._stop.wait(0.05)
+
+        loops = ([sysfs_loop] if (self.power_file or self.freq_file) else []) + ([smi_loop] if self.smi else [])
+        for fn in loops:
+            t = threading.Thread(target=fn, daemon=True)
+            t.start()
+            self._threads.append(t)
+        return self
+
+    def __exit__(self, *exc):
+        if self._stop is not None:
+            self._stop.set()
+        for t in self._threads:
+            t.join(timeout=15)
+        return False
+
+    def summary(self):
+        if self.note:
+            return {"available": False, "note": self.note}
+        stat = lambda v: ({"mean": sum(v) / len(v), "min": min(v), "max": max(v), "samples": len(v)} if v else None)
+        return {"available": True, "power_source": self.power_source, "clock_source": self.clock_source,
+                "power_w": stat(self.power), "power_cap_w": self.cap_w, "sclk_mhz": stat(self.clock)}
+
+
 def prefill_workload(shape, tokens, steps, warmup, dtype, device):
     blocks = build_stack(shape, dtype, device)
     inputs = make_inputs(shape, 1, tokens, 2, dtype, device)
@@ -191,12 +318,25 @@ def prefill_workload(shape, tokens, steps, warmup, dtype, device):
     wall_other = time_steps(blocks, inputs, 1, steps, use_graph=False)
     for blk in blocks:
         blk.merged_prefill = merged
+    # socket power and shader clock as the driver reports them, sampled from a host thread during a pass
+    # of its own (at least about a second of steps), so that the sampling cannot touch the timed figure
+    tele_steps = max(steps, int(3.0 / max(wall / steps, 1e-4)))
+    with GpuTelemetry() as tele:
+        wall_tele = time_steps(blocks, inputs, 0, tele_steps, use_graph=False)
+    telemetry = tele.summary()
+    telemetry["ms_per_step_while_sampling"] = wall_tele / tele_steps * 1e3
     # what the matrix cores sustain on this box with nothing but the kernel's wavefront tile going on:
     # operands in registers, and with the activation fragments read from LDS every k step
     probe = {}
     for name, from_lds in (("registers", False), ("lds_fragments", True)):
-        tf, mhz = ops.mfma_probe(from_lds, device=device)
-        probe[name] = {"tflops": tf, "clock_mhz": mhz, "frac_of_peak": tf / MFMA_BF16_PEAK_TFLOPS}
+        with GpuTelemetry() as tele:
+            until = time.perf_counter() + 2.0          # about two seconds of back-to-back probe launches
+            while True:
+                tf, mhz = ops.mfma_probe(from_lds, device=device)
+                if time.perf_counter() >= until:
+                    break
+        probe[name] = {"tflops": tf, "clock_mhz": mhz, "frac_of_peak": tf / MFMA_BF16_PEAK_TFLOPS,
+                       "telemetry": tele.summary()}
     H, I, Is, K, E = shape["hidden"], shape["inter"], shape["shared_inter"], shape["top_k"], shape["num_experts"]
     flops_layer = 2.0 * tokens * K * 3 * H * I + 2.0 * tokens * 3 * H * Is + 2.0 * tokens * H * E
     gu_ms, gu_n, gu_name = stats["prefill_gateup"]
@@ -217,6 +357,7 @@ def prefill_workload(shape, tokens, steps, warmup, dtype, device):
         # busy compute units' average shader clock during the FFN launches, and the fraction of the
         # MFMA rate that clock allows (the published peak assumes MFMA_PEAK_CLOCK_MHZ)
         ffn_shader_clock_mhz=clock_mhz,
+        telemetry=telemetry,
         mfma_frac_at_clock=(flops_layer * len(blocks) / (ms_per_step / 1e3) / 1e12
                             / (MFMA_BF16_PEAK_TFLOPS * clock_mhz / MFMA_PEAK_CLOCK_MHZ)) if clock_mhz else None,
         # a loop of the same MFMAs on the same wavefront tile and nothing else (sparse_hip_mfma_probe)
@@ -327,6 +468,41 @@ def offload_report(metrics, blocks, wall, n_steps, tokens_per_step, resident_ms)
     )
 
 
+class PolicyCallLog:
+    """Records the calls a stack's blocks make into their residency policy (prefetch budget, plan, execute),
+    in order, with the phase / call id / stage each was made under, so that the same run can be replayed
+    through the CPU oracle of the policy afterwards.  A check beside the measurement, not part of it: the
+    wrappers append to a list and call through."""
+
+    NAMES = ("prefetch_budget", "schedule_prefetch", "execute")
+
+    def __init__(self, blocks):
+        self.calls = []
+        for blk in blocks:
+            res = blk.residency
+            for name in self.NAMES:
+                setattr(res, name, self._wrap(res, name, getattr(res, name)))
+
+    def _wrap(self, res, name, inner):
+        def call(*args):
+            self.calls.append((res.layer_idx, name, tuple(list(a) if isinstance(a, list) else a for a in args),
+                               (res.phase, res.call_id, getattr(res, "stage", "decode"))))
+            return inner(*args)
+        return call
+
+    def oracle_misses(self, cfg, num_layers, num_experts, top_k):
+        """Demand misses the oracle's state machine counts when fed the recorded calls (every copy taken
+        as complete when asked: which copies are late changes waits, not residency, without EPIPE)."""
+        from oracle.ref_layer import RefConfig, RefLayer
+        ref_cfg = RefConfig(**{n: getattr(cfg, n) for n in vars(RefConfig()) if hasattr(cfg, n)})
+        layers = [RefLayer(l, num_experts, top_k, ref_cfg) for l in range(num_layers)]
+        for layer, name, args, (phase, call_id, stage) in self.calls:
+            lay = layers[layer]
+            lay.phase, lay.call_id, lay.stage = phase, call_id, stage
+            getattr(lay, name)(*args)
+        return sum(1 for lay in layers for t in lay.trace if t[0] == "miss")
+
+
 def cached_decode_workload(dtype, device, steps, batch=8, capacity=15, top_m=8, short_steps=None, variants=None):
     """BASELINE configs[3]: Qwen shape, HBM cache of 25 % of each layer's experts, the rest in
     pinned host memory, skewed co-activating routing, rr vs rs (random-init predictor, as the
@@ -385,10 +561,19 @@ def cached_decode_workload(dtype, device, steps, batch=8, capacity=15, top_m=8, 
             engine.prepare({b.layer_idx: b for b in blocks}, SparseContext.rs_bank, batch=batch, dtype=dtype)
             engine.install()
             engine.begin(name)
+        # the two methods the configuration names also record their policy calls, replayed through the CPU
+        # oracle after the timed region: its miss count for the same routing goes beside the product's
+        log = PolicyCallLog(blocks) if name in ("rr", "rs_random_init") else None
         wall = run_phase_steps(blocks, inputs[:n_steps], "decode")   # cold cache, all steps timed
         out[name] = offload_report(metrics, blocks, wall, n_steps, batch, resident_ms)
         out[name]["steps"] = n_steps
         out[name]["shortened"] = n_steps < 512
+        if log is not None:
+            out[name]["oracle_misses"] = log.oracle_misses(blocks[0].residency.cfg, len(blocks),
+                                                           shape["num_experts"], shape["top_k"])
+            print(f"[bench] cached decode: {name}: misses {out[name]['misses']}, oracle on the same routing "
+                  f"{out[name]['oracle_misses']}", file=sys.stderr, flush=True)
+            del log
         if policies:
             out[name]["policy"] = {k: sum(p.stats[k] for p in policies)
                                    for k in ("prefetch_calls", "candidate_scores", "feedback_updates",
@@ -575,7 +760,21 @@ def compact_prefill(r):
             "gateup_us_per_layer_call": r["gateup"]["us_per_layer_call"], "gateup_mfma_frac": r["gateup"]["mfma_frac"],
             "down_us_per_layer_call": r["down"]["us_per_layer_call"], "down_mfma_frac": r["down"]["mfma_frac"],
             "ffn_shader_clock_mhz": r["ffn_shader_clock_mhz"], "mfma_frac_at_clock": r["mfma_frac_at_clock"],
-            "mfma_probe_lds_fragments_frac": r["mfma_probe"]["lds_fragments"]["frac_of_peak"]}
+            "mfma_probe_lds_fragments_frac": r["mfma_probe"]["lds_fragments"]["frac_of_peak"],
+            # socket power / shader clock the driver reported during a pass of the same steps, and during
+            # the probe loop (None where the box exposes neither sysfs files nor amd-smi to this user)
+            "telemetry": _compact_telemetry(r.get("telemetry")),
+            "mfma_probe_telemetry": _compact_telemetry(r["mfma_probe"]["lds_fragments"].get("telemetry"))}
+
+
+def _compact_telemetry(t):
+    if not t or not t.get("available"):
+        return {"available": False, "note": (t or {}).get("note")}
+    p, c = t.get("power_w") or {}, t.get("sclk_mhz") or {}
+    return {"available": True, "power_source": t["power_source"], "clock_source": t["clock_source"],
+            "power_samples": p.get("samples"), "power_w_mean": p.get("mean"), "power_w_max": p.get("max"),
+            "power_cap_w": t.get("power_cap_w"), "sclk_samples": c.get("samples"), "sclk_mhz_mean": c.get("mean"),
+            "sclk_mhz_min": c.get("min"), "sclk_mhz_max": c.get("max")}
 
 
 def main():
@@ -675,6 +874,13 @@ def main():
             except Exception as exc:  # noqa: BLE001
                 cpu[key] = {"error": repr(exc)[:300]}
 
+    if cpu is not None and isinstance(extra.get("cached_decode_qwen"), dict):
+        # the residency policy's CPU oracle replayed on the routing of the two methods the configuration
+        # names: its demand-miss count beside the product's
+        cpu["policy_oracle"] = {name: {"misses": leg.get("misses"), "oracle_misses": leg.get("oracle_misses"),
+                                       "steps": leg.get("steps")}
+                                for name, leg in extra["cached_decode_qwen"].items()
+                                if isinstance(leg, dict) and "oracle_misses" in leg}
     gu = main_res["gateup"]
     ratio = measured_traffic_ratio()
     line = {

@@ -55,3 +55,23 @@ def test_struct_layouts_match_the_header():
     # sparse_hip_experts: ptr, u64, ptr, 4 x i32 ; sparse_hip_seglist: 2 ptr, i32, 256 x i16
     assert ctypes.sizeof(_lib.Experts) == 8 + 8 + 8 + 16
     assert ctypes.sizeof(_lib.SegList) == 8 + 8 + 4 + 2 * 256 + 2 * 256 + 4  # tail padding to 8
+
+
+def test_documented_ctypes_binding_is_current():
+    """The binding shown to the reference's maintainers compiles as Python, names the library's current ABI
+    version and calls only symbols the header declares (the GPU suite executes it)."""
+    text = (ROOT / "INTEGRATION.md").read_text()
+    block = re.search(r"```python\n(.*?)```", text[text.index("## Seam 2"):], re.S).group(1)
+    compile(block, "INTEGRATION.md:seam-2", "exec")
+    assert f"sparse_hip_version() == {_lib.ABI_VERSION}" in block
+    assert f"ABI version {_lib.ABI_VERSION}" in text
+    header_text = HEADER.read_text()
+    assert f"#define SPARSE_HIP_ABI_VERSION {_lib.ABI_VERSION}" in header_text
+    used = set(re.findall(r"_lib\.(sparse_hip_[a-z0-9_]+)", block)) | set(re.findall(r'"(sparse_hip_[a-z0-9_]+)"', block))
+    assert used and used <= set(declared_symbols()), sorted(used - set(declared_symbols()))
+    # struct mirrors in the block have the library's layout
+    ns = {}
+    exec(re.search(r"class Experts.*?\n\n", block, re.S).group(0), {"C": ctypes}, ns)
+    exec(re.search(r"class SegList.*?\n\n", block, re.S).group(0), {"C": ctypes}, ns)
+    assert ctypes.sizeof(ns["Experts"]) == ctypes.sizeof(_lib.Experts)
+    assert ctypes.sizeof(ns["SegList"]) == ctypes.sizeof(_lib.SegList)
