@@ -173,11 +173,17 @@ class GpuTelemetry:
     process per sample (a few a second; it also gives the power where the sysfs file is missing), averaged
     over the XCDs.  What the box does not expose to this user is reported as missing, without figures."""
 
+    enabled = True      # --no-telemetry: no sampling threads and no child processes (runs under a profiler)
+
     def __init__(self, device_index=0, period=0.01):
         import glob
         self.period, self.power, self.clock, self.note = period, [], [], None
         self._stop, self._threads = None, []
         self.hwmon = None
+        if not GpuTelemetry.enabled:
+            self.note = "switched off (--no-telemetry)"
+            self.power_file = self.freq_file = self.smi = self.cap_w = None
+            return
         want = None
         try:
             p = torch.cuda.get_device_properties(device_index)
@@ -247,6 +253,8 @@ class GpuTelemetry:
 
     def __enter__(self):
         import threading
+        if self.note:
+            return self
         self._stop = threading.Event()
 
         def sysfs_loop():
@@ -750,6 +758,37 @@ def cpu_baseline_config1(shape, device, budget_s=6.0):
                        f"{n1} in {dt1:.1f} s on 1 thread (BASELINE configs[0])")
 
 
+def library_gemms(device, dtype=torch.bfloat16, runs=20):
+    """Plain GEMMs of the vendor library through torch at the prefill workload's shapes (no gather, no
+    SwiGLU epilogue, no routing weights): a reference point for the grouped kernels' launch times, not
+    part of any step."""
+    cases = (("dense [4096x2048]x[2048x5632] (shared gate+up as one GEMM)", None, 4096, 2048, 5632),
+             ("dense [4096x2816]x[2816x2048] (shared down)", None, 4096, 2816, 2048),
+             ("bmm 64x[384x2048]x[2048x2816] (routed gate+up, even segments)", 64, 384, 2048, 2816),
+             ("bmm 64x[384x1408]x[1408x2048] (routed down, even segments)", 64, 384, 1408, 2048),
+             ("dense 8192^3", None, 8192, 8192, 8192))
+    out = []
+    for name, batch, m, k, n in cases:
+        lead = (batch,) if batch else ()
+        a = torch.randn(*lead, m, k, device=device, dtype=torch.float32).to(dtype)
+        b = torch.randn(*lead, k, n, device=device, dtype=torch.float32).to(dtype)
+        for _ in range(3):
+            torch.matmul(a, b)
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        start.record()
+        for _ in range(runs):
+            torch.matmul(a, b)
+        stop.record()
+        torch.cuda.synchronize()
+        us = start.elapsed_time(stop) * 1e3 / runs
+        flops = 2.0 * (batch or 1) * m * k * n
+        out.append({"gemm": name, "us": us, "tflops": flops / us / 1e6,
+                    "frac_of_peak": flops / us / 1e6 / MFMA_BF16_PEAK_TFLOPS})
+        del a, b
+    return out
+
+
 def compact_prefill(r):
     """The handful of prefill figures that travel inside ``roofline``."""
     if not r:
@@ -789,6 +828,10 @@ def main():
     ap.add_argument("--only-prefill", action="store_true", help="run just the prefill workload (for profiling)")
     ap.add_argument("--only-decode", type=int, default=0, metavar="BATCH",
                     help="run just the all-resident decode workload at this batch size (for profiling)")
+    ap.add_argument("--no-telemetry", action="store_true",
+                    help="do not sample power and clock (no sampling threads, no amd-smi child processes)")
+    ap.add_argument("--library-gemms", action="store_true",
+                    help="time plain vendor-library GEMMs at the prefill shapes (a reference point) and exit")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also launch a 256 MiB plain copy kernel a few times (yardstick for --pmc byte counters)")
     ap.add_argument("--cached-decode", type=int, default=0, metavar="STEPS",
@@ -808,6 +851,10 @@ def main():
     device = torch.device("cuda:0")
     dtype = torch.bfloat16
 
+    GpuTelemetry.enabled = not args.no_telemetry
+    if args.library_gemms:
+        print(json.dumps({"library_gemms": library_gemms(device)}))
+        return
     if args.only_prefill:
         print(json.dumps(prefill_workload(DEEPSEEK, 4096, max(2, args.steps), args.warmup, dtype, device)))
         return

@@ -8,7 +8,23 @@
 
 #include "sparse_hip.h"
 
+// The kernels here are written for one target.  Two things in them are outside what the language
+// guarantees and hold on gfx950 (and its gfx9 family) only: the raw `s_waitcnt` immediates below use the
+// gfx9 encoding (vmcnt in bits 3:0 and 15:14, expcnt 6:4, lgkmcnt 11:8), and the hand-off between
+// workgroups in the decode kernel relies on device-scope (sc1) stores being written through to memory
+// and acknowledged only then.  Compiling the device code for anything else must fail here.
+#if defined(__HIP_DEVICE_COMPILE__) && !defined(__gfx950__)
+#error "libsparse_hip's kernels are gfx950 code: s_waitcnt immediates and the sc1 write-through hand-off assume it"
+#endif
+
 namespace sparse {
+
+// s_waitcnt immediates, gfx9 encoding, expcnt and lgkmcnt left at "do not wait" (7 and 15).
+constexpr int kWaitVmcnt0 = 0x0F70;    // vmcnt(0)
+constexpr int kWaitVmcnt20 = 0x4F74;   // vmcnt(20): 20 = 0b01'0100 -> bits 15:14 = 01, bits 3:0 = 0100
+static_assert((kWaitVmcnt0 & 0xC00F) == 0 && (kWaitVmcnt0 & 0x0F70) == 0x0F70, "vmcnt(0), nothing else waited for");
+static_assert((((kWaitVmcnt20 >> 14) & 3) << 4 | (kWaitVmcnt20 & 15)) == 20 && (kWaitVmcnt20 & 0x0F70) == 0x0F70,
+              "vmcnt(20), nothing else waited for");
 
 // ---- error plumbing ---------------------------------------------------------
 void set_error(const char* fmt, ...);

@@ -365,7 +365,7 @@ __global__ __launch_bounds__(kDecThreads) void decode_ffn_kernel(const DecodeArg
     int32_t pos[SPARSE_HIP_MAX_TOPK];
 #pragma unroll
     for (int k = 0; k < SPARSE_HIP_MAX_TOPK; ++k) pos[k] = (k < K && t < Ttok) ? a.inv_perm[t * K + k] : 0x7fffffff;
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wavefront's stores have been acknowledged
+    __builtin_amdgcn_s_waitcnt(kWaitVmcnt0);  // this wavefront's stores have been acknowledged
     __syncthreads();
     const int tile = row0 / kDecRows;
     if (threadIdx.x == 0) {

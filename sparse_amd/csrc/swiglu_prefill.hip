@@ -250,7 +250,7 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_ffn_kernel(const Prefil
     // scheduling fences keep exactly that order (copies, half 0, half 1 in every slab).  Slabs past the end refetch the last one
     // instead of branching.
     // s_waitcnt vmcnt(n), other counters untouched
-    constexpr int kWaitVm0 = 0x0F70, kWaitVm20 = kDrainWaits ? kWaitVm0 : 0x4F74;
+    constexpr int kWaitVm0 = kWaitVmcnt0, kWaitVm20 = kDrainWaits ? kWaitVmcnt0 : kWaitVmcnt20;
     const int nk = Kdim / kPfBK;
     bf16x8 wfrag[2][2][4];   // [stage][k half][16-row group]
     stage_slab(0, 0);

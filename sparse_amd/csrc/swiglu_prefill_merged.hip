@@ -75,7 +75,7 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_merged_kernel(const Pfx
   const int xcd = blockIdx.x % kPfXcds;
 
   // s_waitcnt vmcnt(n), other counters untouched
-  constexpr int kWaitVm0 = 0x0F70, kWaitVm20 = kDrainWaits ? kWaitVm0 : 0x4F74;
+  constexpr int kWaitVm0 = kWaitVmcnt0, kWaitVm20 = kDrainWaits ? kWaitVmcnt0 : kWaitVmcnt20;
   const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
       (__attribute__((address_space(3))) uint8_t*)(&lds[0][0])));
 

@@ -348,6 +348,29 @@ def test_combine_folded_into_the_down_projection_gives_the_same_bits(device, sha
     assert int(ws.split_ws[off:].view(torch.int32).abs().sum().item()) == 0
 
 
+def test_folded_combine_soak_at_the_decode_shape(device):
+    """The hand-off inside the down projection's launch (write-through stores, a full wait, a counter) is
+    ordered by the hardware's behaviour rather than by fences, so it gets a longer run than the other
+    bit-equality tests: 500 calls at the Qwen shape over batch 1, 8 and 16, each on new inputs with routing
+    of its own, the folded launch against the separate combine, stopping at the first difference."""
+    from sparse_amd.synthetic import QWEN, make_hidden
+    _mlp, blk = _build(QWEN, torch.bfloat16, device, seed=9)
+    H = QWEN["hidden"]
+    calls = 0
+    for T, n in ((1, 170), (8, 170), (16, 160)):
+        rows = make_hidden(T * n, H, torch.bfloat16, seed=7000 + T).to(device).view(n, T, 1, H)
+        for i in range(n):
+            blk.fold_combine = True
+            got, _ = blk(rows[i])
+            got = got.clone()
+            blk.fold_combine = False
+            want, _ = blk(rows[i])
+            # one comparison per call, on the device: the host only learns whether to stop
+            assert torch.equal(got, want), f"batch {T}, call {i}: folded combine differs from the separate launch"
+            calls += 1
+    assert calls == 500
+
+
 @pytest.mark.parametrize("T", [8, 300])
 def test_segment_timing_counters(device, monkeypatch, T):
     """``SPARSE_EXPERT_TIMING=1`` (utils/eval_core.py:14655-14676): router, routed experts and
