@@ -328,17 +328,20 @@ def prefill_workload(shape, tokens, steps, warmup, dtype, device):
         blk.merged_prefill = merged
     # socket power and shader clock as the driver reports them, sampled from a host thread during a pass
     # of its own (at least about a second of steps), so that the sampling cannot touch the timed figure
-    tele_steps = max(steps, int(3.0 / max(wall / steps, 1e-4)))
-    with GpuTelemetry() as tele:
-        wall_tele = time_steps(blocks, inputs, 0, tele_steps, use_graph=False)
-    telemetry = tele.summary()
-    telemetry["ms_per_step_while_sampling"] = wall_tele / tele_steps * 1e3
+    telemetry = GpuTelemetry().summary()
+    if GpuTelemetry.enabled:
+        tele_steps = max(steps, int(3.0 / max(wall / steps, 1e-4)))
+        with GpuTelemetry() as tele:
+            wall_tele = time_steps(blocks, inputs, 0, tele_steps, use_graph=False)
+        telemetry = tele.summary()
+        telemetry["ms_per_step_while_sampling"] = wall_tele / tele_steps * 1e3
     # what the matrix cores sustain on this box with nothing but the kernel's wavefront tile going on:
     # operands in registers, and with the activation fragments read from LDS every k step
     probe = {}
     for name, from_lds in (("registers", False), ("lds_fragments", True)):
         with GpuTelemetry() as tele:
-            until = time.perf_counter() + 2.0          # about two seconds of back-to-back probe launches
+            # about two seconds of back-to-back probe launches while the power and clock are sampled
+            until = time.perf_counter() + (2.0 if GpuTelemetry.enabled else 0.0)
             while True:
                 tf, mhz = ops.mfma_probe(from_lds, device=device)
                 if time.perf_counter() >= until:
@@ -758,6 +761,52 @@ def cpu_baseline_config1(shape, device, budget_s=6.0):
                        f"{n1} in {dt1:.1f} s on 1 thread (BASELINE configs[0])")
 
 
+def routing_launch_probe(dtype, device, batch=8, replays=50):
+    """The decode routing launch taken apart: the router's workgroup alone (every layer's own gate matrix, and
+    one gate matrix for all layers, i.e. cached), the shared expert's gate/up projections alone, and both in
+    one launch as the block runs them; each as a HIP graph over the stack's layers, microseconds per layer."""
+    from sparse_amd import ops
+    from sparse_amd.synthetic import QWEN
+    blocks = build_stack(QWEN, dtype, device)
+    x = make_inputs(QWEN, batch, 1, 1, dtype, device)[0].view(batch, -1).contiguous()
+    spaces = [b._workspace(batch) for b in blocks]
+    logits = torch.empty((batch, QWEN["num_experts"]), device=device, dtype=blocks[0].logits_dtype)
+
+    def router(blk, ws, shared_up=None):
+        ops.route_decode_packed(x, blk.gate_packed, blk.num_experts, blk.shared_gate_weight is not None, blk.top_k,
+                                blk.norm_topk_prob, logits, ws.shared_gate, ws.topv, ws.topi, ws.perm,
+                                shared_up=shared_up)
+
+    forms = {
+        "router_alone_us": lambda: [router(b, ws) for b, ws in zip(blocks, spaces)],
+        "router_alone_one_gate_matrix_us": lambda: [router(blocks[0], spaces[0]) for _ in blocks],
+        "shared_gate_up_alone_us": lambda: [ops.shared_gate_up(x, b.shared_weights[0], b.shared_weights[1],
+                                                               ws.shared_inter) for b, ws in zip(blocks, spaces)],
+        "router_and_shared_gate_up_us": lambda: [router(b, ws, (b.shared_weights[0], b.shared_weights[1],
+                                                                ws.shared_inter)) for b, ws in zip(blocks, spaces)],
+    }
+    out = {"batch": batch, "layers": len(blocks), "replays": replays}
+    for name, fn in forms.items():
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            fn()
+        for _ in range(3):
+            graph.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(replays):
+            graph.replay()
+        torch.cuda.synchronize()
+        out[name] = (time.perf_counter() - t0) / replays / len(blocks) * 1e6
+        del graph
+    del blocks
+    release_stack()
+    return out
+
+
 def library_gemms(device, dtype=torch.bfloat16, runs=20):
     """Plain GEMMs of the vendor library through torch at the prefill workload's shapes (no gather, no
     SwiGLU epilogue, no routing weights): a reference point for the grouped kernels' launch times, not
@@ -830,6 +879,8 @@ def main():
                     help="run just the all-resident decode workload at this batch size (for profiling)")
     ap.add_argument("--no-telemetry", action="store_true",
                     help="do not sample power and clock (no sampling threads, no amd-smi child processes)")
+    ap.add_argument("--routing-launch-probe", action="store_true",
+                    help="time the decode routing launch's parts (router alone, shared gate/up alone, both) and exit")
     ap.add_argument("--library-gemms", action="store_true",
                     help="time plain vendor-library GEMMs at the prefill shapes (a reference point) and exit")
     ap.add_argument("--calib-copy", action="store_true",
@@ -855,6 +906,17 @@ def main():
     if args.library_gemms:
         print(json.dumps({"library_gemms": library_gemms(device)}))
         return
+    if args.routing_launch_probe:
+        print(json.dumps({"routing_launch_probe": routing_launch_probe(dtype, device)}))
+        return
+    if args.calib_copy:
+        from sparse_amd import ops
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=device).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(4):
+            ops.calib_copy(src, dst)
+        torch.cuda.synchronize()
+        del src, dst
     if args.only_prefill:
         print(json.dumps(prefill_workload(DEEPSEEK, 4096, max(2, args.steps), args.warmup, dtype, device)))
         return
@@ -869,14 +931,6 @@ def main():
     if args.epipe_prefill:
         print(json.dumps({"epipe_prefill_deepseek": epipe_prefill_workload(dtype, device)}))
         return
-    if args.calib_copy:
-        from sparse_amd import ops
-        src = torch.empty(256 << 20, dtype=torch.uint8, device=device).fill_(1)
-        dst = torch.empty_like(src)
-        for _ in range(4):
-            ops.calib_copy(src, dst)
-        torch.cuda.synchronize()
-        del src, dst
     blocks = build_stack(QWEN, dtype, device)
     main_res = decode_workload(blocks, QWEN, 8, args.steps, args.warmup, dtype, device, not args.no_graph)
     extra = {}
