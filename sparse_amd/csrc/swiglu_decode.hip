@@ -258,6 +258,17 @@ __global__ __launch_bounds__(kDecThreads) void decode_ffn_kernel(const DecodeArg
 #undef SP_DEC_MFMA
 #undef SP_DEC_LOAD
 
+  // A launch that also combines: where each token's K routed rows lie is asked for now, so that the answer
+  // is there long before the hand-off needs it (thread -> (token, four columns) of the 32-column tile).
+  constexpr int kPerTok = kDecRows / 4;   // threads per token in the combine: four columns each
+  const int ct = threadIdx.x / kPerTok, cc4 = (threadIdx.x % kPerTok) * 4;
+  int32_t pos[SPARSE_HIP_MAX_TOPK];
+  if (!kGateUp && a.tile_counters != nullptr) {
+#pragma unroll
+    for (int k = 0; k < SPARSE_HIP_MAX_TOPK; ++k)
+      pos[k] = (k < a.topk && ct < a.T) ? a.inv_perm[ct * a.topk + k] : 0x7fffffff;
+  }
+
   // ---- split-K partials meet in LDS ----------------------------------------
   constexpr int NFRAG = kDecTiles * NT;
   __shared__ f32x4 red[kDecWaves][NFRAG * NM][64];
@@ -357,26 +368,14 @@ __global__ __launch_bounds__(kDecThreads) void decode_ffn_kernel(const DecodeArg
     __shared__ int s_last;
     // thread -> (token, four columns); the arithmetic is that of the stand-alone combine step:
     // K ordered adds rounded to bf16, then the shared expert finished from its parts.  Where the
-    // token's rows lie is read before the hand-off, so that the last workgroup's reads of them
-    // do not wait for it.
+    // token's rows lie was asked for before the reduction.
     const int Ttok = a.T, K = a.topk, H = a.Ndim_s;
-    constexpr int kPerTok = kDecRows / 4;   // threads per token: four columns each
-    const int t = threadIdx.x / kPerTok, c4 = (threadIdx.x % kPerTok) * 4;
-    int32_t pos[SPARSE_HIP_MAX_TOPK];
-#pragma unroll
-    for (int k = 0; k < SPARSE_HIP_MAX_TOPK; ++k) pos[k] = (k < K && t < Ttok) ? a.inv_perm[t * K + k] : 0x7fffffff;
-    __builtin_amdgcn_s_waitcnt(kWaitVmcnt0);  // this wavefront's stores have been acknowledged
-    __syncthreads();
-    const int tile = row0 / kDecRows;
-    if (threadIdx.x == 0) {
-      const int nseg = (a.segs.eids_dev != nullptr) ? min(a.segs.count_dev[0], a.segs.n) : a.segs.n;
-      const int prev = __hip_atomic_fetch_add(a.tile_counters + tile, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      s_last = (prev == nseg + split - 1);
-      if (s_last) __hip_atomic_store(a.tile_counters + tile, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    __syncthreads();
-    if (!s_last) return;
-    if (t >= Ttok) return;
+    const int t = ct, c4 = cc4;
+    // how many workgroups this tile has: read now, not between the barrier and the counter
+    const int arrivals = ((a.segs.eids_dev != nullptr) ? min(a.segs.count_dev[0], a.segs.n) : a.segs.n) + split;
+    // ascending row position = ascending expert id: the order of the stand-alone combine's adds.  Sorted
+    // here, while this wavefront's stores are still on their way, by every workgroup: the one that turns out
+    // to be last then has nothing left to do between the counter and its reads.
 #pragma unroll
     for (int i = 1; i < SPARSE_HIP_MAX_TOPK; ++i) {
 #pragma unroll
@@ -386,33 +385,67 @@ __global__ __launch_bounds__(kDecThreads) void decode_ffn_kernel(const DecodeArg
         pos[j] = hi;
       }
     }
-    const int h = row0 + c4;
-    float accv[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int k = 0; k < SPARSE_HIP_MAX_TOPK; ++k) {
-      if (k < K) {
-        const uint64_t v = ld_device_u64(a.out_r + static_cast<size_t>(pos[k]) * H + h);
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-          accv[j] = F::round(accv[j] + F::from_bits(static_cast<uint16_t>(v >> (16 * j))));
-      }
+    __builtin_amdgcn_s_waitcnt(kWaitVmcnt0);  // this wavefront's stores have been acknowledged
+    __syncthreads();
+    const int tile = row0 / kDecRows;
+    if (threadIdx.x == 0) {
+      const int prev = __hip_atomic_fetch_add(a.tile_counters + tile, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      s_last = (prev == arrivals - 1);
+      if (s_last) __hip_atomic_store(a.tile_counters + tile, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
+    __syncthreads();
+    if (!s_last) return;
+    if (t >= Ttok) return;
+    const int h = row0 + c4;
+    // Every read is requested before the first one is consumed: the loads are ordered atomics, which the
+    // compiler neither hoists nor overlaps with the additions that use them, so written row by row each
+    // would cost its own trip to memory.  Rows past K and parts past `split` repeat the first address and
+    // are not used.
     const size_t part_stride = static_cast<size_t>(Ttok) * H;
     const float* src = a.split_sums + static_cast<size_t>(t) * H + h;
-    float sh[4];
-    {
-      const uint64_t lo = ld_device_u64(src), hi = ld_device_u64(src + 2);
-      sh[0] = __uint_as_float(static_cast<uint32_t>(lo));
-      sh[1] = __uint_as_float(static_cast<uint32_t>(lo >> 32));
-      sh[2] = __uint_as_float(static_cast<uint32_t>(hi));
-      sh[3] = __uint_as_float(static_cast<uint32_t>(hi >> 32));
+    uint64_t part_lo[kDecSplit], part_hi[kDecSplit];
+#pragma unroll
+    for (int p = 0; p < kDecSplit; ++p) {
+      const float* s = src + static_cast<size_t>(p < split ? p : 0) * part_stride;
+      part_lo[p] = ld_device_u64(s);
+      part_hi[p] = ld_device_u64(s + 2);
     }
-    for (int p = 1; p < split; ++p) {
-      const uint64_t lo = ld_device_u64(src + p * part_stride), hi = ld_device_u64(src + p * part_stride + 2);
-      sh[0] += __uint_as_float(static_cast<uint32_t>(lo));
-      sh[1] += __uint_as_float(static_cast<uint32_t>(lo >> 32));
-      sh[2] += __uint_as_float(static_cast<uint32_t>(hi));
-      sh[3] += __uint_as_float(static_cast<uint32_t>(hi >> 32));
+    constexpr int kRowGroup = 8;
+    static_assert(SPARSE_HIP_MAX_TOPK % kRowGroup == 0, "row groups must cover the top-k limit");
+    float accv[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int g = 0; g < SPARSE_HIP_MAX_TOPK; g += kRowGroup) {
+      if (g == 0 || g < K) {          // uniform: K is a launch argument
+        uint64_t v[kRowGroup];
+#pragma unroll
+        for (int i = 0; i < kRowGroup; ++i) {
+          const int32_t p = (g + i < K) ? pos[g + i] : pos[0];
+          v[i] = ld_device_u64(a.out_r + static_cast<size_t>(p) * H + h);
+        }
+#pragma unroll
+        for (int i = 0; i < kRowGroup; ++i) {
+          if (g + i < K) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+              accv[j] = F::round(accv[j] + F::from_bits(static_cast<uint16_t>(v[i] >> (16 * j))));
+          }
+        }
+      }
+    }
+    float sh[4];
+#pragma unroll
+    for (int p = 0; p < kDecSplit; ++p) {
+      if (p < split) {
+        const float f0 = __uint_as_float(static_cast<uint32_t>(part_lo[p]));
+        const float f1 = __uint_as_float(static_cast<uint32_t>(part_lo[p] >> 32));
+        const float f2 = __uint_as_float(static_cast<uint32_t>(part_hi[p]));
+        const float f3 = __uint_as_float(static_cast<uint32_t>(part_hi[p] >> 32));
+        if (p == 0) {
+          sh[0] = f0; sh[1] = f1; sh[2] = f2; sh[3] = f3;
+        } else {
+          sh[0] += f0; sh[1] += f1; sh[2] += f2; sh[3] += f3;
+        }
+      }
     }
     const bool gated = a.gate_s != nullptr;
     const float scale = gated ? F::round(sigmoid_f32(F::from_bits(a.gate_s[t]))) : 1.f;
