@@ -403,10 +403,29 @@ __global__ __launch_bounds__(256) void prefill_queue_kernel(const PfxMapArgs a) 
   const int nt = which == 0 ? a.nt_gu : a.nt_dn;
   const int cap = which == 0 ? a.cap_gu : a.cap_dn;
   const int R = total_mt * nt, S = a.mt_shared * (which == 0 ? a.nts_gu : a.nts_dn);
+  // The shared expert's tiles.  Where the tile grid divides evenly, XCD x takes a block of it -- a quarter
+  // of the row tiles by half of the column tiles -- and walks the block down its rows first, so that the
+  // 64 workgroups an XCD runs at a time cover about 8 x 8 tiles: each activation row tile and each weight
+  // tile is then fetched into that L2 once per 8 users.  (Column by column over all row tiles, an XCD reads
+  // the whole activation matrix, four times its L2, once per column tile.)  Otherwise: contiguous shares
+  // of the (column tile, row tile) order.
+  const int nts = which == 0 ? a.nts_gu : a.nts_dn;
+  const bool blocked = a.mt_shared % 4 == 0 && nts % 2 == 0 && nts > 0;
+  const int RG = a.mt_shared / 4, per_xcd = S / kPfXcds;
   for (int h = tid; h < S; h += 256) {
-    const int bn = h / a.mt_shared, bm = h - bn * a.mt_shared;
-    const int x = pfx_share_of(S, h);
-    const int pos = pfx_queue_base(R, S, x) + (h - pfx_start(S, x));
+    int bn, bm, x, local;
+    if (blocked) {
+      x = h / per_xcd;
+      local = h - x * per_xcd;
+      bm = (x & 3) * RG + local % RG;
+      bn = (x >> 2) * (nts / 2) + local / RG;
+    } else {
+      bn = h / a.mt_shared;
+      bm = h - bn * a.mt_shared;
+      x = pfx_share_of(S, h);
+      local = h - pfx_start(S, x);
+    }
+    const int pos = pfx_queue_base(R, S, x) + local;
     if (pos < cap) map[pos] = PfTile{-1, bm * kPfBM, min(kPfBM, a.T - bm * kPfBM), bn};
   }
   if (tid == 0) map[0] = PfTile{0, 0, 0, 0};
