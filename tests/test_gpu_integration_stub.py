@@ -1,7 +1,8 @@
 """The ctypes binding a maintainer of the reference would add at its patch point
 (utils/rs_overlap.py:438-441), executed as it is written: the first Python code block under the
-"Seam 2" heading of INTEGRATION.md is extracted, run against the built library, and its two functions
-are compared with the CPU oracle on a small layer whose sizes are multiples of 64."""
+"Seam 2" heading of the integration guide at the repository root is extracted, run against the built
+library, and its two functions are compared with the CPU oracle on a small layer whose sizes are
+multiples of 64."""
 import os
 import re
 

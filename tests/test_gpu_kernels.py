@@ -367,7 +367,8 @@ def test_pack_router_gate_declines_what_does_not_fit():
 
 # ------------------------------------------------------------------ permute
 @pytest.mark.parametrize("T,E,K", [(1, 60, 4), (8, 60, 4), (32, 60, 4), (255, 64, 6), (256, 64, 6),
-                                    (257, 64, 6), (2048, 64, 6), (4096, 64, 6), (1000, 256, 16), (3, 4, 4)])
+                                    (257, 64, 6), (2048, 64, 6), (4096, 64, 6), (1000, 256, 16), (3, 4, 4),
+                                    (10923, 64, 6), (16384, 60, 4), (20000, 64, 6)])
 def test_permute_build_bit_exact(device, T, E, K):
     ops = _ops()
     g = torch.Generator().manual_seed(T * 7 + E)

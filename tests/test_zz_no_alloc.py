@@ -52,7 +52,8 @@ def _both(lib, topi, E, first_call=False):
 @pytest.mark.parametrize("E,K", [(64, 6), (60, 4)])
 def test_static_scratch_permute_equals_workspace_permute(device, E, K):
     lib = _lib.load()
-    for n, (T, seed) in enumerate(((4096, 1), (700, 2), (9, 3))):  # large, smaller (several blocks), one block
+    # large, then smaller ones (several blocks each), then one block
+    for n, (T, seed) in enumerate(((20000, 1), (4096, 4), (700, 2), (9, 3))):
         topi = _topi(T, K, E, seed, device)
         want, got = _both(lib, topi, E, first_call=(n == 0))
         n_act = int(want[4].item())
