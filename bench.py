@@ -71,6 +71,9 @@ def make_inputs(shape, batch, seq, n, dtype, device):
             for i in range(n)]
 
 
+SETTLE_SECONDS = 0.25
+
+
 def time_steps(blocks, inputs, warmup, steps, use_graph):
     """Wall time of exactly ``steps`` steps, inputs already on the device."""
     static_in = inputs[0].clone()
@@ -93,6 +96,16 @@ def time_steps(blocks, inputs, warmup, steps, use_graph):
         else:
             stack_step(blocks, static_in)
 
+    # Before the warm-up steps proper the device is brought out of its idle power state: untimed steps for a
+    # quarter of a second (the clocks of an idle part take tens of milliseconds to settle, more than a handful
+    # of 2 ms warm-up steps lasts; a 20-step measurement started cold reads 1-3 % slow and varies run to run).
+    settle_until = time.perf_counter() + SETTLE_SECONDS
+    n_settle = 0
+    while time.perf_counter() < settle_until and n_settle < 2000:
+        one(n_settle)
+        n_settle += 1
+        if n_settle % 8 == 0:
+            torch.cuda.synchronize()
     for i in range(warmup):
         one(i)
     torch.cuda.synchronize()
@@ -103,9 +116,10 @@ def time_steps(blocks, inputs, warmup, steps, use_graph):
     return time.perf_counter() - t0
 
 
-def instrumented_pass(blocks, inputs, steps):
+def instrumented_pass(blocks, inputs, steps, per_step=False):
     """Eager pass with HIP events around every kernel launch; also counts the distinct
-    routed experts of every layer call.  Returns (per-kernel stats, mean distinct experts)."""
+    routed experts of every layer call.  Returns (per-kernel stats, mean distinct experts), and with
+    ``per_step`` also the mean over the layers for each step."""
     from sparse_amd import ops
     ops.profile_reset()
     ops.profile_enable(True)
@@ -122,13 +136,24 @@ def instrumented_pass(blocks, inputs, steps):
     finally:
         ops.profile_enable(False)
         ops.profile_reset()
-    return stats, sum(distinct) / max(1, len(distinct))
+    mean = sum(distinct) / max(1, len(distinct))
+    if not per_step:
+        return stats, mean
+    n = len(blocks)
+    return stats, mean, [sum(distinct[i * n:(i + 1) * n]) / n for i in range(steps)]
 
 
 def decode_workload(blocks, shape, batch, steps, warmup, dtype, device, use_graph=True):
     inputs = make_inputs(shape, batch, 1, max(8, min(64, warmup + steps)), dtype, device)
     wall = time_steps(blocks, inputs, warmup, steps, use_graph)
-    stats, mean_u = instrumented_pass(blocks, inputs, min(steps, 16))
+    # per-kernel times and the number of distinct routed experts, on the very inputs the timed steps ran
+    # (the algorithmic bytes of a step depend on how many experts its tokens hit): timed step i read input
+    # (warmup + i) mod len(inputs), so every input is instrumented once and weighted by how often it was timed
+    used = [(warmup + i) % len(inputs) for i in range(steps)]
+    order = sorted(set(used))
+    stats, _mean, per_input = instrumented_pass(blocks, [inputs[j] for j in order], len(order), per_step=True)
+    weight = {j: used.count(j) for j in order}
+    mean_u = sum(per_input[n] * weight[j] for n, j in enumerate(order)) / len(used)
     H, I, Is, K = shape["hidden"], shape["inter"], shape["shared_inter"], shape["top_k"]
     es = 2
     from sparse_amd import ops
@@ -948,7 +973,7 @@ def main():
     if not args.no_extra:
         # the same stack and step in fp16, the dtype of the reference's formal runs
         blocks16 = build_stack(QWEN, torch.float16, device)
-        extra["decode_b8_fp16"] = decode_workload(blocks16, QWEN, 8, max(10, args.steps // 2), args.warmup,
+        extra["decode_b8_fp16"] = decode_workload(blocks16, QWEN, 8, max(20, args.steps // 2), args.warmup,
                                                   torch.float16, device, not args.no_graph)
         del blocks16
         _Workspace._cache.clear()
