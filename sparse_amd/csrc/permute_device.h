@@ -47,10 +47,19 @@ __device__ __forceinline__ void permute_scatter_block(
 #pragma unroll
       for (int w = 0; w < kMaskWords; ++w) total += __popc(mask[tid][w]);
     } else {
-      for (int b = 0; b < num_blocks; ++b) {
-        const int32_t c = block_counts[static_cast<size_t>(b) * E + tid];
-        total += c;
-        if (b < block) before += c;
+      // eight histograms at a time: the loads do not depend on one another, and taken one by one each
+      // would cost its own trip to the L2
+      constexpr int kBatch = 8;
+      for (int b0 = 0; b0 < num_blocks; b0 += kBatch) {
+        int32_t c[kBatch];
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u)
+          c[u] = (b0 + u < num_blocks) ? block_counts[static_cast<size_t>(b0 + u) * E + tid] : 0;
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u) {
+          total += c[u];
+          if (b0 + u < block) before += c[u];
+        }
       }
     }
   }
